@@ -1,0 +1,77 @@
+"""Shared pytest plumbing: the ``gpu`` marker, import paths and small helpers."""
+import ctypes
+import importlib
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def pkg():
+    """The shipped package (directory ``co-rope_amd``; importable as ``corope_amd``)."""
+    return importlib.import_module("corope_amd")
+
+
+@pytest.fixture(scope="session")
+def brute():
+    """ctypes handle on oracle/libbrute_force.so (built on demand with gcc)."""
+    so = os.path.join(ROOT, "oracle", "libbrute_force.so")
+    if not os.path.exists(so):
+        subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle")])
+    lib = ctypes.CDLL(so)
+    dp = ctypes.POINTER(ctypes.c_double)
+    lib.bf_rope_attn_fwd.argtypes = [dp] * 5 + [ctypes.c_int] * 5 + [ctypes.c_double, dp, dp]
+    lib.bf_rope_attn_fwd.restype = ctypes.c_int
+    lib.bf_corope_gqa_fwd.argtypes = [dp] * 4 + [ctypes.c_int] * 5 + [ctypes.c_double, dp, dp]
+    lib.bf_corope_gqa_fwd.restype = ctypes.c_int
+
+    def ptr(a):
+        return a.ctypes.data_as(dp)
+
+    class Brute:
+        @staticmethod
+        def rope_attn(q, k, v, cos_half, sin_half, causal, sm_scale):
+            q, k, v, c, s = (np.ascontiguousarray(t, dtype=np.float64) for t in (q, k, v, cos_half, sin_half))
+            B, H, N, D = q.shape
+            o = np.empty_like(q)
+            lse = np.empty((B, H, N))
+            rc = lib.bf_rope_attn_fwd(ptr(q), ptr(k), ptr(v), ptr(c), ptr(s), B, H, N, D, int(causal),
+                                      float(sm_scale), ptr(o), ptr(lse))
+            assert rc == 0
+            return o, lse
+
+        @staticmethod
+        def corope(q, k, v, inv_freq, sm_scale, want_delta=False):
+            q, k, v, w = (np.ascontiguousarray(t, dtype=np.float64) for t in (q, k, v, inv_freq))
+            B, Hq, N, D = q.shape
+            Hkv = k.shape[1]
+            o = np.empty_like(q)
+            delta = np.zeros((B, Hkv, N, N)) if want_delta else None
+            rc = lib.bf_corope_gqa_fwd(ptr(q), ptr(k), ptr(v), ptr(w), B, Hq, Hkv, N, D, float(sm_scale),
+                                       ptr(o), ptr(delta) if want_delta else None)
+            assert rc == 0
+            return (o, delta) if want_delta else o
+
+    return Brute
+
+
+def seeded(shape, seed, dtype=torch.float32, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g, dtype=torch.float32) * std).to(dtype)
+
+
+def bf16_round(x):
+    """Round to bf16 and come back: the values the HIP kernels actually see."""
+    return x.to(torch.bfloat16).to(torch.float32)
