@@ -1,0 +1,78 @@
+"""ctypes binding of libcorope_amd.so (the gfx950 kernels behind a C ABI).
+
+The shared library is built in-tree by ``build.py``; nothing here falls back to another implementation: if
+the library is missing or a call fails, an exception is raised."""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libcorope_amd.so")
+ABI_VERSION = 1
+
+# status codes of include/corope_amd.h
+OK, E_BADARG, E_UNSUPPORTED, E_ALIGN, E_LAUNCH = 0, -1, -2, -3, -4
+
+_P, _I, _F, _L = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_int64
+
+#: name -> (restype, argtypes); every symbol include/corope_amd.h declares
+SIGNATURES = {
+    "corope_amd_version": (_I, []),
+    "corope_amd_last_error": (ctypes.c_char_p, []),
+    "corope_rope_attn_check": (_I, [_I, _I, _I, _I, _L, _F, _I]),
+    "corope_gqa_check": (_I, [_I, _I, _I, _I, _I, _F, _F]),
+    "corope_rope_attn_fwd": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
+    "corope_rope_attn_bwd_preprocess": (_I, [_P, _P, _P, _I, _I, _I, _I, _P]),
+    "corope_rope_attn_bwd_dkdv": (_I, [_P] * 8 + [_L, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
+    "corope_rope_attn_bwd_dq": (_I, [_P] * 8 + [_L, _P, _I, _I, _I, _I, _F, _I, _P]),
+    "corope_rope_attn_bwd": (_I, [_P] * 9 + [_L, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
+    "corope_gqa_fwd": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P]),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+class CoRopeLibraryError(RuntimeError):
+    """The native library is missing, stale, or a launch failed."""
+
+
+def load():
+    """Open the shared library once and type its entry points."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise CoRopeLibraryError(
+                f"{LIB_PATH} not found: build it with `python co-rope_amd/build.py` (needs hipcc); "
+                "there is no fallback implementation")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            try:
+                fn = getattr(lib, name)
+            except AttributeError as e:
+                raise CoRopeLibraryError(f"{LIB_PATH} does not export {name}; rebuild it") from e
+            fn.restype, fn.argtypes = res, args
+        if lib.corope_amd_version() != ABI_VERSION:
+            raise CoRopeLibraryError(f"{LIB_PATH} has ABI version {lib.corope_amd_version()}, expected {ABI_VERSION}")
+        _lib = lib
+    return _lib
+
+
+def last_error():
+    return load().corope_amd_last_error().decode("utf-8", "replace")
+
+
+def check(rc, what):
+    """Map a status code to the exception the reference's Python layer would raise for the same mistake."""
+    if rc == OK:
+        return
+    msg = f"{what}: {last_error()} (status {rc})"
+    if rc in (E_BADARG, E_UNSUPPORTED, E_ALIGN):
+        raise ValueError(msg)
+    raise CoRopeLibraryError(msg)

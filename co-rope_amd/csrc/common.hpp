@@ -1,0 +1,213 @@
+// Shared device helpers for the gfx950 kernels: vector types, bf16 packing, MFMA wrappers,
+// wave-half exchange and the global->register->LDS staging of rotated / transposed tiles.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace corope {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+constexpr int kWave = 64;
+
+// ---- bf16 <-> fp32 --------------------------------------------------------------------------
+// A 32-bit word holds two bf16: element 0 in the low half, element 1 in the high half.
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+// Round-to-nearest-even pack of two floats into one bf16x2 word (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  f32x2 v = {lo, hi};
+  bf16x2 r = __builtin_convertvector(v, bf16x2);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+// ---- MFMA ------------------------------------------------------------------------------------
+// D(32x32) += A(32x16) * B(16x32), bf16 in, fp32 accumulate.
+//   A operand: lane l holds row (l % 32), contraction slots 8*(l / 32) .. +7
+//   B operand: lane l holds column (l % 32), contraction slots 8*(l / 32) .. +7
+//   D/C      : lane l holds column (l % 32); register i holds row 8*(i / 4) + 4*(l / 32) + (i % 4)
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                 0, 0, 0);
+}
+
+// Row index (0..31) held by accumulator register i of lane-half h in a 32x32 MFMA result.
+__device__ __forceinline__ constexpr int acc_row(int i, int h) { return 8 * (i / 4) + 4 * h + (i % 4); }
+
+// ---- exchange between the two 32-lane halves of a wave ---------------------------------------------
+// Returns the value held by lane (l ^ 32).
+__device__ __forceinline__ float other_half(float x) {
+  uint32_t u = __builtin_bit_cast(uint32_t, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  // r[0] = {x.lo, x.lo}, r[1] = {x.hi, x.hi} over (lanes 0-31, lanes 32-63)
+  uint32_t mine_is_lo = (threadIdx.x & 32) == 0;
+  uint32_t o = mine_is_lo ? r[1] : r[0];
+  return __builtin_bit_cast(float, o);
+}
+__device__ __forceinline__ float half_max(float x) {
+  uint32_t u = __builtin_bit_cast(uint32_t, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+__device__ __forceinline__ float half_sum(float x) {
+  uint32_t u = __builtin_bit_cast(uint32_t, x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// ---- LDS tile layouts -----------------------------------------------------------------------------
+// Row-major tile [rows][D] of bf16 with 16 bytes of padding per row: 16 consecutive rows read at the
+// same column land in 16 different 16-byte bank groups.
+template <int D>
+struct RowTile {
+  static constexpr int kStride = D + 8;  // elements
+  static constexpr int bytes(int rows) { return rows * kStride * 2; }
+  __device__ static __forceinline__ int off(int row, int col) { return row * kStride + col; }
+};
+
+// Transposed tile [D][COLS] of bf16 (the contraction index runs along a row), 16 bytes of padding.
+// Within every group of 16 columns the order is permuted (bits 2 and 3 of the column index swapped) so
+// that the 8 contraction slots an MFMA B-operand built from a 32x32 accumulator expects from lane-half h,
+//   slot j  <->  column 8*(j / 4) + 4*h + (j % 4),
+// are the 8 consecutive elements [8h, 8h+8) of the group: one 16-byte LDS read per MFMA A operand.
+template <int COLS>
+struct TransTile {
+  static constexpr int kStride = COLS + 8;  // elements
+  static constexpr int bytes(int rows) { return rows * kStride * 2; }
+  __device__ static __forceinline__ int pos(int col) {
+    return (col & ~12) | ((col & 4) << 1) | ((col & 8) >> 1);
+  }
+  __device__ static __forceinline__ int off(int d, int col) { return d * kStride + pos(col); }
+};
+
+// ---- staging: a ROWS x D tile with the half-layout rotation applied on the way -----------------------
+// Work unit = one row x 8 rotation pairs: columns [8c, 8c+8) and [D/2 + 8c, D/2 + 8c + 8) of the same row
+// are loaded by the same thread, so the rotation is thread-local.  cos/sin come from fp32 tables of which
+// only the first D/2 columns are used.
+template <int D, int ROWS, int NT>
+struct RotStage {
+  static constexpr int kChunks = D / 16;              // units per row
+  static constexpr int kUnits = ROWS * kChunks;
+  static constexpr int kIters = (kUnits + NT - 1) / NT;
+  u32x4 x1[kIters], x2[kIters];
+  f32x4 c[kIters][2], s[kIters][2];
+
+  // src: first row of the (n, D) bf16 matrix; row0: first tile row; rows >= n_rows are clamped.
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float* __restrict__ cosp,
+                                       const float* __restrict__ sinp, int64_t fstride, int row0, int n_rows) {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      int u = threadIdx.x + it * NT;
+      if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
+      int r = u / kChunks, ch = u % kChunks;
+      int row = min(row0 + r, n_rows - 1);
+      const uint16_t* p = src + (int64_t)row * D + ch * 8;
+      x1[it] = *reinterpret_cast<const u32x4*>(p);
+      x2[it] = *reinterpret_cast<const u32x4*>(p + D / 2);
+      const float* cp = cosp + (int64_t)row * fstride + ch * 8;
+      const float* sp = sinp + (int64_t)row * fstride + ch * 8;
+      c[it][0] = *reinterpret_cast<const f32x4*>(cp);
+      c[it][1] = *reinterpret_cast<const f32x4*>(cp + 4);
+      s[it][0] = *reinterpret_cast<const f32x4*>(sp);
+      s[it][1] = *reinterpret_cast<const f32x4*>(sp + 4);
+    }
+  }
+
+  // Rotates unit `it`: y1 = x1 c - x2 s, y2 = x2 c + x1 s (fp32), rounds to bf16.
+  __device__ __forceinline__ void rotate(int it, u32x4& y1, u32x4& y2) const {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      float a0 = bf16_lo(x1[it][w]), a1 = bf16_hi(x1[it][w]);
+      float b0 = bf16_lo(x2[it][w]), b1 = bf16_hi(x2[it][w]);
+      float c0 = c[it][w / 2][(2 * w) % 4], c1 = c[it][w / 2][(2 * w) % 4 + 1];
+      float s0 = s[it][w / 2][(2 * w) % 4], s1 = s[it][w / 2][(2 * w) % 4 + 1];
+      y1[w] = pack_bf16(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+      y2[w] = pack_bf16(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+    }
+  }
+
+  // Row-major store of the rotated tile.
+  __device__ __forceinline__ void store_rows(uint16_t* lds) const {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      int u = threadIdx.x + it * NT;
+      if (kUnits % NT != 0 && u >= kUnits) continue;
+      int r = u / kChunks, ch = u % kChunks;
+      u32x4 y1, y2;
+      rotate(it, y1, y2);
+      *reinterpret_cast<u32x4*>(lds + RowTile<D>::off(r, ch * 8)) = y1;
+      *reinterpret_cast<u32x4*>(lds + RowTile<D>::off(r, D / 2 + ch * 8)) = y2;
+    }
+  }
+};
+
+// ---- staging: a ROWS x D tile written transposed ([D][ROWS], permuted columns) -----------------------
+// Work unit = 4 rows x 4 columns (four 8-byte global loads), written as four 8-byte LDS rows.
+// Unit u -> dl = u % 4, row group = (u / 4) % (ROWS / 4), dhi = u / ROWS: within a half wave the LDS
+// writes touch every bank once.
+template <int D, int ROWS, int NT>
+struct TransStage {
+  static constexpr int kUnits = ROWS * D / 16;
+  static constexpr int kIters = (kUnits + NT - 1) / NT;
+  static_assert(kUnits % NT == 0 || kIters == 1, "tile/thread shape");
+  u32x2 x[kIters][4];
+
+  __device__ static __forceinline__ void unit(int u, int& rg, int& d0) {
+    int dl = u % 4;
+    rg = (u / 4) % (ROWS / 4);
+    d0 = 4 * (dl + 4 * (u / ROWS));
+  }
+
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, int row0, int n_rows) {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      int u = threadIdx.x + it * NT;
+      if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
+      int rg, d0;
+      unit(u, rg, d0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int row = min(row0 + 4 * rg + j, n_rows - 1);
+        x[it][j] = *reinterpret_cast<const u32x2*>(src + (int64_t)row * D + d0);
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(uint16_t* lds) const {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      int u = threadIdx.x + it * NT;
+      if (kUnits % NT != 0 && u >= kUnits) continue;
+      int rg, d0;
+      unit(u, rg, d0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        // column e of the 4x4 block: rows j = 0..3 packed into 8 bytes
+        uint32_t w0 = x[it][0][e / 2], w1 = x[it][1][e / 2], w2 = x[it][2][e / 2], w3 = x[it][3][e / 2];
+        u32x2 o;
+        if (e % 2 == 0) {
+          o[0] = (w0 & 0xffffu) | (w1 << 16);
+          o[1] = (w2 & 0xffffu) | (w3 << 16);
+        } else {
+          o[0] = (w0 >> 16) | (w1 & 0xffff0000u);
+          o[1] = (w2 >> 16) | (w3 & 0xffff0000u);
+        }
+        *reinterpret_cast<u32x2*>(lds + TransTile<ROWS>::off(d0 + e, 4 * rg)) = o;
+      }
+    }
+  }
+};
+
+}  // namespace corope

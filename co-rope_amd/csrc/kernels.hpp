@@ -1,0 +1,62 @@
+// Parameter blocks and host-side launchers of the gfx950 kernels (internal to the library).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace corope {
+
+struct FwdParams {
+  const uint16_t* q;
+  const uint16_t* k;
+  const uint16_t* v;
+  const float* cos;
+  const float* sin;
+  uint16_t* o;
+  float* lse;
+  int64_t fstride;   // elements between rows of the cos/sin tables
+  float qk_scale;    // sm_scale * log2(e)
+  int N;
+  int BH;            // batch * heads
+  int num_m_blocks;  // filled in by the launcher
+};
+
+struct BwdParams {
+  const uint16_t* q;
+  const uint16_t* k;
+  const uint16_t* v;
+  const uint16_t* o;
+  const uint16_t* d_o;
+  const float* cos;
+  const float* sin;
+  const float* lse;
+  float* delta;
+  uint16_t* dq;
+  uint16_t* dk;
+  uint16_t* dv;
+  int64_t fstride;
+  float sm_scale;
+  float qk_scale;  // sm_scale * log2(e)
+  int N;
+  int BH;
+  int num_blocks;  // filled in by the launcher
+};
+
+struct CoropeParams {
+  const uint16_t* q;
+  const uint16_t* k;
+  const uint16_t* v;
+  uint16_t* o;
+  float sm_scale;
+  float log2_theta;  // inverse frequencies are exp2(-(2 d / D) * log2_theta)
+  int B, Hq, Hkv, N;
+  int num_m_blocks;
+};
+
+hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_bwd_preprocess(const BwdParams& p, int D, hipStream_t stream);
+hipError_t launch_bwd_dkdv(const BwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_corope_gqa_fwd(const CoropeParams& p, int D, hipStream_t stream);
+
+}  // namespace corope

@@ -1,0 +1,120 @@
+"""Fused RoPE flash-attention behind the reference's call surface.
+
+``attention(q, k, v, causal, sm_scale, freqs_cos, freqs_sin[, warp_specialize])`` is positional-only, exactly
+like the reference's ``attention = _attention.apply`` (fused-rope/fused_rope_attn.py:652-780); the last argument is
+accepted and ignored (it selects a Triton code path there).  ``fused_rope_attn`` is a keyword-friendly wrapper.
+
+Forward and backward run hand-written gfx950 kernels through the C ABI in ``include/corope_amd.h``; there is no
+other implementation behind this module."""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_SUPPORTED_D = (64, 128)
+
+
+def _stream_ptr(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _check_inputs(q, k, v, freqs_cos, freqs_sin):
+    # shape constraints of the reference (fused_rope_attn.py:657-661)
+    assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be (B, H, N, D)"
+    d = q.shape[-1]
+    assert d == k.shape[-1] and d == v.shape[-1], "q, k, v must share the head dim"
+    assert q.shape == k.shape == v.shape, "q, k, v must share one shape"
+    if d not in _SUPPORTED_D:
+        raise ValueError(f"head dim {d} not built for gfx950 (supported: {_SUPPORTED_D})")
+    if not (q.is_cuda and k.is_cuda and v.is_cuda and freqs_cos.is_cuda and freqs_sin.is_cuda):
+        raise ValueError("fused RoPE attention runs on the GPU only: all tensors must be on a HIP device")
+    if not (q.dtype == k.dtype == v.dtype == torch.bfloat16):
+        raise ValueError(f"q, k, v must be bfloat16 (got {q.dtype}, {k.dtype}, {v.dtype})")
+    n = q.shape[2]
+    for name, f in (("freqs_cos", freqs_cos), ("freqs_sin", freqs_sin)):
+        if f.dim() != 2 or f.shape[0] < n or f.shape[1] < d // 2:
+            raise ValueError(f"{name} must be (N, D) or (N, D/2) with N >= {n}, got {tuple(f.shape)}")
+
+
+def _freq_table(f):
+    """fp32 table with unit column stride and a row stride the kernels accept."""
+    if f.dtype != torch.float32:
+        f = f.float()
+    if f.stride(1) != 1 or f.stride(0) % 4 != 0 or f.data_ptr() % 16 != 0:
+        f = f.contiguous()
+        if f.stride(0) % 4 != 0:
+            f = torch.nn.functional.pad(f, (0, 4 - f.shape[1] % 4)).contiguous()
+    return f
+
+
+class _FusedRopeAttn(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, q, k, v, causal, sm_scale, freqs_cos, freqs_sin, warp_specialize=True):
+        _check_inputs(q, k, v, freqs_cos, freqs_sin)
+        lib = _lib.load()
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        fc, fs = _freq_table(freqs_cos), _freq_table(freqs_sin)
+        if fc.stride(0) != fs.stride(0):
+            fc, fs = fc.contiguous(), fs.contiguous()
+        B, H, N, D = q.shape
+        o = torch.empty_like(q)
+        M = torch.empty((B, H, N), device=q.device, dtype=torch.float32)
+        with torch.cuda.device(q.device):
+            rc = lib.corope_rope_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
+                                          fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, N, D, float(sm_scale),
+                                          int(bool(causal)), _stream_ptr(q))
+        _lib.check(rc, "corope_rope_attn_fwd")
+        ctx.save_for_backward(q, k, v, o, M, fc, fs)
+        ctx.sm_scale = float(sm_scale)
+        ctx.HEAD_DIM = D
+        ctx.causal = bool(causal)
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, M, fc, fs = ctx.saved_tensors
+        lib = _lib.load()
+        do = do.contiguous()
+        if do.dtype != torch.bfloat16:
+            do = do.to(torch.bfloat16)
+        B, H, N, D = q.shape
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        delta = torch.empty_like(M)
+        with torch.cuda.device(q.device):
+            rc = lib.corope_rope_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
+                                          M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0),
+                                          dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, N, D, ctx.sm_scale,
+                                          int(ctx.causal), _stream_ptr(q))
+        _lib.check(rc, "corope_rope_attn_bwd")
+        return dq, dk, dv, None, None, None, None, None
+
+
+attention = _FusedRopeAttn.apply
+
+
+def fused_rope_attn(q, k, v, freqs_cos, freqs_sin, causal=True, sm_scale=None):
+    """Keyword-friendly form: ``sm_scale`` defaults to 1/sqrt(D)."""
+    if sm_scale is None:
+        sm_scale = q.shape[-1] ** -0.5
+    return attention(q, k, v, causal, sm_scale, freqs_cos, freqs_sin)
+
+
+def rope_attn_forward_with_lse(q, k, v, causal, sm_scale, freqs_cos, freqs_sin):
+    """Forward only, returning (O, M) where M is the saved base-2 log-sum-exp statistic (B, H, N) fp32."""
+    _check_inputs(q, k, v, freqs_cos, freqs_sin)
+    lib = _lib.load()
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    fc, fs = _freq_table(freqs_cos), _freq_table(freqs_sin)
+    if fc.stride(0) != fs.stride(0):
+        fc, fs = fc.contiguous(), fs.contiguous()
+    B, H, N, D = q.shape
+    o = torch.empty_like(q)
+    M = torch.empty((B, H, N), device=q.device, dtype=torch.float32)
+    with torch.cuda.device(q.device):
+        rc = lib.corope_rope_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
+                                      fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, N, D, float(sm_scale),
+                                      int(bool(causal)), _stream_ptr(q))
+    _lib.check(rc, "corope_rope_attn_fwd")
+    return o, M

@@ -1,0 +1,10 @@
+"""Importable alias of the ``co-rope_amd`` package (a hyphen cannot appear in an ``import`` statement)."""
+import importlib
+import os
+import sys
+
+_root = os.path.dirname(os.path.abspath(__file__))
+if _root not in sys.path:
+    sys.path.insert(0, _root)
+_pkg = importlib.import_module("co-rope_amd")
+sys.modules[__name__] = _pkg

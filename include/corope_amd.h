@@ -1,0 +1,100 @@
+/* corope_amd.h -- C ABI of the MI355X (gfx950) fused RoPE-attention library.
+ *
+ * The reference repository (Superposition09m/Co-RoPE) has no C or FFI boundary: its hot path
+ * sits behind two torch.autograd.Function classes that launch Triton kernels.  This library
+ * is the device side of the same two operators; the Python layer in co-rope_amd/ keeps the
+ * reference's call surface and reaches these entry points through ctypes.
+ *
+ * Conventions (all entry points)
+ *   - tensors are device pointers to contiguous row-major (B, H, N, D) bf16 storage;
+ *     D is 64 or 128; pointers are 16-byte aligned;
+ *   - freqs_cos / freqs_sin are fp32 tables with one row per position; only columns
+ *     [0, D/2) are read; `freq_row_stride` is the distance between rows in elements
+ *     (D for the reference's duplicated-half (N, D) table);
+ *   - `lse` is the forward's per-row statistic M = log2(sum_j exp2(s_ij * sm_scale * log2 e)),
+ *     shape (B, H, N) fp32 -- the same base-2 quantity the reference saves
+ *     (fused-rope/fused_rope_attn.py:316-319);
+ *   - the caller owns every buffer; the library never allocates or frees device memory and
+ *     never synchronises; kernels are enqueued on `stream` (a hipStream_t, NULL = default);
+ *   - every argument is validated before the first HIP call; return 0 on success or a
+ *     negative COROPE_E_* code, with a message available from corope_amd_last_error().
+ */
+#ifndef COROPE_AMD_H
+#define COROPE_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define COROPE_OK 0
+#define COROPE_E_BADARG (-1)      /* null pointer, non-positive size, bad scale */
+#define COROPE_E_UNSUPPORTED (-2) /* head dim / group size / sequence length outside the built kernels */
+#define COROPE_E_ALIGN (-3)       /* pointer not 16-byte aligned */
+#define COROPE_E_LAUNCH (-4)      /* HIP reported an error at launch */
+
+/* ABI version of this header (bumped on any signature change). */
+int corope_amd_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char *corope_amd_last_error(void);
+
+/* Argument check only (no HIP call): what corope_rope_attn_fwd/bwd would return for these sizes. */
+int corope_rope_attn_check(int B, int H, int N, int D, int64_t freq_row_stride, float sm_scale, int backward);
+
+/* Argument check only (no HIP call) for corope_gqa_fwd. */
+int corope_gqa_check(int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta);
+
+/* Fused RoPE flash-attention forward.
+ * Replaces the launch of _attn_fwd in _attention.forward
+ * (reference fused-rope/fused_rope_attn.py:222-320 kernel, :702-716 launch).
+ * Writes o (B,H,N,D) bf16 and lse (B,H,N) fp32. */
+int corope_rope_attn_fwd(const void *q, const void *k, const void *v,
+                         const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                         void *o, float *lse,
+                         int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
+/* delta[b,h,i] = sum_d o[b,h,i,d] * do[b,h,i,d]  (fp32).
+ * Replaces _attn_bwd_preprocess (reference fused-rope/fused_rope_attn.py:324-337, launch :753-758). */
+int corope_rope_attn_bwd_preprocess(const void *o, const void *d_o, float *delta,
+                                    int B, int H, int N, int D, void *stream);
+
+/* dK and dV: one workgroup per key block, sweeping the query blocks that attend to it.
+ * Replaces the _attn_bwd_dkdv half of _attn_bwd (reference fused-rope/fused_rope_attn.py:342-404,
+ * :524-579) including the host-side K pre-scale (:746-748), which is folded into the kernel. */
+int corope_rope_attn_bwd_dkdv(const void *q, const void *k, const void *v, const void *d_o,
+                              const float *lse, const float *delta,
+                              const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                              void *dk, void *dv,
+                              int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
+/* dQ: one workgroup per query block, sweeping the key blocks it attends to.
+ * Replaces the _attn_bwd_dq half of _attn_bwd (reference fused-rope/fused_rope_attn.py:409-470, :592-649). */
+int corope_rope_attn_bwd_dq(const void *q, const void *k, const void *v, const void *d_o,
+                            const float *lse, const float *delta,
+                            const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                            void *dq,
+                            int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
+/* Whole backward = preprocess + dkdv + dq on one stream (what _attention.backward launches,
+ * reference fused-rope/fused_rope_attn.py:725-777).  `delta` is caller-provided (B,H,N) fp32 scratch. */
+int corope_rope_attn_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                         const float *lse, float *delta,
+                         const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                         void *dq, void *dk, void *dv,
+                         int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
+/* Co-RoPE grouped-query attention forward (causal only).
+ * q: (B,Hq,N,D), k/v: (B,Hkv,N,D), o: (B,Hq,N,D), group size Hq/Hkv in [1, 8].
+ * Replaces the launch of _corope_fwd_backbone in _attention.forward
+ * (reference corope-exp/flash_attn_co_rope_gqa_triton.py:48-400 kernel, :428-450 launch);
+ * the inverse frequencies theta^(-2d/D) the reference builds with torch (:428) are computed
+ * on the host here and passed to the kernel by value. */
+int corope_gqa_fwd(const void *q, const void *k, const void *v, void *o,
+                   int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COROPE_AMD_H */

@@ -1,0 +1,95 @@
+"""GPU parity of the fused RoPE-attention forward against the CPU oracle (through the C ABI).
+
+Bar: max-abs <= 2e-2 for bf16 outputs against the fp32 oracle evaluated on the same bf16-rounded inputs."""
+import math
+
+import pytest
+import torch
+
+from conftest import bf16_round, seeded
+from oracle import rope_attn_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2          # the stated bar, at the benchmark's temperature sm_scale = 1/sqrt(D)
+TOL_HOT = 1.5e-1     # sm_scale = 0.5 (the reference's verification script, written for fp16 with bound 1e-2):
+                    # score std is 4-6x larger there and bf16 carries 8x less mantissa than fp16
+LN2 = math.log(2.0)
+
+
+def _inputs(B, H, N, D, seed=42, std=1.0):
+    q, k, v = (bf16_round(seeded((B, H, N, D), seed + i, std=std)) for i in range(3))
+    return q, k, v
+
+
+def _run(pkg, q, k, v, causal, scale, c, s):
+    dev = torch.device("cuda:0")
+    o, M = pkg.rope_attn_forward_with_lse(q.to(dev, torch.bfloat16), k.to(dev, torch.bfloat16), v.to(dev, torch.bfloat16),
+                                          causal, scale, c.to(dev), s.to(dev))
+    torch.cuda.synchronize()
+    return o.float().cpu(), M.cpu()
+
+
+# the six cases of the reference's verification script (fused-rope/verification.py:153-161), its C2 benchmark
+# shape, and ragged / tiny sequence lengths
+SHAPES = [(2, 4, 512, 64), (1, 8, 1024, 128), (4, 16, 2048, 64), (4, 8, 1024, 64),
+          (1, 2, 200, 64), (2, 1, 77, 128), (1, 3, 333, 128), (1, 1, 1, 64), (1, 1, 31, 128), (1, 2, 257, 128)]
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,N,D", SHAPES)
+def test_forward_parity(pkg, B, H, N, D, causal):
+    print(f"case B={B} H={H} N={N} D={D} causal={causal}", flush=True)
+    q, k, v = _inputs(B, H, N, D)
+    c, s = O.precompute_freqs_cis(D, N)
+    scale = 1 / math.sqrt(D)
+    o, M = _run(pkg, q, k, v, causal, scale, c, s)
+    ro, rl = O.rope_attn_forward_blocked(q, k, v, causal, scale, c, s)
+    err = (o - ro).abs()
+    print(f"  O max-abs {err.max():.3e} mean-abs {err.mean():.3e}; LSE max-abs {(M * LN2 - rl).abs().max():.3e}")
+    assert torch.isfinite(o).all()
+    assert err.max() <= TOL
+    assert (M * LN2 - rl).abs().max() <= TOL
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,N,D", [(2, 4, 512, 64), (1, 8, 1024, 128), (4, 16, 2048, 64)])
+def test_forward_parity_verification_script_cases(pkg, B, H, N, D, causal):
+    """The six cases of the reference's verification script (fused-rope/verification.py:153-161), sm_scale = 0.5."""
+    print(f"case B={B} H={H} N={N} D={D} causal={causal} sm_scale=0.5", flush=True)
+    q, k, v = _inputs(B, H, N, D)
+    c, s = O.precompute_freqs_cis(D, N)
+    o, M = _run(pkg, q, k, v, causal, 0.5, c, s)
+    ro, rl = O.rope_attn_forward_blocked(q, k, v, causal, 0.5, c, s)
+    err = (o - ro).abs()
+    print(f"  O max-abs {err.max():.3e} mean-abs {err.mean():.3e}; LSE max-abs {(M * LN2 - rl).abs().max():.3e}")
+    assert torch.isfinite(o).all()
+    assert err.max() <= TOL_HOT and err.mean() <= 5e-3
+
+
+def test_identity_rotation_is_plain_attention(pkg):
+    """cos=1, sin=0, N(0, 0.5^2) inputs, sm_scale=0.5: the reference's embedded pytest (fused_rope_attn.py:785-851)."""
+    B, H, N, D = 1, 2, 1024, 64
+    q, k, v = _inputs(B, H, N, D, seed=20, std=0.5)
+    one, zero = torch.ones(N, D), torch.zeros(N, D)
+    o, _ = _run(pkg, q, k, v, True, 0.5, one, zero)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=0.5)
+    assert (o - ref).abs().max() <= 1e-2
+
+
+def test_half_width_table_and_row_stride(pkg):
+    """Only columns [0, D/2) of the tables are read; a (N, D/2) table gives the same result as the (N, D) one."""
+    B, H, N, D = 1, 2, 256, 128
+    q, k, v = _inputs(B, H, N, D, seed=5)
+    c, s = O.precompute_freqs_cis(D, N)
+    o_full, _ = _run(pkg, q, k, v, True, 0.1, c, s)
+    o_half, _ = _run(pkg, q, k, v, True, 0.1, c[:, :D // 2].contiguous(), s[:, :D // 2].contiguous())
+    assert torch.equal(o_full, o_half)
+
+
+def test_deterministic(pkg):
+    B, H, N, D = 2, 4, 512, 128
+    q, k, v = _inputs(B, H, N, D, seed=9)
+    c, s = O.precompute_freqs_cis(D, N)
+    a, ma = _run(pkg, q, k, v, True, 0.09, c, s)
+    b, mb = _run(pkg, q, k, v, True, 0.09, c, s)
+    assert torch.equal(a, b) and torch.equal(ma, mb)
