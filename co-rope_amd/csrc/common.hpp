@@ -210,4 +210,112 @@ struct TransStage {
   }
 };
 
+// ---- staging: a ROWS x D tile copied row-major (no rotation) -------------------------------------------
+template <int D, int ROWS, int NT>
+struct CopyStage {
+  static constexpr int kChunks = D / 8;  // 16-byte units per row
+  static constexpr int kUnits = ROWS * kChunks;
+  static constexpr int kIters = (kUnits + NT - 1) / NT;
+  u32x4 x[kIters];
+
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, int row0, int n_rows) {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      int u = threadIdx.x + it * NT;
+      if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
+      int row = min(row0 + u / kChunks, n_rows - 1);
+      x[it] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * D + (u % kChunks) * 8);
+    }
+  }
+  __device__ __forceinline__ void store_rows(uint16_t* lds) const {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      int u = threadIdx.x + it * NT;
+      if (kUnits % NT != 0 && u >= kUnits) continue;
+      *reinterpret_cast<u32x4*>(lds + RowTile<D>::off(u / kChunks, (u % kChunks) * 8)) = x[it];
+    }
+  }
+};
+
+// ---- transposing LDS read (ds_read_b64_tr_b16) ------------------------------------------------------------
+// The instruction works on blocks of 16 lanes: source lane s supplies 8 bytes E[s][0..3]; result lane L
+// receives { E[4j + L/4][L % 4] : j = 0..3 }.
+//
+// load_a_trans builds the A operand of mfma32 (32 rows m x 16 contraction slots) from a ROW-MAJOR tile
+// T[k][m] whose rows are the contraction index, i.e. it reads the tile transposed.  The contraction slots
+// follow the order in which a 32x32 accumulator hands out its rows when it is re-used as a B operand:
+//   slot j of lane-half h  <->  k = kbase + 8*(j / 4) + 4*h + (j % 4).
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+__device__ __forceinline__ u32x4 load_a_trans(const uint16_t* tile, int stride, int kbase, int m0) {
+  typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+  const int l = threadIdx.x % kWave;
+  const int blk = l / 16, s = l % 16, h = blk / 2;
+  const uint16_t* p = tile + (kbase + 4 * h + s / 4) * stride + m0 + 16 * (blk % 2) + 4 * (s % 4);
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 8 * stride));
+  u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
+  return u32x4{a[0], a[1], b[0], b[1]};
+}
+
+// Loads 32 rows x D of a (rows, D) bf16 matrix as the B operand chunks of mfma32 (lane = row, 8 columns per
+// chunk and lane-half), optionally applying the half-layout rotation first.  KC = D / 16 chunks.
+template <int D, bool ROTATE>
+__device__ __forceinline__ void load_b_rows(u32x4 (&out)[D / 16], const uint16_t* __restrict__ src,
+                                            const float* __restrict__ cosp, const float* __restrict__ sinp,
+                                            int64_t fstride, int row) {
+  constexpr int KC = D / 16;
+  const int lh = (threadIdx.x % kWave) / 32;
+  const uint16_t* xp = src + (int64_t)row * D + 8 * lh;
+  if constexpr (!ROTATE) {
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) out[kc] = *reinterpret_cast<const u32x4*>(xp + 16 * kc);
+  } else {
+    const float* cp = cosp + (int64_t)row * fstride + 8 * lh;
+    const float* sp = sinp + (int64_t)row * fstride + 8 * lh;
+#pragma unroll
+    for (int kc = 0; kc < KC / 2; ++kc) {
+      u32x4 x1 = *reinterpret_cast<const u32x4*>(xp + 16 * kc);
+      u32x4 x2 = *reinterpret_cast<const u32x4*>(xp + D / 2 + 16 * kc);
+      f32x4 c[2] = {*reinterpret_cast<const f32x4*>(cp + 16 * kc), *reinterpret_cast<const f32x4*>(cp + 16 * kc + 4)};
+      f32x4 s[2] = {*reinterpret_cast<const f32x4*>(sp + 16 * kc), *reinterpret_cast<const f32x4*>(sp + 16 * kc + 4)};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        float a0 = bf16_lo(x1[w]), a1 = bf16_hi(x1[w]), b0 = bf16_lo(x2[w]), b1 = bf16_hi(x2[w]);
+        float c0 = c[w / 2][(2 * w) % 4], c1 = c[w / 2][(2 * w) % 4 + 1];
+        float s0 = s[w / 2][(2 * w) % 4], s1 = s[w / 2][(2 * w) % 4 + 1];
+        out[kc][w] = pack_bf16(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+        out[kc + KC / 2][w] = pack_bf16(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+      }
+    }
+  }
+}
+
+// Epilogue for gradients held as a transposed accumulator (lane = row of the output matrix, registers =
+// columns): undoes the rotation, d1 = d1r c + d2r s, d2 = d2r c - d1r s, scales, rounds and stores.
+// acc[db][i] holds column db*32 + 8*(i/4) + 4*h + (i%4) of the lane's row.
+template <int D>
+__device__ __forceinline__ void store_unrotated(const f32x16 (&acc)[D / 32], uint16_t* __restrict__ dst_row,
+                                                const float* __restrict__ cos_row, const float* __restrict__ sin_row,
+                                                float scale) {
+  constexpr int NDB = D / 32;
+  const int lh = (threadIdx.x % kWave) / 32;
+#pragma unroll
+  for (int db = 0; db < NDB / 2; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int col = db * 32 + 8 * g + 4 * lh;
+      f32x4 c = *reinterpret_cast<const f32x4*>(cos_row + col);
+      f32x4 s = *reinterpret_cast<const f32x4*>(sin_row + col);
+      float o1[4], o2[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float r1 = acc[db][4 * g + e] * scale, r2 = acc[db + NDB / 2][4 * g + e] * scale;
+        o1[e] = r1 * c[e] + r2 * s[e];
+        o2[e] = r2 * c[e] - r1 * s[e];
+      }
+      *reinterpret_cast<u32x2*>(dst_row + col) = u32x2{pack_bf16(o1[0], o1[1]), pack_bf16(o1[2], o1[3])};
+      *reinterpret_cast<u32x2*>(dst_row + D / 2 + col) = u32x2{pack_bf16(o2[0], o2[1]), pack_bf16(o2[2], o2[3])};
+    }
+}
+
 }  // namespace corope

@@ -1,6 +1,347 @@
+// Fused half-layout-RoPE flash-attention backward for gfx950: the dK/dV kernel and the dQ kernel.
+//
+// Device counterparts of the reference's _attn_bwd_dkdv / _attn_bwd_dq
+// (fused-rope/fused_rope_attn.py:342-404, :409-470, driver :474-649).  The reference runs both halves in one
+// program and re-rotates Q (resp. K) in registers on every inner iteration; here each half is its own kernel
+// and the streamed operand is rotated once per workgroup per tile while it is staged into LDS.  No atomics:
+// dK/dV are owned by the key block's workgroup, dQ by the query block's.
+//
+// Scaling contract (same as the reference's, :385, :457, :574-575, :643-644, with the host-side K pre-scale
+// :746-748 folded in): P = exp2(s * sm_scale * log2e - M) with M the forward's base-2 statistic;
+// dS = P o (dP - delta); dK_r = sm_scale * dS^T Q_r; dQ_r = sm_scale * dS K_r; both un-rotated in fp32
+// before the single rounding to bf16.
+//
+// Operands that must be read "transposed" (contraction along the sequence axis of a row-major tile) use the
+// gfx950 transposing LDS read, so every tile is staged row-major exactly once.
 #include "common.hpp"
 #include "kernels.hpp"
+
 namespace corope {
-hipError_t launch_bwd_dkdv(const BwdParams&, int, bool, hipStream_t) { return hipErrorNotSupported; }
-hipError_t launch_bwd_dq(const BwdParams&, int, bool, hipStream_t) { return hipErrorNotSupported; }
+
+// ===================================================================================== dK / dV
+// Workgroup = NWAVES waves x 32 keys.  K_r and V rows of the wave stay in registers as B operands.
+// Per query tile (BLOCK_M rows, staged: rotated Q and dO, plus M and delta):
+//   S  = Q_r K_r^T            (A = Q_r rows from LDS,      B = K_r regs)   lane = key, registers = queries
+//   dP = dO V^T               (A = dO rows from LDS,       B = V regs)
+//   P  = exp2(S*c - M), dS = P o (dP - delta)                               (bf16, already B-operand shaped)
+//   dV^T   += dO^T  P         (A = dO tile read transposed, B = P)
+//   dK_r^T += Q_r^T dS        (A = Q_r tile read transposed, B = dS)
+template <int D, int NWAVES, int BLOCK_M>
+struct DkdvCfg {
+  static constexpr int kThreads = NWAVES * kWave;
+  static constexpr int kBlockN = NWAVES * 32;
+  static constexpr int kTileBytes = RowTile<D>::bytes(BLOCK_M);
+  static constexpr int kStatBytes = BLOCK_M * 4;
+  static constexpr int kStageBytes = 2 * kTileBytes + 2 * kStatBytes;
+  static constexpr int kLdsBytes = 2 * kStageBytes;
+};
+
+template <int D, int NWAVES, int BLOCK_M, bool CAUSAL>
+__global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M>;
+  constexpr int NT = Cfg::kThreads;
+  constexpr int KC = D / 16, NDB = D / 32, NQB = BLOCK_M / 32;
+  constexpr int LS = RowTile<D>::kStride;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  const int bh = blockIdx.x % p.BH;
+  const int nb = blockIdx.x / p.BH;  // key block; for causal the low blocks are the heavy ones and start first
+  const int n0 = nb * Cfg::kBlockN;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int lq = lane % 32, lh = lane / 32;
+  const int N = p.N;
+  const int64_t base = (int64_t)bh * N * D;
+  const uint16_t* qg = p.q + base;
+  const uint16_t* dog = p.d_o + base;
+  const float* lseg = p.lse + (int64_t)bh * N;
+  const float* deltag = p.delta + (int64_t)bh * N;
+
+  const int key = n0 + wave * 32 + lq;
+  const int key_c = min(key, N - 1);
+  const int wk_lo = n0 + wave * 32, wk_hi = wk_lo + 31;
+
+  u32x4 kb[KC], vb[KC];
+  load_b_rows<D, true>(kb, p.k + base, p.cos, p.sin, p.fstride, key_c);
+  load_b_rows<D, false>(vb, p.v + base, nullptr, nullptr, 0, key_c);
+
+  const int m_tiles = (N + BLOCK_M - 1) / BLOCK_M;
+  const int mt0 = CAUSAL ? n0 / BLOCK_M : 0;
+
+  RotStage<D, BLOCK_M, NT> qst;
+  CopyStage<D, BLOCK_M, NT> dst;
+  float st_lse = 0.f, st_delta = 0.f;
+  auto load_tile = [&](int m0) {
+    qst.load(qg, p.cos, p.sin, p.fstride, m0, N);
+    dst.load(dog, m0, N);
+    if (threadIdx.x < BLOCK_M) {
+      int qi = m0 + threadIdx.x;
+      // rows past the end: M = +inf makes P = 0, so they contribute nothing
+      st_lse = qi < N ? lseg[qi] : INFINITY;
+      st_delta = qi < N ? deltag[qi] : 0.f;
+    }
+  };
+  auto q_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
+  auto do_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes + Cfg::kTileBytes); };
+  auto lse_tile = [&](int buf) { return reinterpret_cast<float*>(smem + buf * Cfg::kStageBytes + 2 * Cfg::kTileBytes); };
+  auto delta_tile = [&](int buf) {
+    return reinterpret_cast<float*>(smem + buf * Cfg::kStageBytes + 2 * Cfg::kTileBytes + Cfg::kStatBytes);
+  };
+  auto store_tile = [&](int buf) {
+    qst.store_rows(q_tile(buf));
+    dst.store_rows(do_tile(buf));
+    if (threadIdx.x < BLOCK_M) {
+      lse_tile(buf)[threadIdx.x] = st_lse;
+      delta_tile(buf)[threadIdx.x] = st_delta;
+    }
+  };
+
+  f32x16 dvacc[NDB], dkacc[NDB];
+#pragma unroll
+  for (int i = 0; i < NDB; ++i) dvacc[i] = dkacc[i] = f32x16{0};
+
+  if (mt0 < m_tiles) {
+    load_tile(mt0 * BLOCK_M);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  const float scale2 = p.qk_scale;
+  for (int mt = mt0; mt < m_tiles; ++mt) {
+    const int m0 = mt * BLOCK_M;
+    const int cur = (mt - mt0) & 1;
+    if (mt + 1 < m_tiles) load_tile(m0 + BLOCK_M);
+
+    const uint16_t* qs = q_tile(cur);
+    const uint16_t* dos = do_tile(cur);
+    const float* lses = lse_tile(cur);
+    const float* deltas = delta_tile(cur);
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+      const int mq0 = m0 + qb * 32;
+      // queries of this 32-row block that lie above every key of the wave see none of them
+      if (CAUSAL && mq0 + 31 < wk_lo) continue;
+      f32x16 sacc = f32x16{0}, dpacc = f32x16{0};
+      const uint16_t* qrow = qs + RowTile<D>::off(qb * 32 + lq, 8 * lh);
+      const uint16_t* dorow = dos + RowTile<D>::off(qb * 32 + lq, 8 * lh);
+#pragma unroll
+      for (int kc = 0; kc < KC; ++kc)
+        sacc = mfma32(*reinterpret_cast<const u32x4*>(qrow + 16 * kc), kb[kc], sacc);
+#pragma unroll
+      for (int kc = 0; kc < KC; ++kc)
+        dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc), vb[kc], dpacc);
+
+      const bool need_mask = CAUSAL && mq0 < wk_hi;
+      u32x4 pb[2], dsb[2];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 m4 = *reinterpret_cast<const f32x4*>(lses + qb * 32 + 8 * g + 4 * lh);
+        f32x4 d4 = *reinterpret_cast<const f32x4*>(deltas + qb * 32 + 8 * g + 4 * lh);
+        float pv[4], ds[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          pv[e] = fast_exp2(sacc[4 * g + e] * scale2 - m4[e]);
+          if (need_mask && (mq0 + 8 * g + 4 * lh + e) < key) pv[e] = 0.f;
+          ds[e] = pv[e] * (dpacc[4 * g + e] - d4[e]);
+        }
+        pb[g / 2][2 * (g % 2)] = pack_bf16(pv[0], pv[1]);
+        pb[g / 2][2 * (g % 2) + 1] = pack_bf16(pv[2], pv[3]);
+        dsb[g / 2][2 * (g % 2)] = pack_bf16(ds[0], ds[1]);
+        dsb[g / 2][2 * (g % 2) + 1] = pack_bf16(ds[2], ds[3]);
+      }
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) {
+        const int kbase = qb * 32 + 16 * cc;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          dvacc[db] = mfma32(load_a_trans(dos, LS, kbase, db * 32), pb[cc], dvacc[db]);
+          dkacc[db] = mfma32(load_a_trans(qs, LS, kbase, db * 32), dsb[cc], dkacc[db]);
+        }
+      }
+    }
+    if (mt + 1 < m_tiles) store_tile(cur ^ 1);
+    __syncthreads();
+  }
+
+  if (key < N) {
+    uint16_t* dvp = p.dv + base + (int64_t)key * D;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w = {pack_bf16(dvacc[db][4 * g], dvacc[db][4 * g + 1]), pack_bf16(dvacc[db][4 * g + 2], dvacc[db][4 * g + 3])};
+        *reinterpret_cast<u32x2*>(dvp + db * 32 + 8 * g + 4 * lh) = w;
+      }
+    store_unrotated<D>(dkacc, p.dk + base + (int64_t)key * D, p.cos + (int64_t)key * p.fstride,
+                       p.sin + (int64_t)key * p.fstride, p.sm_scale);
+  }
+}
+
+// ===================================================================================== dQ
+// Workgroup = NWAVES waves x 32 queries.  Rotated Q rows and dO rows of the wave stay in registers.
+// Per key tile (BLOCK_N rows, staged: rotated K and V):
+//   S^T  = K_r Q_r^T          (A = K_r rows from LDS, B = Q_r regs)    lane = query, registers = keys
+//   dP^T = V dO^T             (A = V rows from LDS,   B = dO regs)
+//   dS^T = P^T o (dP^T - delta)                                        (bf16, B-operand shaped)
+//   dQ_r^T += K_r^T dS^T      (A = K_r tile read transposed, B = dS^T)
+template <int D, int NWAVES, int BLOCK_N>
+struct DqCfg {
+  static constexpr int kThreads = NWAVES * kWave;
+  static constexpr int kBlockM = NWAVES * 32;
+  static constexpr int kTileBytes = RowTile<D>::bytes(BLOCK_N);
+  static constexpr int kStageBytes = 2 * kTileBytes;
+  static constexpr int kLdsBytes = 2 * kStageBytes;
+};
+
+template <int D, int NWAVES, int BLOCK_N, bool CAUSAL>
+__global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdParams p) {
+  using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
+  constexpr int NT = Cfg::kThreads;
+  constexpr int KC = D / 16, NDB = D / 32, NKB = BLOCK_N / 32;
+  constexpr int LS = RowTile<D>::kStride;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  const int bh = blockIdx.x % p.BH;
+  const int mb = p.num_blocks - 1 - blockIdx.x / p.BH;  // heaviest (last) query blocks first
+  const int m0 = mb * Cfg::kBlockM;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int lq = lane % 32, lh = lane / 32;
+  const int N = p.N;
+  const int64_t base = (int64_t)bh * N * D;
+  const uint16_t* kg = p.k + base;
+  const uint16_t* vg = p.v + base;
+
+  const int q_row = m0 + wave * 32 + lq;
+  const int q_c = min(q_row, N - 1);
+  const int wq_lo = m0 + wave * 32, wq_hi = wq_lo + 31;
+
+  const int n_tiles = CAUSAL ? min((m0 + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, (N + BLOCK_N - 1) / BLOCK_N)
+                             : (N + BLOCK_N - 1) / BLOCK_N;
+  RotStage<D, BLOCK_N, NT> kst;
+  CopyStage<D, BLOCK_N, NT> vst;
+  kst.load(kg, p.cos, p.sin, p.fstride, 0, N);
+  vst.load(vg, 0, N);
+
+  u32x4 qb[KC], dob[KC];
+  load_b_rows<D, true>(qb, p.q + base, p.cos, p.sin, p.fstride, q_c);
+  load_b_rows<D, false>(dob, p.d_o + base, nullptr, nullptr, 0, q_c);
+  const float lse_q = p.lse[(int64_t)bh * N + q_c];
+  const float delta_q = p.delta[(int64_t)bh * N + q_c];
+
+  auto k_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
+  auto v_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes + Cfg::kTileBytes); };
+
+  f32x16 dqacc[NDB];
+#pragma unroll
+  for (int i = 0; i < NDB; ++i) dqacc[i] = f32x16{0};
+
+  kst.store_rows(k_tile(0));
+  vst.store_rows(v_tile(0));
+  __syncthreads();
+
+  const float scale2 = p.qk_scale;
+  for (int t = 0; t < n_tiles; ++t) {
+    const int n0 = t * BLOCK_N;
+    const int cur = t & 1;
+    if (t + 1 < n_tiles) {
+      kst.load(kg, p.cos, p.sin, p.fstride, n0 + BLOCK_N, N);
+      vst.load(vg, n0 + BLOCK_N, N);
+    }
+    const bool active = !CAUSAL || n0 <= wq_hi;
+    if (active) {
+      const uint16_t* ks = k_tile(cur);
+      const uint16_t* vs = v_tile(cur);
+      const bool need_mask = (CAUSAL && n0 + BLOCK_N - 1 > wq_lo) || (!CAUSAL && n0 + BLOCK_N > N);
+      u32x4 dsb[BLOCK_N / 16];
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) {
+        f32x16 sacc = f32x16{0}, dpacc = f32x16{0};
+        const uint16_t* krow = ks + RowTile<D>::off(kb * 32 + lq, 8 * lh);
+        const uint16_t* vrow = vs + RowTile<D>::off(kb * 32 + lq, 8 * lh);
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc)
+          sacc = mfma32(*reinterpret_cast<const u32x4*>(krow + 16 * kc), qb[kc], sacc);
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc)
+          dpacc = mfma32(*reinterpret_cast<const u32x4*>(vrow + 16 * kc), dob[kc], dpacc);
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          float ds[2];
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            float pv = fast_exp2(sacc[i + e] * scale2 - lse_q);
+            if (need_mask) {
+              int kk = n0 + kb * 32 + acc_row(i + e, lh);
+              if (CAUSAL ? kk > q_row : kk >= N) pv = 0.f;
+            }
+            ds[e] = pv * (dpacc[i + e] - delta_q);
+          }
+          dsb[2 * kb + i / 8][(i % 8) / 2] = pack_bf16(ds[0], ds[1]);
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < BLOCK_N / 16; ++c)
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+          dqacc[db] = mfma32(load_a_trans(ks, LS, 16 * c, db * 32), dsb[c], dqacc[db]);
+    }
+    if (t + 1 < n_tiles) {
+      kst.store_rows(k_tile(cur ^ 1));
+      vst.store_rows(v_tile(cur ^ 1));
+    }
+    __syncthreads();
+  }
+
+  if (q_row < N)
+    store_unrotated<D>(dqacc, p.dq + base + (int64_t)q_row * D, p.cos + (int64_t)q_row * p.fstride,
+                       p.sin + (int64_t)q_row * p.fstride, p.sm_scale);
+}
+
+// ===================================================================================== launchers
+template <typename K>
+static hipError_t set_lds(K kern, int bytes) {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+template <int D, bool CAUSAL>
+static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
+  constexpr int NWAVES = 4, BLOCK_M = 64;
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M>;
+  auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = set_lds(kern, Cfg::kLdsBytes);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  p.num_blocks = (p.N + Cfg::kBlockN - 1) / Cfg::kBlockN;
+  hipLaunchKernelGGL(kern, dim3(p.num_blocks * p.BH), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
+  return hipGetLastError();
+}
+
+template <int D, bool CAUSAL>
+static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
+  constexpr int NWAVES = 4, BLOCK_N = 64;
+  using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
+  auto kern = rope_attn_bwd_dq_kernel<D, NWAVES, BLOCK_N, CAUSAL>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = set_lds(kern, Cfg::kLdsBytes);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  p.num_blocks = (p.N + Cfg::kBlockM - 1) / Cfg::kBlockM;
+  hipLaunchKernelGGL(kern, dim3(p.num_blocks * p.BH), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_bwd_dkdv(const BwdParams& p, int D, bool causal, hipStream_t stream) {
+  if (D == 128) return causal ? launch_dkdv_cfg<128, true>(p, stream) : launch_dkdv_cfg<128, false>(p, stream);
+  return causal ? launch_dkdv_cfg<64, true>(p, stream) : launch_dkdv_cfg<64, false>(p, stream);
+}
+
+hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream) {
+  if (D == 128) return causal ? launch_dq_cfg<128, true>(p, stream) : launch_dq_cfg<128, false>(p, stream);
+  return causal ? launch_dq_cfg<64, true>(p, stream) : launch_dq_cfg<64, false>(p, stream);
+}
+
 }  // namespace corope

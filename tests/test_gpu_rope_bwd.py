@@ -1,0 +1,85 @@
+"""GPU parity of the fused RoPE-attention backward (preprocess, dK/dV, dQ) against the CPU oracle.
+
+Everything goes through the torch.autograd.Function, i.e. through the C ABI.  Bar: max-abs <= 2e-2 per tensor
+against the fp32 oracle evaluated on the same bf16-rounded q, k, v, dO."""
+import math
+
+import pytest
+import torch
+
+from conftest import bf16_round, seeded
+from oracle import rope_attn_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def _case(B, H, N, D, seed=42):
+    q, k, v, g = (bf16_round(seeded((B, H, N, D), seed + i)) for i in range(4))
+    c, s = O.precompute_freqs_cis(D, N)
+    return q, k, v, g, c, s
+
+
+def _gpu_fwd_bwd(pkg, q, k, v, g, causal, scale, c, s):
+    dev = torch.device("cuda:0")
+    qd, kd, vd = (t.to(dev, torch.bfloat16).requires_grad_(True) for t in (q, k, v))
+    o = pkg.attention(qd, kd, vd, causal, scale, c.to(dev), s.to(dev))
+    o.backward(g.to(dev, torch.bfloat16))
+    torch.cuda.synchronize()
+    return tuple(t.detach().float().cpu() for t in (o, qd.grad, kd.grad, vd.grad))
+
+
+SHAPES = [(4, 8, 1024, 64), (1, 8, 1024, 128), (2, 4, 512, 64), (2, 2, 256, 128), (1, 2, 200, 64), (2, 1, 77, 128),
+          (1, 2, 257, 128), (1, 1, 1, 64), (1, 1, 130, 64)]
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,N,D", SHAPES)
+def test_backward_parity(pkg, B, H, N, D, causal):
+    print(f"case B={B} H={H} N={N} D={D} causal={causal}", flush=True)
+    q, k, v, g, c, s = _case(B, H, N, D)
+    scale = 1 / math.sqrt(D)
+    o, dq, dk, dv = _gpu_fwd_bwd(pkg, q, k, v, g, causal, scale, c, s)
+    ro, _, rdq, rdk, rdv, _ = O.rope_attn_fwd_bwd_blocked(q, k, v, g, causal, scale, c, s)
+    for name, a, b in (("O", o, ro), ("dQ", dq, rdq), ("dK", dk, rdk), ("dV", dv, rdv)):
+        err = (a - b).abs()
+        print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
+        assert torch.isfinite(a).all(), name
+        assert err.max() <= TOL, name
+
+
+def test_preprocess_delta(pkg):
+    """delta = rowsum(O * dO) in fp32, straight through the C ABI."""
+    import ctypes
+    B, H, N, D = 2, 3, 333, 128
+    dev = torch.device("cuda:0")
+    o = bf16_round(seeded((B, H, N, D), 1)).to(dev, torch.bfloat16)
+    g = bf16_round(seeded((B, H, N, D), 2)).to(dev, torch.bfloat16)
+    delta = torch.full((B, H, N), float("nan"), device=dev)
+    lib = pkg._lib.load()
+    rc = lib.corope_rope_attn_bwd_preprocess(o.data_ptr(), g.data_ptr(), delta.data_ptr(), B, H, N, D,
+                                             torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, pkg._lib.last_error()
+    torch.cuda.synchronize()
+    ref = (o.double() * g.double()).sum(-1)
+    assert (delta.double() - ref).abs().max() < 1e-4
+
+
+def test_backward_identity_rotation(pkg):
+    """cos=1, sin=0: gradients of plain causal attention (the reference's embedded pytest, atol 1e-2)."""
+    B, H, N, D = 1, 2, 512, 64
+    q, k, v, g = (bf16_round(seeded((B, H, N, D), 20 + i, std=0.5)) for i in range(4))
+    one, zero = torch.ones(N, D), torch.zeros(N, D)
+    _, dq, dk, dv = _gpu_fwd_bwd(pkg, q, k, v, g, True, 0.5, one, zero)
+    qr, kr, vr = (t.clone().requires_grad_(True) for t in (q, k, v))
+    ref = torch.nn.functional.scaled_dot_product_attention(qr, kr, vr, is_causal=True, scale=0.5)
+    ref.backward(g)
+    for a, b in ((dq, qr.grad), (dk, kr.grad), (dv, vr.grad)):
+        assert (a - b).abs().max() <= 1e-2
+
+
+def test_backward_deterministic(pkg):
+    q, k, v, g, c, s = _case(2, 4, 512, 128, seed=3)
+    a = _gpu_fwd_bwd(pkg, q, k, v, g, True, 0.09, c, s)
+    b = _gpu_fwd_bwd(pkg, q, k, v, g, True, 0.09, c, s)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
