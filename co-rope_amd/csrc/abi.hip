@@ -175,7 +175,7 @@ int corope_gqa_fwd(const void* q, const void* k, const void* v, void* o, int B, 
   p.v = static_cast<const uint16_t*>(v);
   p.o = static_cast<uint16_t*>(o);
   p.sm_scale = sm_scale;
-  p.log2_theta = std::log2(theta);
+  p.theta = theta;
   p.B = B;
   p.Hq = Hq;
   p.Hkv = Hkv;

@@ -48,7 +48,7 @@ struct CoropeParams {
   const uint16_t* v;
   uint16_t* o;
   float sm_scale;
-  float log2_theta;  // inverse frequencies are exp2(-(2 d / D) * log2_theta)
+  float theta;  // RoPE base; inverse frequencies are theta^(-2d/D)
   int B, Hq, Hkv, N;
   int num_m_blocks;
 };
