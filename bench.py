@@ -1,0 +1,189 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused RoPE flash-attention hot path on one MI355X.
+
+One step = one forward + one backward of the operator (through its public torch.autograd.Function) on the
+metric shape B2 H32 N4096 D128, causal, bf16, synthetic N(0,1) inputs resident in HBM.  Prints ONE JSON line:
+whole-step TFLOP/s by the reference's FLOP model (4*B*H*N^2*D, halved for causal, x2.5 for the backward,
+rotation FLOPs not counted), the roofline of the dominant kernel from per-launch HIP-event timings, and the CPU
+oracle timed on the host cores as a baseline.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--no-cpu-baseline]
+"""
+import argparse
+import importlib
+import json
+import math
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak used for every "fraction of peak" below
+PEAK_HBM_GBS = 8000.0
+
+CONFIGS = {
+    "c2": dict(B=4, H=8, N=1024, D=64, name="C2: fused RoPE flash-attention fwd+bwd B4 H8 N1024 D64 causal bf16"),
+    "c3": dict(B=2, H=32, N=4096, D=128, name="C3: fused RoPE flash-attention fwd+bwd B2 H32 N4096 D128 causal bf16"),
+    "c4": dict(B=1, H=8, N=65536, D=128, name="C4: fused RoPE flash-attention fwd B1 H8 N65536 D128 causal bf16"),
+}
+
+
+def attention_flops(B, H, N, D, mode, causal=True):
+    total = 4.0 * B * H * N * N * D * (0.5 if causal else 1.0)
+    return total * (2.5 if mode == "bwd" else 1.0)
+
+
+def cpu_baseline():
+    """The oracle (an eager-PyTorch port of the reference's rope_attn_pytorch path) at the reference's CPU-runnable
+    configuration: B4 H8 N512 D64 fp32, forward + backward."""
+    import torch
+    from oracle import rope_attn_oracle as O
+    B, H, N, D = 4, 8, 512, 64
+    g = torch.Generator().manual_seed(0)
+    q, k, v, do = (torch.randn(B, H, N, D, generator=g) for _ in range(4))
+    cos, sin = O.precompute_freqs_cis(D, N)
+    scale = 1 / math.sqrt(D)
+
+    def step():
+        _, _, saved = O.rope_attn_forward(q, k, v, True, scale, cos, sin)
+        O.rope_attn_backward(saved, do, True, scale, cos, sin)
+
+    for _ in range(2):
+        step()
+    times = []
+    t_end = time.perf_counter() + 15.0
+    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 40):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    flops = attention_flops(B, H, N, D, "fwd") + attention_flops(B, H, N, D, "bwd")
+    return {"value": round(flops / med * 1e-12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port", "ms_per_step": round(med * 1e3, 3),
+            "sample": f"oracle fwd+bwd at B4 H8 N512 D64 fp32 causal, median of {len(times)} reps after 2 warm-ups, "
+                      f"os.cpu_count()={os.cpu_count()}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="c3", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (every (batch, head) is independent; see DESIGN.md for how "
+                 "the path would shard); run it with --gpus 1")
+
+    import torch
+    pkg = importlib.import_module("corope_amd")
+    lib = pkg._lib.load()
+    dev = torch.device("cuda:0")
+    cfg = CONFIGS[args.config]
+    B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
+    fwd_only = args.config == "c4"
+    scale = 1 / math.sqrt(D)
+    g = torch.Generator().manual_seed(42)
+    q, k, v, do = (torch.randn(B, H, N, D, generator=g).to(dev, torch.bfloat16) for _ in range(4))
+    cos, sin = pkg.precompute_freqs_cis(D, N, 10000.0, device=dev)
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+
+    def step():
+        o = pkg.attention(q, k, v, True, scale, cos, sin)
+        if not fwd_only:
+            o.backward(do)
+            q.grad = k.grad = v.grad = None
+        return o
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    f_fwd, f_bwd = attention_flops(B, H, N, D, "fwd"), (0.0 if fwd_only else attention_flops(B, H, N, D, "bwd"))
+    value = (f_fwd + f_bwd) / (ms_per_step * 1e-3) * 1e-12
+
+    # ---- per-kernel launch durations: HIP events on the launch stream, straight through the C ABI ----------------
+    stream = torch.cuda.current_stream().cuda_stream
+    o = torch.empty_like(q)
+    M = torch.empty(B, H, N, device=dev, dtype=torch.float32)
+    delta = torch.empty_like(M)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    qp, kp, vp, dop = q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr()
+    cp, sp, fs = cos.data_ptr(), sin.data_ptr(), cos.stride(0)
+    launches = [("rope_attn_fwd", lambda: lib.corope_rope_attn_fwd(qp, kp, vp, cp, sp, fs, o.data_ptr(), M.data_ptr(),
+                                                                  B, H, N, D, scale, 1, stream))]
+    if not fwd_only:
+        launches += [
+            ("rope_attn_bwd_preprocess", lambda: lib.corope_rope_attn_bwd_preprocess(o.data_ptr(), dop, delta.data_ptr(),
+                                                                                    B, H, N, D, stream)),
+            ("rope_attn_bwd_dkdv", lambda: lib.corope_rope_attn_bwd_dkdv(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),
+                                                                        cp, sp, fs, dk.data_ptr(), dv.data_ptr(),
+                                                                        B, H, N, D, scale, 1, stream)),
+            ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),
+                                                                    cp, sp, fs, dq.data_ptr(), B, H, N, D, scale, 1, stream)),
+        ]
+    durs = {n: [] for n, _ in launches}
+    for it in range(args.warmup + args.steps):
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(launches) + 1)]
+        evs[0].record()
+        for i, (name, fn) in enumerate(launches):
+            rc = fn()
+            if rc != 0:
+                sys.exit(f"{name} failed: {pkg._lib.last_error()}")
+            evs[i + 1].record()
+        torch.cuda.synchronize()
+        if it >= args.warmup:
+            for i, (name, _) in enumerate(launches):
+                durs[name].append(evs[i].elapsed_time(evs[i + 1]))
+    avg = {n: sum(d) / len(d) for n, d in durs.items()}
+    # algorithmic FLOPs per launch: forward 2 matmul units; dK/dV 4 units (the counted S recompute, dP, dV, dK);
+    # dQ 1 unit (its own S and dP recomputes are overhead on top of the model); preprocess is HBM-bound.
+    unit = 2.0 * B * H * N * N * D * 0.5
+    alg = {"rope_attn_fwd": 2 * unit, "rope_attn_bwd_dkdv": 4 * unit, "rope_attn_bwd_dq": 1 * unit}
+    kernels = {}
+    for n, ms in avg.items():
+        if n in alg:
+            tf = alg[n] / (ms * 1e-3) * 1e-12
+            kernels[n] = {"ms": round(ms, 4), "tflops": round(tf, 1), "frac_of_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
+        else:
+            by = 2.0 * B * H * N * D * 2 + B * H * N * 4
+            kernels[n] = {"ms": round(ms, 4), "gbs": round(by / (ms * 1e-3) * 1e-9, 1),
+                          "frac_of_hbm_peak": round(by / (ms * 1e-3) * 1e-9 / PEAK_HBM_GBS, 4)}
+    dom = max((n for n in avg if n in alg), key=lambda n: avg[n])
+    dom_tf = alg[dom] / (avg[dom] * 1e-3) * 1e-12
+    roofline = {"bound": "mfma", "kernel": dom, "achieved": round(dom_tf, 1), "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(dom_tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "avg_launch_ms": round(avg[dom], 4)}
+    fwd_tf = alg["rope_attn_fwd"] / (avg["rope_attn_fwd"] * 1e-3) * 1e-12
+    out = {
+        "metric": "RoPE-attn fwd+bwd TFLOPS & % bf16 MFMA peak, B2 H32 N4096 D128 causal",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": cfg["name"], "B": B, "H": H, "N": N, "D": D, "causal": True,
+                   "sm_scale": "1/sqrt(D)", "rope_base": 10000.0},
+        "frac_of_bf16_peak": round(value / PEAK_BF16_TFLOPS, 4),
+        "fwd": {"ms": round(avg["rope_attn_fwd"], 4), "tflops": round(fwd_tf, 1),
+                "frac_of_peak": round(fwd_tf / PEAK_BF16_TFLOPS, 4)},
+        "kernels": kernels, "roofline": roofline,
+    }
+    if not fwd_only:
+        bwd_ms = avg["rope_attn_bwd_preprocess"] + avg["rope_attn_bwd_dkdv"] + avg["rope_attn_bwd_dq"]
+        bwd_tf = f_bwd / (bwd_ms * 1e-3) * 1e-12
+        out["bwd"] = {"ms": round(bwd_ms, 4), "tflops": round(bwd_tf, 1), "frac_of_peak": round(bwd_tf / PEAK_BF16_TFLOPS, 4)}
+    out["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,137 @@
+"""CPU-only checks of the drop-in boundary: the shared library loads, exports every symbol the header declares,
+validates its arguments before touching HIP, and the Python layer keeps the reference's call surface."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "corope_amd.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(corope_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_typed(pkg):
+    lib = pkg._lib.load()
+    names = _declared_symbols()
+    assert "corope_rope_attn_fwd" in names and "corope_gqa_fwd" in names and len(names) >= 10
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+    assert sorted(pkg._lib.SIGNATURES) == names, "ctypes table and header disagree"
+    assert lib.corope_amd_version() == pkg._lib.ABI_VERSION
+
+
+def test_header_cites_reference_for_each_entry_point():
+    text = open(HEADER).read()
+    for fn in ("corope_rope_attn_fwd", "corope_rope_attn_bwd_preprocess", "corope_rope_attn_bwd_dkdv",
+               "corope_rope_attn_bwd_dq", "corope_rope_attn_bwd", "corope_gqa_fwd"):
+        before = text[:text.index(f"int {fn}(")]
+        comment = before[before.rindex("/*"):]
+        assert re.search(r"\.py:\d+", comment), f"{fn}: no reference file:line in its comment"
+
+
+@pytest.mark.parametrize("args,code", [
+    ((2, 32, 4096, 128, 128, 0.088, 0), 0),
+    ((4, 8, 1024, 64, 32, 0.125, 1), 0),
+    ((1, 1, 77, 128, 64, 1.0, 0), 0),
+    ((0, 8, 128, 64, 64, 1.0, 0), -1),
+    ((1, 8, -5, 64, 64, 1.0, 0), -1),
+    ((1, 8, 128, 32, 32, 1.0, 0), -2),
+    ((1, 8, 128, 256, 256, 1.0, 0), -2),
+    ((1, 8, 128, 64, 16, 1.0, 0), -1),      # table narrower than D/2
+    ((1, 8, 128, 64, 66, 1.0, 0), -1),      # row stride not a multiple of 4 floats
+    ((1, 8, 128, 64, 64, 0.0, 0), -1),
+    ((1, 8, 128, 64, 64, float("nan"), 0), -1),
+])
+def test_rope_attn_check_codes(pkg, args, code):
+    lib = pkg._lib.load()
+    assert lib.corope_rope_attn_check(*args) == code
+    assert (pkg._lib.last_error() == "") == (code == 0)
+
+
+@pytest.mark.parametrize("args,code", [
+    ((2, 32, 8, 4096, 128, 0.088, 10000.0), 0),
+    ((1, 7, 1, 65, 64, 1.0, 100.0), 0),
+    ((1, 6, 4, 64, 64, 1.0, 1e4), -1),      # Hq not a multiple of Hkv
+    ((1, 18, 2, 64, 64, 1.0, 1e4), -2),     # group of 9
+    ((1, 4, 2, 64, 32, 1.0, 1e4), -2),
+    ((1, 4, 2, 64, 64, 1.0, 0.0), -1),
+    ((1, 4, 2, 0, 64, 1.0, 1e4), -1),
+])
+def test_corope_check_codes(pkg, args, code):
+    assert pkg._lib.load().corope_gqa_check(*args) == code
+
+
+def test_null_and_misaligned_pointers_are_rejected_before_any_launch(pkg):
+    lib = pkg._lib.load()
+    buf = ctypes.create_string_buffer(4096)
+    base = (ctypes.addressof(buf) + 15) & ~15
+    ok, odd = base, base + 2
+    rc = lib.corope_rope_attn_fwd(ok, ok, None, ok, ok, 64, ok, ok, 1, 1, 8, 64, 1.0, 1, None)
+    assert rc == -1 and "null" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_fwd(ok, odd, ok, ok, ok, 64, ok, ok, 1, 1, 8, 64, 1.0, 1, None)
+    assert rc == -3 and "aligned" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_bwd_preprocess(ok, None, ok, 1, 1, 8, 64, None)
+    assert rc == -1
+    rc = lib.corope_gqa_fwd(ok, ok, ok, odd, 1, 2, 1, 8, 64, 1.0, 1e4, None)
+    assert rc == -3
+    with pytest.raises(ValueError):
+        pkg._lib.check(rc, "corope_gqa_fwd")
+
+
+def test_python_surface_matches_reference_order(pkg):
+    # reference: forward(ctx, q, k, v, causal, sm_scale, freqs_cos, freqs_sin, warp_specialize=True)
+    from importlib import import_module
+    ra = import_module("co-rope_amd.rope_attn")
+    cg = import_module("co-rope_amd.corope_gqa")
+    assert list(inspect.signature(ra._FusedRopeAttn.forward).parameters) == [
+        "ctx", "q", "k", "v", "causal", "sm_scale", "freqs_cos", "freqs_sin", "warp_specialize"]
+    assert list(inspect.signature(cg._CoRopeGqaAttn.forward).parameters) == [
+        "ctx", "q", "k", "v", "causal", "sm_scale", "theta", "warp_specialize"]
+    assert list(inspect.signature(pkg.fused_rope_attn).parameters) == [
+        "q", "k", "v", "freqs_cos", "freqs_sin", "causal", "sm_scale"]
+
+
+def test_host_validation_raises_without_a_gpu(pkg):
+    q = torch.zeros(1, 2, 16, 64, dtype=torch.bfloat16)
+    c = torch.ones(16, 64)
+    with pytest.raises(ValueError):          # CPU tensors: there is no CPU fallback
+        pkg.attention(q, q, q, True, 0.125, c, c)
+    with pytest.raises(AssertionError):      # mismatched head dims, as the reference asserts
+        pkg.attention(q, q[..., :32], q, True, 0.125, c, c)
+    with pytest.raises(ValueError):
+        pkg.attention(torch.zeros(1, 2, 16, 32, dtype=torch.bfloat16), torch.zeros(1, 2, 16, 32, dtype=torch.bfloat16),
+                      torch.zeros(1, 2, 16, 32, dtype=torch.bfloat16), True, 0.1, c, c)
+    k = torch.zeros(1, 1, 16, 64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        pkg.corope_attention(q, k, k, False, 1.0, 1e4)          # non-causal
+    with pytest.raises(ValueError):
+        pkg.corope_attention(q, k, k[:, :, :8], True, 1.0, 1e4)  # k/v shape mismatch
+    with pytest.raises(ValueError):
+        pkg.corope_attention(q[0], k[0], k[0], True, 1.0, 1e4)   # rank
+    with pytest.raises(ValueError):
+        pkg.corope_attention(torch.zeros(1, 3, 16, 64, dtype=torch.bfloat16), torch.zeros(1, 2, 16, 64, dtype=torch.bfloat16),
+                             torch.zeros(1, 2, 16, 64, dtype=torch.bfloat16), True, 1.0, 1e4)
+    with pytest.raises(ValueError):
+        pkg.corope_attention(q, k, k, True, 1.0, 1e4)            # CPU tensors
+
+
+def test_freqs_match_oracle(pkg):
+    from oracle import rope_attn_oracle as O
+    c, s = pkg.precompute_freqs_cis(128, 300, 10000.0, device="cpu")
+    rc, rs = O.precompute_freqs_cis(128, 300, 10000.0)
+    assert torch.equal(c, rc) and torch.equal(s, rs) and c.shape == (300, 128)
+
+
+def test_missing_library_fails_loudly(pkg, monkeypatch):
+    monkeypatch.setattr(pkg._lib, "_lib", None)
+    monkeypatch.setattr(pkg._lib, "LIB_PATH", "/nonexistent/libcorope_amd.so")
+    with pytest.raises(pkg._lib.CoRopeLibraryError):
+        pkg._lib.load()
