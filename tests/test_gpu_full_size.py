@@ -1,0 +1,93 @@
+"""Parity at the benchmark's full sizes (C3, C4, C5), checked on sampled query rows (attention rows are independent
+given K and V), on whole heads for the gradients, and through size-independent properties."""
+import math
+
+import pytest
+import torch
+
+from conftest import bf16_round, seeded
+from oracle import corope_gqa_oracle as C
+from oracle import rope_attn_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+LN2 = math.log(2.0)
+
+
+def _rows(N, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    r = torch.randperm(N, generator=g)[:n]
+    return torch.unique(torch.cat([r, torch.tensor([0, 1, 63, 64, N // 2, N - 2, N - 1])]))
+
+
+def test_c3_forward_backward(pkg):
+    """B2 H32 N4096 D128 causal: O/LSE on sampled rows of every head; dQ/dK/dV on whole heads (a subset of heads)."""
+    B, H, N, D = 2, 32, 4096, 128
+    dev = torch.device("cuda:0")
+    q, k, v, g = (bf16_round(seeded((B, H, N, D), 42 + i)) for i in range(4))
+    c, s = O.precompute_freqs_cis(D, N)
+    scale = 1 / math.sqrt(D)
+    qd, kd, vd = (t.to(dev, torch.bfloat16).requires_grad_(True) for t in (q, k, v))
+    o, M = pkg.rope_attn_forward_with_lse(qd.detach(), kd.detach(), vd.detach(), True, scale, c.to(dev), s.to(dev))
+    out = pkg.attention(qd, kd, vd, True, scale, c.to(dev), s.to(dev))
+    out.backward(g.to(dev, torch.bfloat16))
+    torch.cuda.synchronize()
+    assert torch.equal(out.detach(), o)
+    o, M = o.float().cpu(), M.cpu()
+    rows = _rows(N, 96, 1)
+    ro, rl = O.rope_attn_forward_blocked(q, k, v, True, scale, c, s, rows=rows)
+    e_o, e_l = (o[:, :, rows] - ro).abs().max().item(), (M[:, :, rows] * LN2 - rl).abs().max().item()
+    print(f"  C3 O max-abs {e_o:.3e}, LSE max-abs {e_l:.3e} on {rows.numel()} rows x {B * H} heads", flush=True)
+    assert e_o <= TOL and e_l <= TOL
+    assert torch.equal(o[:, :, 0], v[:, :, 0])                                   # row 0 attends to key 0 only
+    dq, dk, dv = (t.grad.float().cpu() for t in (qd, kd, vd))
+    for (b, h) in ((0, 0), (1, 17), (1, 31)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        _, _, rdq, rdk, rdv, _ = O.rope_attn_fwd_bwd_blocked(q[sl], k[sl], v[sl], g[sl], True, scale, c, s)
+        for name, a, r in (("dQ", dq[sl], rdq), ("dK", dk[sl], rdk), ("dV", dv[sl], rdv)):
+            err = (a - r).abs()
+            print(f"  C3 head ({b},{h}) {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e}", flush=True)
+            assert err.max() <= TOL, name
+    # linearity of the backward in dO: grad(2 dO) == 2 grad(dO) exactly (power-of-two scaling commutes with rounding)
+    qd.grad = kd.grad = vd.grad = None
+    out2 = pkg.attention(qd, kd, vd, True, scale, c.to(dev), s.to(dev))
+    out2.backward((2 * g).to(dev, torch.bfloat16))
+    torch.cuda.synchronize()
+    assert torch.equal(qd.grad.float().cpu(), 2 * dq) and torch.equal(vd.grad.float().cpu(), 2 * dv)
+
+
+def test_c4_long_context_forward(pkg):
+    """B1 H8 N65536 D128 causal forward on sampled rows."""
+    B, H, N, D = 1, 8, 65536, 128
+    dev = torch.device("cuda:0")
+    q, k, v = (bf16_round(seeded((B, H, N, D), 7 + i)) for i in range(3))
+    c, s = O.precompute_freqs_cis(D, N)
+    scale = 1 / math.sqrt(D)
+    o, M = pkg.rope_attn_forward_with_lse(q.to(dev, torch.bfloat16), k.to(dev, torch.bfloat16),
+                                          v.to(dev, torch.bfloat16), True, scale, c.to(dev), s.to(dev))
+    torch.cuda.synchronize()
+    o, M = o.float().cpu(), M.cpu()
+    rows = _rows(N, 48, 2)
+    ro, rl = O.rope_attn_forward_blocked(q, k, v, True, scale, c, s, rows=rows)
+    e_o, e_l = (o[:, :, rows] - ro).abs().max().item(), (M[:, :, rows] * LN2 - rl).abs().max().item()
+    print(f"  C4 O max-abs {e_o:.3e}, LSE max-abs {e_l:.3e} on {rows.numel()} rows x {H} heads", flush=True)
+    assert torch.isfinite(o).all() and e_o <= TOL and e_l <= TOL
+
+
+def test_c5_corope_forward(pkg):
+    """B2 Hq32 Hkv8 N4096 D128 Co-RoPE forward on sampled rows of every head."""
+    B, Hq, Hkv, N, D = 2, 32, 8, 4096, 128
+    dev = torch.device("cuda:0")
+    q = bf16_round(seeded((B, Hq, N, D), 3))
+    k, v = bf16_round(seeded((B, Hkv, N, D), 4)), bf16_round(seeded((B, Hkv, N, D), 5))
+    scale = 1 / math.sqrt(D)
+    o = pkg.corope_attention(q.to(dev, torch.bfloat16), k.to(dev, torch.bfloat16), v.to(dev, torch.bfloat16), True,
+                             scale, 10000.0)
+    torch.cuda.synchronize()
+    o = o.float().cpu()
+    rows = _rows(N, 9, 3)
+    ref = C.corope_gqa_forward_rows(q, k, v, True, scale, 10000.0, rows, torch.float32, row_block=16)
+    err = (o[:, :, rows] - ref).abs()
+    print(f"  C5 O max-abs {err.max():.3e} mean-abs {err.mean():.3e} on {rows.numel()} rows x {B * Hq} heads", flush=True)
+    assert torch.isfinite(o).all() and err.max() <= TOL
+    assert torch.equal(o[:, :, 0], v.repeat_interleave(Hq // Hkv, 1)[:, :, 0])
