@@ -68,11 +68,15 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
 // ---- LDS tile layouts -----------------------------------------------------------------------------
-// Row-major tile [rows][D] of bf16 with 16 bytes of padding per row: 16 consecutive rows read at the
-// same column land in 16 different 16-byte bank groups.
-template <int D>
+// Row-major tile [rows][D] of bf16 with PAD elements of padding per row.
+//   PAD = 8  (16 bytes): 16 consecutive rows read at the same column with 16-byte reads land in 16 different
+//                        bank groups -- the layout for tiles read row-wise as MFMA operands;
+//   PAD = 32 (64 bytes): the row stride is 16 dwords past a multiple of 64, so the 4 rows x 32 bytes a 16-lane
+//                        block touches in a transposing read (and the 8 rows of a whole wave) spread over all
+//                        banks -- the layout for tiles read only through load_a_trans.
+template <int D, int PAD = 8>
 struct RowTile {
-  static constexpr int kStride = D + 8;  // elements
+  static constexpr int kStride = D + PAD;  // elements
   static constexpr int bytes(int rows) { return rows * kStride * 2; }
   __device__ static __forceinline__ int off(int row, int col) { return row * kStride + col; }
 };
@@ -122,6 +126,44 @@ struct RotStage {
       c[it][1] = *reinterpret_cast<const f32x4*>(cp + 4);
       s[it][0] = *reinterpret_cast<const f32x4*>(sp);
       s[it][1] = *reinterpret_cast<const f32x4*>(sp + 4);
+    }
+  }
+
+  // Loads iterations [it0, it1) only (same addressing as load()).
+  __device__ __forceinline__ void load_part(int it0, int it1, const uint16_t* __restrict__ src,
+                                            const float* __restrict__ cosp, const float* __restrict__ sinp,
+                                            int64_t fstride, int row0, int n_rows) {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      if (it < it0 || it >= it1) continue;
+      int u = threadIdx.x + it * NT;
+      if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
+      int r = u / kChunks, ch = u % kChunks;
+      int row = min(row0 + r, n_rows - 1);
+      const uint16_t* p = src + (int64_t)row * D + ch * 8;
+      x1[it] = *reinterpret_cast<const u32x4*>(p);
+      x2[it] = *reinterpret_cast<const u32x4*>(p + D / 2);
+      const float* cp = cosp + (int64_t)row * fstride + ch * 8;
+      const float* sp = sinp + (int64_t)row * fstride + ch * 8;
+      c[it][0] = *reinterpret_cast<const f32x4*>(cp);
+      c[it][1] = *reinterpret_cast<const f32x4*>(cp + 4);
+      s[it][0] = *reinterpret_cast<const f32x4*>(sp);
+      s[it][1] = *reinterpret_cast<const f32x4*>(sp + 4);
+    }
+  }
+
+  // Rotates and stores iterations [it0, it1) only.
+  __device__ __forceinline__ void store_rows_part(int it0, int it1, uint16_t* lds) const {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      if (it < it0 || it >= it1) continue;
+      int u = threadIdx.x + it * NT;
+      if (kUnits % NT != 0 && u >= kUnits) continue;
+      int r = u / kChunks, ch = u % kChunks;
+      u32x4 y1, y2;
+      rotate(it, y1, y2);
+      *reinterpret_cast<u32x4*>(lds + RowTile<D>::off(r, ch * 8)) = y1;
+      *reinterpret_cast<u32x4*>(lds + RowTile<D>::off(r, D / 2 + ch * 8)) = y2;
     }
   }
 
@@ -211,7 +253,7 @@ struct TransStage {
 };
 
 // ---- staging: a ROWS x D tile copied row-major (no rotation) -------------------------------------------
-template <int D, int ROWS, int NT>
+template <int D, int ROWS, int NT, int PAD = 8>
 struct CopyStage {
   static constexpr int kChunks = D / 8;  // 16-byte units per row
   static constexpr int kUnits = ROWS * kChunks;
@@ -232,7 +274,27 @@ struct CopyStage {
     for (int it = 0; it < kIters; ++it) {
       int u = threadIdx.x + it * NT;
       if (kUnits % NT != 0 && u >= kUnits) continue;
-      *reinterpret_cast<u32x4*>(lds + RowTile<D>::off(u / kChunks, (u % kChunks) * 8)) = x[it];
+      *reinterpret_cast<u32x4*>(lds + RowTile<D, PAD>::off(u / kChunks, (u % kChunks) * 8)) = x[it];
+    }
+  }
+  // Iterations [it0, it1) only.
+  __device__ __forceinline__ void load_part(int it0, int it1, const uint16_t* __restrict__ src, int row0, int n_rows) {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      if (it < it0 || it >= it1) continue;
+      int u = threadIdx.x + it * NT;
+      if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
+      int row = min(row0 + u / kChunks, n_rows - 1);
+      x[it] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * D + (u % kChunks) * 8);
+    }
+  }
+  __device__ __forceinline__ void store_rows_part(int it0, int it1, uint16_t* lds) const {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it) {
+      if (it < it0 || it >= it1) continue;
+      int u = threadIdx.x + it * NT;
+      if (kUnits % NT != 0 && u >= kUnits) continue;
+      *reinterpret_cast<u32x4*>(lds + RowTile<D, PAD>::off(u / kChunks, (u % kChunks) * 8)) = x[it];
     }
   }
 };

@@ -3,38 +3,95 @@
 // Device counterpart of the reference's _attn_fwd / _attn_fwd_inner
 // (fused-rope/fused_rope_attn.py:222-320, :48-138).
 //
-// One workgroup owns BLOCK_M = 32 * NWAVES query rows of one (batch, head); each wave owns 32 of them.
+// One workgroup owns 256 query rows of one (batch, head); each of its 8 waves owns 32 of them.
 // Scores are produced transposed, S^T = K_r Q_r^T, with 32x32x16 bf16 MFMAs: the rotated K tile is the A
 // operand (read from LDS), the rotated Q rows are the B operand (registers, loaded and rotated once).  In
 // the 32x32 accumulator every lane then holds 16 keys of ONE query, so the online-softmax row statistics
 // are a per-lane reduction plus one exchange between the two halves of the wave, and the bf16 P^T values
-// are already laid out as the B operand of O^T += V^T P^T (V^T read from a transposed LDS tile).
+// are already laid out as the B operand of O^T += V^T P^T (V tile staged row-major, read with the transposing
+// LDS load).
 //
 // K tiles are rotated while they are staged global -> registers -> LDS, once per workgroup per tile
 // (the reference re-rotates per program: :82-99); the next tile's global loads are issued before the
-// current tile's MFMAs and written to the other LDS buffer afterwards (one barrier per tile).
+// current tile's MFMAs and written to the next LDS buffer afterwards (one barrier per tile).
 #include "common.hpp"
 #include "kernels.hpp"
 
 namespace corope {
 
-template <int D, int NWAVES, int BLOCK_N>
+// Workgroup = 8 waves x 32 query rows = 256 rows, two waves per SIMD.
+//
+// Issue schedule.  VALU work only overlaps an MFMA that is already in flight, so a wave that mixes independent VALU
+// instructions into its MFMA stream keeps the matrix pipe busier than one that runs an MFMA phase followed by a
+// VALU phase.  A 64-key tile is therefore consumed as two 32-key halves in four slots of 8 MFMAs each, and every
+// slot carries the VALU work of another stage in the same basic block for the instruction scheduler to mix in:
+//     slot A:  S^T(half 0)          +  rotate K of tile t+1 and write it to LDS, refill the K staging registers
+//     slot B:  S^T(half 1)          +  online softmax of half 0
+//     slot C:  O^T += V^T P^T(h0)   +  online softmax of half 1
+//     slot D:  O^T += V^T P^T(h1)   +  write V of tile t+1 to LDS, refill the V staging registers
+// Scheduling barriers separate the slots and pin the operand prefetches ahead of the MFMAs that use them.
+constexpr int kFwdWaves = 8;
+constexpr int kFwdStages = 2;
+
+template <int D, int BLOCK_N>
 struct FwdCfg {
-  static constexpr int kThreads = NWAVES * kWave;
-  static constexpr int kBlockM = NWAVES * 32;
-  static constexpr int kKBytes = RowTile<D>::bytes(BLOCK_N);
-  static constexpr int kVBytes = TransTile<BLOCK_N>::bytes(D);
+  static constexpr int kThreads = kFwdWaves * kWave;
+  static constexpr int kBlockM = kFwdWaves * 32;
+  static constexpr int kVPad = 32;                                       // V is read only through load_a_trans
+  static constexpr int kKBytes = RowTile<D>::bytes(BLOCK_N);             // K tile, row-major, read row-wise
+  static constexpr int kVBytes = RowTile<D, kVPad>::bytes(BLOCK_N);      // V tile, row-major, read transposed
   static constexpr int kStageBytes = kKBytes + kVBytes;
-  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr int kLdsBytes = kFwdStages * kStageBytes;
 };
 
-template <int D, int NWAVES, int BLOCK_N, bool CAUSAL>
-__global__ __launch_bounds__(NWAVES* kWave) void rope_attn_fwd_kernel(FwdParams p) {
-  using Cfg = FwdCfg<D, NWAVES, BLOCK_N>;
+// State of the online softmax while one 32-key half is processed.
+struct SoftmaxHalf {
+  float mt;     // maximum of the half's raw scores, then the new running maximum
+  float ms;     // new running maximum in the base-2 scaled domain
+  float alpha;  // factor that brings the old accumulators to the new maximum
+  float lsum;   // this lane's share of the half's denominator
+};
+
+// Piece `step` of `n_steps` of the softmax of one half (16 raw scores per lane -> 8 bf16 pairs = two B operands).
+// Step 0 reduces the maximum, step 1 fixes the new running maximum, the others exponentiate.
+__device__ __forceinline__ void softmax_piece(int step, int n_steps, const f32x16& sacc, u32x4 (&pb)[2], SoftmaxHalf& st,
+                                              float m_run, float scale) {
+  if (step == 0) {
+    float mt = fmaxf(sacc[0], sacc[1]);
+#pragma unroll
+    for (int i = 2; i < 16; i += 2) mt = fmaxf(fmaxf(mt, sacc[i]), sacc[i + 1]);
+    st.mt = mt;
+  } else if (step == 1) {
+    st.mt = fmaxf(m_run, half_max(st.mt));
+    st.ms = st.mt * scale;
+    st.alpha = fast_exp2(m_run * scale - st.ms);
+    st.lsum = 0.f;
+  } else {
+    const int n = n_steps - 2;
+    const int lo = (step - 2) * 8 / n, hi = (step - 1) * 8 / n;
+    const bf16x2 ones = __builtin_bit_cast(bf16x2, 0x3f803f80u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (j < lo || j >= hi) continue;
+      float p0 = fast_exp2(sacc[2 * j] * scale - st.ms);
+      float p1 = fast_exp2(sacc[2 * j + 1] * scale - st.ms);
+      uint32_t w = pack_bf16(p0, p1);
+      // the denominator sums the ROUNDED probabilities, i.e. exactly the weights the PV product uses
+      st.lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, st.lsum, false);
+      pb[j / 4][j % 4] = w;
+    }
+  }
+}
+
+template <int D, int BLOCK_N, bool CAUSAL>
+__global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdParams p) {
+  using Cfg = FwdCfg<D, BLOCK_N>;
+  static_assert(BLOCK_N == 64, "the slot schedule is written for two 32-key halves");
   constexpr int NT = Cfg::kThreads;
-  constexpr int KC = D / 16;        // contraction chunks of QK^T
-  constexpr int NKB = BLOCK_N / 32; // 32-key blocks per tile
+  constexpr int KC = D / 16;        // contraction chunks of QK^T = MFMAs per S^T half
   constexpr int NDB = D / 32;       // 32-column blocks of O
+  constexpr int NPV = 2 * NDB;      // MFMAs per PV half
+  constexpr int LSV = RowTile<D, Cfg::kVPad>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
   // Heaviest query blocks first; consecutive workgroup ids walk over (batch, head) so that all blocks of one
@@ -54,34 +111,14 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_fwd_kernel(FwdParams 
                              : (N + BLOCK_N - 1) / BLOCK_N;
 
   RotStage<D, BLOCK_N, NT> kst;
-  TransStage<D, BLOCK_N, NT> vst;
+  CopyStage<D, BLOCK_N, NT, Cfg::kVPad> vst;
   kst.load(kg, p.cos, p.sin, p.fstride, 0, N);
   vst.load(vg, 0, N);
 
   // ---- Q rows of this wave: load, rotate, keep as the B operand ------------------------------------------
   const int q_row = m0 + wave * 32 + lq;           // absolute query index of this lane
   u32x4 qb[KC];
-  {
-    const int qr = min(q_row, N - 1);
-    const uint16_t* qp = qg + (int64_t)qr * D + 8 * lh;
-    const float* cp = p.cos + (int64_t)qr * p.fstride + 8 * lh;
-    const float* sp = p.sin + (int64_t)qr * p.fstride + 8 * lh;
-#pragma unroll
-    for (int kc = 0; kc < KC / 2; ++kc) {
-      u32x4 x1 = *reinterpret_cast<const u32x4*>(qp + 16 * kc);
-      u32x4 x2 = *reinterpret_cast<const u32x4*>(qp + D / 2 + 16 * kc);
-      f32x4 c0 = *reinterpret_cast<const f32x4*>(cp + 16 * kc), c1 = *reinterpret_cast<const f32x4*>(cp + 16 * kc + 4);
-      f32x4 s0 = *reinterpret_cast<const f32x4*>(sp + 16 * kc), s1 = *reinterpret_cast<const f32x4*>(sp + 16 * kc + 4);
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        float a0 = bf16_lo(x1[w]), a1 = bf16_hi(x1[w]), b0 = bf16_lo(x2[w]), b1 = bf16_hi(x2[w]);
-        float cc0 = w < 2 ? c0[2 * w] : c1[2 * w - 4], cc1 = w < 2 ? c0[2 * w + 1] : c1[2 * w - 3];
-        float ss0 = w < 2 ? s0[2 * w] : s1[2 * w - 4], ss1 = w < 2 ? s0[2 * w + 1] : s1[2 * w - 3];
-        qb[kc][w] = pack_bf16(a0 * cc0 - b0 * ss0, a1 * cc1 - b1 * ss1);
-        qb[kc + KC / 2][w] = pack_bf16(b0 * cc0 + a0 * ss0, b1 * cc1 + a1 * ss1);
-      }
-    }
-  }
+  load_b_rows<D, true>(qb, qg, p.cos, p.sin, p.fstride, min(q_row, N - 1));
 
   f32x16 oacc[NDB];
 #pragma unroll
@@ -89,10 +126,17 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_fwd_kernel(FwdParams 
   float m_run = -INFINITY;   // running row maximum of the raw scores (this lane's query)
   float l_run = 0.f;         // this lane's share of the running denominator
 
-  auto ks = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
-  auto vs = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes + Cfg::kKBytes); };
+  auto ks = [&](int t) { return reinterpret_cast<uint16_t*>(smem + (t % kFwdStages) * Cfg::kStageBytes); };
+  auto vs = [&](int t) {
+    return reinterpret_cast<uint16_t*>(smem + (t % kFwdStages) * Cfg::kStageBytes + Cfg::kKBytes);
+  };
+  // Staging registers hold tile t+1 during iteration t: it is written to its LDS buffer during the iteration and the
+  // registers are refilled at once with tile t+2, so a global load has a whole iteration to land.  Row indices
+  // are clamped, which makes tiles past the end harmless to load and store.
   kst.store_rows(ks(0));
-  vst.store(vs(0));
+  vst.store_rows(vs(0));
+  kst.load(kg, p.cos, p.sin, p.fstride, BLOCK_N, N);
+  vst.load(vg, BLOCK_N, N);
   __syncthreads();
 
   const float scale = p.qk_scale;
@@ -100,81 +144,94 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_fwd_kernel(FwdParams 
 
   for (int t = 0; t < n_tiles; ++t) {
     const int n0 = t * BLOCK_N;
-    const int cur = t & 1;
-    if (t + 1 < n_tiles) {
-      kst.load(kg, p.cos, p.sin, p.fstride, n0 + BLOCK_N, N);
-      vst.load(vg, n0 + BLOCK_N, N);
-    }
-    // Tiles entirely above this wave's diagonal contribute nothing to it.
-    const bool active = !CAUSAL || n0 <= wave_q_hi;
-    if (active) {
-      // ---- S^T = K_r Q_r^T -----------------------------------------------------------------------------
-      f32x16 sacc[NKB];
+    const uint16_t* kt = ks(t) + RowTile<D>::off(lq, 8 * lh);
+    const uint16_t* vt = vs(t);
+    auto stage_k = [&]() {
+      kst.store_rows(ks(t + 1));
+      kst.load(kg, p.cos, p.sin, p.fstride, n0 + 2 * BLOCK_N, N);
+    };
+    auto stage_v = [&]() {
+      vst.store_rows(vs(t + 1));
+      vst.load(vg, n0 + 2 * BLOCK_N, N);
+    };
+    auto k_operand = [&](int half, int kc) {
+      return *reinterpret_cast<const u32x4*>(kt + RowTile<D>::off(half * 32, 16 * kc));
+    };
+    auto v_operand = [&](int half, int i) {  // MFMA i of a PV half: output block i % NDB, 16-key chunk i / NDB
+      return load_a_trans(vt, LSV, half * 32 + 16 * (i / NDB), (i % NDB) * 32);
+    };
+    auto mask_scores = [&](f32x16& sacc, int half) {
 #pragma unroll
-      for (int kb = 0; kb < NKB; ++kb) {
-        sacc[kb] = f32x16{0};
-        const uint16_t* kp = ks(cur) + RowTile<D>::off(kb * 32 + lq, 8 * lh);
-#pragma unroll
-        for (int kc = 0; kc < KC; ++kc) {
-          u32x4 a = *reinterpret_cast<const u32x4*>(kp + 16 * kc);
-          sacc[kb] = mfma32(a, qb[kc], sacc[kb]);
-        }
+      for (int i = 0; i < 16; ++i) {
+        int key = n0 + half * 32 + acc_row(i, lh);
+        if (CAUSAL ? key > q_row : key >= N) sacc[i] = -INFINITY;
       }
-      // ---- masking (diagonal tiles, ragged tail) -----------------------------------------------------
-      const bool need_mask = (CAUSAL && n0 + BLOCK_N - 1 > wave_q_lo) || (!CAUSAL && n0 + BLOCK_N > N);
-      if (need_mask) {
-#pragma unroll
-        for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            int key = n0 + kb * 32 + acc_row(i, lh);
-            bool dead = CAUSAL ? key > q_row : key >= N;
-            if (dead) sacc[kb][i] = -INFINITY;
-          }
-      }
-      // ---- online softmax (base 2) -----------------------------------------------------------------
-      float mt = sacc[0][0];
-#pragma unroll
-      for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mt = fmaxf(mt, sacc[kb][i]);
-      mt = half_max(mt);
-      const float m_new = fmaxf(m_run, mt);
-      const float ms = m_new * scale;
-      const float alpha = fast_exp2(m_run * scale - ms);
-      m_run = m_new;
-      float lsum = 0.f;
-      u32x4 pb[BLOCK_N / 16];
-#pragma unroll
-      for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; i += 2) {
-          float p0 = fast_exp2(sacc[kb][i] * scale - ms);
-          float p1 = fast_exp2(sacc[kb][i + 1] * scale - ms);
-          lsum += p0 + p1;
-          pb[2 * kb + i / 8][(i % 8) / 2] = pack_bf16(p0, p1);
-        }
-      l_run = l_run * alpha + lsum;
+    };
+    auto rescale = [&](float alpha) {
       if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
 #pragma unroll
           for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
       }
-      // ---- O^T += V^T P^T ------------------------------------------------------------------------------
+    };
+
+    // Tiles entirely above this wave's diagonal contribute nothing to it; the wave still stages its share.
+    const bool active = !CAUSAL || n0 <= wave_q_hi;
+    const bool need_mask = (CAUSAL && n0 + BLOCK_N - 1 > wave_q_lo) || (!CAUSAL && n0 + BLOCK_N > N);
+    if (active) {
+      f32x16 s0 = f32x16{0}, s1 = f32x16{0};
+      u32x4 pb0[2], pb1[2];
+      SoftmaxHalf st0, st1;
+      u32x4 a[KC];  // A operands, fetched one slot ahead of the MFMAs that consume them
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) {
-        const uint16_t* vp = vs(cur) + (db * 32 + lq) * TransTile<BLOCK_N>::kStride + 8 * lh;
+      for (int kc = 0; kc < KC; ++kc) a[kc] = k_operand(0, kc);
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- slot A: S^T(half 0), K staging on the side --------------------------------------------------------
 #pragma unroll
-        for (int c = 0; c < BLOCK_N / 16; ++c) {
-          u32x4 a = *reinterpret_cast<const u32x4*>(vp + 16 * c);
-          oacc[db] = mfma32(a, pb[c], oacc[db]);
-        }
+      for (int kc = 0; kc < KC; ++kc) {
+        s0 = mfma32(a[kc], qb[kc], s0);
+        a[kc] = k_operand(1, kc);
+        if (kc == 0) stage_k();
       }
-    }
-    if (t + 1 < n_tiles) {
-      kst.store_rows(ks(cur ^ 1));
-      vst.store(vs(cur ^ 1));
+      __builtin_amdgcn_sched_barrier(0);
+      if (need_mask) mask_scores(s0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- slot B: S^T(half 1), softmax of half 0 between the MFMAs ---------------------------------------------
+#pragma unroll
+      for (int kc = 0; kc < KC; ++kc) {
+        s1 = mfma32(a[kc], qb[kc], s1);
+        softmax_piece(kc, KC, s0, pb0, st0, m_run, scale);
+      }
+      m_run = st0.mt;
+      l_run = l_run * st0.alpha + st0.lsum;
+      rescale(st0.alpha);
+      if (need_mask) mask_scores(s1, 1);
+      u32x4 av[NDB];  // transposed V operands, one 16-key chunk ahead
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) av[db] = v_operand(0, db);
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- slot C: O^T += V^T P^T(half 0), softmax of half 1 between the MFMAs -----------------------------------
+#pragma unroll
+      for (int i = 0; i < NPV; ++i) {
+        oacc[i % NDB] = mfma32(av[i % NDB], pb0[i / NDB], oacc[i % NDB]);
+        av[i % NDB] = i + NDB < NPV ? v_operand(0, i + NDB) : v_operand(1, i + NDB - NPV);
+        softmax_piece(i, NPV, s1, pb1, st1, m_run, scale);
+      }
+      m_run = st1.mt;
+      l_run = l_run * st1.alpha + st1.lsum;
+      rescale(st1.alpha);
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- slot D: O^T += V^T P^T(half 1), V staging on the side -------------------------------------------------
+#pragma unroll
+      for (int i = 0; i < NPV; ++i) {
+        oacc[i % NDB] = mfma32(av[i % NDB], pb1[i / NDB], oacc[i % NDB]);
+        if (i + NDB < NPV) av[i % NDB] = v_operand(1, i + NDB);
+        if (i == 0) stage_v();
+      }
+    } else {
+      stage_k();
+      stage_v();
     }
     __syncthreads();
   }
@@ -198,10 +255,10 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_fwd_kernel(FwdParams 
 }
 
 // ---- host-side launch -----------------------------------------------------------------------------------------
-template <int D, int NWAVES, int BLOCK_N, bool CAUSAL>
+template <int D, int BLOCK_N, bool CAUSAL>
 static hipError_t launch_fwd_cfg(FwdParams p, hipStream_t stream) {
-  using Cfg = FwdCfg<D, NWAVES, BLOCK_N>;
-  auto kern = rope_attn_fwd_kernel<D, NWAVES, BLOCK_N, CAUSAL>;
+  using Cfg = FwdCfg<D, BLOCK_N>;
+  auto kern = rope_attn_fwd_kernel<D, BLOCK_N, CAUSAL>;
   static bool attr_set = false;  // per instantiation; benign if raced (same value)
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -216,10 +273,8 @@ static hipError_t launch_fwd_cfg(FwdParams p, hipStream_t stream) {
 }
 
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream) {
-  if (D == 128) {
-    return causal ? launch_fwd_cfg<128, 8, 64, true>(p, stream) : launch_fwd_cfg<128, 8, 64, false>(p, stream);
-  }
-  return causal ? launch_fwd_cfg<64, 8, 64, true>(p, stream) : launch_fwd_cfg<64, 8, 64, false>(p, stream);
+  if (D == 128) return causal ? launch_fwd_cfg<128, 64, true>(p, stream) : launch_fwd_cfg<128, 64, false>(p, stream);
+  return causal ? launch_fwd_cfg<64, 64, true>(p, stream) : launch_fwd_cfg<64, 64, false>(p, stream);
 }
 
 }  // namespace corope

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 import torch
 
+from conftest import within_bar
 from oracle import corope_gqa_oracle as C
 from oracle import rope_attn_oracle as O
 
@@ -64,9 +65,9 @@ def test_kernels_reproduce_rope_fixture(pkg, path):
     o.backward(_t(z["do"]).to(dev, torch.bfloat16))
     torch.cuda.synchronize()
     for name, got in (("o", o), ("dq", q.grad), ("dk", k.grad), ("dv", v.grad)):
-        err = (got.detach().float().cpu() - _t(z[name])).abs().max().item()
+        ok, err = within_bar(got.detach().float().cpu(), _t(z[name]))
         print(f"  {os.path.basename(path)} {name}: max-abs {err:.3e}")
-        assert err <= 2e-2, name
+        assert ok, name
 
 
 @pytest.mark.gpu

@@ -5,7 +5,7 @@ import math
 import pytest
 import torch
 
-from conftest import bf16_round, seeded
+from conftest import bf16_round, seeded, within_bar
 from oracle import corope_gqa_oracle as C
 from oracle import rope_attn_oracle as O
 
@@ -47,7 +47,7 @@ def test_c3_forward_backward(pkg):
         for name, a, r in (("dQ", dq[sl], rdq), ("dK", dk[sl], rdk), ("dV", dv[sl], rdv)):
             err = (a - r).abs()
             print(f"  C3 head ({b},{h}) {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e}", flush=True)
-            assert err.max() <= TOL, name
+            assert within_bar(a, r, TOL)[0], name
     # linearity of the backward in dO: grad(2 dO) == 2 grad(dO) exactly (power-of-two scaling commutes with rounding)
     qd.grad = kd.grad = vd.grad = None
     out2 = pkg.attention(qd, kd, vd, True, scale, c.to(dev), s.to(dev))

@@ -7,7 +7,7 @@ import math
 import pytest
 import torch
 
-from conftest import bf16_round, seeded
+from conftest import bf16_round, seeded, within_bar
 from oracle import rope_attn_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -45,7 +45,7 @@ def test_backward_parity(pkg, B, H, N, D, causal):
         err = (a - b).abs()
         print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
         assert torch.isfinite(a).all(), name
-        assert err.max() <= TOL, name
+        assert within_bar(a, b, TOL)[0], name
 
 
 def test_preprocess_delta(pkg):
