@@ -36,7 +36,7 @@ struct DkdvCfg {
   static constexpr int kLdsBytes = 2 * kStageBytes;
 };
 
-template <int D, int NWAVES, int BLOCK_M, bool CAUSAL>
+template <int D, int NWAVES, int BLOCK_M, bool CAUSAL, bool DO_DV, bool DO_DK>
 __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
   using Cfg = DkdvCfg<D, NWAVES, BLOCK_M>;
   constexpr int NT = Cfg::kThreads;
@@ -60,9 +60,9 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
   const int key_c = min(key, N - 1);
   const int wk_lo = n0 + wave * 32, wk_hi = wk_lo + 31;
 
-  u32x4 kb[KC], vb[KC];
+  u32x4 kb[KC], vb[DO_DK ? KC : 1];
   load_b_rows<D, true>(kb, p.k + base, p.cos, p.sin, p.fstride, key_c);
-  load_b_rows<D, false>(vb, p.v + base, nullptr, nullptr, 0, key_c);
+  if constexpr (DO_DK) load_b_rows<D, false>(vb, p.v + base, nullptr, nullptr, 0, key_c);
 
   const int m_tiles = (N + BLOCK_M - 1) / BLOCK_M;
   const int mt0 = CAUSAL ? n0 / BLOCK_M : 0;
@@ -77,7 +77,7 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
       int qi = m0 + threadIdx.x;
       // rows past the end: M = +inf makes P = 0, so they contribute nothing
       st_lse = qi < N ? lseg[qi] : INFINITY;
-      st_delta = qi < N ? deltag[qi] : 0.f;
+      if constexpr (DO_DK) st_delta = qi < N ? deltag[qi] : 0.f;
     }
   };
   auto q_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
@@ -91,13 +91,16 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
     dst.store_rows(do_tile(buf));
     if (threadIdx.x < BLOCK_M) {
       lse_tile(buf)[threadIdx.x] = st_lse;
-      delta_tile(buf)[threadIdx.x] = st_delta;
+      if constexpr (DO_DK) delta_tile(buf)[threadIdx.x] = st_delta;
     }
   };
 
-  f32x16 dvacc[NDB], dkacc[NDB];
+  f32x16 dvacc[DO_DV ? NDB : 1], dkacc[DO_DK ? NDB : 1];
 #pragma unroll
-  for (int i = 0; i < NDB; ++i) dvacc[i] = dkacc[i] = f32x16{0};
+  for (int i = 0; i < NDB; ++i) {
+    if constexpr (DO_DV) dvacc[i] = f32x16{0};
+    if constexpr (DO_DK) dkacc[i] = f32x16{0};
+  }
 
   if (mt0 < m_tiles) {
     load_tile(mt0 * BLOCK_M);
@@ -126,16 +129,19 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
 #pragma unroll
       for (int kc = 0; kc < KC; ++kc)
         sacc = mfma32(*reinterpret_cast<const u32x4*>(qrow + 16 * kc), kb[kc], sacc);
+      if constexpr (DO_DK) {
 #pragma unroll
-      for (int kc = 0; kc < KC; ++kc)
-        dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc), vb[kc], dpacc);
+        for (int kc = 0; kc < KC; ++kc)
+          dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc), vb[kc], dpacc);
+      }
 
       const bool need_mask = CAUSAL && mq0 < wk_hi;
       u32x4 pb[2], dsb[2];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         f32x4 m4 = *reinterpret_cast<const f32x4*>(lses + qb * 32 + 8 * g + 4 * lh);
-        f32x4 d4 = *reinterpret_cast<const f32x4*>(deltas + qb * 32 + 8 * g + 4 * lh);
+        f32x4 d4 = f32x4{0};
+        if constexpr (DO_DK) d4 = *reinterpret_cast<const f32x4*>(deltas + qb * 32 + 8 * g + 4 * lh);
         float pv[4], ds[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -143,18 +149,22 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
           if (need_mask && (mq0 + 8 * g + 4 * lh + e) < key) pv[e] = 0.f;
           ds[e] = pv[e] * (dpacc[4 * g + e] - d4[e]);
         }
-        pb[g / 2][2 * (g % 2)] = pack_bf16(pv[0], pv[1]);
-        pb[g / 2][2 * (g % 2) + 1] = pack_bf16(pv[2], pv[3]);
-        dsb[g / 2][2 * (g % 2)] = pack_bf16(ds[0], ds[1]);
-        dsb[g / 2][2 * (g % 2) + 1] = pack_bf16(ds[2], ds[3]);
+        if constexpr (DO_DV) {
+          pb[g / 2][2 * (g % 2)] = pack_bf16(pv[0], pv[1]);
+          pb[g / 2][2 * (g % 2) + 1] = pack_bf16(pv[2], pv[3]);
+        }
+        if constexpr (DO_DK) {
+          dsb[g / 2][2 * (g % 2)] = pack_bf16(ds[0], ds[1]);
+          dsb[g / 2][2 * (g % 2) + 1] = pack_bf16(ds[2], ds[3]);
+        }
       }
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc) {
         const int kbase = qb * 32 + 16 * cc;
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-          dvacc[db] = mfma32(load_a_trans(dos, LS, kbase, db * 32), pb[cc], dvacc[db]);
-          dkacc[db] = mfma32(load_a_trans(qs, LS, kbase, db * 32), dsb[cc], dkacc[db]);
+          if constexpr (DO_DV) dvacc[db] = mfma32(load_a_trans(dos, LS, kbase, db * 32), pb[cc], dvacc[db]);
+          if constexpr (DO_DK) dkacc[db] = mfma32(load_a_trans(qs, LS, kbase, db * 32), dsb[cc], dkacc[db]);
         }
       }
     }
@@ -163,16 +173,20 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
   }
 
   if (key < N) {
-    uint16_t* dvp = p.dv + base + (int64_t)key * D;
+    if constexpr (DO_DV) {
+      uint16_t* dvp = p.dv + base + (int64_t)key * D;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
+      for (int db = 0; db < NDB; ++db)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w = {pack_bf16(dvacc[db][4 * g], dvacc[db][4 * g + 1]), pack_bf16(dvacc[db][4 * g + 2], dvacc[db][4 * g + 3])};
-        *reinterpret_cast<u32x2*>(dvp + db * 32 + 8 * g + 4 * lh) = w;
-      }
-    store_unrotated<D>(dkacc, p.dk + base + (int64_t)key * D, p.cos + (int64_t)key * p.fstride,
-                       p.sin + (int64_t)key * p.fstride, p.sm_scale);
+        for (int g = 0; g < 4; ++g) {
+          u32x2 w = {pack_bf16(dvacc[db][4 * g], dvacc[db][4 * g + 1]),
+                     pack_bf16(dvacc[db][4 * g + 2], dvacc[db][4 * g + 3])};
+          *reinterpret_cast<u32x2*>(dvp + db * 32 + 8 * g + 4 * lh) = w;
+        }
+    }
+    if constexpr (DO_DK)
+      store_unrotated<D>(dkacc, p.dk + base + (int64_t)key * D, p.cos + (int64_t)key * p.fstride,
+                         p.sin + (int64_t)key * p.fstride, p.sm_scale);
   }
 }
 
@@ -302,11 +316,13 @@ static hipError_t set_lds(K kern, int bytes) {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
-template <int D, bool CAUSAL>
+// dK and dV are produced by two launches of the same kernel template: with both sets of accumulators resident a
+// wave needs more than 256 registers, which would halve the waves per SIMD.
+template <int D, bool CAUSAL, bool DO_DV, bool DO_DK>
 static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
-  constexpr int NWAVES = 4, BLOCK_M = 64;
+  constexpr int NWAVES = 8, BLOCK_M = 64;
   using Cfg = DkdvCfg<D, NWAVES, BLOCK_M>;
-  auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL>;
+  auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = set_lds(kern, Cfg::kLdsBytes);
@@ -319,8 +335,15 @@ static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
 }
 
 template <int D, bool CAUSAL>
+static hipError_t launch_dkdv_both(const BwdParams& p, hipStream_t stream) {
+  hipError_t e = launch_dkdv_cfg<D, CAUSAL, true, false>(p, stream);
+  if (e != hipSuccess) return e;
+  return launch_dkdv_cfg<D, CAUSAL, false, true>(p, stream);
+}
+
+template <int D, bool CAUSAL>
 static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
-  constexpr int NWAVES = 4, BLOCK_N = 64;
+  constexpr int NWAVES = 8, BLOCK_N = 64;
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
   auto kern = rope_attn_bwd_dq_kernel<D, NWAVES, BLOCK_N, CAUSAL>;
   static bool attr_set = false;
@@ -335,8 +358,8 @@ static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
 }
 
 hipError_t launch_bwd_dkdv(const BwdParams& p, int D, bool causal, hipStream_t stream) {
-  if (D == 128) return causal ? launch_dkdv_cfg<128, true>(p, stream) : launch_dkdv_cfg<128, false>(p, stream);
-  return causal ? launch_dkdv_cfg<64, true>(p, stream) : launch_dkdv_cfg<64, false>(p, stream);
+  if (D == 128) return causal ? launch_dkdv_both<128, true>(p, stream) : launch_dkdv_both<128, false>(p, stream);
+  return causal ? launch_dkdv_both<64, true>(p, stream) : launch_dkdv_both<64, false>(p, stream);
 }
 
 hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream) {
