@@ -35,12 +35,23 @@ struct CoropeFreqs {
   float w[64];  // inverse frequencies divided by 2*pi (revolutions per unit of delta), D/2 entries used
 };
 
-template <int D>
+template <int D, int G>
 struct CoropeCfg {
+  static constexpr int kR = 32 / G;                                    // query rows per wave
+  static constexpr int kRowsWg = kR * kCoWaves;                        // query rows per workgroup
+  static constexpr int kQW = 2 * G;                                    // floats per (row, rotation pair): (q1, q2) per head
   static constexpr int kSStride = kCoBlockN + 4;                       // floats per scratch row
-  static constexpr int kTileBytes = RowTile<D>::bytes(kCoBlockN);       // K tile and V tile, row-major bf16
-  static constexpr int kSBytes = 32 * kSStride * 4;                     // per wave
-  static constexpr int kLdsBytes = 2 * kTileBytes + kCoWaves * kSBytes;
+  static constexpr int kKBytes = RowTile<D>::bytes(kCoBlockN);          // K tile, row-major bf16, read row-wise
+  static constexpr int kVPad = 32;                                     // V tile is read only through the transposing load
+  static constexpr int kVBytes = RowTile<D, kVPad>::bytes(kCoBlockN);
+  static constexpr int kSBytes = 32 * kSStride * 4;                     // score scratch, per wave
+  static constexpr int kQBytes = kRowsWg * (D / 2) * kQW * 4;           // the workgroup's queries as fp32, all heads
+  static constexpr int kWBytes = (D / 2) * 4;                           // inverse frequencies
+  static constexpr int kOffV = kKBytes;
+  static constexpr int kOffS = kOffV + kVBytes;
+  static constexpr int kOffQ = kOffS + kCoWaves * kSBytes;
+  static constexpr int kOffW = kOffQ + kQBytes;
+  static constexpr int kLdsBytes = kOffW + kWBytes;
 };
 
 // Natural-order variant of load_a_trans: slot j of lane-half h <-> k = kbase + 8*h + j.
@@ -57,20 +68,23 @@ __device__ __forceinline__ u32x4 load_a_trans_natural(const uint16_t* tile, int 
 
 template <int D, int G>
 __global__ __launch_bounds__(kCoWaves* kWave) void corope_gqa_fwd_kernel(CoropeParams p, CoropeFreqs fr) {
-  using Cfg = CoropeCfg<D>;
-  constexpr int R = 32 / G;              // query rows per wave
+  using Cfg = CoropeCfg<D, G>;
+  constexpr int R = Cfg::kR;             // query rows per wave
   constexpr int VR = R * G;              // virtual rows in use (<= 32)
-  constexpr int ROWS_WG = R * kCoWaves;  // query rows per workgroup
+  constexpr int ROWS_WG = Cfg::kRowsWg;  // query rows per workgroup
   constexpr int HALF = D / 2, NDB = D / 32;
-  constexpr int LS = RowTile<D>::kStride;
+  constexpr int LSV = RowTile<D, Cfg::kVPad>::kStride;
   constexpr int NT = kCoWaves * kWave;
+  constexpr int QW = Cfg::kQW;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint16_t* ks = reinterpret_cast<uint16_t*>(smem);
-  uint16_t* vs = reinterpret_cast<uint16_t*>(smem + Cfg::kTileBytes);
+  uint16_t* vs = reinterpret_cast<uint16_t*>(smem + Cfg::kOffV);
+  float* qs = reinterpret_cast<float*>(smem + Cfg::kOffQ);
+  float* ws = reinterpret_cast<float*>(smem + Cfg::kOffW);
 
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  float* ss = reinterpret_cast<float*>(smem + 2 * Cfg::kTileBytes + wave * Cfg::kSBytes);
+  float* ss = reinterpret_cast<float*>(smem + Cfg::kOffS + wave * Cfg::kSBytes);
 
   const int n_groups = p.B * p.Hkv;
   const int grp = blockIdx.x % n_groups;                       // (batch, kv head)
@@ -100,7 +114,24 @@ __global__ __launch_bounds__(kCoWaves* kWave) void corope_gqa_fwd_kernel(CoropeP
   const float scale2 = p.sm_scale * 1.4426950408889634f;
   const int t_hi = min(m0 + ROWS_WG - 1, N - 1) / kCoBlockN;
 
-  CopyStage<D, kCoBlockN, NT> kst, vst;
+  // ---- the workgroup's query rows, all heads of the group, as fp32 in LDS: [row][pair d][head][q1, q2] -----------
+  // (wave-uniform operands of the lane = key domain are read from here with broadcast LDS loads)
+  for (int u = threadIdx.x; u < ROWS_WG * G * (HALF / 8); u += NT) {
+    const int ch = u % (HALF / 8), g = (u / (HALF / 8)) % G, row = u / ((HALF / 8) * G);
+    const uint32_t* src = qg + (int64_t)g * q_head_words + (int64_t)min(m0 + row, N - 1) * (D / 2) + ch * 4;
+    u32x4 x1 = *reinterpret_cast<const u32x4*>(src);
+    u32x4 x2 = *reinterpret_cast<const u32x4*>(src + HALF / 2);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float a = e % 2 ? bf16_hi(x1[e / 2]) : bf16_lo(x1[e / 2]);
+      float b2 = e % 2 ? bf16_hi(x2[e / 2]) : bf16_lo(x2[e / 2]);
+      *reinterpret_cast<f32x2*>(qs + ((row * HALF) + ch * 8 + e) * QW + 2 * g) = f32x2{a, b2};
+    }
+  }
+  if (threadIdx.x < HALF) ws[threadIdx.x] = fr.w[threadIdx.x];
+
+  CopyStage<D, kCoBlockN, NT> kst;
+  CopyStage<D, kCoBlockN, NT, Cfg::kVPad> vst;
   for (int t = t_hi; t >= 0; --t) {
     const int n0 = t * kCoBlockN;
     kst.load(kg, n0, N);
@@ -132,14 +163,30 @@ __global__ __launch_bounds__(kCoWaves* kWave) void corope_gqa_fwd_kernel(CoropeP
 #pragma unroll 1
       for (int r = 0; r < R; ++r) {
         const int row = min(row0 + r, N - 1);                   // wave-uniform
-        const uint32_t* qrow = qg + (int64_t)row * (D / 2);
-        // leader logit (head 0 of the group), wave-uniform q values
+        const float* qrow = qs + (wave * R + r) * HALF * QW;     // fp32 (q1, q2) pairs of every head, broadcast reads
+        // leader logit (head 0 of the group)
         float logit = 0.f;
+        {
+          // chunks of 8 pairs, fetched one chunk ahead; the scheduling barrier keeps the (fully unrolled) loop from
+          // hoisting every LDS read to the top and drowning in registers
+          f32x2 qc[8], qn[8];
 #pragma unroll
-        for (int w = 0; w < HALF / 2; ++w) {
-          uint32_t a = qrow[w], bq = qrow[HALF / 2 + w];
-          logit += bf16_lo(a) * k1[2 * w] + bf16_hi(a) * k1[2 * w + 1];
-          logit += bf16_lo(bq) * k2[2 * w] + bf16_hi(bq) * k2[2 * w + 1];
+          for (int e = 0; e < 8; ++e) qc[e] = *reinterpret_cast<const f32x2*>(qrow + e * QW);
+#pragma unroll
+          for (int d8 = 0; d8 < HALF; d8 += 8) {
+            if (d8 + 8 < HALF) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) qn[e] = *reinterpret_cast<const f32x2*>(qrow + (d8 + 8 + e) * QW);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              logit = __builtin_fmaf(qc[e][0], k1[d8 + e], logit);
+              logit = __builtin_fmaf(qc[e][1], k2[d8 + e], logit);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qc[e] = qn[e];
+          }
         }
         float z = 1.f / (1.f + __expf(-logit * p.sm_scale));
         if (key > row) z = 0.f;                                  // gates beyond the diagonal do not count
@@ -158,27 +205,43 @@ __global__ __launch_bounds__(kCoWaves* kWave) void corope_gqa_fwd_kernel(CoropeP
         float acc[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) acc[g] = 0.f;
+        {
+          constexpr int CH = G <= 4 ? 4 : 2;   // rotation pairs per chunk (bounds the registers of the look-ahead)
+          typedef float wvec __attribute__((ext_vector_type(CH)));
+          f32x2 qc[CH][G], qn[CH][G];
+          wvec wc = *reinterpret_cast<const wvec*>(ws), wn = wc;
 #pragma unroll
-        for (int w = 0; w < HALF / 2; ++w) {
-          uint32_t qa[G], qb[G];
+          for (int e = 0; e < CH; ++e)
 #pragma unroll
-          for (int g = 0; g < G; ++g) {
-            qa[g] = qrow[g * q_head_words + w];
-            qb[g] = qrow[g * q_head_words + HALF / 2 + w];
-          }
+            for (int g = 0; g < G; ++g) qc[e][g] = *reinterpret_cast<const f32x2*>(qrow + e * QW + 2 * g);
 #pragma unroll
-          for (int e = 0; e < 2; ++e) {
-            const int d = 2 * w + e;
-            float x = __builtin_amdgcn_fractf(delta * fr.w[d]);
-            float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
-            float r1 = cs * k1[d] + sn * k2[d];
-            float r2 = cs * k2[d] - sn * k1[d];
+          for (int d0 = 0; d0 < HALF; d0 += CH) {
+            if (d0 + CH < HALF) {
+              wn = *reinterpret_cast<const wvec*>(ws + d0 + CH);
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
-              float q1 = e ? bf16_hi(qa[g]) : bf16_lo(qa[g]);
-              float q2 = e ? bf16_hi(qb[g]) : bf16_lo(qb[g]);
-              acc[g] += q1 * r1 + q2 * r2;
+              for (int e = 0; e < CH; ++e)
+#pragma unroll
+                for (int g = 0; g < G; ++g) qn[e][g] = *reinterpret_cast<const f32x2*>(qrow + (d0 + CH + e) * QW + 2 * g);
             }
+#pragma unroll
+            for (int e = 0; e < CH; ++e) {
+              const int d = d0 + e;
+              float x = __builtin_amdgcn_fractf(delta * wc[e]);
+              float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
+              float r1 = __builtin_fmaf(cs, k1[d], sn * k2[d]);
+              float r2 = __builtin_fmaf(cs, k2[d], -(sn * k1[d]));
+#pragma unroll
+              for (int g = 0; g < G; ++g) {
+                acc[g] = __builtin_fmaf(qc[e][g][0], r1, acc[g]);
+                acc[g] = __builtin_fmaf(qc[e][g][1], r2, acc[g]);
+              }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            wc = wn;
+#pragma unroll
+            for (int e = 0; e < CH; ++e)
+#pragma unroll
+              for (int g = 0; g < G; ++g) qc[e][g] = qn[e][g];
           }
         }
 #pragma unroll
@@ -229,7 +292,7 @@ __global__ __launch_bounds__(kCoWaves* kWave) void corope_gqa_fwd_kernel(CoropeP
       for (int c = 0; c < kCoBlockN / 16; ++c)
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
-          oacc[db] = mfma32(load_a_trans_natural(vs, LS, 16 * c, db * 32), pb[c], oacc[db]);
+          oacc[db] = mfma32(load_a_trans_natural(vs, LSV, 16 * c, db * 32), pb[c], oacc[db]);
     }
   }
 
@@ -250,7 +313,7 @@ __global__ __launch_bounds__(kCoWaves* kWave) void corope_gqa_fwd_kernel(CoropeP
 
 template <int D, int G>
 static hipError_t launch_corope_cfg(CoropeParams p, const CoropeFreqs& fr, hipStream_t stream) {
-  using Cfg = CoropeCfg<D>;
+  using Cfg = CoropeCfg<D, G>;
   auto kern = corope_gqa_fwd_kernel<D, G>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -259,7 +322,7 @@ static hipError_t launch_corope_cfg(CoropeParams p, const CoropeFreqs& fr, hipSt
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  constexpr int rows_wg = (32 / G) * kCoWaves;
+  constexpr int rows_wg = Cfg::kRowsWg;
   p.num_m_blocks = (p.N + rows_wg - 1) / rows_wg;
   hipLaunchKernelGGL(kern, dim3(p.num_m_blocks * p.B * p.Hkv), dim3(kCoWaves * kWave), Cfg::kLdsBytes, stream, p, fr);
   return hipGetLastError();
