@@ -8,6 +8,8 @@ rotation FLOPs not counted), the roofline of the dominant kernel from per-launch
 oracle timed on the host cores as a baseline.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--no-cpu-baseline]
+
+(c3 is the metric shape and the default; c2/c4 are the other RoPE-attention shapes; c5 is the Co-RoPE GQA forward.)
 """
 import argparse
 import importlib
@@ -24,6 +26,16 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak used for every "fraction of peak" below
 PEAK_HBM_GBS = 8000.0
+
+# HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE on this
+# benchmark (summary and commands: profiles/rope_attn_c3_hbm_traffic.md); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE
+# by 1.0, the factors a plain 1 GiB device copy gives for the same counters.
+HBM_TRAFFIC_BYTES = {
+    ("c3", "rope_attn_fwd"): int((355229 * 2.0 + 66565) * 1024),
+    ("c3", "rope_attn_bwd_dv"): int((272982 * 2.0 + 65536) * 1024),
+    ("c3", "rope_attn_bwd_dk"): int((391606 * 2.0 + 65561) * 1024),
+    ("c3", "rope_attn_bwd_dq"): int((371726 * 2.0 + 65601) * 1024),
+}
 
 CONFIGS = {
     "c2": dict(B=4, H=8, N=1024, D=64, name="C2: fused RoPE flash-attention fwd+bwd B4 H8 N1024 D64 causal bf16"),
@@ -68,18 +80,82 @@ def cpu_baseline():
                       f"os.cpu_count()={os.cpu_count()}"}
 
 
+def bench_corope(args):
+    """C5: Co-RoPE GQA forward, B2 Hq32 Hkv8 N4096 D128 bf16 causal.  VALU/transcendental-bound: reported as ms,
+    attention-equivalent TFLOP/s and (sin, cos) pairs per second, not as an MFMA fraction."""
+    import torch
+    pkg = importlib.import_module("corope_amd")
+    lib = pkg._lib.load()
+    dev = torch.device("cuda:0")
+    B, Hq, Hkv, N, D = 2, 32, 8, 4096, 128
+    scale = 1 / math.sqrt(D)
+    g = torch.Generator().manual_seed(42)
+    q = torch.randn(B, Hq, N, D, generator=g).to(dev, torch.bfloat16)
+    k, v = (torch.randn(B, Hkv, N, D, generator=g).to(dev, torch.bfloat16) for _ in range(2))
+    o = torch.empty_like(q)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        rc = lib.corope_gqa_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, Hq, Hkv, N, D, scale, 10000.0, stream)
+        if rc != 0:
+            sys.exit(pkg._lib.last_error())
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    evs[0].record()
+    for i in range(args.steps):
+        step()
+        evs[i + 1].record()
+    torch.cuda.synchronize()
+    kms = sum(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps)) / args.steps
+    flops = attention_flops(B, Hq, N, D, "fwd")
+    pairs = B * Hkv * N * (N + 1) / 2 * D / 2
+    # VALU roofline: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz lane-instructions/s; per (sin, cos) pair the kernel issues
+    # 14 + 2G full-rate instructions (2 of them transcendental, counted once here)
+    out = {"metric": "Co-RoPE GQA fwd, B2 Hq32 Hkv8 N4096 D128 causal", "value": round(flops / (ms * 1e-3) * 1e-12, 2),
+           "unit": "TFLOP/s (attention-equivalent)", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "C5: Co-RoPE GQA attention fwd B2 Hq32 Hkv8 N4096 D128 causal bf16", "theta": 10000.0},
+           "sincos_pairs_per_s": round(pairs / (kms * 1e-3), 1), "kernel_ms": round(kms, 4),
+           "roofline": {"bound": "valu", "kernel": "corope_gqa_fwd", "achieved": round(pairs * 22 / (kms * 1e-3) * 1e-12, 3),
+                        "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T lane-instr/s",
+                        "frac": round(pairs * 22 / (kms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4), "traffic": None},
+           "cpu_baseline": None}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--config", default="c3", choices=sorted(CONFIGS))
+    ap.add_argument("--config", default="c3", choices=sorted(CONFIGS) + ["c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every (batch, head) is independent; see DESIGN.md for how "
                  "the path would shard); run it with --gpus 1")
 
+    if args.copy_calibration:
+        import torch
+        a = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda:0").normal_()
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)          # reads 1 GiB, writes 1 GiB per launch
+        torch.cuda.synchronize()
+        del a, b
+    if args.config == "c5":
+        return bench_corope(args)
     import torch
     pkg = importlib.import_module("corope_amd")
     lib = pkg._lib.load()
@@ -126,9 +202,10 @@ def main():
         launches += [
             ("rope_attn_bwd_preprocess", lambda: lib.corope_rope_attn_bwd_preprocess(o.data_ptr(), dop, delta.data_ptr(),
                                                                                     B, H, N, D, stream)),
-            ("rope_attn_bwd_dkdv", lambda: lib.corope_rope_attn_bwd_dkdv(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),
-                                                                        cp, sp, fs, dk.data_ptr(), dv.data_ptr(),
-                                                                        B, H, N, D, scale, 1, stream)),
+            ("rope_attn_bwd_dv", lambda: lib.corope_rope_attn_bwd_dv(qp, kp, dop, M.data_ptr(), cp, sp, fs, dv.data_ptr(),
+                                                                    B, H, N, D, scale, 1, stream)),
+            ("rope_attn_bwd_dk", lambda: lib.corope_rope_attn_bwd_dk(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),
+                                                                    cp, sp, fs, dk.data_ptr(), B, H, N, D, scale, 1, stream)),
             ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),
                                                                     cp, sp, fs, dq.data_ptr(), B, H, N, D, scale, 1, stream)),
         ]
@@ -146,10 +223,11 @@ def main():
             for i, (name, _) in enumerate(launches):
                 durs[name].append(evs[i].elapsed_time(evs[i + 1]))
     avg = {n: sum(d) / len(d) for n, d in durs.items()}
-    # algorithmic FLOPs per launch: forward 2 matmul units; dK/dV 4 units (the counted S recompute, dP, dV, dK);
-    # dQ 1 unit (its own S and dP recomputes are overhead on top of the model); preprocess is HBM-bound.
+    # algorithmic FLOPs per launch (the reference's model: forward 2 matmul units, backward 5): dV kernel 2 units (the
+    # counted S recompute and dV), dK kernel 2 units (dP and dK; its own S recompute is overhead on top of the model),
+    # dQ kernel 1 unit (dQ; its S and dP recomputes are overhead); the preprocess pass is HBM-bound.
     unit = 2.0 * B * H * N * N * D * 0.5
-    alg = {"rope_attn_fwd": 2 * unit, "rope_attn_bwd_dkdv": 4 * unit, "rope_attn_bwd_dq": 1 * unit}
+    alg = {"rope_attn_fwd": 2 * unit, "rope_attn_bwd_dv": 2 * unit, "rope_attn_bwd_dk": 2 * unit, "rope_attn_bwd_dq": 1 * unit}
     kernels = {}
     for n, ms in avg.items():
         if n in alg:
@@ -161,8 +239,9 @@ def main():
                           "frac_of_hbm_peak": round(by / (ms * 1e-3) * 1e-9 / PEAK_HBM_GBS, 4)}
     dom = max((n for n in avg if n in alg), key=lambda n: avg[n])
     dom_tf = alg[dom] / (avg[dom] * 1e-3) * 1e-12
+    traffic = HBM_TRAFFIC_BYTES.get((args.config, dom))
     roofline = {"bound": "mfma", "kernel": dom, "achieved": round(dom_tf, 1), "peak": PEAK_BF16_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(dom_tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "unit": "TFLOP/s", "frac": round(dom_tf / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
                 "avg_launch_ms": round(avg[dom], 4)}
     fwd_tf = alg["rope_attn_fwd"] / (avg["rope_attn_fwd"] * 1e-3) * 1e-12
     out = {
@@ -178,7 +257,8 @@ def main():
         "kernels": kernels, "roofline": roofline,
     }
     if not fwd_only:
-        bwd_ms = avg["rope_attn_bwd_preprocess"] + avg["rope_attn_bwd_dkdv"] + avg["rope_attn_bwd_dq"]
+        bwd_ms = (avg["rope_attn_bwd_preprocess"] + avg["rope_attn_bwd_dv"] + avg["rope_attn_bwd_dk"]
+                  + avg["rope_attn_bwd_dq"])
         bwd_tf = f_bwd / (bwd_ms * 1e-3) * 1e-12
         out["bwd"] = {"ms": round(bwd_ms, 4), "tflops": round(bwd_tf, 1), "frac_of_peak": round(bwd_tf / PEAK_BF16_TFLOPS, 4)}
     out["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline()

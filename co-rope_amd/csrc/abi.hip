@@ -124,17 +124,42 @@ int corope_rope_attn_bwd_preprocess(const void* o, const void* d_o, float* delta
   return launch_status("rope_attn_bwd_preprocess", corope::launch_bwd_preprocess(p, D, static_cast<hipStream_t>(stream)));
 }
 
+int corope_rope_attn_bwd_dv(const void* q, const void* k, const void* d_o, const float* lse, const float* freqs_cos,
+                            const float* freqs_sin, int64_t freq_row_stride, void* dv, int B, int H, int N, int D,
+                            float sm_scale, int causal, void* stream) {
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
+  if (rc) return rc;
+  rc = check_ptrs("rope_attn_bwd_dv", {q, k, d_o, lse, freqs_cos, freqs_sin, dv});
+  if (rc) return rc;
+  corope::BwdParams p = make_bwd(q, k, nullptr, nullptr, d_o, lse, nullptr, freqs_cos, freqs_sin, freq_row_stride,
+                                 nullptr, nullptr, dv, B, H, N, sm_scale);
+  return launch_status("rope_attn_bwd_dv", corope::launch_bwd_dv(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+}
+
+int corope_rope_attn_bwd_dk(const void* q, const void* k, const void* v, const void* d_o, const float* lse,
+                            const float* delta, const float* freqs_cos, const float* freqs_sin,
+                            int64_t freq_row_stride, void* dk, int B, int H, int N, int D, float sm_scale, int causal,
+                            void* stream) {
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
+  if (rc) return rc;
+  rc = check_ptrs("rope_attn_bwd_dk", {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dk});
+  if (rc) return rc;
+  corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
+                                 freq_row_stride, nullptr, dk, nullptr, B, H, N, sm_scale);
+  return launch_status("rope_attn_bwd_dk", corope::launch_bwd_dk(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+}
+
 int corope_rope_attn_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* lse,
                               const float* delta, const float* freqs_cos, const float* freqs_sin,
                               int64_t freq_row_stride, void* dk, void* dv, int B, int H, int N, int D, float sm_scale,
                               int causal, void* stream) {
-  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
+  int rc = check_ptrs("rope_attn_bwd_dkdv", {v, delta, dk, dv});
   if (rc) return rc;
-  rc = check_ptrs("rope_attn_bwd_dkdv", {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dk, dv});
+  rc = corope_rope_attn_bwd_dv(q, k, d_o, lse, freqs_cos, freqs_sin, freq_row_stride, dv, B, H, N, D, sm_scale, causal,
+                               stream);
   if (rc) return rc;
-  corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
-                                 freq_row_stride, nullptr, dk, dv, B, H, N, sm_scale);
-  return launch_status("rope_attn_bwd_dkdv", corope::launch_bwd_dkdv(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+  return corope_rope_attn_bwd_dk(q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dk, B, H, N, D,
+                                 sm_scale, causal, stream);
 }
 
 int corope_rope_attn_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* lse,

@@ -55,7 +55,8 @@ struct CoropeParams {
 
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_preprocess(const BwdParams& p, int D, hipStream_t stream);
-hipError_t launch_bwd_dkdv(const BwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_bwd_dv(const BwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_bwd_dk(const BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_corope_gqa_fwd(const CoropeParams& p, int D, hipStream_t stream);
 

@@ -335,13 +335,6 @@ static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
 }
 
 template <int D, bool CAUSAL>
-static hipError_t launch_dkdv_both(const BwdParams& p, hipStream_t stream) {
-  hipError_t e = launch_dkdv_cfg<D, CAUSAL, true, false>(p, stream);
-  if (e != hipSuccess) return e;
-  return launch_dkdv_cfg<D, CAUSAL, false, true>(p, stream);
-}
-
-template <int D, bool CAUSAL>
 static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
   constexpr int NWAVES = 8, BLOCK_N = 64;
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
@@ -357,9 +350,16 @@ static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_bwd_dkdv(const BwdParams& p, int D, bool causal, hipStream_t stream) {
-  if (D == 128) return causal ? launch_dkdv_both<128, true>(p, stream) : launch_dkdv_both<128, false>(p, stream);
-  return causal ? launch_dkdv_both<64, true>(p, stream) : launch_dkdv_both<64, false>(p, stream);
+hipError_t launch_bwd_dv(const BwdParams& p, int D, bool causal, hipStream_t stream) {
+  if (D == 128)
+    return causal ? launch_dkdv_cfg<128, true, true, false>(p, stream) : launch_dkdv_cfg<128, false, true, false>(p, stream);
+  return causal ? launch_dkdv_cfg<64, true, true, false>(p, stream) : launch_dkdv_cfg<64, false, true, false>(p, stream);
+}
+
+hipError_t launch_bwd_dk(const BwdParams& p, int D, bool causal, hipStream_t stream) {
+  if (D == 128)
+    return causal ? launch_dkdv_cfg<128, true, false, true>(p, stream) : launch_dkdv_cfg<128, false, false, true>(p, stream);
+  return causal ? launch_dkdv_cfg<64, true, false, true>(p, stream) : launch_dkdv_cfg<64, false, false, true>(p, stream);
 }
 
 hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream) {

@@ -60,9 +60,24 @@ int corope_rope_attn_fwd(const void *q, const void *k, const void *v,
 int corope_rope_attn_bwd_preprocess(const void *o, const void *d_o, float *delta,
                                     int B, int H, int N, int D, void *stream);
 
-/* dK and dV: one workgroup per key block, sweeping the query blocks that attend to it.
+/* dV alone: one workgroup per key block, sweeping the query blocks that attend to it; recomputes P from q, k and lse.
+ * Replaces the dV part of _attn_bwd_dkdv (reference fused-rope/fused_rope_attn.py:382-393, :571-572). */
+int corope_rope_attn_bwd_dv(const void *q, const void *k, const void *d_o, const float *lse,
+                            const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                            void *dv,
+                            int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
+/* dK alone: same sweep; recomputes P and dP, forms dS, un-rotates and scales dK in the epilogue.
+ * Replaces the dK part of _attn_bwd_dkdv (reference fused-rope/fused_rope_attn.py:395-401, :573-579). */
+int corope_rope_attn_bwd_dk(const void *q, const void *k, const void *v, const void *d_o,
+                            const float *lse, const float *delta,
+                            const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                            void *dk,
+                            int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
+/* dK and dV = corope_rope_attn_bwd_dv followed by corope_rope_attn_bwd_dk on the same stream.
  * Replaces the _attn_bwd_dkdv half of _attn_bwd (reference fused-rope/fused_rope_attn.py:342-404,
- * :524-579) including the host-side K pre-scale (:746-748), which is folded into the kernel. */
+ * :524-579) including the host-side K pre-scale (:746-748), which is folded into the kernels. */
 int corope_rope_attn_bwd_dkdv(const void *q, const void *k, const void *v, const void *d_o,
                               const float *lse, const float *delta,
                               const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,

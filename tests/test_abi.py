@@ -30,7 +30,8 @@ def test_header_symbols_are_exported_and_typed(pkg):
 
 def test_header_cites_reference_for_each_entry_point():
     text = open(HEADER).read()
-    for fn in ("corope_rope_attn_fwd", "corope_rope_attn_bwd_preprocess", "corope_rope_attn_bwd_dkdv",
+    for fn in ("corope_rope_attn_fwd", "corope_rope_attn_bwd_preprocess", "corope_rope_attn_bwd_dv",
+               "corope_rope_attn_bwd_dk", "corope_rope_attn_bwd_dkdv",
                "corope_rope_attn_bwd_dq", "corope_rope_attn_bwd", "corope_gqa_fwd"):
         before = text[:text.index(f"int {fn}(")]
         comment = before[before.rindex("/*"):]
