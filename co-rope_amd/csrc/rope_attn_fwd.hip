@@ -69,16 +69,14 @@ __device__ __forceinline__ void softmax_piece(int step, int n_steps, const f32x1
   } else {
     const int n = n_steps - 2;
     const int lo = (step - 2) * 8 / n, hi = (step - 1) * 8 / n;
-    const bf16x2 ones = __builtin_bit_cast(bf16x2, 0x3f803f80u);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if (j < lo || j >= hi) continue;
       float p0 = fast_exp2(sacc[2 * j] * scale - st.ms);
       float p1 = fast_exp2(sacc[2 * j + 1] * scale - st.ms);
-      uint32_t w = pack_bf16(p0, p1);
-      // the denominator sums the ROUNDED probabilities, i.e. exactly the weights the PV product uses
-      st.lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), ones, st.lsum, false);
-      pb[j / 4][j % 4] = w;
+      // plain adds: the bf16 dot-product instruction would do this in one op but stalls the MFMA pipe
+      st.lsum += p0 + p1;
+      pb[j / 4][j % 4] = pack_bf16(p0, p1);
     }
   }
 }
