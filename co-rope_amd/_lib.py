@@ -23,6 +23,7 @@ SIGNATURES = {
     "corope_amd_last_error": (ctypes.c_char_p, []),
     "corope_rope_attn_check": (_I, [_I, _I, _I, _I, _L, _F, _I]),
     "corope_gqa_check": (_I, [_I, _I, _I, _I, _I, _F, _F]),
+    "corope_rope_freqs": (_I, [_P, _P, _I, _I, _I, _L, _I, _F, _P]),
     "corope_rope_attn_fwd": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_bwd_preprocess": (_I, [_P, _P, _P, _I, _I, _I, _I, _P]),
     "corope_rope_attn_bwd_dv": (_I, [_P] * 6 + [_L, _P, _I, _I, _I, _I, _F, _I, _P]),

@@ -188,6 +188,20 @@ int corope_rope_attn_bwd(const void* q, const void* k, const void* v, const void
                                  sm_scale, causal, stream);
 }
 
+int corope_rope_freqs(float* freqs_cos, float* freqs_sin, int n_pos, int D, int width, int64_t freq_row_stride, int pos0,
+                      float theta, void* stream) {
+  if (n_pos <= 0 || D <= 0 || D % 2 != 0) return fail(COROPE_E_BADARG, "rope_freqs: n_pos must be positive and D even");
+  if (D > 128) return fail(COROPE_E_UNSUPPORTED, "rope_freqs: head dim %d exceeds 128", D);
+  if (width != D && width != D / 2) return fail(COROPE_E_BADARG, "rope_freqs: width must be D or D/2 (got %d)", width);
+  if (freq_row_stride < width) return fail(COROPE_E_BADARG, "rope_freqs: row stride smaller than the row");
+  if (pos0 < 0 || !(theta > 0.f) || !std::isfinite(theta)) return fail(COROPE_E_BADARG, "rope_freqs: bad pos0 or theta");
+  if ((int64_t)n_pos * (D / 2) >= ((int64_t)1 << 31)) return fail(COROPE_E_UNSUPPORTED, "rope_freqs: table too large");
+  if (freqs_cos == nullptr || freqs_sin == nullptr) return fail(COROPE_E_BADARG, "rope_freqs: null pointer argument");
+  g_err[0] = 0;
+  return launch_status("rope_freqs", corope::launch_rope_freqs(freqs_cos, freqs_sin, n_pos, D, width, freq_row_stride,
+                                                               pos0, theta, static_cast<hipStream_t>(stream)));
+}
+
 int corope_gqa_fwd(const void* q, const void* k, const void* v, void* o, int B, int Hq, int Hkv, int N, int D,
                    float sm_scale, float theta, void* stream) {
   int rc = corope_gqa_check(B, Hq, Hkv, N, D, sm_scale, theta);

@@ -46,6 +46,13 @@ int corope_rope_attn_check(int B, int H, int N, int D, int64_t freq_row_stride, 
 /* Argument check only (no HIP call) for corope_gqa_fwd. */
 int corope_gqa_check(int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta);
 
+/* cos/sin tables on the device: row r holds position pos0 + r, column i the angle (pos0 + r) * theta^(-2i/D);
+ * width = D writes the reference's duplicated-half (n_pos, D) layout, width = D/2 the compact one.
+ * Replaces precompute_freqs_cis (reference fused-rope/rope_attn_pytorch.py:10-49), which the reference runs as
+ * torch ops on the device; pos0 > 0 gives a shard or a decode step its own slice of positions. */
+int corope_rope_freqs(float *freqs_cos, float *freqs_sin, int n_pos, int D, int width, int64_t freq_row_stride,
+                      int pos0, float theta, void *stream);
+
 /* Fused RoPE flash-attention forward.
  * Replaces the launch of _attn_fwd in _attention.forward
  * (reference fused-rope/fused_rope_attn.py:222-320 kernel, :702-716 launch).

@@ -30,7 +30,7 @@ def test_header_symbols_are_exported_and_typed(pkg):
 
 def test_header_cites_reference_for_each_entry_point():
     text = open(HEADER).read()
-    for fn in ("corope_rope_attn_fwd", "corope_rope_attn_bwd_preprocess", "corope_rope_attn_bwd_dv",
+    for fn in ("corope_rope_freqs", "corope_rope_attn_fwd", "corope_rope_attn_bwd_preprocess", "corope_rope_attn_bwd_dv",
                "corope_rope_attn_bwd_dk", "corope_rope_attn_bwd_dkdv",
                "corope_rope_attn_bwd_dq", "corope_rope_attn_bwd", "corope_gqa_fwd"):
         before = text[:text.index(f"int {fn}(")]
@@ -85,6 +85,19 @@ def test_null_and_misaligned_pointers_are_rejected_before_any_launch(pkg):
     assert rc == -3
     with pytest.raises(ValueError):
         pkg._lib.check(rc, "corope_gqa_fwd")
+
+
+def test_rope_freqs_argument_checks(pkg):
+    lib = pkg._lib.load()
+    buf = ctypes.create_string_buffer(4096)
+    ok = (ctypes.addressof(buf) + 15) & ~15
+    assert lib.corope_rope_freqs(ok, ok, 0, 64, 64, 64, 0, 1e4, None) == -1
+    assert lib.corope_rope_freqs(ok, ok, 8, 64, 48, 64, 0, 1e4, None) == -1      # width neither D nor D/2
+    assert lib.corope_rope_freqs(ok, ok, 8, 64, 64, 32, 0, 1e4, None) == -1      # stride < width
+    assert lib.corope_rope_freqs(ok, None, 8, 64, 64, 64, 0, 1e4, None) == -1
+    assert lib.corope_rope_freqs(ok, ok, 8, 64, 64, 64, -1, 1e4, None) == -1
+    with pytest.raises(ValueError):
+        pkg.rope_freqs_device(64, 8, device="cpu")
 
 
 def test_python_surface_matches_reference_order(pkg):

@@ -93,3 +93,28 @@ def test_deterministic(pkg):
     a, ma = _run(pkg, q, k, v, True, 0.09, c, s)
     b, mb = _run(pkg, q, k, v, True, 0.09, c, s)
     assert torch.equal(a, b) and torch.equal(ma, mb)
+
+
+def test_device_freq_tables_match_the_oracle(pkg):
+    """The library's own table kernel against the oracle's precompute_freqs_cis: fp32 angles are formed the same way;
+    the device's cosf/sinf may differ from the host's by a few ulp."""
+    for D, N, theta in ((128, 4096, 10000.0), (64, 777, 500.0)):
+        c, s = pkg.rope_freqs_device(D, N, theta, device="cuda:0")
+        rc, rs = O.precompute_freqs_cis(D, N, theta)
+        assert c.shape == (N, D) and (c.cpu() - rc).abs().max() < 2e-6 and (s.cpu() - rs).abs().max() < 2e-6
+        ch, sh = pkg.rope_freqs_device(D, 100, theta, device="cuda:0", pos0=37, compact=True)
+        assert ch.shape == (100, D // 2)
+        assert torch.equal(ch, c[37:137, :D // 2]) and torch.equal(sh, s[37:137, :D // 2])
+
+
+def test_position_offset_leaves_attention_unchanged(pkg):
+    """Relative-position property on the device path: tables for positions 1000.. give the same O as positions 0.."""
+    B, H, N, D = 1, 2, 320, 128
+    q, k, v = _inputs(B, H, N, D, seed=13)
+    dev = torch.device("cuda:0")
+    c0, s0 = pkg.rope_freqs_device(D, N, device=dev, compact=True)
+    c1, s1 = pkg.rope_freqs_device(D, N, device=dev, pos0=1000, compact=True)
+    qd, kd, vd = (t.to(dev, torch.bfloat16) for t in (q, k, v))
+    o0, _ = pkg.rope_attn_forward_with_lse(qd, kd, vd, True, 0.09, c0, s0)
+    o1, _ = pkg.rope_attn_forward_with_lse(qd, kd, vd, True, 0.09, c1, s1)
+    assert (o0.float() - o1.float()).abs().max() <= 2e-2
