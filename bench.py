@@ -80,6 +80,50 @@ def cpu_baseline():
                       f"os.cpu_count()={os.cpu_count()}"}
 
 
+# the 19 shapes of the reference's comparison harness (fused-rope/bench_compare.py:323-350): (B, H, N, D, name), causal
+SWEEP = [(4, 8, 512, 64, "Small-512"), (4, 8, 1024, 64, "Small-1K"), (2, 8, 2048, 64, "Small-2K"),
+         (2, 8, 4096, 64, "Small-4K"), (1, 8, 8192, 64, "Small-8K"),
+         (4, 32, 512, 128, "Llama7B-512"), (4, 32, 1024, 128, "Llama7B-1K"), (2, 32, 2048, 128, "Llama7B-2K"),
+         (2, 32, 4096, 128, "Llama7B-4K"), (1, 32, 8192, 128, "Llama7B-8K"), (1, 32, 16384, 128, "Llama7B-16K"),
+         (2, 64, 512, 128, "Llama70B-512"), (2, 64, 1024, 128, "Llama70B-1K"), (1, 64, 2048, 128, "Llama70B-2K"),
+         (1, 64, 4096, 128, "Llama70B-4K"), (1, 32, 8192, 128, "Llama70B-8K"),
+         (1, 16, 32768, 128, "Long-32K"), (1, 8, 65536, 128, "Long-64K"), (1, 4, 131072, 128, "Long-128K")]
+
+
+def bench_sweep(args):
+    """Forward and backward-only times (median of HIP-event timings, backward with the forward graph retained, as the
+    reference's harness does) for the reference's 19 shapes; one JSON line per shape."""
+    import torch
+    pkg = importlib.import_module("corope_amd")
+    dev = torch.device("cuda:0")
+    for (B, H, N, D, name) in SWEEP:
+        g = torch.Generator().manual_seed(0)
+        q, k, v, do = (torch.randn(B, H, N, D, generator=g).to(dev, torch.bfloat16) for _ in range(4))
+        cos, sin = pkg.rope_freqs_device(D, N, 10000.0, device=dev)
+        q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+        reps = 30 if N <= 16384 else 8
+
+        def timed(fn):
+            for _ in range(3):
+                fn()
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+            evs[0].record()
+            for i in range(reps):
+                fn()
+                evs[i + 1].record()
+            torch.cuda.synchronize()
+            return statistics.median(evs[i].elapsed_time(evs[i + 1]) for i in range(reps))
+
+        f_ms = timed(lambda: pkg.attention(q, k, v, True, 0.5, cos, sin))
+        o = pkg.attention(q, k, v, True, 0.5, cos, sin)
+        b_ms = timed(lambda: o.backward(do, retain_graph=True))
+        ff, fb = attention_flops(B, H, N, D, "fwd"), attention_flops(B, H, N, D, "bwd")
+        print(json.dumps({"config": name, "B": B, "H": H, "N": N, "D": D, "fwd_ms": round(f_ms, 4),
+                          "fwd_tflops": round(ff / f_ms * 1e-9, 1), "bwd_ms": round(b_ms, 4),
+                          "bwd_tflops": round(fb / b_ms * 1e-9, 1)}), flush=True)
+        del q, k, v, do, o
+
+
 def bench_corope(args):
     """C5: Co-RoPE GQA forward, B2 Hq32 Hkv8 N4096 D128 bf16 causal.  VALU/transcendental-bound: reported as ms,
     attention-equivalent TFLOP/s and (sin, cos) pairs per second, not as an MFMA fraction."""
@@ -139,6 +183,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="c3", choices=sorted(CONFIGS) + ["c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sweep", action="store_true",
+                    help="time the reference harness's 19 shapes instead (one JSON line per shape)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
@@ -154,6 +200,8 @@ def main():
             b.copy_(a)          # reads 1 GiB, writes 1 GiB per launch
         torch.cuda.synchronize()
         del a, b
+    if args.sweep:
+        return bench_sweep(args)
     if args.config == "c5":
         return bench_corope(args)
     import torch
