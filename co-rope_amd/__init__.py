@@ -6,7 +6,7 @@ from . import _lib
 from .corope_gqa import attention as corope_attention
 from .corope_gqa import corope_attn_gqa
 from .freqs import precompute_freqs_cis, rope_freqs_device
-from .rope_attn import attention, fused_rope_attn, rope_attn_forward_with_lse
+from .rope_attn import attention, fused_rope_attn, rope_attn_forward_with_lse, rope_rotate
 
-__all__ = ["attention", "fused_rope_attn", "rope_attn_forward_with_lse", "corope_attention", "corope_attn_gqa",
+__all__ = ["attention", "fused_rope_attn", "rope_attn_forward_with_lse", "rope_rotate", "corope_attention", "corope_attn_gqa",
            "precompute_freqs_cis", "rope_freqs_device", "_lib"]

@@ -25,6 +25,10 @@ SIGNATURES = {
     "corope_gqa_check": (_I, [_I, _I, _I, _I, _I, _F, _F]),
     "corope_rope_freqs": (_I, [_P, _P, _I, _I, _I, _L, _I, _F, _P]),
     "corope_rope_attn_fwd": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
+    "corope_rope_attn_fwd_workspace_bytes": (_L, [_I, _I, _I, _I]),
+    "corope_rope_attn_fwd_ws": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P, _L, _P]),
+    "corope_rope_attn_fwd_prerotated": (_I, [_P, _P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
+    "corope_rope_rotate": (_I, [_P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _P]),
     "corope_rope_attn_bwd_preprocess": (_I, [_P, _P, _P, _I, _I, _I, _I, _P]),
     "corope_rope_attn_bwd_dv": (_I, [_P] * 6 + [_L, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_bwd_dk": (_I, [_P] * 8 + [_L, _P, _I, _I, _I, _I, _F, _I, _P]),

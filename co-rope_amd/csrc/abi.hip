@@ -91,12 +91,24 @@ int corope_gqa_check(int B, int Hq, int Hkv, int N, int D, float sm_scale, float
   return COROPE_OK;
 }
 
-int corope_rope_attn_fwd(const void* q, const void* k, const void* v, const float* freqs_cos, const float* freqs_sin,
-                         int64_t freq_row_stride, void* o, float* lse, int B, int H, int N, int D, float sm_scale,
-                         int causal, void* stream) {
+}  // extern "C" (reopened below)
+
+namespace {
+
+// Workspace of the two-launch forward: rotated K (bf16, same shape as k), then one float per 64-key tile.
+int64_t fwd_ws_krot_bytes(int B, int H, int N, int D) { return (((int64_t)B * H * N * D * 2) + 255) / 256 * 256; }
+int64_t fwd_ws_bytes(int B, int H, int N, int D) {
+  return fwd_ws_krot_bytes(B, H, N, D) + (int64_t)B * H * ((N + 63) / 64) * 4;
+}
+
+// k_rot / tile_kmax null: single launch.  workspace non-null: rotate K into it first.
+int rope_attn_fwd_impl(const char* what, const void* q, const void* k, const void* v, const float* freqs_cos,
+                       const float* freqs_sin, int64_t freq_row_stride, void* o, float* lse, int B, int H, int N, int D,
+                       float sm_scale, int causal, const void* k_rot, const float* tile_kmax, void* workspace,
+                       int64_t workspace_bytes, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
   if (rc) return rc;
-  rc = check_ptrs("rope_attn_fwd", {q, k, v, freqs_cos, freqs_sin, o, lse});
+  rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse});
   if (rc) return rc;
   corope::FwdParams p{};
   p.q = static_cast<const uint16_t*>(q);
@@ -110,7 +122,73 @@ int corope_rope_attn_fwd(const void* q, const void* k, const void* v, const floa
   p.qk_scale = sm_scale * kLog2e;
   p.N = N;
   p.BH = B * H;
-  return launch_status("rope_attn_fwd", corope::launch_rope_attn_fwd(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+  p.k_rot = static_cast<const uint16_t*>(k_rot);
+  p.tile_kmax = tile_kmax;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (workspace != nullptr) {
+    rc = check_ptrs(what, {workspace});
+    if (rc) return rc;
+    if (workspace_bytes < fwd_ws_bytes(B, H, N, D))
+      return fail(COROPE_E_BADARG, "%s: workspace of %lld bytes, %lld needed", what, (long long)workspace_bytes,
+                  (long long)fwd_ws_bytes(B, H, N, D));
+    uint16_t* ws_k = static_cast<uint16_t*>(workspace);
+    float* ws_max = reinterpret_cast<float*>(static_cast<char*>(workspace) + fwd_ws_krot_bytes(B, H, N, D));
+    rc = launch_status(what, corope::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, ws_k, ws_max, p.BH, N, D, st));
+    if (rc) return rc;
+    p.k_rot = ws_k;
+    p.tile_kmax = ws_max;
+  }
+  return launch_status(what, corope::launch_rope_attn_fwd(p, D, causal != 0, st));
+}
+
+}  // namespace
+
+extern "C" {
+
+int corope_rope_attn_fwd(const void* q, const void* k, const void* v, const float* freqs_cos, const float* freqs_sin,
+                         int64_t freq_row_stride, void* o, float* lse, int B, int H, int N, int D, float sm_scale,
+                         int causal, void* stream) {
+  return rope_attn_fwd_impl("rope_attn_fwd", q, k, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, H, N, D, sm_scale,
+                            causal, nullptr, nullptr, nullptr, 0, stream);
+}
+
+int64_t corope_rope_attn_fwd_workspace_bytes(int B, int H, int N, int D) {
+  if (corope_rope_attn_check(B, H, N, D, D, 1.f, 0)) return -1;
+  return fwd_ws_bytes(B, H, N, D);
+}
+
+int corope_rope_attn_fwd_ws(const void* q, const void* k, const void* v, const float* freqs_cos, const float* freqs_sin,
+                            int64_t freq_row_stride, void* o, float* lse, int B, int H, int N, int D, float sm_scale,
+                            int causal, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (workspace == nullptr) return fail(COROPE_E_BADARG, "rope_attn_fwd_ws: null workspace");
+  return rope_attn_fwd_impl("rope_attn_fwd_ws", q, k, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, H, N, D,
+                            sm_scale, causal, nullptr, nullptr, workspace, workspace_bytes, stream);
+}
+
+int corope_rope_attn_fwd_prerotated(const void* q, const void* k_rot, const float* tile_kmax, const void* v,
+                                    const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* o,
+                                    float* lse, int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
+  int rc = check_ptrs("rope_attn_fwd_prerotated", {k_rot});
+  if (rc) return rc;
+  if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
+    return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "rope_attn_fwd_prerotated: tile_kmax %p is null or misaligned",
+                (const void*)tile_kmax);
+  return rope_attn_fwd_impl("rope_attn_fwd_prerotated", q, k_rot, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, H,
+                            N, D, sm_scale, causal, k_rot, tile_kmax, nullptr, 0, stream);
+}
+
+int corope_rope_rotate(const void* x, const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* y,
+                       float* tile_max, int B, int H, int N, int D, void* stream) {
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, 1.f, 0);
+  if (rc) return rc;
+  rc = check_ptrs("rope_rotate", {x, freqs_cos, freqs_sin, y});
+  if (rc) return rc;
+  if (tile_max != nullptr && (reinterpret_cast<uintptr_t>(tile_max) & 3u))
+    return fail(COROPE_E_ALIGN, "rope_rotate: tile_max %p is not 4-byte aligned", (void*)tile_max);
+  return launch_status("rope_rotate",
+                       corope::launch_rope_rotate(static_cast<const uint16_t*>(x), freqs_cos, freqs_sin, freq_row_stride,
+                                                  static_cast<uint16_t*>(y), tile_max, B * H, N, D,
+                                                  static_cast<hipStream_t>(stream)));
 }
 
 int corope_rope_attn_bwd_preprocess(const void* o, const void* d_o, float* delta, int B, int H, int N, int D,

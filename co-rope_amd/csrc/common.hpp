@@ -67,6 +67,15 @@ __device__ __forceinline__ float half_sum(float x) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
+// ---- addressing ------------------------------------------------------------------------------------
+// base + a 32-bit unsigned byte offset.  With a wave-uniform base this is the "scalar base + 32-bit vector offset"
+// form of the global load, which needs one address register per lane instead of two and no 64-bit arithmetic.
+// Callers guarantee that one (batch, head) slice and the cos/sin tables stay below 4 GiB.
+template <typename T>
+__device__ __forceinline__ const T* byte_offset(const T* base, uint32_t bytes) {
+  return reinterpret_cast<const T*>(reinterpret_cast<const char*>(base) + bytes);
+}
+
 // ---- LDS tile layouts -----------------------------------------------------------------------------
 // Row-major tile [rows][D] of bf16 with PAD elements of padding per row.
 //   PAD = 8  (16 bytes): 16 consecutive rows read at the same column with 16-byte reads land in 16 different
@@ -117,11 +126,12 @@ struct RotStage {
       if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
       int r = u / kChunks, ch = u % kChunks;
       int row = min(row0 + r, n_rows - 1);
-      const uint16_t* p = src + (int64_t)row * D + ch * 8;
+      const uint16_t* p = byte_offset(src, (uint32_t)row * (D * 2) + ch * 16);
       x1[it] = *reinterpret_cast<const u32x4*>(p);
       x2[it] = *reinterpret_cast<const u32x4*>(p + D / 2);
-      const float* cp = cosp + (int64_t)row * fstride + ch * 8;
-      const float* sp = sinp + (int64_t)row * fstride + ch * 8;
+      const uint32_t foff = ((uint32_t)row * (uint32_t)fstride + ch * 8) * 4;
+      const float* cp = byte_offset(cosp, foff);
+      const float* sp = byte_offset(sinp, foff);
       c[it][0] = *reinterpret_cast<const f32x4*>(cp);
       c[it][1] = *reinterpret_cast<const f32x4*>(cp + 4);
       s[it][0] = *reinterpret_cast<const f32x4*>(sp);
@@ -140,11 +150,12 @@ struct RotStage {
       if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
       int r = u / kChunks, ch = u % kChunks;
       int row = min(row0 + r, n_rows - 1);
-      const uint16_t* p = src + (int64_t)row * D + ch * 8;
+      const uint16_t* p = byte_offset(src, (uint32_t)row * (D * 2) + ch * 16);
       x1[it] = *reinterpret_cast<const u32x4*>(p);
       x2[it] = *reinterpret_cast<const u32x4*>(p + D / 2);
-      const float* cp = cosp + (int64_t)row * fstride + ch * 8;
-      const float* sp = sinp + (int64_t)row * fstride + ch * 8;
+      const uint32_t foff = ((uint32_t)row * (uint32_t)fstride + ch * 8) * 4;
+      const float* cp = byte_offset(cosp, foff);
+      const float* sp = byte_offset(sinp, foff);
       c[it][0] = *reinterpret_cast<const f32x4*>(cp);
       c[it][1] = *reinterpret_cast<const f32x4*>(cp + 4);
       s[it][0] = *reinterpret_cast<const f32x4*>(sp);
@@ -266,7 +277,7 @@ struct CopyStage {
       int u = threadIdx.x + it * NT;
       if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
       int row = min(row0 + u / kChunks, n_rows - 1);
-      x[it] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * D + (u % kChunks) * 8);
+      x[it] = *reinterpret_cast<const u32x4*>(byte_offset(src, (uint32_t)row * (D * 2) + (u % kChunks) * 16));
     }
   }
   __device__ __forceinline__ void store_rows(uint16_t* lds) const {
@@ -285,7 +296,7 @@ struct CopyStage {
       int u = threadIdx.x + it * NT;
       if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
       int row = min(row0 + u / kChunks, n_rows - 1);
-      x[it] = *reinterpret_cast<const u32x4*>(src + (int64_t)row * D + (u % kChunks) * 8);
+      x[it] = *reinterpret_cast<const u32x4*>(byte_offset(src, (uint32_t)row * (D * 2) + (u % kChunks) * 16));
     }
   }
   __device__ __forceinline__ void store_rows_part(int it0, int it1, uint16_t* lds) const {

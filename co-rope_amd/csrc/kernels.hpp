@@ -10,6 +10,8 @@ struct FwdParams {
   const uint16_t* q;
   const uint16_t* k;
   const uint16_t* v;
+  const uint16_t* k_rot;   // K already rotated (same layout as k), or null: rotate K tiles inside the kernel
+  const float* tile_kmax;  // with k_rot: largest rotated-key norm of every 64-key tile, [BH][ceil(N / 64)]
   const float* cos;
   const float* sin;
   uint16_t* o;
@@ -53,6 +55,9 @@ struct CoropeParams {
   int num_m_blocks;
 };
 
+// y = rotated x for a (BH, N, D) tensor; tile_max (may be null) receives [BH][ceil(N / 64)] largest row norms.
+hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
+                              float* tile_max, int BH, int N, int D, hipStream_t stream);
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_preprocess(const BwdParams& p, int D, hipStream_t stream);
 hipError_t launch_bwd_dv(const BwdParams& p, int D, bool causal, hipStream_t stream);

@@ -17,6 +17,8 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
+#include <type_traits>
+
 namespace corope {
 
 // Workgroup = 8 waves x 32 query rows = 256 rows, two waves per SIMD.
@@ -25,10 +27,10 @@ namespace corope {
 // instructions into its MFMA stream keeps the matrix pipe busier than one that runs an MFMA phase followed by a
 // VALU phase.  A 64-key tile is therefore consumed as two 32-key halves in four slots of 8 MFMAs each, and every
 // slot carries the VALU work of another stage in the same basic block for the instruction scheduler to mix in:
-//     slot A:  S^T(half 0)          +  rotate K of tile t+1 and write it to LDS, refill the K staging registers
+//     slot A:  S^T(half 0)          +  rotate K / copy V of tile t+1 into LDS, refill the staging registers (tile t+2)
 //     slot B:  S^T(half 1)          +  online softmax of half 0
 //     slot C:  O^T += V^T P^T(h0)   +  online softmax of half 1
-//     slot D:  O^T += V^T P^T(h1)   +  write V of tile t+1 to LDS, refill the V staging registers
+//     slot D:  O^T += V^T P^T(h1)
 // Scheduling barriers separate the slots and pin the operand prefetches ahead of the MFMAs that use them.
 constexpr int kFwdWaves = 8;
 constexpr int kFwdStages = 2;
@@ -44,44 +46,86 @@ struct FwdCfg {
   static constexpr int kLdsBytes = kFwdStages * kStageBytes;
 };
 
-// State of the online softmax while one 32-key half is processed.
-struct SoftmaxHalf {
-  float mt;     // maximum of the half's raw scores, then the new running maximum
-  float ms;     // new running maximum in the base-2 scaled domain
-  float alpha;  // factor that brings the old accumulators to the new maximum
-  float lsum;   // this lane's share of the half's denominator
-};
+// ---- online softmax with a lazily updated reference maximum -------------------------------------------------------
+// Probabilities are formed against a per-row reference m_ref that is NOT the running maximum: p = exp2(s*c - m_ref*c).
+// Any finite reference gives the same normalised result (numerator and denominator carry the same factor), so the
+// reference only has to stay close enough to the true maximum for p to remain a comfortable fp32 / bf16 number.  The
+// fast path therefore skips the maximum altogether (no reduction, no cross-lane exchange, no accumulator rescale, no
+// dependency between the scores and the first exponential); it only watches the half's partial denominator, and when
+// that grows past kLsumLimit -- some score is ~2^20 above the reference, or the reference is still -inf on the first
+// tile, which shows up as inf/NaN -- the half is redone on the slow path, which moves the reference to the true maximum
+// and rescales the accumulators like a classic online softmax.
+constexpr float kLsumLimit = 1048576.f;
 
-// Piece `step` of `n_steps` of the softmax of one half (16 raw scores per lane -> 8 bf16 pairs = two B operands).
-// Step 0 reduces the maximum, step 1 fixes the new running maximum, the others exponentiate.
-__device__ __forceinline__ void softmax_piece(int step, int n_steps, const f32x16& sacc, u32x4 (&pb)[2], SoftmaxHalf& st,
-                                              float m_run, float scale) {
-  if (step == 0) {
-    float mt = fmaxf(sacc[0], sacc[1]);
+// Fast-path piece `step` of `n_steps`: exponentiates 8 / n_steps score pairs of a half.
+__device__ __forceinline__ void softmax_fast_piece(int step, int n_steps, const f32x16& sacc, u32x4 (&pb)[2], float& lsum,
+                                                   float scale, float ms) {
+  const int lo = step * 8 / n_steps, hi = (step + 1) * 8 / n_steps;
+  asm volatile("" : "+v"(ms));  // the piece starts here, not wherever the scheduler would like to hoist it
 #pragma unroll
-    for (int i = 2; i < 16; i += 2) mt = fmaxf(fmaxf(mt, sacc[i]), sacc[i + 1]);
-    st.mt = mt;
-  } else if (step == 1) {
-    st.mt = fmaxf(m_run, half_max(st.mt));
-    st.ms = st.mt * scale;
-    st.alpha = fast_exp2(m_run * scale - st.ms);
-    st.lsum = 0.f;
-  } else {
-    const int n = n_steps - 2;
-    const int lo = (step - 2) * 8 / n, hi = (step - 1) * 8 / n;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      if (j < lo || j >= hi) continue;
-      float p0 = fast_exp2(sacc[2 * j] * scale - st.ms);
-      float p1 = fast_exp2(sacc[2 * j + 1] * scale - st.ms);
-      // plain adds: the bf16 dot-product instruction would do this in one op but stalls the MFMA pipe
-      st.lsum += p0 + p1;
-      pb[j / 4][j % 4] = pack_bf16(p0, p1);
-    }
+  for (int j = 0; j < 8; ++j) {
+    if (j < lo || j >= hi) continue;
+    float p0 = fast_exp2(sacc[2 * j] * scale - ms);
+    float p1 = fast_exp2(sacc[2 * j + 1] * scale - ms);
+    // plain adds: the bf16 dot-product instruction would do this in one op but stalls the MFMA pipe
+    lsum += p0 + p1;
+    uint32_t w = pack_bf16(p0, p1);
+    asm volatile("" : "+v"(w));  // keeps the piece between the two MFMAs it is written between
+    pb[j / 4][j % 4] = w;
   }
 }
 
-template <int D, int BLOCK_N, bool CAUSAL>
+// Slow path of one half: classic online-softmax step.  Returns the factor the accumulators must be multiplied by.
+__device__ __forceinline__ float softmax_slow_half(const f32x16& sacc, u32x4 (&pb)[2], float& m_ref, float& l_run,
+                                                   float scale) {
+  float mt = fmaxf(sacc[0], sacc[1]);
+#pragma unroll
+  for (int i = 2; i < 16; i += 2) mt = fmaxf(fmaxf(mt, sacc[i]), sacc[i + 1]);
+  const float m_new = fmaxf(m_ref, half_max(mt));
+  const float ms = m_new * scale;
+  const float alpha = fast_exp2(m_ref * scale - ms);
+  float lsum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    float p0 = fast_exp2(sacc[2 * j] * scale - ms);
+    float p1 = fast_exp2(sacc[2 * j + 1] * scale - ms);
+    lsum += p0 + p1;
+    pb[j / 4][j % 4] = pack_bf16(p0, p1);
+  }
+  l_run = l_run * alpha + lsum;
+  m_ref = m_new;
+  return alpha;
+}
+
+// How a tile's softmax is run.
+//   kChecked: fast pieces, each half verified afterwards (its denominator share must stay below kLsumLimit) and redone on
+//             the slow path if not -- needs no prior knowledge of the keys, costs two data-dependent branches per tile;
+//   kFast:    fast pieces, no verification -- only for tiles whose scores are known in advance not to exceed the reference
+//             maximum by more than kLazyMargin (in the base-2 domain).  Probabilities then stay below 2^kLazyMargin and
+//             the fp32 sums below 2^(kLazyMargin + log2 N + log2 max|v|), far from overflow; bf16 has fp32's exponent
+//             range, so P loses nothing either.
+enum TileMode { kChecked, kFast };
+constexpr float kLazyMargin = 64.f;
+
+// K staging: rotate on the way to LDS, or plain copy of an already rotated K.
+template <int D, int ROWS, int NT, bool PREROT>
+struct KStage : RotStage<D, ROWS, NT> {};
+template <int D, int ROWS, int NT>
+struct KStage<D, ROWS, NT, true> : CopyStage<D, ROWS, NT, 8> {
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float*, const float*, int64_t, int row0,
+                                       int n_rows) {
+    CopyStage<D, ROWS, NT, 8>::load(src, row0, n_rows);
+  }
+};
+
+// PREROT = false: K tiles are rotated inside the kernel, softmax in kChecked mode (a single launch, no workspace).
+// PREROT = true:  K was rotated by rope_rotate_kernel, which also left the largest key norm of every 64-key tile; with the
+//                 norm of the lane's own (rotated) query that bounds every score of the tile (Cauchy-Schwarz), so a tile
+//                 is classified before it is touched: when the bound is within kLazyMargin of the reference maximum the
+//                 tile runs in kFast mode as it is (no data-dependent branch inside the tile); otherwise its scores are
+//                 computed once just for their maximum, the reference moves there (accumulators rescaled), and the tile
+//                 then runs in kFast mode all the same.
+template <int D, int BLOCK_N, bool CAUSAL, bool PREROT>
 __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdParams p) {
   using Cfg = FwdCfg<D, BLOCK_N>;
   static_assert(BLOCK_N == 64, "the slot schedule is written for two 32-key halves");
@@ -89,6 +133,7 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
   constexpr int KC = D / 16;        // contraction chunks of QK^T = MFMAs per S^T half
   constexpr int NDB = D / 32;       // 32-column blocks of O
   constexpr int NPV = 2 * NDB;      // MFMAs per PV half
+  constexpr int KA = 4;             // K operands in flight
   constexpr int LSV = RowTile<D, Cfg::kVPad>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -102,13 +147,13 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
   const int N = p.N;
 
   const uint16_t* qg = p.q + (int64_t)bh * N * D;
-  const uint16_t* kg = p.k + (int64_t)bh * N * D;
+  const uint16_t* kg = (PREROT ? p.k_rot : p.k) + (int64_t)bh * N * D;
   const uint16_t* vg = p.v + (int64_t)bh * N * D;
 
-  const int n_tiles = CAUSAL ? min((m0 + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, (N + BLOCK_N - 1) / BLOCK_N)
-                             : (N + BLOCK_N - 1) / BLOCK_N;
+  const int n_k_tiles = (N + BLOCK_N - 1) / BLOCK_N;
+  const int n_tiles = CAUSAL ? min((m0 + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, n_k_tiles) : n_k_tiles;
 
-  RotStage<D, BLOCK_N, NT> kst;
+  KStage<D, BLOCK_N, NT, PREROT> kst;
   CopyStage<D, BLOCK_N, NT, Cfg::kVPad> vst;
   kst.load(kg, p.cos, p.sin, p.fstride, 0, N);
   vst.load(vg, 0, N);
@@ -118,10 +163,27 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
   u32x4 qb[KC];
   load_b_rows<D, true>(qb, qg, p.cos, p.sin, p.fstride, min(q_row, N - 1));
 
+  const float scale = p.qk_scale;
+  // PREROT: |q_r| * scale (a little generous), times a tile's largest key norm = upper bound of its scaled scores.
+  float q_bound = 0.f;
+  const float* tile_kmax = nullptr;
+  if constexpr (PREROT) {
+    float ss = 0.f;
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        float x0 = bf16_lo(qb[kc][w]), x1 = bf16_hi(qb[kc][w]);
+        ss += x0 * x0 + x1 * x1;
+      }
+    q_bound = __builtin_sqrtf(half_sum(ss)) * scale * 1.01f;
+    tile_kmax = p.tile_kmax + (int64_t)bh * n_k_tiles;
+  }
+
   f32x16 oacc[NDB];
 #pragma unroll
   for (int i = 0; i < NDB; ++i) oacc[i] = f32x16{0};
-  float m_run = -INFINITY;   // running row maximum of the raw scores (this lane's query)
+  float m_run = -INFINITY;   // reference maximum of the raw scores (this lane's query); see the softmax notes above
   float l_run = 0.f;         // this lane's share of the running denominator
 
   auto ks = [&](int t) { return reinterpret_cast<uint16_t*>(smem + (t % kFwdStages) * Cfg::kStageBytes); };
@@ -137,19 +199,18 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
   vst.load(vg, BLOCK_N, N);
   __syncthreads();
 
-  const float scale = p.qk_scale;
   const int wave_q_lo = m0 + wave * 32, wave_q_hi = wave_q_lo + 31;
 
   for (int t = 0; t < n_tiles; ++t) {
     const int n0 = t * BLOCK_N;
     const uint16_t* kt = ks(t) + RowTile<D>::off(lq, 8 * lh);
     const uint16_t* vt = vs(t);
-    auto stage_k = [&]() {
+    // All of the staging happens at one point of the iteration: tile t+1 goes from the staging registers to its LDS
+    // buffer and the registers are refilled with tile t+2 straight away.
+    auto stage_next = [&]() {
       kst.store_rows(ks(t + 1));
-      kst.load(kg, p.cos, p.sin, p.fstride, n0 + 2 * BLOCK_N, N);
-    };
-    auto stage_v = [&]() {
       vst.store_rows(vs(t + 1));
+      kst.load(kg, p.cos, p.sin, p.fstride, n0 + 2 * BLOCK_N, N);
       vst.load(vg, n0 + 2 * BLOCK_N, N);
     };
     auto k_operand = [&](int half, int kc) {
@@ -166,45 +227,50 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
       }
     };
     auto rescale = [&](float alpha) {
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
-        for (int db = 0; db < NDB; ++db)
+      for (int db = 0; db < NDB; ++db)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
-      }
+        for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
     };
 
-    // Tiles entirely above this wave's diagonal contribute nothing to it; the wave still stages its share.
-    const bool active = !CAUSAL || n0 <= wave_q_hi;
-    const bool need_mask = (CAUSAL && n0 + BLOCK_N - 1 > wave_q_lo) || (!CAUSAL && n0 + BLOCK_N > N);
-    if (active) {
+    // One tile in four slots of 8 MFMAs (see the schedule at the top of the file).
+    auto run_tile = [&](auto mode_c, const bool MASK) {
+      constexpr TileMode MODE = decltype(mode_c)::value;
       f32x16 s0 = f32x16{0}, s1 = f32x16{0};
       u32x4 pb0[2], pb1[2];
-      SoftmaxHalf st0, st1;
-      u32x4 a[KC];  // A operands, fetched one slot ahead of the MFMAs that consume them
+      float lsum0 = 0.f, lsum1 = 0.f;
+      float ms_ref = m_run * scale;
+      u32x4 a[KA];  // ring of A operands, fetched KA MFMAs ahead of their use
 #pragma unroll
-      for (int kc = 0; kc < KC; ++kc) a[kc] = k_operand(0, kc);
+      for (int kc = 0; kc < KA; ++kc) a[kc] = k_operand(0, kc);
       __builtin_amdgcn_sched_barrier(0);
-      // ---- slot A: S^T(half 0), K staging on the side --------------------------------------------------------
+      // ---- slot A: S^T(half 0), staging on the side --------------------------------------------------------------
 #pragma unroll
       for (int kc = 0; kc < KC; ++kc) {
-        s0 = mfma32(a[kc], qb[kc], s0);
-        a[kc] = k_operand(1, kc);
-        if (kc == 0) stage_k();
+        s0 = mfma32(a[kc % KA], qb[kc], s0);
+        a[kc % KA] = kc + KA < KC ? k_operand(0, kc + KA) : k_operand(1, kc + KA - KC);
+        if (kc == 0) stage_next();
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (need_mask) mask_scores(s0, 0);
+      if (MASK) mask_scores(s0, 0);
       __builtin_amdgcn_sched_barrier(0);
       // ---- slot B: S^T(half 1), softmax of half 0 between the MFMAs ---------------------------------------------
 #pragma unroll
       for (int kc = 0; kc < KC; ++kc) {
-        s1 = mfma32(a[kc], qb[kc], s1);
-        softmax_piece(kc, KC, s0, pb0, st0, m_run, scale);
+        s1 = mfma32(a[kc % KA], qb[kc], s1);
+        if (kc + KA < KC) a[kc % KA] = k_operand(1, kc + KA);
+        softmax_fast_piece(kc, KC, s0, pb0, lsum0, scale, ms_ref);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      m_run = st0.mt;
-      l_run = l_run * st0.alpha + st0.lsum;
-      rescale(st0.alpha);
-      if (need_mask) mask_scores(s1, 1);
+      if (MODE == kChecked) {
+        if (__builtin_amdgcn_ballot_w64(!(lsum0 <= kLsumLimit))) {
+          rescale(softmax_slow_half(s0, pb0, m_run, l_run, scale));
+        } else {
+          l_run += lsum0;
+        }
+        ms_ref = m_run * scale;
+      }
+      if (MASK) mask_scores(s1, 1);
       u32x4 av[NDB];  // transposed V operands, one 16-key chunk ahead
 #pragma unroll
       for (int db = 0; db < NDB; ++db) av[db] = v_operand(0, db);
@@ -214,22 +280,61 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
       for (int i = 0; i < NPV; ++i) {
         oacc[i % NDB] = mfma32(av[i % NDB], pb0[i / NDB], oacc[i % NDB]);
         av[i % NDB] = i + NDB < NPV ? v_operand(0, i + NDB) : v_operand(1, i + NDB - NPV);
-        softmax_piece(i, NPV, s1, pb1, st1, m_run, scale);
+        softmax_fast_piece(i, NPV, s1, pb1, lsum1, scale, ms_ref);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      m_run = st1.mt;
-      l_run = l_run * st1.alpha + st1.lsum;
-      rescale(st1.alpha);
+      if (MODE == kChecked) {
+        if (__builtin_amdgcn_ballot_w64(!(lsum1 <= kLsumLimit))) {
+          rescale(softmax_slow_half(s1, pb1, m_run, l_run, scale));
+        } else {
+          l_run += lsum1;
+        }
+      }
+      if (MODE == kFast) l_run += lsum0 + lsum1;
       __builtin_amdgcn_sched_barrier(0);
-      // ---- slot D: O^T += V^T P^T(half 1), V staging on the side -------------------------------------------------
+      // ---- slot D: O^T += V^T P^T(half 1) ------------------------------------------------------------------------
 #pragma unroll
       for (int i = 0; i < NPV; ++i) {
         oacc[i % NDB] = mfma32(av[i % NDB], pb1[i / NDB], oacc[i % NDB]);
         if (i + NDB < NPV) av[i % NDB] = v_operand(1, i + NDB);
-        if (i == 0) stage_v();
+      }
+    };
+    // Moves the reference maximum of every row to the true maximum over this tile (and what came before).
+    auto raise_reference = [&](const bool MASK) {
+      f32x16 s0 = f32x16{0}, s1 = f32x16{0};
+#pragma unroll
+      for (int kc = 0; kc < KC; ++kc) {
+        s0 = mfma32(k_operand(0, kc), qb[kc], s0);
+        s1 = mfma32(k_operand(1, kc), qb[kc], s1);
+      }
+      if (MASK) {
+        mask_scores(s0, 0);
+        mask_scores(s1, 1);
+      }
+      float mt = fmaxf(s0[0], s1[0]);
+#pragma unroll
+      for (int i = 1; i < 16; ++i) mt = fmaxf(fmaxf(mt, s0[i]), s1[i]);
+      const float m_new = fmaxf(m_run, half_max(mt));
+      const float alpha = fast_exp2((m_run - m_new) * scale);   // m_new is finite: every row sees key 0 of tile 0
+      l_run *= alpha;
+      rescale(alpha);
+      m_run = m_new;
+    };
+
+    // Tiles entirely above this wave's diagonal contribute nothing to it; the wave still stages its share.
+    const bool active = !CAUSAL || n0 <= wave_q_hi;
+    const bool need_mask = (CAUSAL && n0 + BLOCK_N - 1 > wave_q_lo) || (!CAUSAL && n0 + BLOCK_N > N);
+    if (active) {
+      if constexpr (PREROT) {
+        // tile_kmax[t] is wave-uniform; a tile is fast only if no lane can exceed its reference by kLazyMargin
+        const float bound = q_bound * tile_kmax[t];
+        if (__builtin_amdgcn_ballot_w64(!(bound <= m_run * scale + kLazyMargin))) raise_reference(need_mask);
+        run_tile(std::integral_constant<TileMode, kFast>{}, need_mask);
+      } else {
+        run_tile(std::integral_constant<TileMode, kChecked>{}, need_mask);
       }
     } else {
-      stage_k();
-      stage_v();
+      stage_next();
     }
     __syncthreads();
   }
@@ -253,10 +358,10 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
 }
 
 // ---- host-side launch -----------------------------------------------------------------------------------------
-template <int D, int BLOCK_N, bool CAUSAL>
+template <int D, int BLOCK_N, bool CAUSAL, bool PREROT>
 static hipError_t launch_fwd_cfg(FwdParams p, hipStream_t stream) {
   using Cfg = FwdCfg<D, BLOCK_N>;
-  auto kern = rope_attn_fwd_kernel<D, BLOCK_N, CAUSAL>;
+  auto kern = rope_attn_fwd_kernel<D, BLOCK_N, CAUSAL, PREROT>;
   static bool attr_set = false;  // per instantiation; benign if raced (same value)
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -270,9 +375,15 @@ static hipError_t launch_fwd_cfg(FwdParams p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <int D>
+static hipError_t launch_fwd_d(const FwdParams& p, bool causal, hipStream_t stream) {
+  if (p.k_rot)
+    return causal ? launch_fwd_cfg<D, 64, true, true>(p, stream) : launch_fwd_cfg<D, 64, false, true>(p, stream);
+  return causal ? launch_fwd_cfg<D, 64, true, false>(p, stream) : launch_fwd_cfg<D, 64, false, false>(p, stream);
+}
+
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream) {
-  if (D == 128) return causal ? launch_fwd_cfg<128, 64, true>(p, stream) : launch_fwd_cfg<128, 64, false>(p, stream);
-  return causal ? launch_fwd_cfg<64, 64, true>(p, stream) : launch_fwd_cfg<64, 64, false>(p, stream);
+  return D == 128 ? launch_fwd_d<128>(p, causal, stream) : launch_fwd_d<64>(p, causal, stream);
 }
 
 }  // namespace corope

@@ -48,24 +48,48 @@ def _freq_table(f):
     return f
 
 
+# Sequences at least this long take the two-launch forward (K rotated once into a scratch buffer, then attention on
+# the rotated copy); shorter ones the single launch, where every K tile is rotated by few query blocks anyway.
+TWO_LAUNCH_MIN_N = 1024
+
+
+def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None):
+    """Runs the forward kernels; returns (o, M, fc, fs) with the tables in the form the kernels were given."""
+    lib = _lib.load()
+    fc, fs = _freq_table(freqs_cos), _freq_table(freqs_sin)
+    if fc.stride(0) != fs.stride(0):
+        fc, fs = fc.contiguous(), fs.contiguous()
+    B, H, N, D = q.shape
+    o = torch.empty_like(q)
+    M = torch.empty((B, H, N), device=q.device, dtype=torch.float32)
+    if two_launch is None:
+        two_launch = N >= TWO_LAUNCH_MIN_N
+    with torch.cuda.device(q.device):
+        if two_launch:
+            nbytes = lib.corope_rope_attn_fwd_workspace_bytes(B, H, N, D)
+            if nbytes < 0:
+                _lib.check(lib.corope_rope_attn_check(B, H, N, D, fc.stride(0), float(sm_scale), 0), "corope_rope_attn_check")
+            ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+            rc = lib.corope_rope_attn_fwd_ws(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
+                                             fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, N, D, float(sm_scale),
+                                             int(bool(causal)), ws.data_ptr(), nbytes, _stream_ptr(q))
+            _lib.check(rc, "corope_rope_attn_fwd_ws")
+        else:
+            rc = lib.corope_rope_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
+                                          fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, N, D, float(sm_scale),
+                                          int(bool(causal)), _stream_ptr(q))
+            _lib.check(rc, "corope_rope_attn_fwd")
+    return o, M, fc, fs
+
+
 class _FusedRopeAttn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, causal, sm_scale, freqs_cos, freqs_sin, warp_specialize=True):
         _check_inputs(q, k, v, freqs_cos, freqs_sin)
-        lib = _lib.load()
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        fc, fs = _freq_table(freqs_cos), _freq_table(freqs_sin)
-        if fc.stride(0) != fs.stride(0):
-            fc, fs = fc.contiguous(), fs.contiguous()
         B, H, N, D = q.shape
-        o = torch.empty_like(q)
-        M = torch.empty((B, H, N), device=q.device, dtype=torch.float32)
-        with torch.cuda.device(q.device):
-            rc = lib.corope_rope_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
-                                          fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, N, D, float(sm_scale),
-                                          int(bool(causal)), _stream_ptr(q))
-        _lib.check(rc, "corope_rope_attn_fwd")
+        o, M, fc, fs = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin)
         ctx.save_for_backward(q, k, v, o, M, fc, fs)
         ctx.sm_scale = float(sm_scale)
         ctx.HEAD_DIM = D
@@ -101,20 +125,29 @@ def fused_rope_attn(q, k, v, freqs_cos, freqs_sin, causal=True, sm_scale=None):
     return attention(q, k, v, causal, sm_scale, freqs_cos, freqs_sin)
 
 
-def rope_attn_forward_with_lse(q, k, v, causal, sm_scale, freqs_cos, freqs_sin):
-    """Forward only, returning (O, M) where M is the saved base-2 log-sum-exp statistic (B, H, N) fp32."""
+def rope_attn_forward_with_lse(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None):
+    """Forward only, returning (O, M) where M is the saved base-2 log-sum-exp statistic (B, H, N) fp32.
+    ``two_launch`` forces (True / False) or leaves to the length rule (None) the choice of forward path."""
     _check_inputs(q, k, v, freqs_cos, freqs_sin)
-    lib = _lib.load()
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    o, M, _, _ = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch)
+    return o, M
+
+
+def rope_rotate(x, freqs_cos, freqs_sin, with_tile_max=False):
+    """Half-layout rotation of x (B, H, N, D) bf16 on the device (fp32 arithmetic, one rounding to bf16).
+    Returns y, or (y, tile_max) with the largest rotated-row norm of every 64-row tile, (B, H, ceil(N/64)) fp32."""
+    _check_inputs(x, x, x, freqs_cos, freqs_sin)
+    lib = _lib.load()
+    x = x.contiguous()
     fc, fs = _freq_table(freqs_cos), _freq_table(freqs_sin)
     if fc.stride(0) != fs.stride(0):
         fc, fs = fc.contiguous(), fs.contiguous()
-    B, H, N, D = q.shape
-    o = torch.empty_like(q)
-    M = torch.empty((B, H, N), device=q.device, dtype=torch.float32)
-    with torch.cuda.device(q.device):
-        rc = lib.corope_rope_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
-                                      fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, N, D, float(sm_scale),
-                                      int(bool(causal)), _stream_ptr(q))
-    _lib.check(rc, "corope_rope_attn_fwd")
-    return o, M
+    B, H, N, D = x.shape
+    y = torch.empty_like(x)
+    tm = torch.empty((B, H, (N + 63) // 64), device=x.device, dtype=torch.float32) if with_tile_max else None
+    with torch.cuda.device(x.device):
+        rc = lib.corope_rope_rotate(x.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0), y.data_ptr(),
+                                    tm.data_ptr() if with_tile_max else None, B, H, N, D, _stream_ptr(x))
+    _lib.check(rc, "corope_rope_rotate")
+    return (y, tm) if with_tile_max else y

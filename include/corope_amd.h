@@ -62,6 +62,34 @@ int corope_rope_attn_fwd(const void *q, const void *k, const void *v,
                          void *o, float *lse,
                          int B, int H, int N, int D, float sm_scale, int causal, void *stream);
 
+/* Two-launch forward for long sequences: rotates K once into `workspace` (with the largest key norm of every
+ * 64-key tile), then runs the attention kernel on the rotated copy, whose inner loop reads no cos/sin tables and
+ * takes no data-dependent branch on tiles the norms prove harmless.  Same results as corope_rope_attn_fwd
+ * (the rotated K is rounded to bf16 exactly as the single-launch kernel rounds it).  The reference rotates K
+ * inside every program instead (fused-rope/fused_rope_attn.py:82-99); same launch site as above (:702-716).
+ * workspace: device memory, 16-byte aligned, at least corope_rope_attn_fwd_workspace_bytes(B,H,N,D) bytes; it is
+ * scratch, nothing in it has to survive the call. */
+int64_t corope_rope_attn_fwd_workspace_bytes(int B, int H, int N, int D); /* -1 for unsupported sizes */
+int corope_rope_attn_fwd_ws(const void *q, const void *k, const void *v,
+                            const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                            void *o, float *lse,
+                            int B, int H, int N, int D, float sm_scale, int causal,
+                            void *workspace, int64_t workspace_bytes, void *stream);
+
+/* y = half-layout rotation of x (B,H,N,D) bf16, fp32 arithmetic, rounded to bf16; tile_max (may be NULL) receives
+ * [B*H][ceil(N/64)] floats, the largest norm of a rotated row in every 64-row tile.
+ * Replaces apply_rotary_emb (reference fused-rope/rope_attn_pytorch.py:60-91). */
+int corope_rope_rotate(const void *x, const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                       void *y, float *tile_max, int B, int H, int N, int D, void *stream);
+
+/* Attention on a K that corope_rope_rotate already rotated (k_rot, with its tile_max as tile_kmax): the second
+ * launch of corope_rope_attn_fwd_ws on its own, for callers that keep the rotated K (a key cache) or time the two
+ * launches separately.  q is still rotated inside the kernel.  Same reference site as corope_rope_attn_fwd. */
+int corope_rope_attn_fwd_prerotated(const void *q, const void *k_rot, const float *tile_kmax, const void *v,
+                                    const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                                    void *o, float *lse,
+                                    int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
 /* delta[b,h,i] = sum_d o[b,h,i,d] * do[b,h,i,d]  (fp32).
  * Replaces _attn_bwd_preprocess (reference fused-rope/fused_rope_attn.py:324-337, launch :753-758). */
 int corope_rope_attn_bwd_preprocess(const void *o, const void *d_o, float *delta,

@@ -21,10 +21,10 @@ def _inputs(B, H, N, D, seed=42, std=1.0):
     return q, k, v
 
 
-def _run(pkg, q, k, v, causal, scale, c, s):
+def _run(pkg, q, k, v, causal, scale, c, s, two_launch=None):
     dev = torch.device("cuda:0")
     o, M = pkg.rope_attn_forward_with_lse(q.to(dev, torch.bfloat16), k.to(dev, torch.bfloat16), v.to(dev, torch.bfloat16),
-                                          causal, scale, c.to(dev), s.to(dev))
+                                          causal, scale, c.to(dev), s.to(dev), two_launch)
     torch.cuda.synchronize()
     return o.float().cpu(), M.cpu()
 
@@ -35,14 +35,16 @@ SHAPES = [(2, 4, 512, 64), (1, 8, 1024, 128), (4, 16, 2048, 64), (4, 8, 1024, 64
           (1, 2, 200, 64), (2, 1, 77, 128), (1, 3, 333, 128), (1, 1, 1, 64), (1, 1, 31, 128), (1, 2, 257, 128)]
 
 
+# two_launch: False = single launch (K rotated inside the kernel), True = K rotated once into a workspace first
+@pytest.mark.parametrize("two_launch", [False, True])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,N,D", SHAPES)
-def test_forward_parity(pkg, B, H, N, D, causal):
-    print(f"case B={B} H={H} N={N} D={D} causal={causal}", flush=True)
+def test_forward_parity(pkg, B, H, N, D, causal, two_launch):
+    print(f"case B={B} H={H} N={N} D={D} causal={causal} two_launch={two_launch}", flush=True)
     q, k, v = _inputs(B, H, N, D)
     c, s = O.precompute_freqs_cis(D, N)
     scale = 1 / math.sqrt(D)
-    o, M = _run(pkg, q, k, v, causal, scale, c, s)
+    o, M = _run(pkg, q, k, v, causal, scale, c, s, two_launch)
     ro, rl = O.rope_attn_forward_blocked(q, k, v, causal, scale, c, s)
     err = (o - ro).abs()
     print(f"  O max-abs {err.max():.3e} mean-abs {err.mean():.3e}; LSE max-abs {(M * LN2 - rl).abs().max():.3e}")
@@ -51,14 +53,15 @@ def test_forward_parity(pkg, B, H, N, D, causal):
     assert (M * LN2 - rl).abs().max() <= TOL
 
 
+@pytest.mark.parametrize("two_launch", [False, True])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,N,D", [(2, 4, 512, 64), (1, 8, 1024, 128), (4, 16, 2048, 64)])
-def test_forward_parity_verification_script_cases(pkg, B, H, N, D, causal):
+def test_forward_parity_verification_script_cases(pkg, B, H, N, D, causal, two_launch):
     """The six cases of the reference's verification script (fused-rope/verification.py:153-161), sm_scale = 0.5."""
-    print(f"case B={B} H={H} N={N} D={D} causal={causal} sm_scale=0.5", flush=True)
+    print(f"case B={B} H={H} N={N} D={D} causal={causal} sm_scale=0.5 two_launch={two_launch}", flush=True)
     q, k, v = _inputs(B, H, N, D)
     c, s = O.precompute_freqs_cis(D, N)
-    o, M = _run(pkg, q, k, v, causal, 0.5, c, s)
+    o, M = _run(pkg, q, k, v, causal, 0.5, c, s, two_launch)
     ro, rl = O.rope_attn_forward_blocked(q, k, v, causal, 0.5, c, s)
     err = (o - ro).abs()
     print(f"  O max-abs {err.max():.3e} mean-abs {err.mean():.3e}; LSE max-abs {(M * LN2 - rl).abs().max():.3e}")
@@ -118,3 +121,61 @@ def test_position_offset_leaves_attention_unchanged(pkg):
     o0, _ = pkg.rope_attn_forward_with_lse(qd, kd, vd, True, 0.09, c0, s0)
     o1, _ = pkg.rope_attn_forward_with_lse(qd, kd, vd, True, 0.09, c1, s1)
     assert (o0.float() - o1.float()).abs().max() <= 2e-2
+
+
+def test_rotate_pass_matches_the_oracle(pkg):
+    """corope_rope_rotate: y against the oracle's apply_rotary_emb (fp32, rounded to bf16 -- at most one bf16 ulp apart
+    where the device contracts a multiply-add), tile_max against the norms of the y it wrote."""
+    dev = torch.device("cuda:0")
+    for B, H, N, D in ((2, 3, 200, 128), (1, 2, 64, 64), (1, 1, 1, 128), (2, 2, 513, 64)):
+        print(f"case rotate B={B} H={H} N={N} D={D}", flush=True)
+        x = bf16_round(seeded((B, H, N, D), 3, std=2.0))
+        c, s = O.precompute_freqs_cis(D, N)
+        y, tm = pkg.rope_rotate(x.to(dev, torch.bfloat16), c.to(dev), s.to(dev), with_tile_max=True)
+        y, tm = y.float().cpu(), tm.cpu()
+        ref = O.apply_rotary_emb(x, c, s)
+        assert ((y - ref).abs() <= ref.abs() / 128 + 1e-30).all()   # within one bf16 ulp of the fp32 value
+        assert (y == bf16_round(ref)).float().mean() > 0.99
+        norms = y.norm(dim=-1)
+        pad = (-N) % 64
+        want = torch.nn.functional.pad(norms, (0, pad)).reshape(B, H, -1, 64).amax(-1)
+        assert tm.shape == want.shape and torch.allclose(tm, want, rtol=1e-5, atol=0)
+        y_only = pkg.rope_rotate(x.to(dev, torch.bfloat16), c.to(dev), s.to(dev))
+        assert torch.equal(y_only.float().cpu(), y)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("case", ["large_norms", "outlier_keys", "growing_scores", "tiny_scores"])
+def test_two_launch_softmax_modes(pkg, case, causal):
+    """Inputs that push tiles of the two-launch forward onto each of its softmax modes: the per-tile score bound
+    (query norm x largest key norm of the tile) decides, so large norms, a few huge keys, and scores that keep
+    growing along the sequence all force the exact mode on some tiles while others stay on the unchecked one."""
+    B, H, N, D = 1, 2, 640, 128
+    q, k, v = _inputs(B, H, N, D, seed=31)
+    scale = 1 / math.sqrt(D)
+    if case == "large_norms":
+        q, k = bf16_round(q * 2), bf16_round(k * 2)
+    elif case == "outlier_keys":
+        k[:, :, 0] *= 8      # an attention-sink-like first key
+        k[:, :, 300] *= 16
+        k = bf16_round(k)
+    elif case == "growing_scores":
+        ramp = torch.linspace(0.2, 3.0, N).reshape(1, 1, N, 1)
+        k = bf16_round(k * ramp)
+    elif case == "tiny_scores":
+        q, k = bf16_round(q * 1e-3), bf16_round(k * 1e-3)
+    c, s = O.precompute_freqs_cis(D, N)
+    print(f"case modes {case} causal={causal}", flush=True)
+    o, M = _run(pkg, q, k, v, causal, scale, c, s, True)
+    o1, M1 = _run(pkg, q, k, v, causal, scale, c, s, False)
+    ro, rl = O.rope_attn_forward_blocked(q, k, v, causal, scale, c, s)
+    for name, got, lse in (("two-launch", o, M), ("single", o1, M1)):
+        err = (got - ro).abs()
+        print(f"  {name}: O max-abs {err.max():.3e} mean-abs {err.mean():.3e} LSE {(lse * LN2 - rl).abs().max():.3e}")
+        assert torch.isfinite(got).all()
+        # sharp softmaxes amplify the bf16 rounding of the rotated operands: a looser max bound, a tight mean bound
+        assert err.max() <= TOL_HOT and err.mean() <= 5e-3
+        assert ((lse * LN2 - rl).abs() <= 2e-2 + rl.abs() / 128).all()
+    # both paths round the rotated operands identically; only the softmax bookkeeping differs between them (P is rounded
+    # to bf16 relative to different reference maxima), which can flip the bf16 rounding of an output: one ulp of slack
+    assert ((o - o1).abs() <= 5e-3 + o.abs() / 64).all() and (M - M1).abs().max() * LN2 <= 1e-3
