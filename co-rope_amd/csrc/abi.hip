@@ -138,6 +138,7 @@ int rope_attn_fwd_impl(const char* what, const void* q, const void* k, const voi
     p.k_rot = ws_k;
     p.tile_kmax = ws_max;
   }
+  if (p.k_rot != nullptr) return launch_status(what, corope::launch_rope_attn_fwd_prerotated(p, D, causal != 0, st));
   return launch_status(what, corope::launch_rope_attn_fwd(p, D, causal != 0, st));
 }
 

@@ -330,6 +330,22 @@ __device__ __forceinline__ u32x4 load_a_trans(const uint16_t* tile, int stride, 
   return u32x4{a[0], a[1], b[0], b[1]};
 }
 
+// The same read with the address split into its per-lane part and the rest: a_trans_lane_offset(stride) elements are
+// added to the tile once (per lane), load_a_trans_at then needs only compile-time offsets on top of that pointer.
+__device__ __forceinline__ int a_trans_lane_offset(int stride) {
+  const int l = threadIdx.x % kWave;
+  const int blk = l / 16, s = l % 16, h = blk / 2;
+  return (4 * h + s / 4) * stride + 16 * (blk % 2) + 4 * (s % 4);
+}
+__device__ __forceinline__ u32x4 load_a_trans_at(const uint16_t* lane_tile, int stride, int kbase, int m0) {
+  typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+  const uint16_t* p = lane_tile + kbase * stride + m0;
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 8 * stride));
+  u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
+  return u32x4{a[0], a[1], b[0], b[1]};
+}
+
 // Loads 32 rows x D of a (rows, D) bf16 matrix as the B operand chunks of mfma32 (lane = row, 8 columns per
 // chunk and lane-half), optionally applying the half-layout rotation first.  KC = D / 16 chunks.
 template <int D, bool ROTATE>

@@ -58,6 +58,7 @@ struct CoropeParams {
 // y = rotated x for a (BH, N, D) tensor; tile_max (may be null) receives [BH][ceil(N / 64)] largest row norms.
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
                               float* tile_max, int BH, int N, int D, hipStream_t stream);
+hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream);  // needs k_rot
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_preprocess(const BwdParams& p, int D, hipStream_t stream);
 hipError_t launch_bwd_dv(const BwdParams& p, int D, bool causal, hipStream_t stream);

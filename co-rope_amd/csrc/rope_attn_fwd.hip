@@ -97,35 +97,10 @@ __device__ __forceinline__ float softmax_slow_half(const f32x16& sacc, u32x4 (&p
   return alpha;
 }
 
-// How a tile's softmax is run.
-//   kChecked: fast pieces, each half verified afterwards (its denominator share must stay below kLsumLimit) and redone on
-//             the slow path if not -- needs no prior knowledge of the keys, costs two data-dependent branches per tile;
-//   kFast:    fast pieces, no verification -- only for tiles whose scores are known in advance not to exceed the reference
-//             maximum by more than kLazyMargin (in the base-2 domain).  Probabilities then stay below 2^kLazyMargin and
-//             the fp32 sums below 2^(kLazyMargin + log2 N + log2 max|v|), far from overflow; bf16 has fp32's exponent
-//             range, so P loses nothing either.
-enum TileMode { kChecked, kFast };
-constexpr float kLazyMargin = 64.f;
-
-// K staging: rotate on the way to LDS, or plain copy of an already rotated K.
-template <int D, int ROWS, int NT, bool PREROT>
-struct KStage : RotStage<D, ROWS, NT> {};
-template <int D, int ROWS, int NT>
-struct KStage<D, ROWS, NT, true> : CopyStage<D, ROWS, NT, 8> {
-  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float*, const float*, int64_t, int row0,
-                                       int n_rows) {
-    CopyStage<D, ROWS, NT, 8>::load(src, row0, n_rows);
-  }
-};
-
-// PREROT = false: K tiles are rotated inside the kernel, softmax in kChecked mode (a single launch, no workspace).
-// PREROT = true:  K was rotated by rope_rotate_kernel, which also left the largest key norm of every 64-key tile; with the
-//                 norm of the lane's own (rotated) query that bounds every score of the tile (Cauchy-Schwarz), so a tile
-//                 is classified before it is touched: when the bound is within kLazyMargin of the reference maximum the
-//                 tile runs in kFast mode as it is (no data-dependent branch inside the tile); otherwise its scores are
-//                 computed once just for their maximum, the reference moves there (accumulators rescaled), and the tile
-//                 then runs in kFast mode all the same.
-template <int D, int BLOCK_N, bool CAUSAL, bool PREROT>
+// This kernel knows nothing about the keys in advance, so every half runs the fast pieces and is verified afterwards
+// (two data-dependent branches per tile); the two-launch forward in rope_attn_fwd_pipe.hip gets the same guarantee
+// from key norms computed beforehand and has no such branch.
+template <int D, int BLOCK_N, bool CAUSAL>
 __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdParams p) {
   using Cfg = FwdCfg<D, BLOCK_N>;
   static_assert(BLOCK_N == 64, "the slot schedule is written for two 32-key halves");
@@ -147,13 +122,13 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
   const int N = p.N;
 
   const uint16_t* qg = p.q + (int64_t)bh * N * D;
-  const uint16_t* kg = (PREROT ? p.k_rot : p.k) + (int64_t)bh * N * D;
+  const uint16_t* kg = p.k + (int64_t)bh * N * D;
   const uint16_t* vg = p.v + (int64_t)bh * N * D;
 
   const int n_k_tiles = (N + BLOCK_N - 1) / BLOCK_N;
   const int n_tiles = CAUSAL ? min((m0 + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, n_k_tiles) : n_k_tiles;
 
-  KStage<D, BLOCK_N, NT, PREROT> kst;
+  RotStage<D, BLOCK_N, NT> kst;
   CopyStage<D, BLOCK_N, NT, Cfg::kVPad> vst;
   kst.load(kg, p.cos, p.sin, p.fstride, 0, N);
   vst.load(vg, 0, N);
@@ -164,22 +139,6 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
   load_b_rows<D, true>(qb, qg, p.cos, p.sin, p.fstride, min(q_row, N - 1));
 
   const float scale = p.qk_scale;
-  // PREROT: |q_r| * scale (a little generous), times a tile's largest key norm = upper bound of its scaled scores.
-  float q_bound = 0.f;
-  const float* tile_kmax = nullptr;
-  if constexpr (PREROT) {
-    float ss = 0.f;
-#pragma unroll
-    for (int kc = 0; kc < KC; ++kc)
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        float x0 = bf16_lo(qb[kc][w]), x1 = bf16_hi(qb[kc][w]);
-        ss += x0 * x0 + x1 * x1;
-      }
-    q_bound = __builtin_sqrtf(half_sum(ss)) * scale * 1.01f;
-    tile_kmax = p.tile_kmax + (int64_t)bh * n_k_tiles;
-  }
-
   f32x16 oacc[NDB];
 #pragma unroll
   for (int i = 0; i < NDB; ++i) oacc[i] = f32x16{0};
@@ -200,7 +159,6 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
   __syncthreads();
 
   const int wave_q_lo = m0 + wave * 32, wave_q_hi = wave_q_lo + 31;
-
   for (int t = 0; t < n_tiles; ++t) {
     const int n0 = t * BLOCK_N;
     const uint16_t* kt = ks(t) + RowTile<D>::off(lq, 8 * lh);
@@ -234,8 +192,7 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
     };
 
     // One tile in four slots of 8 MFMAs (see the schedule at the top of the file).
-    auto run_tile = [&](auto mode_c, const bool MASK) {
-      constexpr TileMode MODE = decltype(mode_c)::value;
+    auto run_tile = [&](const bool MASK) {
       f32x16 s0 = f32x16{0}, s1 = f32x16{0};
       u32x4 pb0[2], pb1[2];
       float lsum0 = 0.f, lsum1 = 0.f;
@@ -262,7 +219,7 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
         softmax_fast_piece(kc, KC, s0, pb0, lsum0, scale, ms_ref);
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (MODE == kChecked) {
+      {
         if (__builtin_amdgcn_ballot_w64(!(lsum0 <= kLsumLimit))) {
           rescale(softmax_slow_half(s0, pb0, m_run, l_run, scale));
         } else {
@@ -283,14 +240,13 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
         softmax_fast_piece(i, NPV, s1, pb1, lsum1, scale, ms_ref);
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (MODE == kChecked) {
+      {
         if (__builtin_amdgcn_ballot_w64(!(lsum1 <= kLsumLimit))) {
           rescale(softmax_slow_half(s1, pb1, m_run, l_run, scale));
         } else {
           l_run += lsum1;
         }
       }
-      if (MODE == kFast) l_run += lsum0 + lsum1;
       __builtin_amdgcn_sched_barrier(0);
       // ---- slot D: O^T += V^T P^T(half 1) ------------------------------------------------------------------------
 #pragma unroll
@@ -299,40 +255,11 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
         if (i + NDB < NPV) av[i % NDB] = v_operand(1, i + NDB);
       }
     };
-    // Moves the reference maximum of every row to the true maximum over this tile (and what came before).
-    auto raise_reference = [&](const bool MASK) {
-      f32x16 s0 = f32x16{0}, s1 = f32x16{0};
-#pragma unroll
-      for (int kc = 0; kc < KC; ++kc) {
-        s0 = mfma32(k_operand(0, kc), qb[kc], s0);
-        s1 = mfma32(k_operand(1, kc), qb[kc], s1);
-      }
-      if (MASK) {
-        mask_scores(s0, 0);
-        mask_scores(s1, 1);
-      }
-      float mt = fmaxf(s0[0], s1[0]);
-#pragma unroll
-      for (int i = 1; i < 16; ++i) mt = fmaxf(fmaxf(mt, s0[i]), s1[i]);
-      const float m_new = fmaxf(m_run, half_max(mt));
-      const float alpha = fast_exp2((m_run - m_new) * scale);   // m_new is finite: every row sees key 0 of tile 0
-      l_run *= alpha;
-      rescale(alpha);
-      m_run = m_new;
-    };
-
     // Tiles entirely above this wave's diagonal contribute nothing to it; the wave still stages its share.
     const bool active = !CAUSAL || n0 <= wave_q_hi;
     const bool need_mask = (CAUSAL && n0 + BLOCK_N - 1 > wave_q_lo) || (!CAUSAL && n0 + BLOCK_N > N);
     if (active) {
-      if constexpr (PREROT) {
-        // tile_kmax[t] is wave-uniform; a tile is fast only if no lane can exceed its reference by kLazyMargin
-        const float bound = q_bound * tile_kmax[t];
-        if (__builtin_amdgcn_ballot_w64(!(bound <= m_run * scale + kLazyMargin))) raise_reference(need_mask);
-        run_tile(std::integral_constant<TileMode, kFast>{}, need_mask);
-      } else {
-        run_tile(std::integral_constant<TileMode, kChecked>{}, need_mask);
-      }
+      run_tile(need_mask);
     } else {
       stage_next();
     }
@@ -358,10 +285,10 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
 }
 
 // ---- host-side launch -----------------------------------------------------------------------------------------
-template <int D, int BLOCK_N, bool CAUSAL, bool PREROT>
+template <int D, int BLOCK_N, bool CAUSAL>
 static hipError_t launch_fwd_cfg(FwdParams p, hipStream_t stream) {
   using Cfg = FwdCfg<D, BLOCK_N>;
-  auto kern = rope_attn_fwd_kernel<D, BLOCK_N, CAUSAL, PREROT>;
+  auto kern = rope_attn_fwd_kernel<D, BLOCK_N, CAUSAL>;
   static bool attr_set = false;  // per instantiation; benign if raced (same value)
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -375,15 +302,9 @@ static hipError_t launch_fwd_cfg(FwdParams p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int D>
-static hipError_t launch_fwd_d(const FwdParams& p, bool causal, hipStream_t stream) {
-  if (p.k_rot)
-    return causal ? launch_fwd_cfg<D, 64, true, true>(p, stream) : launch_fwd_cfg<D, 64, false, true>(p, stream);
-  return causal ? launch_fwd_cfg<D, 64, true, false>(p, stream) : launch_fwd_cfg<D, 64, false, false>(p, stream);
-}
-
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream) {
-  return D == 128 ? launch_fwd_d<128>(p, causal, stream) : launch_fwd_d<64>(p, causal, stream);
+  if (D == 128) return causal ? launch_fwd_cfg<128, 64, true>(p, stream) : launch_fwd_cfg<128, 64, false>(p, stream);
+  return causal ? launch_fwd_cfg<64, 64, true>(p, stream) : launch_fwd_cfg<64, 64, false>(p, stream);
 }
 
 }  // namespace corope
