@@ -256,16 +256,30 @@ def main():
         launches = [("rope_attn_fwd", lambda: lib.corope_rope_attn_fwd(qp, kp, vp, cp, sp, fs, o.data_ptr(), M.data_ptr(),
                                                                       B, H, N, D, scale, 1, stream))]
     if not fwd_only:
-        launches += [
-            ("rope_attn_bwd_preprocess", lambda: lib.corope_rope_attn_bwd_preprocess(o.data_ptr(), dop, delta.data_ptr(),
-                                                                                    B, H, N, D, stream)),
-            ("rope_attn_bwd_dv", lambda: lib.corope_rope_attn_bwd_dv(qp, kp, dop, M.data_ptr(), cp, sp, fs, dv.data_ptr(),
-                                                                    B, H, N, D, scale, 1, stream)),
-            ("rope_attn_bwd_dk", lambda: lib.corope_rope_attn_bwd_dk(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),
-                                                                    cp, sp, fs, dk.data_ptr(), B, H, N, D, scale, 1, stream)),
-            ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),
-                                                                    cp, sp, fs, dq.data_ptr(), B, H, N, D, scale, 1, stream)),
-        ]
+        launches += [("rope_attn_bwd_preprocess", lambda: lib.corope_rope_attn_bwd_preprocess(
+            o.data_ptr(), dop, delta.data_ptr(), B, H, N, D, stream))]
+        if N >= pkg.rope_attn.TWO_LAUNCH_MIN_N:   # the backward the operator takes at this length: rotate q and k first
+            q_rot = torch.empty_like(q)
+            qr, kr = q_rot.data_ptr(), k_rot.data_ptr()
+            launches += [
+                ("rope_rotate_q", lambda: lib.corope_rope_rotate(qp, cp, sp, fs, qr, None, B, H, N, D, stream)),
+                ("rope_rotate_k_bwd", lambda: lib.corope_rope_rotate(kp, cp, sp, fs, kr, None, B, H, N, D, stream)),
+                ("rope_attn_bwd_dv", lambda: lib.corope_rope_attn_bwd_dv_prerotated(
+                    qr, kr, dop, M.data_ptr(), cp, sp, fs, dv.data_ptr(), B, H, N, D, scale, 1, stream)),
+                ("rope_attn_bwd_dk", lambda: lib.corope_rope_attn_bwd_dk_prerotated(
+                    qr, kr, vp, dop, M.data_ptr(), delta.data_ptr(), cp, sp, fs, dk.data_ptr(), B, H, N, D, scale, 1, stream)),
+                ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq_prerotated(
+                    qr, kr, vp, dop, M.data_ptr(), delta.data_ptr(), cp, sp, fs, dq.data_ptr(), B, H, N, D, scale, 1, stream)),
+            ]
+        else:
+            launches += [
+                ("rope_attn_bwd_dv", lambda: lib.corope_rope_attn_bwd_dv(qp, kp, dop, M.data_ptr(), cp, sp, fs, dv.data_ptr(),
+                                                                        B, H, N, D, scale, 1, stream)),
+                ("rope_attn_bwd_dk", lambda: lib.corope_rope_attn_bwd_dk(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),
+                                                                        cp, sp, fs, dk.data_ptr(), B, H, N, D, scale, 1, stream)),
+                ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),
+                                                                        cp, sp, fs, dq.data_ptr(), B, H, N, D, scale, 1, stream)),
+            ]
     durs = {n: [] for n, _ in launches}
     for it in range(args.warmup + args.steps):
         evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(launches) + 1)]
@@ -315,8 +329,7 @@ def main():
         "kernels": kernels, "roofline": roofline,
     }
     if not fwd_only:
-        bwd_ms = (avg["rope_attn_bwd_preprocess"] + avg["rope_attn_bwd_dv"] + avg["rope_attn_bwd_dk"]
-                  + avg["rope_attn_bwd_dq"])
+        bwd_ms = sum(ms for n, ms in avg.items() if n not in ("rope_rotate_k", "rope_attn_fwd"))
         bwd_tf = f_bwd / (bwd_ms * 1e-3) * 1e-12
         out["bwd"] = {"ms": round(bwd_ms, 4), "tflops": round(bwd_tf, 1), "frac_of_peak": round(bwd_tf / PEAK_BF16_TFLOPS, 4)}
     out["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline()

@@ -203,29 +203,76 @@ int corope_rope_attn_bwd_preprocess(const void* o, const void* d_o, float* delta
   return launch_status("rope_attn_bwd_preprocess", corope::launch_bwd_preprocess(p, D, static_cast<hipStream_t>(stream)));
 }
 
-int corope_rope_attn_bwd_dv(const void* q, const void* k, const void* d_o, const float* lse, const float* freqs_cos,
-                            const float* freqs_sin, int64_t freq_row_stride, void* dv, int B, int H, int N, int D,
-                            float sm_scale, int causal, void* stream) {
+}  // extern "C" (reopened below)
+
+namespace {
+
+int64_t bwd_ws_tensor_bytes(int B, int H, int N, int D) { return (((int64_t)B * H * N * D * 2) + 255) / 256 * 256; }
+
+// prerot: q and k are copies that corope_rope_rotate rotated.
+void mark_prerotated(corope::BwdParams& p, bool prerot) {
+  if (prerot) {
+    p.q_rot = p.q;
+    p.k_rot = p.k;
+  }
+}
+
+int bwd_dv_impl(const char* what, bool prerot, const void* q, const void* k, const void* d_o, const float* lse,
+                const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* dv, int B, int H, int N,
+                int D, float sm_scale, int causal, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
-  rc = check_ptrs("rope_attn_bwd_dv", {q, k, d_o, lse, freqs_cos, freqs_sin, dv});
+  rc = check_ptrs(what, {q, k, d_o, lse, freqs_cos, freqs_sin, dv});
   if (rc) return rc;
   corope::BwdParams p = make_bwd(q, k, nullptr, nullptr, d_o, lse, nullptr, freqs_cos, freqs_sin, freq_row_stride,
                                  nullptr, nullptr, dv, B, H, N, sm_scale);
-  return launch_status("rope_attn_bwd_dv", corope::launch_bwd_dv(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+  mark_prerotated(p, prerot);
+  return launch_status(what, corope::launch_bwd_dv(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+}
+
+int bwd_dk_impl(const char* what, bool prerot, const void* q, const void* k, const void* v, const void* d_o,
+                const float* lse, const float* delta, const float* freqs_cos, const float* freqs_sin,
+                int64_t freq_row_stride, void* dk, int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
+  if (rc) return rc;
+  rc = check_ptrs(what, {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dk});
+  if (rc) return rc;
+  corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
+                                 freq_row_stride, nullptr, dk, nullptr, B, H, N, sm_scale);
+  mark_prerotated(p, prerot);
+  return launch_status(what, corope::launch_bwd_dk(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+}
+
+int bwd_dq_impl(const char* what, bool prerot, const void* q, const void* k, const void* v, const void* d_o,
+                const float* lse, const float* delta, const float* freqs_cos, const float* freqs_sin,
+                int64_t freq_row_stride, void* dq, int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
+  if (rc) return rc;
+  rc = check_ptrs(what, {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dq});
+  if (rc) return rc;
+  corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
+                                 freq_row_stride, dq, nullptr, nullptr, B, H, N, sm_scale);
+  mark_prerotated(p, prerot);
+  return launch_status(what, corope::launch_bwd_dq(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+}
+
+}  // namespace
+
+extern "C" {
+
+int corope_rope_attn_bwd_dv(const void* q, const void* k, const void* d_o, const float* lse, const float* freqs_cos,
+                            const float* freqs_sin, int64_t freq_row_stride, void* dv, int B, int H, int N, int D,
+                            float sm_scale, int causal, void* stream) {
+  return bwd_dv_impl("rope_attn_bwd_dv", false, q, k, d_o, lse, freqs_cos, freqs_sin, freq_row_stride, dv, B, H, N, D,
+                     sm_scale, causal, stream);
 }
 
 int corope_rope_attn_bwd_dk(const void* q, const void* k, const void* v, const void* d_o, const float* lse,
                             const float* delta, const float* freqs_cos, const float* freqs_sin,
                             int64_t freq_row_stride, void* dk, int B, int H, int N, int D, float sm_scale, int causal,
                             void* stream) {
-  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
-  if (rc) return rc;
-  rc = check_ptrs("rope_attn_bwd_dk", {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dk});
-  if (rc) return rc;
-  corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
-                                 freq_row_stride, nullptr, dk, nullptr, B, H, N, sm_scale);
-  return launch_status("rope_attn_bwd_dk", corope::launch_bwd_dk(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+  return bwd_dk_impl("rope_attn_bwd_dk", false, q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dk, B,
+                     H, N, D, sm_scale, causal, stream);
 }
 
 int corope_rope_attn_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* lse,
@@ -245,13 +292,31 @@ int corope_rope_attn_bwd_dq(const void* q, const void* k, const void* v, const v
                             const float* delta, const float* freqs_cos, const float* freqs_sin,
                             int64_t freq_row_stride, void* dq, int B, int H, int N, int D, float sm_scale, int causal,
                             void* stream) {
-  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
-  if (rc) return rc;
-  rc = check_ptrs("rope_attn_bwd_dq", {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dq});
-  if (rc) return rc;
-  corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
-                                 freq_row_stride, dq, nullptr, nullptr, B, H, N, sm_scale);
-  return launch_status("rope_attn_bwd_dq", corope::launch_bwd_dq(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+  return bwd_dq_impl("rope_attn_bwd_dq", false, q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, B,
+                     H, N, D, sm_scale, causal, stream);
+}
+
+int corope_rope_attn_bwd_dv_prerotated(const void* q_rot, const void* k_rot, const void* d_o, const float* lse,
+                                       const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* dv,
+                                       int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
+  return bwd_dv_impl("rope_attn_bwd_dv_prerotated", true, q_rot, k_rot, d_o, lse, freqs_cos, freqs_sin, freq_row_stride,
+                     dv, B, H, N, D, sm_scale, causal, stream);
+}
+
+int corope_rope_attn_bwd_dk_prerotated(const void* q_rot, const void* k_rot, const void* v, const void* d_o,
+                                       const float* lse, const float* delta, const float* freqs_cos,
+                                       const float* freqs_sin, int64_t freq_row_stride, void* dk, int B, int H, int N,
+                                       int D, float sm_scale, int causal, void* stream) {
+  return bwd_dk_impl("rope_attn_bwd_dk_prerotated", true, q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin,
+                     freq_row_stride, dk, B, H, N, D, sm_scale, causal, stream);
+}
+
+int corope_rope_attn_bwd_dq_prerotated(const void* q_rot, const void* k_rot, const void* v, const void* d_o,
+                                       const float* lse, const float* delta, const float* freqs_cos,
+                                       const float* freqs_sin, int64_t freq_row_stride, void* dq, int B, int H, int N,
+                                       int D, float sm_scale, int causal, void* stream) {
+  return bwd_dq_impl("rope_attn_bwd_dq_prerotated", true, q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin,
+                     freq_row_stride, dq, B, H, N, D, sm_scale, causal, stream);
 }
 
 int corope_rope_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
@@ -265,6 +330,40 @@ int corope_rope_attn_bwd(const void* q, const void* k, const void* v, const void
   if (rc) return rc;
   return corope_rope_attn_bwd_dq(q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, B, H, N, D,
                                  sm_scale, causal, stream);
+}
+
+int64_t corope_rope_attn_bwd_workspace_bytes(int B, int H, int N, int D) {
+  if (corope_rope_attn_check(B, H, N, D, D, 1.f, 1)) return -1;
+  return 2 * bwd_ws_tensor_bytes(B, H, N, D);
+}
+
+int corope_rope_attn_bwd_ws(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                            const float* lse, float* delta, const float* freqs_cos, const float* freqs_sin,
+                            int64_t freq_row_stride, void* dq, void* dk, void* dv, int B, int H, int N, int D,
+                            float sm_scale, int causal, void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
+  if (rc) return rc;
+  rc = check_ptrs("rope_attn_bwd_ws", {workspace});
+  if (rc) return rc;
+  if (workspace_bytes < 2 * bwd_ws_tensor_bytes(B, H, N, D))
+    return fail(COROPE_E_BADARG, "rope_attn_bwd_ws: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
+                (long long)(2 * bwd_ws_tensor_bytes(B, H, N, D)));
+  void* q_rot = workspace;
+  void* k_rot = static_cast<char*>(workspace) + bwd_ws_tensor_bytes(B, H, N, D);
+  rc = corope_rope_rotate(q, freqs_cos, freqs_sin, freq_row_stride, q_rot, nullptr, B, H, N, D, stream);
+  if (rc) return rc;
+  rc = corope_rope_rotate(k, freqs_cos, freqs_sin, freq_row_stride, k_rot, nullptr, B, H, N, D, stream);
+  if (rc) return rc;
+  rc = corope_rope_attn_bwd_preprocess(o, d_o, delta, B, H, N, D, stream);
+  if (rc) return rc;
+  rc = corope_rope_attn_bwd_dv_prerotated(q_rot, k_rot, d_o, lse, freqs_cos, freqs_sin, freq_row_stride, dv, B, H, N, D,
+                                          sm_scale, causal, stream);
+  if (rc) return rc;
+  rc = corope_rope_attn_bwd_dk_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dk, B,
+                                          H, N, D, sm_scale, causal, stream);
+  if (rc) return rc;
+  return corope_rope_attn_bwd_dq_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq,
+                                            B, H, N, D, sm_scale, causal, stream);
 }
 
 int corope_rope_freqs(float* freqs_cos, float* freqs_sin, int n_pos, int D, int width, int64_t freq_row_stride, int pos0,

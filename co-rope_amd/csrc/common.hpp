@@ -310,6 +310,18 @@ struct CopyStage {
   }
 };
 
+// Staging of a tile whose rows take part in QK^T: rotated on the way to LDS (PREROT = false), or copied from a tensor
+// that rope_rotate_kernel rotated beforehand (PREROT = true; the tables are then not touched).
+template <int D, int ROWS, int NT, bool PREROT>
+struct RopeStage : RotStage<D, ROWS, NT> {};
+template <int D, int ROWS, int NT>
+struct RopeStage<D, ROWS, NT, true> : CopyStage<D, ROWS, NT, 8> {
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float*, const float*, int64_t, int row0,
+                                       int n_rows) {
+    CopyStage<D, ROWS, NT, 8>::load(src, row0, n_rows);
+  }
+};
+
 // ---- transposing LDS read (ds_read_b64_tr_b16) ------------------------------------------------------------
 // The instruction works on blocks of 16 lanes: source lane s supplies 8 bytes E[s][0..3]; result lane L
 // receives { E[4j + L/4][L % 4] : j = 0..3 }.

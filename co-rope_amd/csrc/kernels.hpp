@@ -29,6 +29,8 @@ struct BwdParams {
   const uint16_t* v;
   const uint16_t* o;
   const uint16_t* d_o;
+  const uint16_t* q_rot;  // Q and K already rotated (same layout as q, k), or both null: rotate tiles inside the kernels
+  const uint16_t* k_rot;
   const float* cos;
   const float* sin;
   const float* lse;

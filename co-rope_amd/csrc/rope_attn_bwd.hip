@@ -26,22 +26,27 @@ namespace corope {
 //   P  = exp2(S*c - M), dS = P o (dP - delta)                               (bf16, already B-operand shaped)
 //   dV^T   += dO^T  P         (A = dO tile read transposed, B = P)
 //   dK_r^T += Q_r^T dS        (A = Q_r tile read transposed, B = dS)
-template <int D, int NWAVES, int BLOCK_M>
+// DO_PAD: row padding of the dO tile.  The dV-only kernel reads dO through the transposing load alone and takes the
+// padding that is conflict-free for it (32); the dK kernel reads dO row-wise (8).
+template <int D, int NWAVES, int BLOCK_M, int DO_PAD>
 struct DkdvCfg {
   static constexpr int kThreads = NWAVES * kWave;
   static constexpr int kBlockN = NWAVES * 32;
   static constexpr int kTileBytes = RowTile<D>::bytes(BLOCK_M);
+  static constexpr int kDoTileBytes = RowTile<D, DO_PAD>::bytes(BLOCK_M);
   static constexpr int kStatBytes = BLOCK_M * 4;
-  static constexpr int kStageBytes = 2 * kTileBytes + 2 * kStatBytes;
+  static constexpr int kStageBytes = kTileBytes + kDoTileBytes + 2 * kStatBytes;
   static constexpr int kLdsBytes = 2 * kStageBytes;
 };
 
-template <int D, int NWAVES, int BLOCK_M, bool CAUSAL, bool DO_DV, bool DO_DK>
+// PREROT: Q and K come from copies that rope_rotate_kernel rotated beforehand (no table reads in the loop).
+template <int D, int NWAVES, int BLOCK_M, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
 __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
-  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M>;
+  constexpr int DO_PAD = DO_DK ? 8 : 32;
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_PAD>;
   constexpr int NT = Cfg::kThreads;
   constexpr int KC = D / 16, NDB = D / 32, NQB = BLOCK_M / 32;
-  constexpr int LS = RowTile<D>::kStride;
+  constexpr int LS = RowTile<D>::kStride, LSDO = RowTile<D, DO_PAD>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
   const int bh = blockIdx.x % p.BH;
@@ -51,7 +56,7 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
   const int lq = lane % 32, lh = lane / 32;
   const int N = p.N;
   const int64_t base = (int64_t)bh * N * D;
-  const uint16_t* qg = p.q + base;
+  const uint16_t* qg = (PREROT ? p.q_rot : p.q) + base;
   const uint16_t* dog = p.d_o + base;
   const float* lseg = p.lse + (int64_t)bh * N;
   const float* deltag = p.delta + (int64_t)bh * N;
@@ -61,14 +66,14 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
   const int wk_lo = n0 + wave * 32, wk_hi = wk_lo + 31;
 
   u32x4 kb[KC], vb[DO_DK ? KC : 1];
-  load_b_rows<D, true>(kb, p.k + base, p.cos, p.sin, p.fstride, key_c);
+  load_b_rows<D, !PREROT>(kb, (PREROT ? p.k_rot : p.k) + base, p.cos, p.sin, p.fstride, key_c);
   if constexpr (DO_DK) load_b_rows<D, false>(vb, p.v + base, nullptr, nullptr, 0, key_c);
 
   const int m_tiles = (N + BLOCK_M - 1) / BLOCK_M;
   const int mt0 = CAUSAL ? n0 / BLOCK_M : 0;
 
-  RotStage<D, BLOCK_M, NT> qst;
-  CopyStage<D, BLOCK_M, NT> dst;
+  RopeStage<D, BLOCK_M, NT, PREROT> qst;
+  CopyStage<D, BLOCK_M, NT, DO_PAD> dst;
   float st_lse = 0.f, st_delta = 0.f;
   auto load_tile = [&](int m0) {
     qst.load(qg, p.cos, p.sin, p.fstride, m0, N);
@@ -82,9 +87,11 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
   };
   auto q_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
   auto do_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes + Cfg::kTileBytes); };
-  auto lse_tile = [&](int buf) { return reinterpret_cast<float*>(smem + buf * Cfg::kStageBytes + 2 * Cfg::kTileBytes); };
+  auto lse_tile = [&](int buf) {
+    return reinterpret_cast<float*>(smem + buf * Cfg::kStageBytes + Cfg::kTileBytes + Cfg::kDoTileBytes);
+  };
   auto delta_tile = [&](int buf) {
-    return reinterpret_cast<float*>(smem + buf * Cfg::kStageBytes + 2 * Cfg::kTileBytes + Cfg::kStatBytes);
+    return reinterpret_cast<float*>(smem + buf * Cfg::kStageBytes + Cfg::kTileBytes + Cfg::kDoTileBytes + Cfg::kStatBytes);
   };
   auto store_tile = [&](int buf) {
     qst.store_rows(q_tile(buf));
@@ -125,7 +132,7 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
       if (CAUSAL && mq0 + 31 < wk_lo) continue;
       f32x16 sacc = f32x16{0}, dpacc = f32x16{0};
       const uint16_t* qrow = qs + RowTile<D>::off(qb * 32 + lq, 8 * lh);
-      const uint16_t* dorow = dos + RowTile<D>::off(qb * 32 + lq, 8 * lh);
+      const uint16_t* dorow = dos + RowTile<D, DO_PAD>::off(qb * 32 + lq, 8 * lh);
 #pragma unroll
       for (int kc = 0; kc < KC; ++kc)
         sacc = mfma32(*reinterpret_cast<const u32x4*>(qrow + 16 * kc), kb[kc], sacc);
@@ -135,7 +142,16 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
           dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc), vb[kc], dpacc);
       }
 
-      const bool need_mask = CAUSAL && mq0 < wk_hi;
+      // Causal mask on the raw scores, under a wave-uniform branch of its own (written into the exponential loop it
+      // is turned into compare + select on every tile).  Register i holds query mq0 + 8*(i/4) + 4*lh + i%4; the
+      // lane-dependent part of the threshold goes into one opaque value so that the 16 thresholds stay immediates.
+      if (CAUSAL && mq0 < wk_hi) {
+        int rel = key - mq0 - 4 * lh;
+        asm volatile("" : "+v"(rel));
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (8 * (i / 4) + i % 4 < rel) sacc[i] = -INFINITY;
+      }
       u32x4 pb[2], dsb[2];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -146,7 +162,6 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           pv[e] = fast_exp2(sacc[4 * g + e] * scale2 - m4[e]);
-          if (need_mask && (mq0 + 8 * g + 4 * lh + e) < key) pv[e] = 0.f;
           ds[e] = pv[e] * (dpacc[4 * g + e] - d4[e]);
         }
         if constexpr (DO_DV) {
@@ -163,7 +178,7 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
         const int kbase = qb * 32 + 16 * cc;
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-          if constexpr (DO_DV) dvacc[db] = mfma32(load_a_trans(dos, LS, kbase, db * 32), pb[cc], dvacc[db]);
+          if constexpr (DO_DV) dvacc[db] = mfma32(load_a_trans(dos, LSDO, kbase, db * 32), pb[cc], dvacc[db]);
           if constexpr (DO_DK) dkacc[db] = mfma32(load_a_trans(qs, LS, kbase, db * 32), dsb[cc], dkacc[db]);
         }
       }
@@ -206,7 +221,7 @@ struct DqCfg {
   static constexpr int kLdsBytes = 2 * kStageBytes;
 };
 
-template <int D, int NWAVES, int BLOCK_N, bool CAUSAL>
+template <int D, int NWAVES, int BLOCK_N, bool CAUSAL, bool PREROT>
 __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdParams p) {
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
   constexpr int NT = Cfg::kThreads;
@@ -221,22 +236,23 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdPara
   const int lq = lane % 32, lh = lane / 32;
   const int N = p.N;
   const int64_t base = (int64_t)bh * N * D;
-  const uint16_t* kg = p.k + base;
+  const uint16_t* kg = (PREROT ? p.k_rot : p.k) + base;
   const uint16_t* vg = p.v + base;
 
   const int q_row = m0 + wave * 32 + lq;
   const int q_c = min(q_row, N - 1);
   const int wq_lo = m0 + wave * 32, wq_hi = wq_lo + 31;
+  const int key_limit = CAUSAL ? q_row : N - 1;   // last key this lane's query attends to
 
   const int n_tiles = CAUSAL ? min((m0 + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, (N + BLOCK_N - 1) / BLOCK_N)
                              : (N + BLOCK_N - 1) / BLOCK_N;
-  RotStage<D, BLOCK_N, NT> kst;
+  RopeStage<D, BLOCK_N, NT, PREROT> kst;
   CopyStage<D, BLOCK_N, NT> vst;
   kst.load(kg, p.cos, p.sin, p.fstride, 0, N);
   vst.load(vg, 0, N);
 
   u32x4 qb[KC], dob[KC];
-  load_b_rows<D, true>(qb, p.q + base, p.cos, p.sin, p.fstride, q_c);
+  load_b_rows<D, !PREROT>(qb, (PREROT ? p.q_rot : p.q) + base, p.cos, p.sin, p.fstride, q_c);
   load_b_rows<D, false>(dob, p.d_o + base, nullptr, nullptr, 0, q_c);
   const float lse_q = p.lse[(int64_t)bh * N + q_c];
   const float delta_q = p.delta[(int64_t)bh * N + q_c];
@@ -277,16 +293,21 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdPara
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
           dpacc = mfma32(*reinterpret_cast<const u32x4*>(vrow + 16 * kc), dob[kc], dpacc);
+        // mask on the raw scores under a wave-uniform branch of its own; register i holds key
+        // n0 + 32*kb + 8*(i/4) + 4*lh + i%4, the lane-dependent part of the threshold goes into one opaque value
+        if (need_mask) {
+          int rel = key_limit - n0 - 4 * lh;
+          asm volatile("" : "+v"(rel));
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            if (kb * 32 + 8 * (i / 4) + i % 4 > rel) sacc[i] = -INFINITY;
+        }
 #pragma unroll
         for (int i = 0; i < 16; i += 2) {
           float ds[2];
 #pragma unroll
           for (int e = 0; e < 2; ++e) {
             float pv = fast_exp2(sacc[i + e] * scale2 - lse_q);
-            if (need_mask) {
-              int kk = n0 + kb * 32 + acc_row(i + e, lh);
-              if (CAUSAL ? kk > q_row : kk >= N) pv = 0.f;
-            }
             ds[e] = pv * (dpacc[i + e] - delta_q);
           }
           dsb[2 * kb + i / 8][(i % 8) / 2] = pack_bf16(ds[0], ds[1]);
@@ -318,11 +339,11 @@ static hipError_t set_lds(K kern, int bytes) {
 
 // dK and dV are produced by two launches of the same kernel template: with both sets of accumulators resident a
 // wave needs more than 256 registers, which would halve the waves per SIMD.
-template <int D, bool CAUSAL, bool DO_DV, bool DO_DK>
+template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
 static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
   constexpr int NWAVES = 8, BLOCK_M = 64;
-  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M>;
-  auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK>;
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? 8 : 32>;
+  auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK, PREROT>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = set_lds(kern, Cfg::kLdsBytes);
@@ -334,11 +355,11 @@ static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int D, bool CAUSAL>
+template <int D, bool CAUSAL, bool PREROT>
 static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
   constexpr int NWAVES = 8, BLOCK_N = 64;
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
-  auto kern = rope_attn_bwd_dq_kernel<D, NWAVES, BLOCK_N, CAUSAL>;
+  auto kern = rope_attn_bwd_dq_kernel<D, NWAVES, BLOCK_N, CAUSAL, PREROT>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = set_lds(kern, Cfg::kLdsBytes);
@@ -350,21 +371,36 @@ static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// Dispatch on the run-time switches (head dim, causal, pre-rotated operands present).
+template <bool DO_DV, bool DO_DK>
+static hipError_t launch_dkdv(const BwdParams& p, int D, bool causal, hipStream_t stream) {
+  const bool pre = p.q_rot != nullptr && p.k_rot != nullptr;
+#define COROPE_DKDV(DD, CC, PP) launch_dkdv_cfg<DD, CC, DO_DV, DO_DK, PP>(p, stream)
+  if (D == 128) {
+    if (pre) return causal ? COROPE_DKDV(128, true, true) : COROPE_DKDV(128, false, true);
+    return causal ? COROPE_DKDV(128, true, false) : COROPE_DKDV(128, false, false);
+  }
+  if (pre) return causal ? COROPE_DKDV(64, true, true) : COROPE_DKDV(64, false, true);
+  return causal ? COROPE_DKDV(64, true, false) : COROPE_DKDV(64, false, false);
+#undef COROPE_DKDV
+}
+
 hipError_t launch_bwd_dv(const BwdParams& p, int D, bool causal, hipStream_t stream) {
-  if (D == 128)
-    return causal ? launch_dkdv_cfg<128, true, true, false>(p, stream) : launch_dkdv_cfg<128, false, true, false>(p, stream);
-  return causal ? launch_dkdv_cfg<64, true, true, false>(p, stream) : launch_dkdv_cfg<64, false, true, false>(p, stream);
+  return launch_dkdv<true, false>(p, D, causal, stream);
 }
 
 hipError_t launch_bwd_dk(const BwdParams& p, int D, bool causal, hipStream_t stream) {
-  if (D == 128)
-    return causal ? launch_dkdv_cfg<128, true, false, true>(p, stream) : launch_dkdv_cfg<128, false, false, true>(p, stream);
-  return causal ? launch_dkdv_cfg<64, true, false, true>(p, stream) : launch_dkdv_cfg<64, false, false, true>(p, stream);
+  return launch_dkdv<false, true>(p, D, causal, stream);
 }
 
 hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream) {
-  if (D == 128) return causal ? launch_dq_cfg<128, true>(p, stream) : launch_dq_cfg<128, false>(p, stream);
-  return causal ? launch_dq_cfg<64, true>(p, stream) : launch_dq_cfg<64, false>(p, stream);
+  const bool pre = p.q_rot != nullptr && p.k_rot != nullptr;
+  if (D == 128) {
+    if (pre) return causal ? launch_dq_cfg<128, true, true>(p, stream) : launch_dq_cfg<128, false, true>(p, stream);
+    return causal ? launch_dq_cfg<128, true, false>(p, stream) : launch_dq_cfg<128, false, false>(p, stream);
+  }
+  if (pre) return causal ? launch_dq_cfg<64, true, true>(p, stream) : launch_dq_cfg<64, false, true>(p, stream);
+  return causal ? launch_dq_cfg<64, true, false>(p, stream) : launch_dq_cfg<64, false, false>(p, stream);
 }
 
 }  // namespace corope

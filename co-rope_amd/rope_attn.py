@@ -107,10 +107,18 @@ class _FusedRopeAttn(torch.autograd.Function):
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         delta = torch.empty_like(M)
         with torch.cuda.device(q.device):
-            rc = lib.corope_rope_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
-                                          M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0),
-                                          dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, N, D, ctx.sm_scale,
-                                          int(ctx.causal), _stream_ptr(q))
+            if N >= TWO_LAUNCH_MIN_N:   # rotate q and k once, then run the kernels on the rotated copies
+                nbytes = lib.corope_rope_attn_bwd_workspace_bytes(B, H, N, D)
+                ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+                rc = lib.corope_rope_attn_bwd_ws(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
+                                                 M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(),
+                                                 fc.stride(0), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, N, D,
+                                                 ctx.sm_scale, int(ctx.causal), ws.data_ptr(), nbytes, _stream_ptr(q))
+            else:
+                rc = lib.corope_rope_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
+                                              M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0),
+                                              dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, N, D, ctx.sm_scale,
+                                              int(ctx.causal), _stream_ptr(q))
         _lib.check(rc, "corope_rope_attn_bwd")
         return dq, dk, dv, None, None, None, None, None
 

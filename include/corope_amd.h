@@ -135,6 +135,38 @@ int corope_rope_attn_bwd(const void *q, const void *k, const void *v, const void
                          void *dq, void *dk, void *dv,
                          int B, int H, int N, int D, float sm_scale, int causal, void *stream);
 
+/* Backward on pre-rotated operands: q_rot and k_rot are copies of q and k that corope_rope_rotate rotated; the
+ * kernels then read no cos/sin tables in their inner loops (the tables are still needed once per output row, to
+ * rotate dK and dQ back).  Same results as the plain entry points (the rotated copies are rounded to bf16 exactly
+ * as the kernels round them when they rotate a tile themselves).  Reference sites as for corope_rope_attn_bwd_dv,
+ * _dk and _dq. */
+int corope_rope_attn_bwd_dv_prerotated(const void *q_rot, const void *k_rot, const void *d_o, const float *lse,
+                                       const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                                       void *dv,
+                                       int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+int corope_rope_attn_bwd_dk_prerotated(const void *q_rot, const void *k_rot, const void *v, const void *d_o,
+                                       const float *lse, const float *delta,
+                                       const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                                       void *dk,
+                                       int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+int corope_rope_attn_bwd_dq_prerotated(const void *q_rot, const void *k_rot, const void *v, const void *d_o,
+                                       const float *lse, const float *delta,
+                                       const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                                       void *dq,
+                                       int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
+/* Whole backward for long sequences: rotates q and k once into `workspace`, then preprocess, dV, dK, dQ on the
+ * rotated copies.  Replaces _attention.backward like corope_rope_attn_bwd (reference
+ * fused-rope/fused_rope_attn.py:720-777).  workspace: device memory, 16-byte aligned, at least
+ * corope_rope_attn_bwd_workspace_bytes(B,H,N,D) bytes, scratch. */
+int64_t corope_rope_attn_bwd_workspace_bytes(int B, int H, int N, int D); /* -1 for unsupported sizes */
+int corope_rope_attn_bwd_ws(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                            const float *lse, float *delta,
+                            const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                            void *dq, void *dk, void *dv,
+                            int B, int H, int N, int D, float sm_scale, int causal,
+                            void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Co-RoPE grouped-query attention forward (causal only).
  * q: (B,Hq,N,D), k/v: (B,Hkv,N,D), o: (B,Hq,N,D), group size Hq/Hkv in [1, 8].
  * Replaces the launch of _corope_fwd_backbone in _attention.forward

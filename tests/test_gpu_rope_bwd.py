@@ -33,10 +33,14 @@ SHAPES = [(4, 8, 1024, 64), (1, 8, 1024, 128), (2, 4, 512, 64), (2, 2, 256, 128)
           (1, 2, 257, 128), (1, 1, 1, 64), (1, 1, 130, 64)]
 
 
+# two_launch: False = every kernel rotates its own tiles, True = q and k are rotated once into a workspace first
+# (the operator picks by sequence length; the threshold is moved here so that every shape takes both paths)
+@pytest.mark.parametrize("two_launch", [False, True])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,N,D", SHAPES)
-def test_backward_parity(pkg, B, H, N, D, causal):
-    print(f"case B={B} H={H} N={N} D={D} causal={causal}", flush=True)
+def test_backward_parity(pkg, monkeypatch, B, H, N, D, causal, two_launch):
+    print(f"case B={B} H={H} N={N} D={D} causal={causal} two_launch={two_launch}", flush=True)
+    monkeypatch.setattr(pkg.rope_attn, "TWO_LAUNCH_MIN_N", 1 if two_launch else 1 << 30)
     q, k, v, g, c, s = _case(B, H, N, D)
     scale = 1 / math.sqrt(D)
     o, dq, dk, dv = _gpu_fwd_bwd(pkg, q, k, v, g, causal, scale, c, s)
@@ -83,3 +87,22 @@ def test_backward_deterministic(pkg):
     a = _gpu_fwd_bwd(pkg, q, k, v, g, True, 0.09, c, s)
     b = _gpu_fwd_bwd(pkg, q, k, v, g, True, 0.09, c, s)
     assert all(torch.equal(x, y) for x, y in zip(a, b))
+
+
+def test_backward_paths_agree(pkg, monkeypatch):
+    """The rotated copies are rounded exactly as the kernels round the tiles they rotate themselves, and the backward
+    kernels do the same arithmetic on them: gradients of the two paths are identical bit for bit (given one O, M)."""
+    B, H, N, D = 1, 2, 320, 128
+    q, k, v, g, c, s = _case(B, H, N, D, seed=3)
+    dev = torch.device("cuda:0")
+    grads = []
+    for two_launch in (False, True):
+        monkeypatch.setattr(pkg.rope_attn, "TWO_LAUNCH_MIN_N", 1 << 30)     # same forward for both
+        qd, kd, vd = (t.to(dev, torch.bfloat16).requires_grad_(True) for t in (q, k, v))
+        o = pkg.attention(qd, kd, vd, True, 0.09, c.to(dev), s.to(dev))
+        monkeypatch.setattr(pkg.rope_attn, "TWO_LAUNCH_MIN_N", 1 if two_launch else 1 << 30)
+        o.backward(g.to(dev, torch.bfloat16))
+        torch.cuda.synchronize()
+        grads.append([t.grad.float().cpu() for t in (qd, kd, vd)])
+    for a, b, name in zip(grads[0], grads[1], ("dQ", "dK", "dV")):
+        assert torch.equal(a, b), name
