@@ -130,16 +130,16 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
       const int mq0 = m0 + qb * 32;
       // queries of this 32-row block that lie above every key of the wave see none of them
       if (CAUSAL && mq0 + 31 < wk_lo) continue;
-      f32x16 sacc = f32x16{0}, dpacc = f32x16{0};
+      f32x16 sacc, dpacc = f32x16{0};   // the first MFMA of each product takes a literal zero as its accumulator
       const uint16_t* qrow = qs + RowTile<D>::off(qb * 32 + lq, 8 * lh);
       const uint16_t* dorow = dos + RowTile<D, DO_PAD>::off(qb * 32 + lq, 8 * lh);
 #pragma unroll
       for (int kc = 0; kc < KC; ++kc)
-        sacc = mfma32(*reinterpret_cast<const u32x4*>(qrow + 16 * kc), kb[kc], sacc);
+        sacc = mfma32(*reinterpret_cast<const u32x4*>(qrow + 16 * kc), kb[kc], kc == 0 ? f32x16{0} : sacc);
       if constexpr (DO_DK) {
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
-          dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc), vb[kc], dpacc);
+          dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc), vb[kc], kc == 0 ? f32x16{0} : dpacc);
       }
 
       // Causal mask on the raw scores, under a wave-uniform branch of its own (written into the exponential loop it
@@ -284,15 +284,15 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdPara
       u32x4 dsb[BLOCK_N / 16];
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb) {
-        f32x16 sacc = f32x16{0}, dpacc = f32x16{0};
+        f32x16 sacc, dpacc;   // the first MFMA of each product takes a literal zero as its accumulator
         const uint16_t* krow = ks + RowTile<D>::off(kb * 32 + lq, 8 * lh);
         const uint16_t* vrow = vs + RowTile<D>::off(kb * 32 + lq, 8 * lh);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
-          sacc = mfma32(*reinterpret_cast<const u32x4*>(krow + 16 * kc), qb[kc], sacc);
+          sacc = mfma32(*reinterpret_cast<const u32x4*>(krow + 16 * kc), qb[kc], kc == 0 ? f32x16{0} : sacc);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
-          dpacc = mfma32(*reinterpret_cast<const u32x4*>(vrow + 16 * kc), dob[kc], dpacc);
+          dpacc = mfma32(*reinterpret_cast<const u32x4*>(vrow + 16 * kc), dob[kc], kc == 0 ? f32x16{0} : dpacc);
         // mask on the raw scores under a wave-uniform branch of its own; register i holds key
         // n0 + 32*kb + 8*(i/4) + 4*lh + i%4, the lane-dependent part of the threshold goes into one opaque value
         if (need_mask) {
