@@ -245,25 +245,22 @@ def main():
     qp, kp, vp, dop = q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr()
     cp, sp, fs = cos.data_ptr(), sin.data_ptr(), cos.stride(0)
     if N >= pkg.rope_attn.TWO_LAUNCH_MIN_N:   # the forward the operator takes at this length: rotate K, then attention
-        k_rot = torch.empty_like(k)
+        k_rot, q_rot = torch.empty_like(k), torch.empty_like(q)
         kmax = torch.empty(B, H, (N + 63) // 64, device=dev, dtype=torch.float32)
         launches = [("rope_rotate_k", lambda: lib.corope_rope_rotate(kp, cp, sp, fs, k_rot.data_ptr(), kmax.data_ptr(),
                                                                      B, H, N, D, stream)),
                     ("rope_attn_fwd", lambda: lib.corope_rope_attn_fwd_prerotated(
-                        qp, k_rot.data_ptr(), kmax.data_ptr(), vp, cp, sp, fs, o.data_ptr(), M.data_ptr(), B, H, N, D,
-                        scale, 1, stream))]
+                        qp, k_rot.data_ptr(), kmax.data_ptr(), vp, cp, sp, fs, o.data_ptr(), M.data_ptr(),
+                        None if fwd_only else q_rot.data_ptr(), B, H, N, D, scale, 1, stream))]
     else:
         launches = [("rope_attn_fwd", lambda: lib.corope_rope_attn_fwd(qp, kp, vp, cp, sp, fs, o.data_ptr(), M.data_ptr(),
                                                                       B, H, N, D, scale, 1, stream))]
     if not fwd_only:
         launches += [("rope_attn_bwd_preprocess", lambda: lib.corope_rope_attn_bwd_preprocess(
             o.data_ptr(), dop, delta.data_ptr(), B, H, N, D, stream))]
-        if N >= pkg.rope_attn.TWO_LAUNCH_MIN_N:   # the backward the operator takes at this length: rotate q and k first
-            q_rot = torch.empty_like(q)
-            qr, kr = q_rot.data_ptr(), k_rot.data_ptr()
+        if N >= pkg.rope_attn.TWO_LAUNCH_MIN_N:   # the backward the operator takes at this length: on the rotated q, k
+            qr, kr = q_rot.data_ptr(), k_rot.data_ptr()   # which the forward kept
             launches += [
-                ("rope_rotate_q", lambda: lib.corope_rope_rotate(qp, cp, sp, fs, qr, None, B, H, N, D, stream)),
-                ("rope_rotate_k_bwd", lambda: lib.corope_rope_rotate(kp, cp, sp, fs, kr, None, B, H, N, D, stream)),
                 ("rope_attn_bwd_dv", lambda: lib.corope_rope_attn_bwd_dv_prerotated(
                     qr, kr, dop, M.data_ptr(), cp, sp, fs, dv.data_ptr(), B, H, N, D, scale, 1, stream)),
                 ("rope_attn_bwd_dk", lambda: lib.corope_rope_attn_bwd_dk_prerotated(

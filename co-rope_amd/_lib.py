@@ -27,7 +27,8 @@ SIGNATURES = {
     "corope_rope_attn_fwd": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_fwd_workspace_bytes": (_L, [_I, _I, _I, _I]),
     "corope_rope_attn_fwd_ws": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P, _L, _P]),
-    "corope_rope_attn_fwd_prerotated": (_I, [_P, _P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
+    "corope_rope_attn_fwd_prerotated": (_I, [_P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
+    "corope_rope_attn_fwd_train": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_rotate": (_I, [_P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _P]),
     "corope_rope_attn_bwd_preprocess": (_I, [_P, _P, _P, _I, _I, _I, _I, _P]),
     "corope_rope_attn_bwd_dv": (_I, [_P] * 6 + [_L, _P, _I, _I, _I, _I, _F, _I, _P]),
@@ -38,6 +39,7 @@ SIGNATURES = {
     "corope_rope_attn_bwd_dv_prerotated": (_I, [_P] * 6 + [_L, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_bwd_dk_prerotated": (_I, [_P] * 8 + [_L, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_bwd_dq_prerotated": (_I, [_P] * 8 + [_L, _P, _I, _I, _I, _I, _F, _I, _P]),
+    "corope_rope_attn_bwd_prerotated": (_I, [_P] * 9 + [_L, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_bwd_workspace_bytes": (_L, [_I, _I, _I, _I]),
     "corope_rope_attn_bwd_ws": (_I, [_P] * 9 + [_L, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P, _L, _P]),
     "corope_gqa_fwd": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P]),

@@ -76,6 +76,9 @@ int corope_rope_attn_check(int B, int H, int N, int D, int64_t freq_row_stride, 
     return fail(COROPE_E_BADARG, "rope_attn: freq_row_stride %lld must be >= D/2 and a multiple of 4", (long long)freq_row_stride);
   if (!(sm_scale > 0.f) || !std::isfinite(sm_scale)) return fail(COROPE_E_BADARG, "rope_attn: sm_scale must be positive and finite");
   if ((int64_t)B * H * N * D >= ((int64_t)1 << 40)) return fail(COROPE_E_UNSUPPORTED, "rope_attn: tensor too large");
+  // staging loads address a (batch, head) slab and the tables with 32-bit byte offsets
+  if ((int64_t)N * D * 2 >= ((int64_t)1 << 32) || (int64_t)N * freq_row_stride * 4 >= ((int64_t)1 << 32))
+    return fail(COROPE_E_UNSUPPORTED, "rope_attn: one (batch, head) slab or a cos/sin table exceeds 4 GiB");
   g_err[0] = 0;
   return COROPE_OK;
 }
@@ -104,8 +107,8 @@ int64_t fwd_ws_bytes(int B, int H, int N, int D) {
 // k_rot / tile_kmax null: single launch.  workspace non-null: rotate K into it first.
 int rope_attn_fwd_impl(const char* what, const void* q, const void* k, const void* v, const float* freqs_cos,
                        const float* freqs_sin, int64_t freq_row_stride, void* o, float* lse, int B, int H, int N, int D,
-                       float sm_scale, int causal, const void* k_rot, const float* tile_kmax, void* workspace,
-                       int64_t workspace_bytes, void* stream) {
+                       float sm_scale, int causal, const void* k_rot, const float* tile_kmax, void* q_rot_out,
+                       void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
   if (rc) return rc;
   rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse});
@@ -124,6 +127,7 @@ int rope_attn_fwd_impl(const char* what, const void* q, const void* k, const voi
   p.BH = B * H;
   p.k_rot = static_cast<const uint16_t*>(k_rot);
   p.tile_kmax = tile_kmax;
+  p.q_rot_out = static_cast<uint16_t*>(q_rot_out);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (workspace != nullptr) {
     rc = check_ptrs(what, {workspace});
@@ -150,7 +154,7 @@ int corope_rope_attn_fwd(const void* q, const void* k, const void* v, const floa
                          int64_t freq_row_stride, void* o, float* lse, int B, int H, int N, int D, float sm_scale,
                          int causal, void* stream) {
   return rope_attn_fwd_impl("rope_attn_fwd", q, k, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, H, N, D, sm_scale,
-                            causal, nullptr, nullptr, nullptr, 0, stream);
+                            causal, nullptr, nullptr, nullptr, nullptr, 0, stream);
 }
 
 int64_t corope_rope_attn_fwd_workspace_bytes(int B, int H, int N, int D) {
@@ -163,19 +167,36 @@ int corope_rope_attn_fwd_ws(const void* q, const void* k, const void* v, const f
                             int causal, void* workspace, int64_t workspace_bytes, void* stream) {
   if (workspace == nullptr) return fail(COROPE_E_BADARG, "rope_attn_fwd_ws: null workspace");
   return rope_attn_fwd_impl("rope_attn_fwd_ws", q, k, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, H, N, D,
-                            sm_scale, causal, nullptr, nullptr, workspace, workspace_bytes, stream);
+                            sm_scale, causal, nullptr, nullptr, nullptr, workspace, workspace_bytes, stream);
 }
 
 int corope_rope_attn_fwd_prerotated(const void* q, const void* k_rot, const float* tile_kmax, const void* v,
                                     const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* o,
-                                    float* lse, int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
+                                    float* lse, void* q_rot_out, int B, int H, int N, int D, float sm_scale, int causal,
+                                    void* stream) {
   int rc = check_ptrs("rope_attn_fwd_prerotated", {k_rot});
   if (rc) return rc;
+  if (q_rot_out != nullptr && !aligned16(q_rot_out))
+    return fail(COROPE_E_ALIGN, "rope_attn_fwd_prerotated: q_rot_out %p is not 16-byte aligned", q_rot_out);
   if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
     return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "rope_attn_fwd_prerotated: tile_kmax %p is null or misaligned",
                 (const void*)tile_kmax);
   return rope_attn_fwd_impl("rope_attn_fwd_prerotated", q, k_rot, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, H,
-                            N, D, sm_scale, causal, k_rot, tile_kmax, nullptr, 0, stream);
+                            N, D, sm_scale, causal, k_rot, tile_kmax, q_rot_out, nullptr, 0, stream);
+}
+
+int corope_rope_attn_fwd_train(const void* q, const void* k, const void* v, const float* freqs_cos, const float* freqs_sin,
+                               int64_t freq_row_stride, void* o, float* lse, void* q_rot, void* k_rot, float* tile_kmax,
+                               int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
+  int rc = check_ptrs("rope_attn_fwd_train", {q_rot, k_rot});
+  if (rc) return rc;
+  if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
+    return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "rope_attn_fwd_train: tile_kmax %p is null or misaligned",
+                (const void*)tile_kmax);
+  rc = corope_rope_rotate(k, freqs_cos, freqs_sin, freq_row_stride, k_rot, tile_kmax, B, H, N, D, stream);
+  if (rc) return rc;
+  return corope_rope_attn_fwd_prerotated(q, k_rot, tile_kmax, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, q_rot, B, H,
+                                         N, D, sm_scale, causal, stream);
 }
 
 int corope_rope_rotate(const void* x, const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* y,
@@ -332,6 +353,22 @@ int corope_rope_attn_bwd(const void* q, const void* k, const void* v, const void
                                  sm_scale, causal, stream);
 }
 
+int corope_rope_attn_bwd_prerotated(const void* q_rot, const void* k_rot, const void* v, const void* o, const void* d_o,
+                                    const float* lse, float* delta, const float* freqs_cos, const float* freqs_sin,
+                                    int64_t freq_row_stride, void* dq, void* dk, void* dv, int B, int H, int N, int D,
+                                    float sm_scale, int causal, void* stream) {
+  int rc = corope_rope_attn_bwd_preprocess(o, d_o, delta, B, H, N, D, stream);
+  if (rc) return rc;
+  rc = corope_rope_attn_bwd_dv_prerotated(q_rot, k_rot, d_o, lse, freqs_cos, freqs_sin, freq_row_stride, dv, B, H, N, D,
+                                          sm_scale, causal, stream);
+  if (rc) return rc;
+  rc = corope_rope_attn_bwd_dk_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dk, B,
+                                          H, N, D, sm_scale, causal, stream);
+  if (rc) return rc;
+  return corope_rope_attn_bwd_dq_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq,
+                                            B, H, N, D, sm_scale, causal, stream);
+}
+
 int64_t corope_rope_attn_bwd_workspace_bytes(int B, int H, int N, int D) {
   if (corope_rope_attn_check(B, H, N, D, D, 1.f, 1)) return -1;
   return 2 * bwd_ws_tensor_bytes(B, H, N, D);
@@ -354,16 +391,8 @@ int corope_rope_attn_bwd_ws(const void* q, const void* k, const void* v, const v
   if (rc) return rc;
   rc = corope_rope_rotate(k, freqs_cos, freqs_sin, freq_row_stride, k_rot, nullptr, B, H, N, D, stream);
   if (rc) return rc;
-  rc = corope_rope_attn_bwd_preprocess(o, d_o, delta, B, H, N, D, stream);
-  if (rc) return rc;
-  rc = corope_rope_attn_bwd_dv_prerotated(q_rot, k_rot, d_o, lse, freqs_cos, freqs_sin, freq_row_stride, dv, B, H, N, D,
-                                          sm_scale, causal, stream);
-  if (rc) return rc;
-  rc = corope_rope_attn_bwd_dk_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dk, B,
-                                          H, N, D, sm_scale, causal, stream);
-  if (rc) return rc;
-  return corope_rope_attn_bwd_dq_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq,
-                                            B, H, N, D, sm_scale, causal, stream);
+  return corope_rope_attn_bwd_prerotated(q_rot, k_rot, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, dk,
+                                         dv, B, H, N, D, sm_scale, causal, stream);
 }
 
 int corope_rope_freqs(float* freqs_cos, float* freqs_sin, int n_pos, int D, int width, int64_t freq_row_stride, int pos0,

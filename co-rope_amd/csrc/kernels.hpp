@@ -12,6 +12,7 @@ struct FwdParams {
   const uint16_t* v;
   const uint16_t* k_rot;   // K already rotated (same layout as k), or null: rotate K tiles inside the kernel
   const float* tile_kmax;  // with k_rot: largest rotated-key norm of every 64-key tile, [BH][ceil(N / 64)]
+  uint16_t* q_rot_out;     // with k_rot, optional: receives the rotated Q (same layout as q), for a backward on rotated operands
   const float* cos;
   const float* sin;
   uint16_t* o;

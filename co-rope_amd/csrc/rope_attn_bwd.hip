@@ -341,7 +341,7 @@ static hipError_t set_lds(K kern, int bytes) {
 // wave needs more than 256 registers, which would halve the waves per SIMD.
 template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
 static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
-  constexpr int NWAVES = 8, BLOCK_M = 64;
+  constexpr int NWAVES = 8, BLOCK_M = (PREROT && !DO_DK) ? 128 : 64;   // the larger tile pays off (and fits) for dV on pre-rotated operands only
   using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? 8 : 32>;
   auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK, PREROT>;
   static bool attr_set = false;

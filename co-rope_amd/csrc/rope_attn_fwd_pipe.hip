@@ -117,6 +117,11 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
   const int q_row = m0 + wave * 32 + lq;           // absolute query index of this lane
   u32x4 qb[M];
   load_b_rows<D, true>(qb, qg, p.cos, p.sin, p.fstride, min(q_row, N - 1));
+  if (p.q_rot_out != nullptr && q_row < N) {   // the rotated rows, exactly as the MFMAs see them
+    uint16_t* dst = p.q_rot_out + ((int64_t)bh * N + q_row) * D + 8 * lh;
+#pragma unroll
+    for (int kc = 0; kc < M; ++kc) *reinterpret_cast<u32x4*>(dst + 16 * kc) = qb[kc];
+  }
 
   const float scale = p.qk_scale;
   // Largest |q_r| * scale of the wave's rows (a little generous): times a tile's largest key norm it bounds the

@@ -53,8 +53,9 @@ def _freq_table(f):
 TWO_LAUNCH_MIN_N = 1024
 
 
-def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None):
-    """Runs the forward kernels; returns (o, M, fc, fs) with the tables in the form the kernels were given."""
+def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, keep_rotated=False):
+    """Runs the forward kernels; returns (o, M, fc, fs, rotated) with the tables in the form the kernels were given.
+    ``rotated`` is (q_rot, k_rot) when ``keep_rotated`` was asked for and the two-launch path ran, else None."""
     lib = _lib.load()
     fc, fs = _freq_table(freqs_cos), _freq_table(freqs_sin)
     if fc.stride(0) != fs.stride(0):
@@ -64,8 +65,18 @@ def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None):
     M = torch.empty((B, H, N), device=q.device, dtype=torch.float32)
     if two_launch is None:
         two_launch = N >= TWO_LAUNCH_MIN_N
+    rotated = None
     with torch.cuda.device(q.device):
-        if two_launch:
+        if two_launch and keep_rotated:
+            q_rot, k_rot = torch.empty_like(q), torch.empty_like(k)
+            kmax = torch.empty((B, H, (N + 63) // 64), device=q.device, dtype=torch.float32)
+            rc = lib.corope_rope_attn_fwd_train(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
+                                                fc.stride(0), o.data_ptr(), M.data_ptr(), q_rot.data_ptr(), k_rot.data_ptr(),
+                                                kmax.data_ptr(), B, H, N, D, float(sm_scale), int(bool(causal)),
+                                                _stream_ptr(q))
+            _lib.check(rc, "corope_rope_attn_fwd_train")
+            rotated = (q_rot, k_rot)
+        elif two_launch:
             nbytes = lib.corope_rope_attn_fwd_workspace_bytes(B, H, N, D)
             if nbytes < 0:
                 _lib.check(lib.corope_rope_attn_check(B, H, N, D, fc.stride(0), float(sm_scale), 0), "corope_rope_attn_check")
@@ -79,7 +90,7 @@ def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None):
                                           fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, N, D, float(sm_scale),
                                           int(bool(causal)), _stream_ptr(q))
             _lib.check(rc, "corope_rope_attn_fwd")
-    return o, M, fc, fs
+    return o, M, fc, fs, rotated
 
 
 class _FusedRopeAttn(torch.autograd.Function):
@@ -89,8 +100,15 @@ class _FusedRopeAttn(torch.autograd.Function):
         _check_inputs(q, k, v, freqs_cos, freqs_sin)
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         B, H, N, D = q.shape
-        o, M, fc, fs = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin)
-        ctx.save_for_backward(q, k, v, o, M, fc, fs)
+        # when a gradient will be asked for, the forward keeps its rotated q and k for the backward and the originals
+        # are not saved (the reference saves q and k, fused_rope_attn.py:718, and re-rotates them in its backward)
+        o, M, fc, fs, rotated = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin,
+                                         keep_rotated=any(ctx.needs_input_grad[:3]))
+        ctx.rotated = rotated is not None
+        if ctx.rotated:
+            ctx.save_for_backward(rotated[0], rotated[1], v, o, M, fc, fs)
+        else:
+            ctx.save_for_backward(q, k, v, o, M, fc, fs)
         ctx.sm_scale = float(sm_scale)
         ctx.HEAD_DIM = D
         ctx.causal = bool(causal)
@@ -107,7 +125,13 @@ class _FusedRopeAttn(torch.autograd.Function):
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         delta = torch.empty_like(M)
         with torch.cuda.device(q.device):
-            if N >= TWO_LAUNCH_MIN_N:   # rotate q and k once, then run the kernels on the rotated copies
+            if ctx.rotated:             # q, k are the rotated copies the forward kept
+                rc = lib.corope_rope_attn_bwd_prerotated(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                                         do.data_ptr(), M.data_ptr(), delta.data_ptr(), fc.data_ptr(),
+                                                         fs.data_ptr(), fc.stride(0), dq.data_ptr(), dk.data_ptr(),
+                                                         dv.data_ptr(), B, H, N, D, ctx.sm_scale, int(ctx.causal),
+                                                         _stream_ptr(q))
+            elif N >= TWO_LAUNCH_MIN_N:   # rotate q and k once, then run the kernels on the rotated copies
                 nbytes = lib.corope_rope_attn_bwd_workspace_bytes(B, H, N, D)
                 ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
                 rc = lib.corope_rope_attn_bwd_ws(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
@@ -138,7 +162,7 @@ def rope_attn_forward_with_lse(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, 
     ``two_launch`` forces (True / False) or leaves to the length rule (None) the choice of forward path."""
     _check_inputs(q, k, v, freqs_cos, freqs_sin)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    o, M, _, _ = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch)
+    o, M, _, _, _ = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch)
     return o, M
 
 

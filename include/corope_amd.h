@@ -84,11 +84,22 @@ int corope_rope_rotate(const void *x, const float *freqs_cos, const float *freqs
 
 /* Attention on a K that corope_rope_rotate already rotated (k_rot, with its tile_max as tile_kmax): the second
  * launch of corope_rope_attn_fwd_ws on its own, for callers that keep the rotated K (a key cache) or time the two
- * launches separately.  q is still rotated inside the kernel.  Same reference site as corope_rope_attn_fwd. */
+ * launches separately.  q is still rotated inside the kernel; q_rot_out (may be NULL) receives the rotated q.
+ * Same reference site as corope_rope_attn_fwd. */
 int corope_rope_attn_fwd_prerotated(const void *q, const void *k_rot, const float *tile_kmax, const void *v,
                                     const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
-                                    void *o, float *lse,
+                                    void *o, float *lse, void *q_rot_out,
                                     int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
+/* Forward for training: like corope_rope_attn_fwd_ws, but the rotated operands are outputs the caller keeps --
+ * q_rot and k_rot, (B,H,N,D) bf16 -- so that the backward (corope_rope_attn_bwd_prerotated) needs no rotation pass and
+ * the original q and k need not be saved (the reference saves q and k and re-rotates them in every inner iteration of
+ * its backward, fused-rope/fused_rope_attn.py:718, :367-380).  tile_kmax: scratch, B*H*ceil(N/64) floats.
+ * Same launch site as corope_rope_attn_fwd. */
+int corope_rope_attn_fwd_train(const void *q, const void *k, const void *v,
+                               const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                               void *o, float *lse, void *q_rot, void *k_rot, float *tile_kmax,
+                               int B, int H, int N, int D, float sm_scale, int causal, void *stream);
 
 /* delta[b,h,i] = sum_d o[b,h,i,d] * do[b,h,i,d]  (fp32).
  * Replaces _attn_bwd_preprocess (reference fused-rope/fused_rope_attn.py:324-337, launch :753-758). */
@@ -154,6 +165,14 @@ int corope_rope_attn_bwd_dq_prerotated(const void *q_rot, const void *k_rot, con
                                        const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
                                        void *dq,
                                        int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
+/* Whole backward on rotated operands kept from corope_rope_attn_fwd_train (or made by corope_rope_rotate): preprocess,
+ * dV, dK, dQ.  Replaces _attention.backward like corope_rope_attn_bwd (reference fused-rope/fused_rope_attn.py:720-777). */
+int corope_rope_attn_bwd_prerotated(const void *q_rot, const void *k_rot, const void *v, const void *o, const void *d_o,
+                                    const float *lse, float *delta,
+                                    const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                                    void *dq, void *dk, void *dv,
+                                    int B, int H, int N, int D, float sm_scale, int causal, void *stream);
 
 /* Whole backward for long sequences: rotates q and k once into `workspace`, then preprocess, dV, dK, dQ on the
  * rotated copies.  Replaces _attention.backward like corope_rope_attn_bwd (reference

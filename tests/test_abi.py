@@ -50,6 +50,9 @@ def test_header_cites_reference_for_each_entry_point():
     ((1, 8, 128, 64, 66, 1.0, 0), -1),      # row stride not a multiple of 4 floats
     ((1, 8, 128, 64, 64, 0.0, 0), -1),
     ((1, 8, 128, 64, 64, float("nan"), 0), -1),
+    ((1, 1, 1 << 24, 128, 64, 1.0, 0), -2),   # one (batch, head) slab of 4 GiB: past the 32-bit staging offsets
+    ((1, 1, 1 << 22, 128, 256, 1.0, 0), -2),  # cos/sin table of 4 GiB
+    ((1, 1, 1 << 22, 128, 64, 1.0, 0), 0),
 ])
 def test_rope_attn_check_codes(pkg, args, code):
     lib = pkg._lib.load()

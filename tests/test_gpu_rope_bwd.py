@@ -106,3 +106,25 @@ def test_backward_paths_agree(pkg, monkeypatch):
         grads.append([t.grad.float().cpu() for t in (qd, kd, vd)])
     for a, b, name in zip(grads[0], grads[1], ("dQ", "dK", "dV")):
         assert torch.equal(a, b), name
+    # third path: the forward keeps its rotated q and k and the backward runs on them (another forward kernel, so O and
+    # M differ in the last bit and the gradients agree to rounding, not bit for bit)
+    monkeypatch.setattr(pkg.rope_attn, "TWO_LAUNCH_MIN_N", 1)
+    qd, kd, vd = (t.to(dev, torch.bfloat16).requires_grad_(True) for t in (q, k, v))
+    pkg.attention(qd, kd, vd, True, 0.09, c.to(dev), s.to(dev)).backward(g.to(dev, torch.bfloat16))
+    torch.cuda.synchronize()
+    for a, t, name in zip(grads[0], (qd, kd, vd), ("dQ", "dK", "dV")):
+        assert ((a - t.grad.float().cpu()).abs() <= 5e-3 + a.abs() / 64).all(), name
+
+
+def test_forward_keeps_rotated_operands(pkg):
+    """corope_rope_attn_fwd_train leaves q_rot and k_rot equal to what corope_rope_rotate produces (bit for bit)."""
+    B, H, N, D = 2, 2, 300, 128
+    q, k, v, g, c, s = _case(B, H, N, D, seed=8)
+    dev = torch.device("cuda:0")
+    qd, kd, vd = (t.to(dev, torch.bfloat16) for t in (q, k, v))
+    cd, sd = c.to(dev), s.to(dev)
+    o, M, _, _, rot = pkg.rope_attn._forward(qd, kd, vd, True, 0.09, cd, sd, two_launch=True, keep_rotated=True)
+    o2, M2 = pkg.rope_attn_forward_with_lse(qd, kd, vd, True, 0.09, cd, sd, two_launch=True)
+    torch.cuda.synchronize()
+    assert torch.equal(rot[0], pkg.rope_rotate(qd, cd, sd)) and torch.equal(rot[1], pkg.rope_rotate(kd, cd, sd))
+    assert torch.equal(o, o2) and torch.equal(M, M2)
