@@ -265,10 +265,9 @@ def main():
         if N >= pkg.rope_attn.TWO_LAUNCH_MIN_N:   # the backward the operator takes at this length: on the rotated q, k
             qr, kr = q_rot.data_ptr(), k_rot.data_ptr()   # which the forward kept
             launches += [
-                ("rope_attn_bwd_dv", lambda: lib.corope_rope_attn_bwd_dv_prerotated(
-                    qr, kr, dop, M.data_ptr(), cp, sp, fs, dv.data_ptr(), B, H, N, D, scale, 1, stream)),
-                ("rope_attn_bwd_dk", lambda: lib.corope_rope_attn_bwd_dk_prerotated(
-                    qr, kr, vp, dop, M.data_ptr(), delta.data_ptr(), cp, sp, fs, dk.data_ptr(), B, H, N, D, scale, 1, stream)),
+                ("rope_attn_bwd_dkdv", lambda: lib.corope_rope_attn_bwd_dkdv_prerotated(
+                    qr, kr, vp, dop, M.data_ptr(), delta.data_ptr(), cp, sp, fs, dk.data_ptr(), dv.data_ptr(), B, H, N, D,
+                    scale, 1, stream)),
                 ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq_prerotated(
                     qr, kr, vp, dop, M.data_ptr(), delta.data_ptr(), cp, sp, fs, dq.data_ptr(), B, H, N, D, scale, 1, stream)),
             ]
@@ -295,11 +294,12 @@ def main():
             for i, (name, _) in enumerate(launches):
                 durs[name].append(evs[i].elapsed_time(evs[i + 1]))
     avg = {n: sum(d) / len(d) for n, d in durs.items()}
-    # algorithmic FLOPs per launch (the reference's model: forward 2 matmul units, backward 5): dV kernel 2 units (the
-    # counted S recompute and dV), dK kernel 2 units (dP and dK; its own S recompute is overhead on top of the model),
-    # dQ kernel 1 unit (dQ; its S and dP recomputes are overhead); the preprocess pass is HBM-bound.
+    # algorithmic FLOPs per launch (the reference's model: forward 2 matmul units, backward 5): fused dK+dV kernel 4 units
+    # (the counted S recompute, dP, dV, dK) -- as two launches: dV 2 units, dK 2 units (its own S recompute is overhead on
+    # top of the model); dQ kernel 1 unit (dQ; its S and dP recomputes are overhead); the preprocess pass is HBM-bound.
     unit = 2.0 * B * H * N * N * D * 0.5
-    alg = {"rope_attn_fwd": 2 * unit, "rope_attn_bwd_dv": 2 * unit, "rope_attn_bwd_dk": 2 * unit, "rope_attn_bwd_dq": 1 * unit}
+    alg = {"rope_attn_fwd": 2 * unit, "rope_attn_bwd_dkdv": 4 * unit, "rope_attn_bwd_dv": 2 * unit, "rope_attn_bwd_dk": 2 * unit,
+           "rope_attn_bwd_dq": 1 * unit}
     kernels = {}
     for n, ms in avg.items():
         if n in alg:

@@ -332,6 +332,21 @@ int corope_rope_attn_bwd_dk_prerotated(const void* q_rot, const void* k_rot, con
                      freq_row_stride, dk, B, H, N, D, sm_scale, causal, stream);
 }
 
+int corope_rope_attn_bwd_dkdv_prerotated(const void* q_rot, const void* k_rot, const void* v, const void* d_o,
+                                         const float* lse, const float* delta, const float* freqs_cos,
+                                         const float* freqs_sin, int64_t freq_row_stride, void* dk, void* dv, int B, int H,
+                                         int N, int D, float sm_scale, int causal, void* stream) {
+  const char* what = "rope_attn_bwd_dkdv_prerotated";
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
+  if (rc) return rc;
+  rc = check_ptrs(what, {q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, dk, dv});
+  if (rc) return rc;
+  corope::BwdParams p = make_bwd(q_rot, k_rot, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
+                                 freq_row_stride, nullptr, dk, dv, B, H, N, sm_scale);
+  mark_prerotated(p, true);
+  return launch_status(what, corope::launch_bwd_dkdv_fused(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+}
+
 int corope_rope_attn_bwd_dq_prerotated(const void* q_rot, const void* k_rot, const void* v, const void* d_o,
                                        const float* lse, const float* delta, const float* freqs_cos,
                                        const float* freqs_sin, int64_t freq_row_stride, void* dq, int B, int H, int N,
@@ -359,11 +374,8 @@ int corope_rope_attn_bwd_prerotated(const void* q_rot, const void* k_rot, const 
                                     float sm_scale, int causal, void* stream) {
   int rc = corope_rope_attn_bwd_preprocess(o, d_o, delta, B, H, N, D, stream);
   if (rc) return rc;
-  rc = corope_rope_attn_bwd_dv_prerotated(q_rot, k_rot, d_o, lse, freqs_cos, freqs_sin, freq_row_stride, dv, B, H, N, D,
-                                          sm_scale, causal, stream);
-  if (rc) return rc;
-  rc = corope_rope_attn_bwd_dk_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dk, B,
-                                          H, N, D, sm_scale, causal, stream);
+  rc = corope_rope_attn_bwd_dkdv_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dk,
+                                            dv, B, H, N, D, sm_scale, causal, stream);
   if (rc) return rc;
   return corope_rope_attn_bwd_dq_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq,
                                             B, H, N, D, sm_scale, causal, stream);

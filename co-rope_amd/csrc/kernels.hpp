@@ -66,6 +66,7 @@ hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStrea
 hipError_t launch_bwd_preprocess(const BwdParams& p, int D, hipStream_t stream);
 hipError_t launch_bwd_dv(const BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_dk(const BwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_bwd_dkdv_fused(const BwdParams& p, int D, bool causal, hipStream_t stream);  // dK and dV in one launch
 hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_corope_gqa_fwd(const CoropeParams& p, int D, hipStream_t stream);
 hipError_t launch_rope_freqs(float* cosp, float* sinp, int n_pos, int D, int width, int64_t row_stride, int pos0,

@@ -28,7 +28,9 @@ namespace corope {
 //   dK_r^T += Q_r^T dS        (A = Q_r tile read transposed, B = dS)
 // DO_PAD: row padding of the dO tile.  The dV-only kernel reads dO through the transposing load alone and takes the
 // padding that is conflict-free for it (32); the dK kernel reads dO row-wise (8).
-template <int D, int NWAVES, int BLOCK_M, int DO_PAD>
+// V_LDS: the workgroup's V rows live in LDS (behind the two tile stages) instead of registers -- the fused dK+dV kernel,
+// whose two sets of accumulators leave no room for them.
+template <int D, int NWAVES, int BLOCK_M, int DO_PAD, bool V_LDS>
 struct DkdvCfg {
   static constexpr int kThreads = NWAVES * kWave;
   static constexpr int kBlockN = NWAVES * 32;
@@ -36,14 +38,16 @@ struct DkdvCfg {
   static constexpr int kDoTileBytes = RowTile<D, DO_PAD>::bytes(BLOCK_M);
   static constexpr int kStatBytes = BLOCK_M * 4;
   static constexpr int kStageBytes = kTileBytes + kDoTileBytes + 2 * kStatBytes;
-  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr int kVRowsBytes = V_LDS ? RowTile<D>::bytes(kBlockN) : 0;
+  static constexpr int kLdsBytes = 2 * kStageBytes + kVRowsBytes;
 };
 
 // PREROT: Q and K come from copies that rope_rotate_kernel rotated beforehand (no table reads in the loop).
 template <int D, int NWAVES, int BLOCK_M, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
 __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
   constexpr int DO_PAD = DO_DK ? 8 : 32;
-  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_PAD>;
+  constexpr bool V_LDS = DO_DV && DO_DK;
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_PAD, V_LDS>;
   constexpr int NT = Cfg::kThreads;
   constexpr int KC = D / 16, NDB = D / 32, NQB = BLOCK_M / 32;
   constexpr int LS = RowTile<D>::kStride, LSDO = RowTile<D, DO_PAD>::kStride;
@@ -65,9 +69,15 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
   const int key_c = min(key, N - 1);
   const int wk_lo = n0 + wave * 32, wk_hi = wk_lo + 31;
 
-  u32x4 kb[KC], vb[DO_DK ? KC : 1];
+  u32x4 kb[KC], vb[(DO_DK && !V_LDS) ? KC : 1];
   load_b_rows<D, !PREROT>(kb, (PREROT ? p.k_rot : p.k) + base, p.cos, p.sin, p.fstride, key_c);
-  if constexpr (DO_DK) load_b_rows<D, false>(vb, p.v + base, nullptr, nullptr, 0, key_c);
+  if constexpr (DO_DK && !V_LDS) load_b_rows<D, false>(vb, p.v + base, nullptr, nullptr, 0, key_c);
+  uint16_t* vrows = reinterpret_cast<uint16_t*>(smem + 2 * Cfg::kStageBytes);   // V_LDS: the block's V rows, row-major
+  if constexpr (V_LDS) {
+    CopyStage<D, Cfg::kBlockN, NT> vcp;
+    vcp.load(p.v + base, n0, N);
+    vcp.store_rows(vrows);    // visible after the barrier that ends the prologue
+  }
 
   const int m_tiles = (N + BLOCK_M - 1) / BLOCK_M;
   const int mt0 = CAUSAL ? n0 / BLOCK_M : 0;
@@ -139,7 +149,9 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
       if constexpr (DO_DK) {
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
-          dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc), vb[kc], kc == 0 ? f32x16{0} : dpacc);
+          dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc),
+                         V_LDS ? *reinterpret_cast<const u32x4*>(vrows + RowTile<D>::off(wave * 32 + lq, 8 * lh + 16 * kc)) : vb[V_LDS ? 0 : kc],
+                         kc == 0 ? f32x16{0} : dpacc);
       }
 
       // Causal mask on the raw scores, under a wave-uniform branch of its own (written into the exponential loop it
@@ -342,7 +354,7 @@ static hipError_t set_lds(K kern, int bytes) {
 template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
 static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
   constexpr int NWAVES = 8, BLOCK_M = (PREROT && !DO_DK) ? 128 : 64;   // the larger tile pays off (and fits) for dV on pre-rotated operands only
-  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? 8 : 32>;
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? 8 : 32, DO_DV && DO_DK>;
   auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK, PREROT>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -383,6 +395,10 @@ static hipError_t launch_dkdv(const BwdParams& p, int D, bool causal, hipStream_
   if (pre) return causal ? COROPE_DKDV(64, true, true) : COROPE_DKDV(64, false, true);
   return causal ? COROPE_DKDV(64, true, false) : COROPE_DKDV(64, false, false);
 #undef COROPE_DKDV
+}
+
+hipError_t launch_bwd_dkdv_fused(const BwdParams& p, int D, bool causal, hipStream_t stream) {
+  return launch_dkdv<true, true>(p, D, causal, stream);
 }
 
 hipError_t launch_bwd_dv(const BwdParams& p, int D, bool causal, hipStream_t stream) {

@@ -160,6 +160,14 @@ int corope_rope_attn_bwd_dk_prerotated(const void *q_rot, const void *k_rot, con
                                        const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
                                        void *dk,
                                        int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+/* dK and dV in one launch (S is recomputed once for both; the workgroup's V rows sit in LDS to make room for the two
+ * sets of accumulators): the fused form of the two entry points above, same results bit for bit.  Replaces
+ * _attn_bwd_dkdv (reference fused-rope/fused_rope_attn.py:342-404). */
+int corope_rope_attn_bwd_dkdv_prerotated(const void *q_rot, const void *k_rot, const void *v, const void *d_o,
+                                         const float *lse, const float *delta,
+                                         const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                                         void *dk, void *dv,
+                                         int B, int H, int N, int D, float sm_scale, int causal, void *stream);
 int corope_rope_attn_bwd_dq_prerotated(const void *q_rot, const void *k_rot, const void *v, const void *d_o,
                                        const float *lse, const float *delta,
                                        const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
