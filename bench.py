@@ -248,7 +248,8 @@ def main():
     dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
     qp, kp, vp, dop = q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr()
     cp, sp, fs = cos.data_ptr(), sin.data_ptr(), cos.stride(0)
-    if N >= pkg.rope_attn.TWO_LAUNCH_MIN_N:   # the forward the operator takes at this length: rotate K, then attention
+    rotated = pkg.rope_attn.use_rotated_path(N, D, training=not fwd_only)
+    if rotated:   # the forward the operator takes at this shape: rotate K, then attention
         k_rot, q_rot = torch.empty_like(k), torch.empty_like(q)
         kmax = torch.empty(B, H, (N + 63) // 64, device=dev, dtype=torch.float32)
         launches = [("rope_rotate_k", lambda: lib.corope_rope_rotate(kp, cp, sp, fs, k_rot.data_ptr(), kmax.data_ptr(),
@@ -262,7 +263,7 @@ def main():
     if not fwd_only:
         launches += [("rope_attn_bwd_preprocess", lambda: lib.corope_rope_attn_bwd_preprocess(
             o.data_ptr(), dop, delta.data_ptr(), B, H, N, D, stream))]
-        if N >= pkg.rope_attn.TWO_LAUNCH_MIN_N:   # the backward the operator takes at this length: on the rotated q, k
+        if rotated:   # the backward the operator takes at this shape: on the rotated q, k
             qr, kr = q_rot.data_ptr(), k_rot.data_ptr()   # which the forward kept
             launches += [
                 ("rope_attn_bwd_dkdv", lambda: lib.corope_rope_attn_bwd_dkdv_prerotated(

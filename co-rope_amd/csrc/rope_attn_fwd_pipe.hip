@@ -40,6 +40,7 @@ constexpr int kPipeBlockN = 64;
 // p stays below 2^kPipeMargin and the fp32 sums below 2^(kPipeMargin + log2 N + log2 max|v|): far from overflow, and
 // bf16 has fp32's exponent range, so P loses nothing either.
 constexpr float kPipeMargin = 64.f;
+constexpr float kPipeLift = 40.f;
 
 template <int D>
 struct FwdPipeCfg {
@@ -182,6 +183,19 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
   // last tile this wave's rows can see
   const int t_last = __builtin_amdgcn_readfirstlane(CAUSAL ? min(n_tiles - 1, wave_q_hi / BLOCK_N) : n_tiles - 1);
 
+  // Reference value (raw-score units) that puts every tile this wave will see within the margin.
+  float lift_target;
+  {
+    uint32_t kall = 0;
+    for (int t0 = 0; t0 <= t_last; t0 += kWave) {
+      const int tt = t0 + lane;
+      kall = max(kall, tt <= t_last ? tile_kmax_bits[tt] : 0u);   // non-negative floats order like their bit patterns
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) kall = max(kall, (uint32_t)__shfl_xor((int)kall, m));
+    lift_target = (q_bound_wave * __builtin_bit_cast(float, kall) - kPipeMargin) / scale;
+  }
+
   // Bit patterns of non-negative floats order like the floats: the per-tile test "bound > reference + margin" is
   // kmax_bits > thr_bits with thr = (min over rows of m_run * scale + margin) / q_bound_wave, recomputed when the
   // reference moves.  Lane i of kvec holds the key-norm maximum of tile kvec_base + i.
@@ -292,7 +306,12 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
       float mt = fmaxf(r0[0], r1[0]);
 #pragma unroll
       for (int i = 1; i < 16; ++i) mt = fmaxf(fmaxf(mt, r0[i]), r1[i]);
-      const float m_new = fmaxf(m_run, half_max(mt));
+      float m_new = fmaxf(m_run, half_max(mt));
+      // Lift the reference towards the largest bound any later tile of this wave can show, so that the test above does
+      // not fire again (with the Cauchy-Schwarz bound 2-3x above the scores actually seen, hot logits would otherwise
+      // send most tiles through this block).  Never further than kPipeLift above the true maximum: the row's largest
+      // probability stays above 2^-kPipeLift, far inside fp32 / bf16 range.
+      m_new = fmaxf(m_new, fminf(lift_target, m_new + kPipeLift / scale));
       const float alpha = fast_exp2((m_run - m_new) * scale);   // m_new is finite: every row sees key 0 of tile 0
       l_run = (l_run + lsum) * alpha;
       lsum = 0.f;

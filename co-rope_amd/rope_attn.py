@@ -51,6 +51,14 @@ def _freq_table(f):
 # Sequences at least this long take the two-launch forward (K rotated once into a scratch buffer, then attention on
 # the rotated copy); shorter ones the single launch, where every K tile is rotated by few query blocks anyway.
 TWO_LAUNCH_MIN_N = 1024
+# When a gradient will be asked for, the rotated copies also feed the backward (fused dK+dV, no tables in its loops), which
+# pays off earlier: from N * D >= this (N = 512 at D = 128, N = 1024 at D = 64; measured crossover on MI355X).
+TRAIN_ROTATED_MIN_ND = 65536
+
+
+def use_rotated_path(N, D, training):
+    """Whether the operator rotates the operands ahead of the attention kernels at this shape."""
+    return N >= TWO_LAUNCH_MIN_N or (training and N * D >= TRAIN_ROTATED_MIN_ND)
 
 
 def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, keep_rotated=False):
@@ -64,7 +72,7 @@ def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, k
     o = torch.empty_like(q)
     M = torch.empty((B, H, N), device=q.device, dtype=torch.float32)
     if two_launch is None:
-        two_launch = N >= TWO_LAUNCH_MIN_N
+        two_launch = use_rotated_path(N, D, training=keep_rotated)
     rotated = None
     with torch.cuda.device(q.device):
         if two_launch and keep_rotated:
@@ -131,7 +139,7 @@ class _FusedRopeAttn(torch.autograd.Function):
                                                          fs.data_ptr(), fc.stride(0), dq.data_ptr(), dk.data_ptr(),
                                                          dv.data_ptr(), B, H, N, D, ctx.sm_scale, int(ctx.causal),
                                                          _stream_ptr(q))
-            elif N >= TWO_LAUNCH_MIN_N:   # rotate q and k once, then run the kernels on the rotated copies
+            elif use_rotated_path(N, D, training=True):   # rotate q and k once, then run the kernels on the rotated copies
                 nbytes = lib.corope_rope_attn_bwd_workspace_bytes(B, H, N, D)
                 ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
                 rc = lib.corope_rope_attn_bwd_ws(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),

@@ -20,6 +20,12 @@ def _case(B, H, N, D, seed=42):
     return q, k, v, g, c, s
 
 
+def _force_path(monkeypatch, pkg, rotated):
+    """Moves the operator's shape thresholds so that every shape takes (rotated=True) or avoids the rotated-operand path."""
+    monkeypatch.setattr(pkg.rope_attn, "TWO_LAUNCH_MIN_N", 1 if rotated else 1 << 30)
+    monkeypatch.setattr(pkg.rope_attn, "TRAIN_ROTATED_MIN_ND", 1 if rotated else 1 << 60)
+
+
 def _gpu_fwd_bwd(pkg, q, k, v, g, causal, scale, c, s):
     dev = torch.device("cuda:0")
     qd, kd, vd = (t.to(dev, torch.bfloat16).requires_grad_(True) for t in (q, k, v))
@@ -40,7 +46,7 @@ SHAPES = [(4, 8, 1024, 64), (1, 8, 1024, 128), (2, 4, 512, 64), (2, 2, 256, 128)
 @pytest.mark.parametrize("B,H,N,D", SHAPES)
 def test_backward_parity(pkg, monkeypatch, B, H, N, D, causal, two_launch):
     print(f"case B={B} H={H} N={N} D={D} causal={causal} two_launch={two_launch}", flush=True)
-    monkeypatch.setattr(pkg.rope_attn, "TWO_LAUNCH_MIN_N", 1 if two_launch else 1 << 30)
+    _force_path(monkeypatch, pkg, two_launch)
     q, k, v, g, c, s = _case(B, H, N, D)
     scale = 1 / math.sqrt(D)
     o, dq, dk, dv = _gpu_fwd_bwd(pkg, q, k, v, g, causal, scale, c, s)
@@ -97,10 +103,10 @@ def test_backward_paths_agree(pkg, monkeypatch):
     dev = torch.device("cuda:0")
     grads = []
     for two_launch in (False, True):
-        monkeypatch.setattr(pkg.rope_attn, "TWO_LAUNCH_MIN_N", 1 << 30)     # same forward for both
+        _force_path(monkeypatch, pkg, False)     # same forward for both
         qd, kd, vd = (t.to(dev, torch.bfloat16).requires_grad_(True) for t in (q, k, v))
         o = pkg.attention(qd, kd, vd, True, 0.09, c.to(dev), s.to(dev))
-        monkeypatch.setattr(pkg.rope_attn, "TWO_LAUNCH_MIN_N", 1 if two_launch else 1 << 30)
+        _force_path(monkeypatch, pkg, two_launch)
         o.backward(g.to(dev, torch.bfloat16))
         torch.cuda.synchronize()
         grads.append([t.grad.float().cpu() for t in (qd, kd, vd)])
@@ -108,7 +114,7 @@ def test_backward_paths_agree(pkg, monkeypatch):
         assert torch.equal(a, b), name
     # third path: the forward keeps its rotated q and k and the backward runs on them (another forward kernel, so O and
     # M differ in the last bit and the gradients agree to rounding, not bit for bit)
-    monkeypatch.setattr(pkg.rope_attn, "TWO_LAUNCH_MIN_N", 1)
+    _force_path(monkeypatch, pkg, True)
     qd, kd, vd = (t.to(dev, torch.bfloat16).requires_grad_(True) for t in (q, k, v))
     pkg.attention(qd, kd, vd, True, 0.09, c.to(dev), s.to(dev)).backward(g.to(dev, torch.bfloat16))
     torch.cuda.synchronize()
