@@ -122,9 +122,37 @@ def bench_sweep(args):
         o = pkg.attention(q, k, v, True, 0.5, cos, sin)
         b_ms = timed(lambda: o.backward(do, retain_graph=True))
         ff, fb = attention_flops(B, H, N, D, "fwd"), attention_flops(B, H, N, D, "bwd")
-        print(json.dumps({"config": name, "B": B, "H": H, "N": N, "D": D, "fwd_ms": round(f_ms, 4),
-                          "fwd_tflops": round(ff / f_ms * 1e-9, 1), "bwd_ms": round(b_ms, 4),
-                          "bwd_tflops": round(fb / b_ms * 1e-9, 1)}), flush=True)
+        row = {"config": name, "B": B, "H": H, "N": N, "D": D, "fwd_ms": round(f_ms, 4),
+               "fwd_tflops": round(ff / f_ms * 1e-9, 1), "bwd_ms": round(b_ms, 4), "bwd_tflops": round(fb / b_ms * 1e-9, 1)}
+        if args.lanes:
+            # the reference harness's comparison lanes (fused-rope/bench_compare.py:98-260), on this GPU:
+            #   unfused = a separate rotation pass over q and k, then the same attention kernels with identity tables
+            #             (backward: those kernels plus the inverse rotation of dq and dk, timed as two more passes);
+            #   sdpa    = the same rotation passes, then PyTorch's scaled_dot_product_attention.
+            qd, kd, vd = q.detach(), k.detach(), v.detach()
+            one, zero = torch.ones_like(cos), torch.zeros_like(sin)
+            rot_ms = timed(lambda: (pkg.rope_rotate(qd, cos, sin), pkg.rope_rotate(kd, cos, sin)))
+            qr = pkg.rope_rotate(qd, cos, sin).requires_grad_(True)
+            kr = pkg.rope_rotate(kd, cos, sin).requires_grad_(True)
+            uf_ms = rot_ms + timed(lambda: pkg.attention(qr, kr, v, True, 0.5, one, zero))
+            ou = pkg.attention(qr, kr, v, True, 0.5, one, zero)
+            ub_ms = rot_ms + timed(lambda: ou.backward(do, retain_graph=True))
+            row.update({"unfused_fwd_ms": round(uf_ms, 4), "unfused_bwd_ms": round(ub_ms, 4),
+                        "fwd_speedup_vs_unfused": round(uf_ms / f_ms, 3), "bwd_speedup_vs_unfused": round(ub_ms / b_ms, 3),
+                        "cos_sim_vs_unfused": round(float(torch.nn.functional.cosine_similarity(
+                            o.detach().float().flatten(), ou.detach().float().flatten(), dim=0)), 6)})
+            try:
+                sdpa = torch.nn.functional.scaled_dot_product_attention
+                sf_ms = rot_ms + timed(lambda: sdpa(qr, kr, v, is_causal=True, scale=0.5))
+                osd = sdpa(qr, kr, v, is_causal=True, scale=0.5)
+                sb_ms = rot_ms + timed(lambda: osd.backward(do, retain_graph=True))
+                row.update({"sdpa_fwd_ms": round(sf_ms, 4), "sdpa_bwd_ms": round(sb_ms, 4),
+                            "fwd_speedup_vs_sdpa": round(sf_ms / f_ms, 3), "bwd_speedup_vs_sdpa": round(sb_ms / b_ms, 3)})
+                del osd
+            except Exception as e:   # a shape PyTorch's kernels do not take on this build
+                row["sdpa_error"] = type(e).__name__
+            del qr, kr, ou
+        print(json.dumps(row), flush=True)
         del q, k, v, do, o
 
 
@@ -189,6 +217,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sweep", action="store_true",
                     help="time the reference harness's 19 shapes instead (one JSON line per shape)")
+    ap.add_argument("--lanes", action="store_true",
+                    help="with --sweep: also time the unfused lanes (separate rotation + identity-table attention, PyTorch SDPA)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
