@@ -57,6 +57,7 @@ corope::BwdParams make_bwd(const void* q, const void* k, const void* v, const vo
   p.qk_scale = sm_scale * kLog2e;
   p.N = N;
   p.BH = B * H;
+  p.H = p.Hkv = H;
   return p;
 }
 
@@ -108,7 +109,7 @@ int64_t fwd_ws_bytes(int B, int H, int N, int D) {
 int rope_attn_fwd_impl(const char* what, const void* q, const void* k, const void* v, const float* freqs_cos,
                        const float* freqs_sin, int64_t freq_row_stride, void* o, float* lse, int B, int H, int N, int D,
                        float sm_scale, int causal, const void* k_rot, const float* tile_kmax, void* q_rot_out,
-                       void* workspace, int64_t workspace_bytes, void* stream) {
+                       void* workspace, int64_t workspace_bytes, void* stream, int Hkv = 0) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
   if (rc) return rc;
   rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse});
@@ -125,6 +126,8 @@ int rope_attn_fwd_impl(const char* what, const void* q, const void* k, const voi
   p.qk_scale = sm_scale * kLog2e;
   p.N = N;
   p.BH = B * H;
+  p.H = H;
+  p.Hkv = Hkv > 0 ? Hkv : H;
   p.k_rot = static_cast<const uint16_t*>(k_rot);
   p.tile_kmax = tile_kmax;
   p.q_rot_out = static_cast<uint16_t*>(q_rot_out);
@@ -405,6 +408,55 @@ int corope_rope_attn_bwd_ws(const void* q, const void* k, const void* v, const v
   if (rc) return rc;
   return corope_rope_attn_bwd_prerotated(q_rot, k_rot, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, dk,
                                          dv, B, H, N, D, sm_scale, causal, stream);
+}
+
+int corope_rope_attn_fwd_gqa(const void* q, const void* k, const void* v, const float* freqs_cos, const float* freqs_sin,
+                             int64_t freq_row_stride, void* o, float* lse, void* q_rot, void* k_rot, float* tile_kmax, int B,
+                             int Hq, int Hkv, int N, int D, float sm_scale, int causal, void* stream) {
+  const char* what = "rope_attn_fwd_gqa";
+  if (Hkv <= 0 || Hq % Hkv != 0) return fail(COROPE_E_BADARG, "%s: Hq=%d is not a multiple of Hkv=%d", what, Hq, Hkv);
+  if (k_rot == nullptr) {
+    if (q_rot != nullptr) return fail(COROPE_E_BADARG, "%s: q_rot without k_rot", what);
+    return rope_attn_fwd_impl(what, q, k, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, Hq, N, D, sm_scale, causal,
+                              nullptr, nullptr, nullptr, nullptr, 0, stream, Hkv);
+  }
+  int rc = check_ptrs(what, {k_rot});
+  if (rc) return rc;
+  if (q_rot != nullptr && !aligned16(q_rot)) return fail(COROPE_E_ALIGN, "%s: q_rot %p is not 16-byte aligned", what, q_rot);
+  if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
+    return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "%s: tile_kmax %p is null or misaligned", what,
+                (const void*)tile_kmax);
+  rc = corope_rope_rotate(k, freqs_cos, freqs_sin, freq_row_stride, k_rot, tile_kmax, B, Hkv, N, D, stream);
+  if (rc) return rc;
+  return rope_attn_fwd_impl(what, q, k_rot, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, Hq, N, D, sm_scale, causal,
+                            k_rot, tile_kmax, q_rot, nullptr, 0, stream, Hkv);
+}
+
+int corope_rope_attn_bwd_gqa(const void* q, const void* k, int prerotated, const void* v, const void* o, const void* d_o,
+                             const float* lse, float* delta, const float* freqs_cos, const float* freqs_sin,
+                             int64_t freq_row_stride, void* dq, void* dk, void* dv, int B, int Hq, int Hkv, int N, int D,
+                             float sm_scale, int causal, void* stream) {
+  const char* what = "rope_attn_bwd_gqa";
+  if (Hkv <= 0 || Hq % Hkv != 0) return fail(COROPE_E_BADARG, "%s: Hq=%d is not a multiple of Hkv=%d", what, Hq, Hkv);
+  int rc = corope_rope_attn_check(B, Hq, N, D, freq_row_stride, sm_scale, 1);
+  if (rc) return rc;
+  rc = check_ptrs(what, {q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv});
+  if (rc) return rc;
+  rc = corope_rope_attn_bwd_preprocess(o, d_o, delta, B, Hq, N, D, stream);
+  if (rc) return rc;
+  corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, dk, dv, B, Hq,
+                                 N, sm_scale);
+  p.Hkv = Hkv;
+  mark_prerotated(p, prerotated != 0);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (prerotated) {
+    rc = launch_status(what, corope::launch_bwd_dkdv_fused(p, D, causal != 0, st));
+  } else {
+    rc = launch_status(what, corope::launch_bwd_dv(p, D, causal != 0, st));
+    if (rc == 0) rc = launch_status(what, corope::launch_bwd_dk(p, D, causal != 0, st));
+  }
+  if (rc) return rc;
+  return launch_status(what, corope::launch_bwd_dq(p, D, causal != 0, st));
 }
 
 int corope_rope_freqs(float* freqs_cos, float* freqs_sin, int n_pos, int D, int width, int64_t freq_row_stride, int pos0,

@@ -76,6 +76,11 @@ __device__ __forceinline__ const T* byte_offset(const T* base, uint32_t bytes) {
   return reinterpret_cast<const T*>(reinterpret_cast<const char*>(base) + bytes);
 }
 
+// Grouped-query attention: slab (batch, query head) -> slab (batch, key/value head) of tensors with Hkv heads.
+__device__ __forceinline__ int kv_slab(int bh, int H, int Hkv) {
+  return H == Hkv ? bh : (bh / H) * Hkv + (bh % H) / (H / Hkv);
+}
+
 // ---- LDS tile layouts -----------------------------------------------------------------------------
 // Row-major tile [rows][D] of bf16 with PAD elements of padding per row.
 //   PAD = 8  (16 bytes): 16 consecutive rows read at the same column with 16-byte reads land in 16 different

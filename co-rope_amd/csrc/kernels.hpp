@@ -20,7 +20,9 @@ struct FwdParams {
   int64_t fstride;   // elements between rows of the cos/sin tables
   float qk_scale;    // sm_scale * log2(e)
   int N;
-  int BH;            // batch * heads
+  int BH;            // batch * query heads
+  int H, Hkv;        // query heads and key/value heads per batch (grouped-query attention when Hkv < H; k, v, k_rot and
+                     // tile_kmax then have B * Hkv slabs and query head h reads key/value head h / (H / Hkv))
   int num_m_blocks;  // filled in by the launcher
 };
 
@@ -43,7 +45,8 @@ struct BwdParams {
   float sm_scale;
   float qk_scale;  // sm_scale * log2(e)
   int N;
-  int BH;
+  int BH;          // batch * query heads
+  int H, Hkv;      // as in FwdParams; dk, dv have B * Hkv slabs and sum over the query heads of their group
   int num_blocks;  // filled in by the launcher
 };
 

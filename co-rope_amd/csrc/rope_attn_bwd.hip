@@ -53,17 +53,18 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
   constexpr int LS = RowTile<D>::kStride, LSDO = RowTile<D, DO_PAD>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
-  const int bh = blockIdx.x % p.BH;
-  const int nb = blockIdx.x / p.BH;  // key block; for causal the low blocks are the heavy ones and start first
+  // The workgroup owns a key block of one key/value slab and sweeps the query tiles of every query head of its group
+  // (one head without grouped-query attention), accumulating dK and dV over all of them.
+  const int BHkv = p.BH / p.H * p.Hkv, GQ = p.H / p.Hkv;
+  const int bkv = blockIdx.x % BHkv;
+  const int nb = blockIdx.x / BHkv;  // key block; for causal the low blocks are the heavy ones and start first
   const int n0 = nb * Cfg::kBlockN;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int lq = lane % 32, lh = lane / 32;
   const int N = p.N;
-  const int64_t base = (int64_t)bh * N * D;
-  const uint16_t* qg = (PREROT ? p.q_rot : p.q) + base;
-  const uint16_t* dog = p.d_o + base;
-  const float* lseg = p.lse + (int64_t)bh * N;
-  const float* deltag = p.delta + (int64_t)bh * N;
+  const int64_t base = (int64_t)bkv * N * D;                           // k, v, dk, dv
+  const int q_slab0 = (bkv / p.Hkv) * p.H + (bkv % p.Hkv) * GQ;        // first query head of the group
+  const uint16_t* q_all = PREROT ? p.q_rot : p.q;
 
   const int key = n0 + wave * 32 + lq;
   const int key_c = min(key, N - 1);
@@ -79,20 +80,23 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
     vcp.store_rows(vrows);    // visible after the barrier that ends the prologue
   }
 
-  const int m_tiles = (N + BLOCK_M - 1) / BLOCK_M;
-  const int mt0 = CAUSAL ? n0 / BLOCK_M : 0;
-
   RopeStage<D, BLOCK_M, NT, PREROT> qst;
   CopyStage<D, BLOCK_M, NT, DO_PAD> dst;
   float st_lse = 0.f, st_delta = 0.f;
-  auto load_tile = [&](int m0) {
-    qst.load(qg, p.cos, p.sin, p.fstride, m0, N);
-    dst.load(dog, m0, N);
+  const int m_tiles = (N + BLOCK_M - 1) / BLOCK_M;
+  const int mt0 = CAUSAL ? n0 / BLOCK_M : 0;
+  const int tiles_per_head = max(m_tiles - mt0, 0), n_iter = GQ * tiles_per_head;
+  // iteration it -> query head q_slab0 + it / tiles_per_head, query tile mt0 + it % tiles_per_head
+  auto tile_m0 = [&](int it) { return (mt0 + it % tiles_per_head) * BLOCK_M; };
+  auto load_tile = [&](int it) {
+    const int qs = q_slab0 + it / tiles_per_head, m0 = tile_m0(it);
+    qst.load(q_all + (int64_t)qs * N * D, p.cos, p.sin, p.fstride, m0, N);
+    dst.load(p.d_o + (int64_t)qs * N * D, m0, N);
     if (threadIdx.x < BLOCK_M) {
       int qi = m0 + threadIdx.x;
       // rows past the end: M = +inf makes P = 0, so they contribute nothing
-      st_lse = qi < N ? lseg[qi] : INFINITY;
-      if constexpr (DO_DK) st_delta = qi < N ? deltag[qi] : 0.f;
+      st_lse = qi < N ? p.lse[(int64_t)qs * N + qi] : INFINITY;
+      if constexpr (DO_DK) st_delta = qi < N ? p.delta[(int64_t)qs * N + qi] : 0.f;
     }
   };
   auto q_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
@@ -119,17 +123,17 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
     if constexpr (DO_DK) dkacc[i] = f32x16{0};
   }
 
-  if (mt0 < m_tiles) {
-    load_tile(mt0 * BLOCK_M);
+  if (n_iter > 0) {
+    load_tile(0);
     store_tile(0);
   }
   __syncthreads();
 
   const float scale2 = p.qk_scale;
-  for (int mt = mt0; mt < m_tiles; ++mt) {
-    const int m0 = mt * BLOCK_M;
-    const int cur = (mt - mt0) & 1;
-    if (mt + 1 < m_tiles) load_tile(m0 + BLOCK_M);
+  for (int it = 0; it < n_iter; ++it) {
+    const int m0 = tile_m0(it);
+    const int cur = it & 1;
+    if (it + 1 < n_iter) load_tile(it + 1);
 
     const uint16_t* qs = q_tile(cur);
     const uint16_t* dos = do_tile(cur);
@@ -195,7 +199,7 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
         }
       }
     }
-    if (mt + 1 < m_tiles) store_tile(cur ^ 1);
+    if (it + 1 < n_iter) store_tile(cur ^ 1);
     __syncthreads();
   }
 
@@ -248,8 +252,9 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdPara
   const int lq = lane % 32, lh = lane / 32;
   const int N = p.N;
   const int64_t base = (int64_t)bh * N * D;
-  const uint16_t* kg = (PREROT ? p.k_rot : p.k) + base;
-  const uint16_t* vg = p.v + base;
+  const int64_t kv_base = (int64_t)kv_slab(bh, p.H, p.Hkv) * N * D;   // key/value slab of this query head
+  const uint16_t* kg = (PREROT ? p.k_rot : p.k) + kv_base;
+  const uint16_t* vg = p.v + kv_base;
 
   const int q_row = m0 + wave * 32 + lq;
   const int q_c = min(q_row, N - 1);
@@ -363,7 +368,7 @@ static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
     attr_set = true;
   }
   p.num_blocks = (p.N + Cfg::kBlockN - 1) / Cfg::kBlockN;
-  hipLaunchKernelGGL(kern, dim3(p.num_blocks * p.BH), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
+  hipLaunchKernelGGL(kern, dim3(p.num_blocks * (p.BH / p.H * p.Hkv)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
 }
 

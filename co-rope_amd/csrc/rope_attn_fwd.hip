@@ -122,8 +122,9 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
   const int N = p.N;
 
   const uint16_t* qg = p.q + (int64_t)bh * N * D;
-  const uint16_t* kg = p.k + (int64_t)bh * N * D;
-  const uint16_t* vg = p.v + (int64_t)bh * N * D;
+  const int kvs = kv_slab(bh, p.H, p.Hkv);   // key/value slab of this query head
+  const uint16_t* kg = p.k + (int64_t)kvs * N * D;
+  const uint16_t* vg = p.v + (int64_t)kvs * N * D;
 
   const int n_k_tiles = (N + BLOCK_N - 1) / BLOCK_N;
   const int n_tiles = CAUSAL ? min((m0 + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, n_k_tiles) : n_k_tiles;

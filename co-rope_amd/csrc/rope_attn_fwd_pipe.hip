@@ -103,8 +103,9 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
   const int N = p.N;
 
   const uint16_t* qg = p.q + (int64_t)bh * N * D;
-  const uint16_t* kg = p.k_rot + (int64_t)bh * N * D;
-  const uint16_t* vg = p.v + (int64_t)bh * N * D;
+  const int kvs = kv_slab(bh, p.H, p.Hkv);   // key/value slab of this query head
+  const uint16_t* kg = p.k_rot + (int64_t)kvs * N * D;
+  const uint16_t* vg = p.v + (int64_t)kvs * N * D;
 
   const int n_k_tiles = (N + BLOCK_N - 1) / BLOCK_N;
   const int n_tiles = CAUSAL ? min((m0 + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, n_k_tiles) : n_k_tiles;
@@ -139,7 +140,7 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
       }
     q_bound_wave = __builtin_sqrtf(wave_reduce_max(half_sum(ss))) * scale * 1.01f;
   }
-  const uint32_t* tile_kmax_bits = reinterpret_cast<const uint32_t*>(p.tile_kmax) + (int64_t)bh * n_k_tiles;
+  const uint32_t* tile_kmax_bits = reinterpret_cast<const uint32_t*>(p.tile_kmax) + (int64_t)kvs * n_k_tiles;
 
   f32x16 oacc[NDB];
 #pragma unroll

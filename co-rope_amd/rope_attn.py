@@ -24,7 +24,10 @@ def _check_inputs(q, k, v, freqs_cos, freqs_sin):
     assert q.dim() == 4 and k.dim() == 4 and v.dim() == 4, "q, k, v must be (B, H, N, D)"
     d = q.shape[-1]
     assert d == k.shape[-1] and d == v.shape[-1], "q, k, v must share the head dim"
-    assert q.shape == k.shape == v.shape, "q, k, v must share one shape"
+    # grouped-query attention (an extension: the reference requires one shape): k, v may have fewer heads
+    assert k.shape == v.shape, "k and v must share one shape"
+    assert q.shape[0] == k.shape[0] and q.shape[2:] == k.shape[2:], "q and k must agree in batch, sequence and head dim"
+    assert q.shape[1] % k.shape[1] == 0, "the number of query heads must be a multiple of the number of key/value heads"
     if d not in _SUPPORTED_D:
         raise ValueError(f"head dim {d} not built for gfx950 (supported: {_SUPPORTED_D})")
     if not (q.is_cuda and k.is_cuda and v.is_cuda and freqs_cos.is_cuda and freqs_sin.is_cuda):
@@ -74,8 +77,22 @@ def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, k
     if two_launch is None:
         two_launch = use_rotated_path(N, D, training=keep_rotated)
     rotated = None
+    Hkv = k.shape[1]
     with torch.cuda.device(q.device):
-        if two_launch and keep_rotated:
+        if Hkv != H:   # grouped-query attention: one entry point covers the three forms
+            q_rot = torch.empty_like(q) if (two_launch and keep_rotated) else None
+            k_rot = torch.empty_like(k) if two_launch else None
+            kmax = torch.empty((B, Hkv, (N + 63) // 64), device=q.device, dtype=torch.float32) if two_launch else None
+            rc = lib.corope_rope_attn_fwd_gqa(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
+                                              fc.stride(0), o.data_ptr(), M.data_ptr(),
+                                              q_rot.data_ptr() if q_rot is not None else None,
+                                              k_rot.data_ptr() if k_rot is not None else None,
+                                              kmax.data_ptr() if kmax is not None else None, B, H, Hkv, N, D,
+                                              float(sm_scale), int(bool(causal)), _stream_ptr(q))
+            _lib.check(rc, "corope_rope_attn_fwd_gqa")
+            if q_rot is not None:
+                rotated = (q_rot, k_rot)
+        elif two_launch and keep_rotated:
             q_rot, k_rot = torch.empty_like(q), torch.empty_like(k)
             kmax = torch.empty((B, H, (N + 63) // 64), device=q.device, dtype=torch.float32)
             rc = lib.corope_rope_attn_fwd_train(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
@@ -133,7 +150,12 @@ class _FusedRopeAttn(torch.autograd.Function):
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         delta = torch.empty_like(M)
         with torch.cuda.device(q.device):
-            if ctx.rotated:             # q, k are the rotated copies the forward kept
+            if k.shape[1] != H:         # grouped-query attention
+                rc = lib.corope_rope_attn_bwd_gqa(q.data_ptr(), k.data_ptr(), int(ctx.rotated), v.data_ptr(), o.data_ptr(),
+                                                  do.data_ptr(), M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(),
+                                                  fc.stride(0), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H,
+                                                  k.shape[1], N, D, ctx.sm_scale, int(ctx.causal), _stream_ptr(q))
+            elif ctx.rotated:           # q, k are the rotated copies the forward kept
                 rc = lib.corope_rope_attn_bwd_prerotated(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                                          do.data_ptr(), M.data_ptr(), delta.data_ptr(), fc.data_ptr(),
                                                          fs.data_ptr(), fc.stride(0), dq.data_ptr(), dk.data_ptr(),

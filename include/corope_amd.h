@@ -194,6 +194,24 @@ int corope_rope_attn_bwd_ws(const void *q, const void *k, const void *v, const v
                             int B, int H, int N, int D, float sm_scale, int causal,
                             void *workspace, int64_t workspace_bytes, void *stream);
 
+/* Grouped-query form of the operator: q (B,Hq,N,D), k and v (B,Hkv,N,D), Hq a multiple of Hkv; query head h reads
+ * key/value head h / (Hq/Hkv); dk and dv (B,Hkv,N,D) are sums over the query heads of their group (the key block's
+ * workgroup sweeps all of them, no atomics).  The reference's RoPE operator requires Hq == Hkv
+ * (fused-rope/fused_rope_attn.py:657-661); the indexing follows its plain attention tutorial and the group
+ * reduction its archived GQA experiment (assets/flashattn-gqa/triton_gqa.py:605-666).
+ * forward: k_rot NULL = single launch (q_rot and tile_kmax must be NULL too); otherwise K is rotated into k_rot
+ * (B,Hkv,N,D) with tile_kmax (B*Hkv*ceil(N/64) floats, scratch) and q_rot (may be NULL) receives the rotated q.
+ * backward: prerotated != 0 means q and k are those rotated copies (fused dK+dV kernel); delta (B,Hq,N) is scratch. */
+int corope_rope_attn_fwd_gqa(const void *q, const void *k, const void *v,
+                             const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                             void *o, float *lse, void *q_rot, void *k_rot, float *tile_kmax,
+                             int B, int Hq, int Hkv, int N, int D, float sm_scale, int causal, void *stream);
+int corope_rope_attn_bwd_gqa(const void *q, const void *k, int prerotated, const void *v, const void *o, const void *d_o,
+                             const float *lse, float *delta,
+                             const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                             void *dq, void *dk, void *dv,
+                             int B, int Hq, int Hkv, int N, int D, float sm_scale, int causal, void *stream);
+
 /* Co-RoPE grouped-query attention forward (causal only).
  * q: (B,Hq,N,D), k/v: (B,Hkv,N,D), o: (B,Hq,N,D), group size Hq/Hkv in [1, 8].
  * Replaces the launch of _corope_fwd_backbone in _attention.forward

@@ -90,6 +90,22 @@ def test_null_and_misaligned_pointers_are_rejected_before_any_launch(pkg):
         pkg._lib.check(rc, "corope_gqa_fwd")
 
 
+def test_grouped_query_argument_checks(pkg):
+    """Head-count and pointer checks of the grouped-query entry points happen before any launch."""
+    lib = pkg._lib.load()
+    ok = 4096
+    rc = lib.corope_rope_attn_fwd_gqa(ok, ok, ok, ok, ok, 64, ok, ok, None, None, None, 1, 6, 4, 8, 64, 1.0, 1, None)
+    assert rc == -1 and "multiple" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_fwd_gqa(ok, ok, ok, ok, ok, 64, ok, ok, ok, None, None, 1, 8, 2, 8, 64, 1.0, 1, None)
+    assert rc == -1 and "q_rot without k_rot" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_fwd_gqa(ok, ok, ok, ok, ok, 64, ok, ok, None, ok, None, 1, 8, 2, 8, 64, 1.0, 1, None)
+    assert rc == -1 and "tile_kmax" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_bwd_gqa(ok, ok, 1, ok, ok, ok, ok, ok, ok, ok, 64, ok, ok, ok, 1, 8, 3, 8, 64, 1.0, 1, None)
+    assert rc == -1 and "multiple" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_bwd_gqa(ok, ok, 1, ok, ok, ok, ok, ok, ok, ok, 64, ok, None, ok, 1, 8, 2, 8, 64, 1.0, 1, None)
+    assert rc == -1 and "null" in pkg._lib.last_error()
+
+
 def test_rope_freqs_argument_checks(pkg):
     lib = pkg._lib.load()
     buf = ctypes.create_string_buffer(4096)

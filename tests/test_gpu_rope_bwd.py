@@ -134,3 +134,29 @@ def test_forward_keeps_rotated_operands(pkg):
     torch.cuda.synchronize()
     assert torch.equal(rot[0], pkg.rope_rotate(qd, cd, sd)) and torch.equal(rot[1], pkg.rope_rotate(kd, cd, sd))
     assert torch.equal(o, o2) and torch.equal(M, M2)
+
+
+@pytest.mark.parametrize("two_launch", [False, True])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,Hq,Hkv,N,D", [(1, 8, 2, 320, 128), (2, 4, 1, 200, 64), (1, 6, 3, 1024, 128), (1, 4, 4, 130, 64)])
+def test_grouped_query_parity(pkg, monkeypatch, B, Hq, Hkv, N, D, causal, two_launch):
+    """Grouped-query form (k, v with fewer heads): forward and all three gradients against the oracle run on k, v repeated
+    over their groups, with dK, dV summed back over the group (the definition of sharing a key/value head)."""
+    print(f"case gqa B={B} Hq={Hq} Hkv={Hkv} N={N} D={D} causal={causal} two_launch={two_launch}", flush=True)
+    _force_path(monkeypatch, pkg, two_launch)
+    G = Hq // Hkv
+    q, g = (bf16_round(seeded((B, Hq, N, D), 50 + i)) for i in range(2))
+    k, v = (bf16_round(seeded((B, Hkv, N, D), 60 + i)) for i in range(2))
+    c, s = O.precompute_freqs_cis(D, N)
+    scale = 1 / math.sqrt(D)
+    o, dq, dk, dv = _gpu_fwd_bwd(pkg, q, k, v, g, causal, scale, c, s)
+    kx, vx = k.repeat_interleave(G, dim=1), v.repeat_interleave(G, dim=1)
+    ro, _, rdq, rdk, rdv, _ = O.rope_attn_fwd_bwd_blocked(q, kx, vx, g, causal, scale, c, s)
+    rdk, rdv = (t.reshape(B, Hkv, G, N, D).sum(2) for t in (rdk, rdv))
+    for name, a, b in (("O", o, ro), ("dQ", dq, rdq), ("dK", dk, rdk), ("dV", dv, rdv)):
+        err = (a - b).abs()
+        print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
+        assert a.shape == b.shape and torch.isfinite(a).all(), name
+        # dK, dV are sums of G per-head gradients whose bf16 rounding errors (rotated operands, P, dS) are independent:
+        # the per-tensor bar scales with sqrt(G) for them
+        assert within_bar(a, b, TOL * (math.sqrt(G) if name in ("dK", "dV") else 1.0))[0], name
