@@ -291,19 +291,20 @@ def main():
         launches = [("rope_attn_fwd", lambda: lib.corope_rope_attn_fwd(qp, kp, vp, cp, sp, fs, o.data_ptr(), M.data_ptr(),
                                                                       B, H, N, D, scale, 1, stream))]
     if not fwd_only:
-        launches += [("rope_attn_bwd_preprocess", lambda: lib.corope_rope_attn_bwd_preprocess(
-            o.data_ptr(), dop, delta.data_ptr(), B, H, N, D, stream))]
-        if rotated:   # the backward the operator takes at this shape: on the rotated q, k
-            qr, kr = q_rot.data_ptr(), k_rot.data_ptr()   # which the forward kept
+        if rotated:   # the backward the operator takes at this shape: on the rotated q, k the forward kept; the dQ kernel
+            qr, kr = q_rot.data_ptr(), k_rot.data_ptr()   # computes delta on its way, the fused dK+dV kernel follows
             launches += [
+                ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq_prerotated(
+                    qr, kr, vp, o.data_ptr(), dop, M.data_ptr(), delta.data_ptr(), cp, sp, fs, dq.data_ptr(), B, H, N, D,
+                    scale, 1, stream)),
                 ("rope_attn_bwd_dkdv", lambda: lib.corope_rope_attn_bwd_dkdv_prerotated(
                     qr, kr, vp, dop, M.data_ptr(), delta.data_ptr(), cp, sp, fs, dk.data_ptr(), dv.data_ptr(), B, H, N, D,
                     scale, 1, stream)),
-                ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq_prerotated(
-                    qr, kr, vp, dop, M.data_ptr(), delta.data_ptr(), cp, sp, fs, dq.data_ptr(), B, H, N, D, scale, 1, stream)),
             ]
         else:
             launches += [
+                ("rope_attn_bwd_preprocess", lambda: lib.corope_rope_attn_bwd_preprocess(
+                    o.data_ptr(), dop, delta.data_ptr(), B, H, N, D, stream)),
                 ("rope_attn_bwd_dv", lambda: lib.corope_rope_attn_bwd_dv(qp, kp, dop, M.data_ptr(), cp, sp, fs, dv.data_ptr(),
                                                                         B, H, N, D, scale, 1, stream)),
                 ("rope_attn_bwd_dk", lambda: lib.corope_rope_attn_bwd_dk(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),

@@ -267,14 +267,17 @@ int bwd_dk_impl(const char* what, bool prerot, const void* q, const void* k, con
   return launch_status(what, corope::launch_bwd_dk(p, D, causal != 0, static_cast<hipStream_t>(stream)));
 }
 
+// o non-null: the kernel computes delta from o and d_o for its rows and WRITES it to `delta`.
 int bwd_dq_impl(const char* what, bool prerot, const void* q, const void* k, const void* v, const void* d_o,
                 const float* lse, const float* delta, const float* freqs_cos, const float* freqs_sin,
-                int64_t freq_row_stride, void* dq, int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
+                int64_t freq_row_stride, void* dq, int B, int H, int N, int D, float sm_scale, int causal, void* stream,
+                const void* o = nullptr) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
   rc = check_ptrs(what, {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dq});
   if (rc) return rc;
-  corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
+  if (o != nullptr && !aligned16(o)) return fail(COROPE_E_ALIGN, "%s: pointer %p is not 16-byte aligned", what, o);
+  corope::BwdParams p = make_bwd(q, k, v, o, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
                                  freq_row_stride, dq, nullptr, nullptr, B, H, N, sm_scale);
   mark_prerotated(p, prerot);
   return launch_status(what, corope::launch_bwd_dq(p, D, causal != 0, static_cast<hipStream_t>(stream)));
@@ -350,12 +353,12 @@ int corope_rope_attn_bwd_dkdv_prerotated(const void* q_rot, const void* k_rot, c
   return launch_status(what, corope::launch_bwd_dkdv_fused(p, D, causal != 0, static_cast<hipStream_t>(stream)));
 }
 
-int corope_rope_attn_bwd_dq_prerotated(const void* q_rot, const void* k_rot, const void* v, const void* d_o,
-                                       const float* lse, const float* delta, const float* freqs_cos,
-                                       const float* freqs_sin, int64_t freq_row_stride, void* dq, int B, int H, int N,
-                                       int D, float sm_scale, int causal, void* stream) {
+int corope_rope_attn_bwd_dq_prerotated(const void* q_rot, const void* k_rot, const void* v, const void* o, const void* d_o,
+                                       const float* lse, float* delta, const float* freqs_cos, const float* freqs_sin,
+                                       int64_t freq_row_stride, void* dq, int B, int H, int N, int D, float sm_scale,
+                                       int causal, void* stream) {
   return bwd_dq_impl("rope_attn_bwd_dq_prerotated", true, q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin,
-                     freq_row_stride, dq, B, H, N, D, sm_scale, causal, stream);
+                     freq_row_stride, dq, B, H, N, D, sm_scale, causal, stream, o);
 }
 
 int corope_rope_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
@@ -375,13 +378,15 @@ int corope_rope_attn_bwd_prerotated(const void* q_rot, const void* k_rot, const 
                                     const float* lse, float* delta, const float* freqs_cos, const float* freqs_sin,
                                     int64_t freq_row_stride, void* dq, void* dk, void* dv, int B, int H, int N, int D,
                                     float sm_scale, int causal, void* stream) {
-  int rc = corope_rope_attn_bwd_preprocess(o, d_o, delta, B, H, N, D, stream);
+  // two launches: the dQ kernel computes delta for the rows it owns on its way (no separate pass over o and dO), the
+  // fused dK+dV kernel reads it afterwards
+  int rc = check_ptrs("rope_attn_bwd_prerotated", {o});
   if (rc) return rc;
-  rc = corope_rope_attn_bwd_dkdv_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dk,
-                                            dv, B, H, N, D, sm_scale, causal, stream);
+  rc = corope_rope_attn_bwd_dq_prerotated(q_rot, k_rot, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, B,
+                                          H, N, D, sm_scale, causal, stream);
   if (rc) return rc;
-  return corope_rope_attn_bwd_dq_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq,
-                                            B, H, N, D, sm_scale, causal, stream);
+  return corope_rope_attn_bwd_dkdv_prerotated(q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dk,
+                                              dv, B, H, N, D, sm_scale, causal, stream);
 }
 
 int64_t corope_rope_attn_bwd_workspace_bytes(int B, int H, int N, int D) {

@@ -272,7 +272,24 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdPara
   load_b_rows<D, !PREROT>(qb, (PREROT ? p.q_rot : p.q) + base, p.cos, p.sin, p.fstride, q_c);
   load_b_rows<D, false>(dob, p.d_o + base, nullptr, nullptr, 0, q_c);
   const float lse_q = p.lse[(int64_t)bh * N + q_c];
-  const float delta_q = p.delta[(int64_t)bh * N + q_c];
+  // delta_i = sum_d o_id * do_id (reference _attn_bwd_preprocess, :324-337): read from the preprocess pass, or -- when the
+  // caller hands over O instead -- computed here for the rows this workgroup owns and written out for the dK kernel,
+  // which then has to run after this one.
+  float delta_q;
+  if (p.o != nullptr) {
+    u32x4 ob[KC];
+    load_b_rows<D, false>(ob, p.o + base, nullptr, nullptr, 0, q_c);
+    float acc = 0.f;
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
+        acc += bf16_lo(ob[kc][w]) * bf16_lo(dob[kc][w]) + bf16_hi(ob[kc][w]) * bf16_hi(dob[kc][w]);
+    delta_q = half_sum(acc);
+    if (lh == 0 && q_row < N) p.delta[(int64_t)bh * N + q_row] = delta_q;
+  } else {
+    delta_q = p.delta[(int64_t)bh * N + q_c];
+  }
 
   auto k_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
   auto v_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes + Cfg::kTileBytes); };

@@ -150,7 +150,9 @@ int corope_rope_attn_bwd(const void *q, const void *k, const void *v, const void
  * kernels then read no cos/sin tables in their inner loops (the tables are still needed once per output row, to
  * rotate dK and dQ back).  Same results as the plain entry points (the rotated copies are rounded to bf16 exactly
  * as the kernels round them when they rotate a tile themselves).  Reference sites as for corope_rope_attn_bwd_dv,
- * _dk and _dq. */
+ * _dk and _dq.  The dQ entry point takes o as well: NULL = delta is read (from the preprocess pass); non-NULL = delta is
+ * computed from o and d_o for the rows each workgroup owns and WRITTEN to `delta`, which replaces the preprocess pass
+ * (reference :324-337) when this launch comes before the dK launch. */
 int corope_rope_attn_bwd_dv_prerotated(const void *q_rot, const void *k_rot, const void *d_o, const float *lse,
                                        const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
                                        void *dv,
@@ -168,8 +170,8 @@ int corope_rope_attn_bwd_dkdv_prerotated(const void *q_rot, const void *k_rot, c
                                          const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
                                          void *dk, void *dv,
                                          int B, int H, int N, int D, float sm_scale, int causal, void *stream);
-int corope_rope_attn_bwd_dq_prerotated(const void *q_rot, const void *k_rot, const void *v, const void *d_o,
-                                       const float *lse, const float *delta,
+int corope_rope_attn_bwd_dq_prerotated(const void *q_rot, const void *k_rot, const void *v, const void *o,
+                                       const void *d_o, const float *lse, float *delta,
                                        const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
                                        void *dq,
                                        int B, int H, int N, int D, float sm_scale, int causal, void *stream);

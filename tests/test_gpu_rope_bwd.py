@@ -97,7 +97,9 @@ def test_backward_deterministic(pkg):
 
 def test_backward_paths_agree(pkg, monkeypatch):
     """The rotated copies are rounded exactly as the kernels round the tiles they rotate themselves, and the backward
-    kernels do the same arithmetic on them: gradients of the two paths are identical bit for bit (given one O, M)."""
+    kernels do the same arithmetic on them: given one O and M, dV of the two paths is identical bit for bit.  dQ and dK
+    also depend on delta = rowsum(O o dO), which the rotated-operand path sums inside the dQ kernel in another order than
+    the preprocess pass: they agree to the last bit or two of that fp32 sum, i.e. to one bf16 ulp after rounding."""
     B, H, N, D = 1, 2, 320, 128
     q, k, v, g, c, s = _case(B, H, N, D, seed=3)
     dev = torch.device("cuda:0")
@@ -111,7 +113,11 @@ def test_backward_paths_agree(pkg, monkeypatch):
         torch.cuda.synchronize()
         grads.append([t.grad.float().cpu() for t in (qd, kd, vd)])
     for a, b, name in zip(grads[0], grads[1], ("dQ", "dK", "dV")):
-        assert torch.equal(a, b), name
+        if name == "dV":
+            assert torch.equal(a, b), name
+        else:
+            # (row 0 of dQ is analytically zero: dp - delta is pure rounding noise there, hence the absolute term)
+            assert ((a - b).abs() <= 1e-5 + a.abs() / 128).all() and (a == b).float().mean() > 0.98, name
     # third path: the forward keeps its rotated q and k and the backward runs on them (another forward kernel, so O and
     # M differ in the last bit and the gradients agree to rounding, not bit for bit)
     _force_path(monkeypatch, pkg, True)
