@@ -35,10 +35,9 @@ SUSTAINED_BF16_TFLOPS = 1520.0
 # benchmark (summary and commands: profiles/rope_attn_c3_hbm_traffic.md); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE
 # by 1.0, the factors a plain 1 GiB device copy gives for the same counters.
 HBM_TRAFFIC_BYTES = {
-    ("c3", "rope_attn_fwd"): int((259785 * 2.0 + 132101) * 1024),
-    ("c3", "rope_attn_bwd_dv"): int((205670 * 2.0 + 65538) * 1024),
-    ("c3", "rope_attn_bwd_dk"): int((272134 * 2.0 + 65573) * 1024),
-    ("c3", "rope_attn_bwd_dq"): int((306059 * 2.0 + 65562) * 1024),
+    ("c3", "rope_attn_fwd"): int((252746 * 2.0 + 132101) * 1024),
+    ("c3", "rope_attn_bwd_dq"): int((330591 * 2.0 + 66565) * 1024),
+    ("c3", "rope_attn_bwd_dkdv"): int((285381 * 2.0 + 137995) * 1024),
 }
 
 CONFIGS = {
