@@ -222,8 +222,8 @@ def main():
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        sys.exit("bench.py: this build runs on ONE GPU (every (batch, head) is independent; see DESIGN.md for how "
-                 "the path would shard); run it with --gpus 1")
+        sys.exit("bench.py: this build runs on ONE GPU (every (batch, head) is independent, so the path would shard over "
+                 "batch x heads without any exchange); run it with --gpus 1")
 
     if args.copy_calibration:
         import torch

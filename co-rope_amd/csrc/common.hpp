@@ -1,5 +1,5 @@
 // Shared device helpers for the gfx950 kernels: vector types, bf16 packing, MFMA wrappers,
-// wave-half exchange and the global->register->LDS staging of rotated / transposed tiles.
+// wave-half exchange, the global->register->LDS staging of rotated / copied tiles and the transposing LDS read.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -44,15 +44,6 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 __device__ __forceinline__ constexpr int acc_row(int i, int h) { return 8 * (i / 4) + 4 * h + (i % 4); }
 
 // ---- exchange between the two 32-lane halves of a wave ---------------------------------------------
-// Returns the value held by lane (l ^ 32).
-__device__ __forceinline__ float other_half(float x) {
-  uint32_t u = __builtin_bit_cast(uint32_t, x);
-  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  // r[0] = {x.lo, x.lo}, r[1] = {x.hi, x.hi} over (lanes 0-31, lanes 32-63)
-  uint32_t mine_is_lo = (threadIdx.x & 32) == 0;
-  uint32_t o = mine_is_lo ? r[1] : r[0];
-  return __builtin_bit_cast(float, o);
-}
 __device__ __forceinline__ float half_max(float x) {
   uint32_t u = __builtin_bit_cast(uint32_t, x);
   auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
@@ -95,21 +86,6 @@ struct RowTile {
   __device__ static __forceinline__ int off(int row, int col) { return row * kStride + col; }
 };
 
-// Transposed tile [D][COLS] of bf16 (the contraction index runs along a row), 16 bytes of padding.
-// Within every group of 16 columns the order is permuted (bits 2 and 3 of the column index swapped) so
-// that the 8 contraction slots an MFMA B-operand built from a 32x32 accumulator expects from lane-half h,
-//   slot j  <->  column 8*(j / 4) + 4*h + (j % 4),
-// are the 8 consecutive elements [8h, 8h+8) of the group: one 16-byte LDS read per MFMA A operand.
-template <int COLS>
-struct TransTile {
-  static constexpr int kStride = COLS + 8;  // elements
-  static constexpr int bytes(int rows) { return rows * kStride * 2; }
-  __device__ static __forceinline__ int pos(int col) {
-    return (col & ~12) | ((col & 4) << 1) | ((col & 8) >> 1);
-  }
-  __device__ static __forceinline__ int off(int d, int col) { return d * kStride + pos(col); }
-};
-
 // ---- staging: a ROWS x D tile with the half-layout rotation applied on the way -----------------------
 // Work unit = one row x 8 rotation pairs: columns [8c, 8c+8) and [D/2 + 8c, D/2 + 8c + 8) of the same row
 // are loaded by the same thread, so the rotation is thread-local.  cos/sin come from fp32 tables of which
@@ -144,45 +120,6 @@ struct RotStage {
     }
   }
 
-  // Loads iterations [it0, it1) only (same addressing as load()).
-  __device__ __forceinline__ void load_part(int it0, int it1, const uint16_t* __restrict__ src,
-                                            const float* __restrict__ cosp, const float* __restrict__ sinp,
-                                            int64_t fstride, int row0, int n_rows) {
-#pragma unroll
-    for (int it = 0; it < kIters; ++it) {
-      if (it < it0 || it >= it1) continue;
-      int u = threadIdx.x + it * NT;
-      if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
-      int r = u / kChunks, ch = u % kChunks;
-      int row = min(row0 + r, n_rows - 1);
-      const uint16_t* p = byte_offset(src, (uint32_t)row * (D * 2) + ch * 16);
-      x1[it] = *reinterpret_cast<const u32x4*>(p);
-      x2[it] = *reinterpret_cast<const u32x4*>(p + D / 2);
-      const uint32_t foff = ((uint32_t)row * (uint32_t)fstride + ch * 8) * 4;
-      const float* cp = byte_offset(cosp, foff);
-      const float* sp = byte_offset(sinp, foff);
-      c[it][0] = *reinterpret_cast<const f32x4*>(cp);
-      c[it][1] = *reinterpret_cast<const f32x4*>(cp + 4);
-      s[it][0] = *reinterpret_cast<const f32x4*>(sp);
-      s[it][1] = *reinterpret_cast<const f32x4*>(sp + 4);
-    }
-  }
-
-  // Rotates and stores iterations [it0, it1) only.
-  __device__ __forceinline__ void store_rows_part(int it0, int it1, uint16_t* lds) const {
-#pragma unroll
-    for (int it = 0; it < kIters; ++it) {
-      if (it < it0 || it >= it1) continue;
-      int u = threadIdx.x + it * NT;
-      if (kUnits % NT != 0 && u >= kUnits) continue;
-      int r = u / kChunks, ch = u % kChunks;
-      u32x4 y1, y2;
-      rotate(it, y1, y2);
-      *reinterpret_cast<u32x4*>(lds + RowTile<D>::off(r, ch * 8)) = y1;
-      *reinterpret_cast<u32x4*>(lds + RowTile<D>::off(r, D / 2 + ch * 8)) = y2;
-    }
-  }
-
   // Rotates unit `it`: y1 = x1 c - x2 s, y2 = x2 c + x1 s (fp32), rounds to bf16.
   __device__ __forceinline__ void rotate(int it, u32x4& y1, u32x4& y2) const {
 #pragma unroll
@@ -211,63 +148,6 @@ struct RotStage {
   }
 };
 
-// ---- staging: a ROWS x D tile written transposed ([D][ROWS], permuted columns) -----------------------
-// Work unit = 4 rows x 4 columns (four 8-byte global loads), written as four 8-byte LDS rows.
-// Unit u -> dl = u % 4, row group = (u / 4) % (ROWS / 4), dhi = u / ROWS: within a half wave the LDS
-// writes touch every bank once.
-template <int D, int ROWS, int NT>
-struct TransStage {
-  static constexpr int kUnits = ROWS * D / 16;
-  static constexpr int kIters = (kUnits + NT - 1) / NT;
-  static_assert(kUnits % NT == 0 || kIters == 1, "tile/thread shape");
-  u32x2 x[kIters][4];
-
-  __device__ static __forceinline__ void unit(int u, int& rg, int& d0) {
-    int dl = u % 4;
-    rg = (u / 4) % (ROWS / 4);
-    d0 = 4 * (dl + 4 * (u / ROWS));
-  }
-
-  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, int row0, int n_rows) {
-#pragma unroll
-    for (int it = 0; it < kIters; ++it) {
-      int u = threadIdx.x + it * NT;
-      if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
-      int rg, d0;
-      unit(u, rg, d0);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int row = min(row0 + 4 * rg + j, n_rows - 1);
-        x[it][j] = *reinterpret_cast<const u32x2*>(src + (int64_t)row * D + d0);
-      }
-    }
-  }
-
-  __device__ __forceinline__ void store(uint16_t* lds) const {
-#pragma unroll
-    for (int it = 0; it < kIters; ++it) {
-      int u = threadIdx.x + it * NT;
-      if (kUnits % NT != 0 && u >= kUnits) continue;
-      int rg, d0;
-      unit(u, rg, d0);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        // column e of the 4x4 block: rows j = 0..3 packed into 8 bytes
-        uint32_t w0 = x[it][0][e / 2], w1 = x[it][1][e / 2], w2 = x[it][2][e / 2], w3 = x[it][3][e / 2];
-        u32x2 o;
-        if (e % 2 == 0) {
-          o[0] = (w0 & 0xffffu) | (w1 << 16);
-          o[1] = (w2 & 0xffffu) | (w3 << 16);
-        } else {
-          o[0] = (w0 >> 16) | (w1 & 0xffff0000u);
-          o[1] = (w2 >> 16) | (w3 & 0xffff0000u);
-        }
-        *reinterpret_cast<u32x2*>(lds + TransTile<ROWS>::off(d0 + e, 4 * rg)) = o;
-      }
-    }
-  }
-};
-
 // ---- staging: a ROWS x D tile copied row-major (no rotation) -------------------------------------------
 template <int D, int ROWS, int NT, int PAD = 8>
 struct CopyStage {
@@ -288,26 +168,6 @@ struct CopyStage {
   __device__ __forceinline__ void store_rows(uint16_t* lds) const {
 #pragma unroll
     for (int it = 0; it < kIters; ++it) {
-      int u = threadIdx.x + it * NT;
-      if (kUnits % NT != 0 && u >= kUnits) continue;
-      *reinterpret_cast<u32x4*>(lds + RowTile<D, PAD>::off(u / kChunks, (u % kChunks) * 8)) = x[it];
-    }
-  }
-  // Iterations [it0, it1) only.
-  __device__ __forceinline__ void load_part(int it0, int it1, const uint16_t* __restrict__ src, int row0, int n_rows) {
-#pragma unroll
-    for (int it = 0; it < kIters; ++it) {
-      if (it < it0 || it >= it1) continue;
-      int u = threadIdx.x + it * NT;
-      if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
-      int row = min(row0 + u / kChunks, n_rows - 1);
-      x[it] = *reinterpret_cast<const u32x4*>(byte_offset(src, (uint32_t)row * (D * 2) + (u % kChunks) * 16));
-    }
-  }
-  __device__ __forceinline__ void store_rows_part(int it0, int it1, uint16_t* lds) const {
-#pragma unroll
-    for (int it = 0; it < kIters; ++it) {
-      if (it < it0 || it >= it1) continue;
       int u = threadIdx.x + it * NT;
       if (kUnits % NT != 0 && u >= kUnits) continue;
       *reinterpret_cast<u32x4*>(lds + RowTile<D, PAD>::off(u / kChunks, (u % kChunks) * 8)) = x[it];
