@@ -146,6 +146,7 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
 #pragma unroll
   for (int i = 0; i < NDB; ++i) oacc[i] = f32x16{0};
   float m_run = -INFINITY;   // reference maximum of the raw scores (this lane's query)
+  float m_true = -INFINITY;  // largest raw score seen by the reference moves (at most the row's true running maximum)
   float l_run = 0.f;         // this lane's share of the denominator up to the last move of the reference
   float lsum = 0.f;          // ... and since then
   f32x16 s1;                 // scores of the second half of the previous tile (softmax half done)
@@ -307,12 +308,13 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
       float mt = fmaxf(r0[0], r1[0]);
 #pragma unroll
       for (int i = 1; i < 16; ++i) mt = fmaxf(fmaxf(mt, r0[i]), r1[i]);
-      float m_new = fmaxf(m_run, half_max(mt));
       // Lift the reference towards the largest bound any later tile of this wave can show, so that the test above does
       // not fire again (with the Cauchy-Schwarz bound 2-3x above the scores actually seen, hot logits would otherwise
-      // send most tiles through this block).  Never further than kPipeLift above the true maximum: the row's largest
-      // probability stays above 2^-kPipeLift, far inside fp32 / bf16 range.
-      m_new = fmaxf(m_new, fminf(lift_target, m_new + kPipeLift / scale));
+      // send most tiles through this block).  Never further than kPipeLift above the largest score actually seen in
+      // this block so far (m_true, a lower bound of the row's running maximum): the row's largest probability stays
+      // above 2^-kPipeLift, far inside fp32 / bf16 range, however often the block runs.
+      m_true = fmaxf(m_true, half_max(mt));
+      const float m_new = fmaxf(m_run, fmaxf(m_true, fminf(lift_target, m_true + kPipeLift / scale)));
       const float alpha = fast_exp2((m_run - m_new) * scale);   // m_new is finite: every row sees key 0 of tile 0
       l_run = (l_run + lsum) * alpha;
       lsum = 0.f;

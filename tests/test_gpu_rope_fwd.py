@@ -145,7 +145,7 @@ def test_rotate_pass_matches_the_oracle(pkg):
 
 
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("case", ["large_norms", "outlier_keys", "growing_scores", "tiny_scores"])
+@pytest.mark.parametrize("case", ["large_norms", "outlier_keys", "growing_scores", "tiny_scores", "huge_norms_hot"])
 def test_two_launch_softmax_modes(pkg, case, causal):
     """Inputs that push tiles of the two-launch forward onto each of its softmax modes: the per-tile score bound
     (query norm x largest key norm of the tile) decides, so large norms, a few huge keys, and scores that keep
@@ -164,6 +164,10 @@ def test_two_launch_softmax_modes(pkg, case, causal):
         k = bf16_round(k * ramp)
     elif case == "tiny_scores":
         q, k = bf16_round(q * 1e-3), bf16_round(k * 1e-3)
+    elif case == "huge_norms_hot":
+        # logits with a standard deviation of ~18 nats and a norm bound ~120 nats above the largest logit: the reference
+        # has to move on most tiles and must not be lifted out of reach of the scores that actually occur
+        q, k, scale = bf16_round(q * 1.8), bf16_round(k * 1.8), 0.5
     c, s = O.precompute_freqs_cis(D, N)
     print(f"case modes {case} causal={causal}", flush=True)
     o, M = _run(pkg, q, k, v, causal, scale, c, s, True)
@@ -174,8 +178,13 @@ def test_two_launch_softmax_modes(pkg, case, causal):
         print(f"  {name}: O max-abs {err.max():.3e} mean-abs {err.mean():.3e} LSE {(lse * LN2 - rl).abs().max():.3e}")
         assert torch.isfinite(got).all()
         # sharp softmaxes amplify the bf16 rounding of the rotated operands: a looser max bound, a tight mean bound
-        assert err.max() <= TOL_HOT and err.mean() <= 5e-3
-        assert ((lse * LN2 - rl).abs() <= 2e-2 + rl.abs() / 128).all()
+        # (logits with an 18-nat spread turn the bf16 rounding of the rotated operands, ~0.2 nats there, straight into
+        # 20 % changes of single probabilities: that case only has to stay finite and near the oracle on average)
+        hot = case == "huge_norms_hot"
+        assert err.max() <= (0.5 if hot else TOL_HOT) and err.mean() <= (1e-2 if hot else 5e-3)
+        assert ((lse * LN2 - rl).abs() <= (0.3 if hot else 2e-2) + rl.abs() / 128).all()
     # both paths round the rotated operands identically; only the softmax bookkeeping differs between them (P is rounded
     # to bf16 relative to different reference maxima), which can flip the bf16 rounding of an output: one ulp of slack
-    assert ((o - o1).abs() <= 5e-3 + o.abs() / 64).all() and (M - M1).abs().max() * LN2 <= 1e-3
+    print(f"  paths: O max-abs diff {(o - o1).abs().max():.3e}, M max-abs diff {(M - M1).abs().max():.3e}")
+    hot = case == "huge_norms_hot"
+    assert ((o - o1).abs() <= (3e-2 if hot else 5e-3) + o.abs() / 64).all() and (M - M1).abs().max() * LN2 <= (1e-2 if hot else 1e-3)
