@@ -2,9 +2,10 @@
 
 ``attention(q, k, v, causal, sm_scale, theta[, warp_specialize])`` mirrors the reference's
 ``_attention.apply`` (corope-exp/flash_attn_co_rope_gqa_triton.py:403-456, :580), including its validation
-errors (:407-425).  The forward is a hand-written gfx950 kernel reached through the C ABI.  The reference's own
-"fused" operator falls back to a dense PyTorch backward (:459-577); that backward is not part of this library yet,
-so differentiating through this operator raises."""
+errors (:407-425).  Forward and backward are hand-written gfx950 kernels reached through the C ABI.  The reference's
+own "fused" operator falls back to a dense PyTorch backward with (B, Hq, N, N, D/2) temporaries (:459-577); the
+backward here produces the same gradients from q, k, v and dO with N*N fp32 scalars per head of scratch memory
+(``backward_workspace_bytes`` says how much)."""
 from __future__ import annotations
 
 import torch
@@ -41,14 +42,47 @@ class _CoRopeGqaAttn(torch.autograd.Function):
             rc = lib.corope_gqa_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, Hq, Hkv, N, D,
                                     float(sm_scale), float(theta), torch.cuda.current_stream(q.device).cuda_stream)
         _lib.check(rc, "corope_gqa_fwd")
+        ctx.save_for_backward(q, k, v)   # what the reference keeps (:451), minus inv_freq: theta is enough
         ctx.group_size = Hq // Hkv
         ctx.sm_scale = sm_scale
+        ctx.theta = theta
         ctx.causal = causal
         return o
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("Co-RoPE GQA backward is not provided by the gfx950 library")
+        q, k, v = ctx.saved_tensors
+        dq, dk, dv = corope_gqa_backward(q, k, v, grad_output, ctx.sm_scale, ctx.theta)
+        return dq, dk, dv, None, None, None, None
+
+
+def backward_workspace_bytes(B, Hq, Hkv, N, D):
+    """Scratch memory the backward needs: (3 * B * Hkv + 2 * B * Hq) * N * N fp32 values."""
+    n = _lib.load().corope_gqa_bwd_workspace_bytes(B, Hq, Hkv, N, D)
+    if n < 0:
+        raise ValueError(_lib.last_error() or "unsupported Co-RoPE shape")
+    return n
+
+
+def corope_gqa_backward(q, k, v, grad_output, sm_scale, theta, workspace=None):
+    """(dq, dk, dv) of the Co-RoPE GQA attention for upstream gradient ``grad_output`` (reference :459-577).
+
+    ``workspace`` may be a caller-owned uint8/float tensor of at least ``backward_workspace_bytes`` bytes."""
+    lib = _lib.load()
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    q, k, v, d_o = q.contiguous(), k.contiguous(), v.contiguous(), grad_output.to(q.dtype).contiguous()
+    need = backward_workspace_bytes(B, Hq, Hkv, N, D)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    have = workspace.numel() * workspace.element_size()
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    with torch.cuda.device(q.device):
+        rc = lib.corope_gqa_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), d_o.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                dv.data_ptr(), B, Hq, Hkv, N, D, float(sm_scale), float(theta), workspace.data_ptr(),
+                                have, torch.cuda.current_stream(q.device).cuda_stream)
+    _lib.check(rc, "corope_gqa_bwd")
+    return dq, dk, dv
 
 
 attention = _CoRopeGqaAttn.apply

@@ -498,4 +498,38 @@ int corope_gqa_fwd(const void* q, const void* k, const void* v, void* o, int B, 
   return launch_status("corope_gqa_fwd", corope::launch_corope_gqa_fwd(p, D, static_cast<hipStream_t>(stream)));
 }
 
+int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D) {
+  if (corope_gqa_check(B, Hq, Hkv, N, D, 1.f, 2.f)) return -1;
+  return 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N);
+}
+
+int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* d_o, void* dq, void* dk, void* dv, int B,
+                   int Hq, int Hkv, int N, int D, float sm_scale, float theta, void* workspace, int64_t workspace_bytes,
+                   void* stream) {
+  int rc = corope_gqa_check(B, Hq, Hkv, N, D, sm_scale, theta);
+  if (rc) return rc;
+  rc = check_ptrs("corope_gqa_bwd", {q, k, v, d_o, dq, dk, dv, workspace});
+  if (rc) return rc;
+  if ((int64_t)B * Hkv > 65535) return fail(COROPE_E_UNSUPPORTED, "corope_gqa_bwd: B * Hkv = %lld exceeds 65535", (long long)B * Hkv);
+  const int64_t need = 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N);
+  if (workspace_bytes < need)
+    return fail(COROPE_E_BADARG, "corope_gqa_bwd: workspace of %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
+  corope::CoropeBwdParams p{};
+  p.q = static_cast<const uint16_t*>(q);
+  p.k = static_cast<const uint16_t*>(k);
+  p.v = static_cast<const uint16_t*>(v);
+  p.d_o = static_cast<const uint16_t*>(d_o);
+  p.dq = static_cast<uint16_t*>(dq);
+  p.dk = static_cast<uint16_t*>(dk);
+  p.dv = static_cast<uint16_t*>(dv);
+  p.sm_scale = sm_scale;
+  p.theta = theta;
+  p.B = B;
+  p.Hq = Hq;
+  p.Hkv = Hkv;
+  p.N = N;
+  return launch_status("corope_gqa_bwd", corope::launch_corope_gqa_bwd(p, D, static_cast<float*>(workspace),
+                                                                       static_cast<hipStream_t>(stream)));
+}
+
 }  // extern "C"

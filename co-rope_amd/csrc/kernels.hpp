@@ -61,6 +61,19 @@ struct CoropeParams {
   int num_m_blocks;
 };
 
+struct CoropeBwdParams {
+  const uint16_t* q;    // (B, Hq, N, D)
+  const uint16_t* k;    // (B, Hkv, N, D)
+  const uint16_t* v;
+  const uint16_t* d_o;  // (B, Hq, N, D)
+  uint16_t* dq;
+  uint16_t* dk;
+  uint16_t* dv;
+  float sm_scale;
+  float theta;
+  int B, Hq, Hkv, N;
+};
+
 // y = rotated x for a (BH, N, D) tensor; tile_max (may be null) receives [BH][ceil(N / 64)] largest row norms.
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
                               float* tile_max, int BH, int N, int D, hipStream_t stream);
@@ -72,6 +85,8 @@ hipError_t launch_bwd_dk(const BwdParams& p, int D, bool causal, hipStream_t str
 hipError_t launch_bwd_dkdv_fused(const BwdParams& p, int D, bool causal, hipStream_t stream);  // dK and dV in one launch
 hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_corope_gqa_fwd(const CoropeParams& p, int D, hipStream_t stream);
+int64_t corope_gqa_bwd_workspace_floats(int B, int Hq, int Hkv, int N);
+hipError_t launch_corope_gqa_bwd(const CoropeBwdParams& p, int D, float* workspace, hipStream_t stream);
 hipError_t launch_rope_freqs(float* cosp, float* sinp, int n_pos, int D, int width, int64_t row_stride, int pos0,
                              float theta, hipStream_t stream);
 

@@ -223,6 +223,20 @@ int corope_rope_attn_bwd_gqa(const void *q, const void *k, int prerotated, const
 int corope_gqa_fwd(const void *q, const void *k, const void *v, void *o,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void *stream);
 
+/* Bytes of device workspace corope_gqa_bwd needs for these sizes (-1 for sizes corope_gqa_check rejects):
+ * N*N floats per key/value head for the accumulated gates, the sigmoid slopes and the gate gradients, and per query
+ * head for the attention weights and the score gradients. */
+int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D);
+
+/* Co-RoPE grouped-query attention backward (causal only): dq (B,Hq,N,D), dk/dv (B,Hkv,N,D) from q, k, v and dO.
+ * Replaces _attention.backward (reference corope-exp/flash_attn_co_rope_gqa_triton.py:459-577), which recomputes the
+ * forward densely in PyTorch with (B,Hq,N,N,D/2) temporaries; the same gradients (including the path through the
+ * leader head's gates, :548-561) are produced here with N*N scalars per head in `workspace`.  Like the reference's, it
+ * takes neither the forward's output nor its row statistics.  The workspace need not be initialised. */
+int corope_gqa_bwd(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
+                   int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta,
+                   void *workspace, int64_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -48,8 +48,12 @@ def _check_shapes(q, k, v, causal):
     return q.shape[1] // k.shape[1]
 
 
-def corope_gqa_forward(q, k, v, causal, sm_scale, theta, compute_dtype=torch.float32, return_aux=False):
-    """Dense Co-RoPE GQA forward; O has shape (B, Hq, N, D) in ``compute_dtype``."""
+def corope_gqa_forward(q, k, v, causal, sm_scale, theta, compute_dtype=torch.float32, return_aux=False,
+                       detach_gates=False):
+    """Dense Co-RoPE GQA forward; O has shape (B, Hq, N, D) in ``compute_dtype``.
+
+    ``detach_gates`` cuts the position offsets out of the autograd graph (same output, gradients without the path
+    through the leader's sigmoid gates); tests use it to show that this path is material on their inputs."""
     G = _check_shapes(q, k, v, causal)
     cd = compute_dtype
     q, k, v = q.to(cd), k.to(cd), v.to(cd)
@@ -64,6 +68,8 @@ def corope_gqa_forward(q, k, v, causal, sm_scale, theta, compute_dtype=torch.flo
     z = torch.sigmoid(torch.einsum("bhqd,bhkd->bhqk", lead, k) * sm_scale)
     a = torch.cumsum(z, dim=-1).repeat_interleave(G, dim=1)          # (B, Hq, N, N)
     delta = torch.diagonal(a, dim1=-2, dim2=-1).unsqueeze(-1) - a
+    if detach_gates:
+        delta = delta.detach()
 
     h = D // 2
     q1, q2 = q[..., :h].unsqueeze(3), q[..., h:].unsqueeze(3)        # (B,Hq,N,1,h)

@@ -1,0 +1,111 @@
+"""GPU parity of the Co-RoPE GQA backward against autograd through the dense CPU oracle (through the C ABI).
+
+The oracle's gradients come from torch.autograd over its dense fp64 forward, which is how the reference checks its
+own manual backward (corope-exp/corope_attn_gqa_pytorch.py:326-355).  Bar: max-abs <= 2e-2 for the bf16 gradients,
+scaled by sqrt(G) for dK and dV, which sum G heads' contributions before the one rounding."""
+import math
+
+import pytest
+import torch
+
+from conftest import bf16_round, seeded
+from oracle import corope_gqa_oracle as C
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def _inputs(B, Hq, Hkv, N, D, seed=42):
+    return (bf16_round(seeded((B, Hq, N, D), seed)), bf16_round(seeded((B, Hkv, N, D), seed + 1)),
+            bf16_round(seeded((B, Hkv, N, D), seed + 2)), bf16_round(seeded((B, Hq, N, D), seed + 3)))
+
+
+def _oracle_grads(q, k, v, d_o, scale, theta):
+    q, k, v = (t.double().requires_grad_(True) for t in (q, k, v))
+    o = C.corope_gqa_forward(q, k, v, True, scale, theta, torch.float64)
+    return [g.float() for g in torch.autograd.grad(o, (q, k, v), d_o.double())]
+
+
+def _gpu_grads(pkg, q, k, v, d_o, scale, theta):
+    dev = torch.device("cuda:0")
+    qg, kg, vg = (t.to(dev, torch.bfloat16).requires_grad_(True) for t in (q, k, v))
+    o = pkg.corope_attention(qg, kg, vg, True, scale, theta)
+    o.backward(d_o.to(dev, torch.bfloat16))
+    torch.cuda.synchronize()
+    return [t.grad.float().cpu() for t in (qg, kg, vg)]
+
+
+def _compare(got, ref, G):
+    for name, a, b, bar in zip(("dQ", "dK", "dV"), got, ref, (TOL, TOL * math.sqrt(G), TOL * math.sqrt(G))):
+        err = (a - b).abs()
+        print(f"  {name} max-abs {err.max():.3e} mean-abs {err.mean():.3e} (max |ref| {b.abs().max():.3f})", flush=True)
+        assert torch.isfinite(a).all()
+        assert err.max() <= bar, name
+
+
+# (B, Hq, Hkv, N, D): every group size, ragged lengths around the 16/32/64 tile edges, both head dims
+CASES = [(1, 4, 2, 32, 64), (2, 4, 2, 64, 64), (1, 2, 2, 96, 64), (1, 6, 2, 100, 64), (1, 8, 2, 130, 128),
+         (1, 8, 1, 150, 64), (2, 5, 1, 77, 128), (1, 3, 1, 64, 128), (1, 7, 1, 65, 64), (1, 4, 1, 1, 64),
+         (1, 1, 1, 33, 128)]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,N,D", CASES)
+def test_corope_backward_parity(pkg, B, Hq, Hkv, N, D):
+    print(f"case B={B} Hq={Hq} Hkv={Hkv} N={N} D={D}", flush=True)
+    q, k, v, d_o = _inputs(B, Hq, Hkv, N, D)
+    scale = 1 / math.sqrt(D)
+    _compare(_gpu_grads(pkg, q, k, v, d_o, scale, 10000.0), _oracle_grads(q, k, v, d_o, scale, 10000.0), Hq // Hkv)
+
+
+def test_corope_backward_unit_scale_small_theta(pkg):
+    """sm_scale = 1 and a small base: fast rotations make the path through the gates a large part of dQ and dK."""
+    q, k, v, d_o = _inputs(1, 4, 2, 48, 64, seed=7)
+    q, k = bf16_round(q * 0.3), bf16_round(k * 0.3)
+    _compare(_gpu_grads(pkg, q, k, v, d_o, 1.0, 100.0), _oracle_grads(q, k, v, d_o, 1.0, 100.0), 2)
+
+
+def test_corope_backward_gate_path_is_material_and_right(pkg):
+    """On this input the gradient through the leader's gates is a large part of dQ and dK (the oracle with the
+    position offsets cut out of the graph differs by far more than the bar), so parity here pins that path; a
+    central finite difference through the dense forward pins the oracle's own gradient for one leader coordinate."""
+    q, k, v, d_o = _inputs(1, 4, 2, 48, 64, seed=7)
+    q, k = bf16_round(q * 0.3), bf16_round(k * 0.3)
+    full = _oracle_grads(q, k, v, d_o, 1.0, 100.0)
+    qd, kd, vd = (t.double().requires_grad_(True) for t in (q, k, v))
+    o = C.corope_gqa_forward(qd, kd, vd, True, 1.0, 100.0, torch.float64, detach_gates=True)
+    cut = [g.float() for g in torch.autograd.grad(o, (qd, kd, vd), d_o.double())]
+    assert (full[0] - cut[0]).abs().max() > 10 * TOL and (full[1] - cut[1]).abs().max() > 10 * TOL
+    assert torch.equal(full[0][:, 1::2], cut[0][:, 1::2])   # only the leaders' queries feed the gates
+    got = _gpu_grads(pkg, q, k, v, d_o, 1.0, 100.0)
+    _compare(got, full, 2)
+    eps, idx = 1e-4, (0, 0, 40, 5)
+    qp, qm = q.double(), q.double()
+    qp[idx] += eps
+    qm[idx] -= eps
+
+    def loss(qq):
+        return (C.corope_gqa_forward(qq, k.double(), v.double(), True, 1.0, 100.0, torch.float64) * d_o.double()).sum()
+
+    fd = float((loss(qp) - loss(qm)) / (2 * eps))
+    print(f"  finite difference {fd:.5f}, autograd {float(full[0][idx]):.5f}, gpu {float(got[0][idx]):.5f}")
+    assert abs(fd - float(full[0][idx])) <= 1e-5 * max(1.0, abs(fd))
+    assert abs(fd - float(got[0][idx])) <= TOL
+
+
+def test_corope_backward_caller_workspace_and_reuse(pkg):
+    """A caller-owned workspace filled with garbage gives the same gradients; a short one is refused."""
+    import importlib
+    mod = importlib.import_module("corope_amd.corope_gqa")
+    dev = torch.device("cuda:0")
+    B, Hq, Hkv, N, D = 1, 4, 2, 70, 64
+    q, k, v, d_o = (t.to(dev, torch.bfloat16) for t in _inputs(B, Hq, Hkv, N, D, seed=3))
+    need = mod.backward_workspace_bytes(B, Hq, Hkv, N, D)
+    assert need == 4 * N * N * (3 * B * Hkv + 2 * B * Hq)
+    a = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4)
+    ws = torch.full((need // 4 + 64,), float("nan"), device=dev)
+    b = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4, workspace=ws)
+    torch.cuda.synchronize()
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    with pytest.raises(ValueError):
+        mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4, workspace=ws[: need // 4 - 1])
