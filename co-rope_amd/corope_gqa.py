@@ -57,7 +57,7 @@ class _CoRopeGqaAttn(torch.autograd.Function):
 
 
 def backward_workspace_bytes(B, Hq, Hkv, N, D):
-    """Scratch memory the backward needs: (3 * B * Hkv + 2 * B * Hq) * N * N fp32 values."""
+    """Scratch memory the backward needs: (2 * B * Hkv + 3 * B * Hq) * N * N fp32 values."""
     n = _lib.load().corope_gqa_bwd_workspace_bytes(B, Hq, Hkv, N, D)
     if n < 0:
         raise ValueError(_lib.last_error() or "unsupported Co-RoPE shape")

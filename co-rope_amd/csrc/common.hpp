@@ -5,6 +5,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+#include <utility>
+
 namespace corope {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -282,6 +285,17 @@ __device__ __forceinline__ void store_unrotated(const f32x16 (&acc)[D / 32], uin
       *reinterpret_cast<u32x2*>(dst_row + col) = u32x2{pack_bf16(o1[0], o1[1]), pack_bf16(o1[2], o1[3])};
       *reinterpret_cast<u32x2*>(dst_row + D / 2 + col) = u32x2{pack_bf16(o2[0], o2[1]), pack_bf16(o2[2], o2[3])};
     }
+}
+
+// f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
+// in the body, so register arrays indexed with it never look dynamically indexed to the optimiser.
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
 }
 
 }  // namespace corope

@@ -17,13 +17,16 @@
 //                   dz_it = sum_{j < t} G_ij,   W_it = dz_it z_it (1 - z_it)   (gradient of the leader's logit),
 //                   dqL_i += c sum_t W_it k_t,   dk_t += c sum_i W_it qL_i.
 //
-// Four kernels, each a plain loop nest over (query row, key) pairs with one wave per row (or per few keys):
-//   gates   (lane = key):   z, delta by a right-to-left suffix scan             -> DELTA, ZP   [group][N][N]
-//   scores  (lane = key):   S, P, dP, dS for all heads of the group             -> P, DS       [head][N][N]
-//   dq      (lane = pair):  dq, G and its prefix sum, W, leader's dq            -> W           [group][N][N]
+// Three kernels, each a plain loop nest over (query row, key) pairs with one wave per row (or per few keys):
+//   scores  (lane = key):   right to left: z, delta by a suffix scan, S, dS/ddelta, dP and the row's softmax statistics;
+//                           left to right: P, dS, G and its prefix sum, W              -> DELTA, W [group][N][N]
+//                                                                                         P, DS, (DP) [head][N][N]
+//   dq      (lane = pair):  dq of every head, plus the leader's gate path
 //   dkdv    (lane = pair):  dk, dv for 32 keys per workgroup, tiles of the matrices staged through LDS
-// "lane = key" makes every dot product over d a per-lane loop (no reductions); "lane = pair" makes every sum over keys
-// or queries a per-lane accumulation (the only cross-lane reduction left is G_ij, one per (i, j)).
+// "lane = key" makes every dot product over d a per-lane loop and every sum over keys a lane-local accumulation that
+// is reduced once per row; "lane = pair" makes every sum over keys or queries a per-lane accumulation.  The angle
+// is shared by the group and rotation is linear, so sines and cosines are evaluated once per (i, j, d) in each kernel
+// and applied to one vector: the key (scores, dq) or the dS-weighted sum of the group's queries (dk).
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -34,16 +37,16 @@ struct CoropeBwdFreqs {
   float rad[64];     // w_d
 };
 
-// Workspace layout, in floats; NN = N * N.
+// Workspace layout, in floats; NN = N * N.  Only the causal triangle of each matrix is written and read.
 struct CoropeBwdWs {
   float* base;
   int64_t NN;
   int n_groups, n_heads;
   __device__ __host__ float* delta(int g) const { return base + (int64_t)g * NN; }
-  __device__ __host__ float* zp(int g) const { return base + (int64_t)(n_groups + g) * NN; }
-  __device__ __host__ float* w(int g) const { return base + (int64_t)(2 * n_groups + g) * NN; }
-  __device__ __host__ float* p(int h) const { return base + (int64_t)(3 * n_groups + h) * NN; }
-  __device__ __host__ float* ds(int h) const { return base + (int64_t)(3 * n_groups + n_heads + h) * NN; }
+  __device__ __host__ float* w(int g) const { return base + (int64_t)(n_groups + g) * NN; }
+  __device__ __host__ float* p(int h) const { return base + (int64_t)(2 * n_groups + h) * NN; }               // S, then P
+  __device__ __host__ float* ds(int h) const { return base + (int64_t)(2 * n_groups + n_heads + h) * NN; }    // dS/ddelta, then dS
+  __device__ __host__ float* dp(int h) const { return base + (int64_t)(2 * n_groups + 2 * n_heads + h) * NN; }
 };
 
 __device__ __forceinline__ float wave_sum(float x) {
@@ -57,7 +60,7 @@ __device__ __forceinline__ float wave_max(float x) {
   return x;
 }
 
-// One (N, D) bf16 row as D/8 16-byte words in registers; element e as float.
+// One (N, D) bf16 row as D/8 16-byte words in registers; element e as float (one shift or mask per use).
 template <int D>
 struct RowRegs {
   u32x4 w[D / 8];
@@ -74,236 +77,289 @@ struct RowRegs {
 __device__ __forceinline__ float bf16_to_f(uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
 __device__ __forceinline__ uint16_t f_to_bf16(float x) { return (uint16_t)(pack_bf16(x, 0.f) & 0xffffu); }
 
-// ---------------------------------------------------------------------------------------------------- gates
-// One wave per (group, query row i), lane = key inside a 64-key chunk, chunks from the diagonal to the left.
-template <int D>
-__global__ __launch_bounds__(kWave) void corope_bwd_gates_kernel(CoropeBwdParams p, CoropeBwdWs ws) {
-  __shared__ float ql[D];
-  const int i = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
-  const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv, G = p.Hq / p.Hkv;
-  const uint16_t* qrow = p.q + (((int64_t)b * p.Hq + kvh * G) * N + i) * D;   // the leader's row
-  const uint16_t* kbase = p.k + (int64_t)g * N * D;
-  for (int d = lane; d < D; d += kWave) ql[d] = bf16_to_f(qrow[d]);
-  __syncthreads();
-  float* drow = ws.delta(g) + (int64_t)i * N;
-  float* zrow = ws.zp(g) + (int64_t)i * N;
-  float carry = 0.f;   // sum of z over the keys to the right of the current chunk (up to the diagonal)
-  for (int c = i / kWave; c >= 0; --c) {
-    const int j = c * kWave + lane;
-    const bool valid = j <= i;
-    RowRegs<D> kr;
-    kr.load(kbase + (int64_t)(valid ? j : i) * D);
-    float dot = 0.f;
-#pragma unroll
-    for (int d = 0; d < D; ++d) dot = __builtin_fmaf(ql[d], kr.at(d), dot);
-    const float z = valid ? 1.f / (1.f + __expf(-dot * p.sm_scale)) : 0.f;
-    float s = z;   // inclusive suffix sum over the lanes (keys) at and to the right of this one
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      const float t = __shfl_down(s, off);
-      if (lane + off < kWave) s += t;
-    }
-    if (valid) {
-      drow[j] = carry + s - z;   // z of the keys strictly to the right, up to and including the diagonal
-      zrow[j] = z * (1.f - z);
-    }
-    carry += __shfl(s, 0);
-  }
-}
-
 // ---------------------------------------------------------------------------------------------------- scores
-// One wave per (group, query row i), all G heads at once, lane = key.  Four sweeps over the row's keys: raw scores and
-// their maxima; exponentials and their sums; P, dP and rowsum(P o dP); dS.  Only the first sweep evaluates sines and
-// cosines.  The row sum is taken from P and dP themselves, as the reference does (:526-528), so the forward's rounded
-// output is not an input of the backward.
+// One wave per (group, query row i), all G heads at once, lane = key.  The row's queries and upstream gradients sit in
+// LDS as fp32 and are read with broadcast loads, a few rotation pairs ahead of their use (the scheduling barriers keep
+// the fully unrolled loops from pulling every LDS read to the top).
 template <int D, int G>
-__global__ __launch_bounds__(kWave) void corope_bwd_scores_kernel(CoropeBwdParams p, CoropeBwdWs ws, CoropeBwdFreqs fr) {
-  constexpr int HALF = D / 2;
-  __shared__ float qs[HALF][G][2];   // (q1, q2) of every head per rotation pair
-  __shared__ float dos[D][G];        // dO of every head per column
-  const int i = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void corope_bwd_scores_kernel(CoropeBwdParams p, CoropeBwdWs ws, CoropeBwdFreqs fr) {
+  constexpr int HALF = D / 2, QW = 2 * G;
+  constexpr int CH = G <= 4 ? 4 : 2;                                  // rotation pairs per look-ahead chunk
+  __shared__ __attribute__((aligned(16))) float ql[D];                // the leader's row
+  __shared__ __attribute__((aligned(16))) float qs[HALF * QW];        // [pair d][head][q1, q2]
+  __shared__ __attribute__((aligned(16))) float dos[D * G];           // [column][head]
+  __shared__ __attribute__((aligned(16))) float wsm[HALF * 2];        // [pair d][turns, radians]
+  const int i = p.N - 1 - blockIdx.x, g = blockIdx.y, lane = threadIdx.x;   // longest rows first
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
   const int head0 = b * p.Hq + kvh * G;   // first head of the group, as a (batch, head) slab index
 #pragma unroll
   for (int h = 0; h < G; ++h) {
     const int64_t off = ((int64_t)(head0 + h) * N + i) * D;
     for (int d = lane; d < D; d += kWave) {
-      qs[d % HALF][h][d / HALF] = bf16_to_f(p.q[off + d]);
-      dos[d][h] = bf16_to_f(p.d_o[off + d]);
+      const float qv = bf16_to_f(p.q[off + d]);
+      qs[(d % HALF) * QW + 2 * h + d / HALF] = qv;
+      if (h == 0) ql[d] = qv;
+      dos[d * G + h] = bf16_to_f(p.d_o[off + d]);
     }
+  }
+  if (lane < HALF) {
+    wsm[2 * lane] = fr.turns[lane];
+    wsm[2 * lane + 1] = fr.rad[lane];
   }
   __syncthreads();
   const uint16_t* kbase = p.k + (int64_t)g * N * D;
   const uint16_t* vbase = p.v + (int64_t)g * N * D;
-  const float* drow = ws.delta(g) + (int64_t)i * N;
+  const int64_t rowoff = (int64_t)i * N;
   const int n_chunks = i / kWave + 1;
 
-  // ---- sweep 1: raw scores ---------------------------------------------------------------------------------------
-  float mx[G];
+  // ---- right to left: gates, delta, raw scores, dS/ddelta, dP, lane-local softmax statistics -------------------------
+  float m_run[G], l_run[G], pd_run[G];   // per lane: largest score, sum of exp(s - m), sum of exp(s - m) dP
 #pragma unroll
-  for (int h = 0; h < G; ++h) mx[h] = -INFINITY;
-  for (int c = 0; c < n_chunks; ++c) {
+  for (int h = 0; h < G; ++h) {
+    m_run[h] = -INFINITY;
+    l_run[h] = pd_run[h] = 0.f;
+  }
+  float carry = 0.f;   // sum of z over the keys to the right of the current chunk (up to the diagonal)
+#pragma unroll 1
+  for (int c = n_chunks - 1; c >= 0; --c) {
     const int j = c * kWave + lane;
     const bool valid = j <= i;
+    const int jc = valid ? j : i;
+    asm volatile("" ::: "memory");   // the LDS operands are loop-invariant: keep their loads inside the iteration
     RowRegs<D> kr;
-    kr.load(kbase + (int64_t)(valid ? j : i) * D);
-    const float delta = valid ? drow[j] : 0.f;
-    float acc[G];
+    kr.load(kbase + (int64_t)jc * D);
+    // leader logit
+    float logit = 0.f;
+    {
+      const f32x4* q4 = reinterpret_cast<const f32x4*>(ql);
+      f32x4 qa = q4[0], qb = q4[1], na = qa, nb = qb;
+      static_for<D / 8>([&](auto c8_c) __attribute__((always_inline)) {
+        constexpr int c8 = decltype(c8_c)::value;
+        if (c8 + 1 < D / 8) {
+          na = q4[2 * c8 + 2];
+          nb = q4[2 * c8 + 3];
+        }
 #pragma unroll
-    for (int h = 0; h < G; ++h) acc[h] = 0.f;
+        for (int e = 0; e < 4; ++e) logit = __builtin_fmaf(qa[e], kr.at(8 * c8 + e), logit);
 #pragma unroll
-    for (int d = 0; d < HALF; ++d) {
-      const float x = __builtin_amdgcn_fractf(delta * fr.turns[d]);
-      const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
-      const float k1 = kr.at(d), k2 = kr.at(d + HALF);
-      const float kt1 = __builtin_fmaf(cs, k1, sn * k2), kt2 = __builtin_fmaf(cs, k2, -(sn * k1));
-#pragma unroll
-      for (int h = 0; h < G; ++h) acc[h] = __builtin_fmaf(qs[d][h][0], kt1, __builtin_fmaf(qs[d][h][1], kt2, acc[h]));
+        for (int e = 0; e < 4; ++e) logit = __builtin_fmaf(qb[e], kr.at(8 * c8 + 4 + e), logit);
+        __builtin_amdgcn_sched_barrier(0);
+        qa = na;
+        qb = nb;
+      });
     }
+    const float z = valid ? 1.f / (1.f + __expf(-logit * p.sm_scale)) : 0.f;
+    float suf = z;   // inclusive suffix sum over the lanes (keys) at and to the right of this one
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-      const float s = acc[h] * p.sm_scale;
-      if (valid) {
-        ws.p(head0 + h)[(int64_t)i * N + j] = s;
-        mx[h] = fmaxf(mx[h], s);
-      }
+    for (int off = 1; off < kWave; off <<= 1) {
+      const float t = __shfl_down(suf, off);
+      if (lane + off < kWave) suf += t;
     }
-  }
-#pragma unroll
-  for (int h = 0; h < G; ++h) mx[h] = wave_max(mx[h]);
+    const float delta = carry + suf - z;   // gates strictly to the right, up to and including the diagonal
+    carry += __shfl(suf, 0);
 
-  // ---- sweep 2: exponentials -------------------------------------------------------------------------------------
-  float inv_l[G];
+    // rotated dot products of every head, and their derivative with respect to delta
+    float acc[G], gacc[G];
 #pragma unroll
-  for (int h = 0; h < G; ++h) inv_l[h] = 0.f;
-  for (int c = 0; c < n_chunks; ++c) {
-    const int j = c * kWave + lane;
-    if (j <= i) {
+    for (int h = 0; h < G; ++h) acc[h] = gacc[h] = 0.f;
+    {
+      f32x2 qc[CH][G], qn[CH][G], wc[CH], wn[CH];
+#pragma unroll
+      for (int e = 0; e < CH; ++e) {
+        wc[e] = wn[e] = *reinterpret_cast<const f32x2*>(wsm + 2 * e);
+#pragma unroll
+        for (int h = 0; h < G; ++h) qc[e][h] = qn[e][h] = *reinterpret_cast<const f32x2*>(qs + e * QW + 2 * h);
+      }
+      static_for<HALF / CH>([&](auto step_c) __attribute__((always_inline)) {
+        constexpr int d0 = decltype(step_c)::value * CH;
+        if (d0 + CH < HALF) {
+#pragma unroll
+          for (int e = 0; e < CH; ++e) {
+            wn[e] = *reinterpret_cast<const f32x2*>(wsm + 2 * (d0 + CH + e));
+#pragma unroll
+            for (int h = 0; h < G; ++h) qn[e][h] = *reinterpret_cast<const f32x2*>(qs + (d0 + CH + e) * QW + 2 * h);
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < CH; ++e) {
+          const int d = d0 + e;
+          const float x = __builtin_amdgcn_fractf(delta * wc[e][0]);
+          const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
+          const float k1 = kr.at(d), k2 = kr.at(d + HALF);
+          const float r1 = __builtin_fmaf(cs, k1, sn * k2), r2 = __builtin_fmaf(cs, k2, -(sn * k1));
+          const float t1 = wc[e][1] * r2, t2 = wc[e][1] * r1;
+#pragma unroll
+          for (int h = 0; h < G; ++h) {
+            acc[h] = __builtin_fmaf(qc[e][h][0], r1, __builtin_fmaf(qc[e][h][1], r2, acc[h]));
+            gacc[h] = __builtin_fmaf(qc[e][h][0], t1, __builtin_fmaf(-qc[e][h][1], t2, gacc[h]));
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int e = 0; e < CH; ++e) {
+          wc[e] = wn[e];
+#pragma unroll
+          for (int h = 0; h < G; ++h) qc[e][h] = qn[e][h];
+        }
+      });
+    }
+    // the sums are used only under `valid` below: pin them here, or the whole chain is sunk into that branch, away
+    // from the loads that feed it
+#pragma unroll
+    for (int h = 0; h < G; ++h) asm volatile("" : "+v"(acc[h]), "+v"(gacc[h]));
+    // dP = dO . v
+    float dpv[G];
+#pragma unroll
+    for (int h = 0; h < G; ++h) dpv[h] = 0.f;
+    {
+      RowRegs<D> vr;
+      vr.load(vbase + (int64_t)jc * D);
+      const f32x4* d4 = reinterpret_cast<const f32x4*>(dos);   // 4 columns x G heads = G vectors per step
+      f32x4 dc[G], dn[G];
+#pragma unroll
+      for (int u = 0; u < G; ++u) dc[u] = dn[u] = d4[u];
+      static_for<D / 4>([&](auto step_c) __attribute__((always_inline)) {
+        constexpr int d0 = decltype(step_c)::value * 4;
+        if (d0 + 4 < D) {
+#pragma unroll
+          for (int u = 0; u < G; ++u) dn[u] = d4[(d0 + 4) / 4 * G + u];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float vv = vr.at(d0 + e);
+#pragma unroll
+          for (int h = 0; h < G; ++h) dpv[h] = __builtin_fmaf(dc[(e * G + h) / 4][(e * G + h) % 4], vv, dpv[h]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < G; ++u) dc[u] = dn[u];
+      });
+    }
+#pragma unroll
+    for (int h = 0; h < G; ++h) asm volatile("" : "+v"(dpv[h]));
+    if (valid) {
+      ws.delta(g)[rowoff + j] = delta;
+      ws.w(g)[rowoff + j] = z * (1.f - z);   // the sigmoid's slope; replaced by W in the second sweep
 #pragma unroll
       for (int h = 0; h < G; ++h) {
-        float* pp = ws.p(head0 + h) + (int64_t)i * N + j;
-        const float e = __expf(*pp - mx[h]);
-        *pp = e;
-        inv_l[h] += e;
+        const float s = acc[h] * p.sm_scale;
+        ws.p(head0 + h)[rowoff + j] = s;
+        ws.ds(head0 + h)[rowoff + j] = gacc[h] * p.sm_scale;
+        ws.dp(head0 + h)[rowoff + j] = dpv[h];
+        const float m_new = fmaxf(m_run[h], s);
+        const float a = __expf(m_run[h] - m_new), e = __expf(s - m_new);
+        l_run[h] = __builtin_fmaf(l_run[h], a, e);
+        pd_run[h] = __builtin_fmaf(pd_run[h], a, e * dpv[h]);
+        m_run[h] = m_new;
       }
     }
   }
+  // row statistics: largest score, 1 / sum of exponentials, rowsum(P o dP)
+  float m_row[G], inv_l[G], dsum[G];
 #pragma unroll
-  for (int h = 0; h < G; ++h) inv_l[h] = 1.f / wave_sum(inv_l[h]);
+  for (int h = 0; h < G; ++h) {
+    m_row[h] = wave_max(m_run[h]);   // finite: lane 0 of chunk 0 always holds a key
+    const float f = m_run[h] == -INFINITY ? 0.f : __expf(m_run[h] - m_row[h]);
+    const float l = wave_sum(l_run[h] * f), pd = wave_sum(pd_run[h] * f);
+    inv_l[h] = 1.f / l;
+    dsum[h] = pd * inv_l[h];
+  }
 
-  // ---- sweep 3: P, dP = dO . v (parked in DS), rowsum(P o dP) ------------------------------------------------------
-  float dsum[G];
-#pragma unroll
-  for (int h = 0; h < G; ++h) dsum[h] = 0.f;
+  // ---- left to right: P, dS, G_ij = sum_h dS dS/ddelta, its running sum over the keys, W ------------------------------
+  float gcarry = 0.f;
+#pragma unroll 1
   for (int c = 0; c < n_chunks; ++c) {
     const int j = c * kWave + lane;
     const bool valid = j <= i;
-    RowRegs<D> vr;
-    vr.load(vbase + (int64_t)(valid ? j : i) * D);
-    float dp[G];
-#pragma unroll
-    for (int h = 0; h < G; ++h) dp[h] = 0.f;
-#pragma unroll
-    for (int d = 0; d < D; ++d) {
-      const float vv = vr.at(d);
-#pragma unroll
-      for (int h = 0; h < G; ++h) dp[h] = __builtin_fmaf(dos[d][h], vv, dp[h]);
-    }
+    float gij = 0.f, slope = 0.f;
     if (valid) {
+      slope = ws.w(g)[rowoff + j];
 #pragma unroll
       for (int h = 0; h < G; ++h) {
-        const int64_t at = (int64_t)i * N + j;
-        const float pr = ws.p(head0 + h)[at] * inv_l[h];
-        ws.p(head0 + h)[at] = pr;
-        ws.ds(head0 + h)[at] = dp[h];
-        dsum[h] = __builtin_fmaf(pr, dp[h], dsum[h]);
+        float* pp = ws.p(head0 + h) + rowoff + j;
+        float* dd = ws.ds(head0 + h) + rowoff + j;
+        const float pr = __expf(*pp - m_row[h]) * inv_l[h];
+        const float dsv = pr * (ws.dp(head0 + h)[rowoff + j] - dsum[h]);
+        gij = __builtin_fmaf(dsv, *dd, gij);
+        *pp = pr;
+        *dd = dsv;
       }
     }
-  }
+    float pre = gij;   // inclusive prefix sum over the lanes (keys) at and to the left of this one
 #pragma unroll
-  for (int h = 0; h < G; ++h) dsum[h] = wave_sum(dsum[h]);
-
-  // ---- sweep 4: dS = P (dP - rowsum(P o dP)) -----------------------------------------------------------------------
-  for (int c = 0; c < n_chunks; ++c) {
-    const int j = c * kWave + lane;
-    if (j <= i) {
-#pragma unroll
-      for (int h = 0; h < G; ++h) {
-        const int64_t at = (int64_t)i * N + j;
-        ws.ds(head0 + h)[at] = ws.p(head0 + h)[at] * (ws.ds(head0 + h)[at] - dsum[h]);
-      }
+    for (int off = 1; off < kWave; off <<= 1) {
+      const float t = __shfl_up(pre, off);
+      if (lane >= off) pre += t;
     }
+    if (valid) ws.w(g)[rowoff + j] = (gcarry + pre - gij) * slope;   // (sum of G over the keys j < t) z'(t)
+    gcarry += __shfl(pre, kWave - 1);
   }
 }
 
 // ---------------------------------------------------------------------------------------------------- dq
-// One wave per (group, query row i), lane = rotation pair (d, d + D/2), keys in ascending order so that the prefix sum
-// of G is a running scalar.  The key chunk is staged in LDS; the row's scalars (delta, z(1-z), dS per head) are loaded
-// with lane = key and handed out with readlane.
+// One wave per (group, query row i), lane = rotation pair (d, d + D/2).  The key chunk is staged in LDS; the row's
+// scalars (delta, W, dS per head) are loaded with lane = key and handed out with readlane.
 template <int D, int G>
 __global__ __launch_bounds__(kWave) void corope_bwd_dq_kernel(CoropeBwdParams p, CoropeBwdWs ws, CoropeBwdFreqs fr) {
   constexpr int HALF = D / 2;
   __shared__ __attribute__((aligned(16))) uint16_t kch[kWave][D];   // 64 keys x D, bf16
-  const int i = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+  const int i = p.N - 1 - blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
   const int head0 = b * p.Hq + kvh * G;
   const bool act = lane < HALF;           // D = 64 leaves the upper half of the wave without a pair
   const int dpair = act ? lane : 0;
-  const float w_turn = fr.turns[dpair], w_rad = act ? fr.rad[dpair] : 0.f;
-  float q1[G], q2[G], dq1[G], dq2[G];
+  const float w_turn = fr.turns[dpair];
+  float dq1[G], dq2[G];
 #pragma unroll
-  for (int h = 0; h < G; ++h) {
-    const int64_t off = ((int64_t)(head0 + h) * N + i) * D;
-    q1[h] = bf16_to_f(p.q[off + dpair]);
-    q2[h] = bf16_to_f(p.q[off + dpair + HALF]);
-    dq1[h] = dq2[h] = 0.f;
-  }
-  float dql1 = 0.f, dql2 = 0.f;   // the leader's extra gradient through its logits
-  float gprefix = 0.f;            // sum of G_ij over the keys already visited
+  for (int h = 0; h < G; ++h) dq1[h] = dq2[h] = 0.f;
+  float dql1 = 0.f, dql2 = 0.f;   // the leader's extra gradient through its gates
   const uint16_t* kbase = p.k + (int64_t)g * N * D;
   const int64_t rowoff = (int64_t)i * N;
   const int n_chunks = i / kWave + 1;
-  for (int c = 0; c < n_chunks; ++c) {
-    const int j0 = c * kWave, jl = j0 + lane;
+  // the next chunk's key row and scalars are fetched into registers while the current chunk is consumed
+  u32x4 kv[D / 8];
+  int dnext, wnext, dsnext[G];
+  auto fetch = [&](int c) __attribute__((always_inline)) {
+    const int jl = c * kWave + lane;
     const bool valid = jl <= i;
+    const uint16_t* src = kbase + (int64_t)(valid ? jl : i) * D;
+#pragma unroll
+    for (int v8 = 0; v8 < D / 8; ++v8) kv[v8] = *reinterpret_cast<const u32x4*>(src + 8 * v8);
+    dnext = valid ? __builtin_bit_cast(int, ws.delta(g)[rowoff + jl]) : 0;
+    wnext = valid ? __builtin_bit_cast(int, ws.w(g)[rowoff + jl]) : 0;
+#pragma unroll
+    for (int h = 0; h < G; ++h) dsnext[h] = valid ? __builtin_bit_cast(int, ws.ds(head0 + h)[rowoff + jl]) : 0;
+  };
+  fetch(0);
+#pragma unroll 1
+  for (int c = 0; c < n_chunks; ++c) {
+    const int j0 = c * kWave;
     __syncthreads();   // the previous chunk's keys are no longer needed
-    {
-      const uint16_t* src = kbase + (int64_t)(valid ? jl : i) * D;
 #pragma unroll
-      for (int v8 = 0; v8 < D / 8; ++v8)
-        *reinterpret_cast<u32x4*>(&kch[lane][8 * v8]) = *reinterpret_cast<const u32x4*>(src + 8 * v8);
-    }
-    const float dvec = valid ? ws.delta(g)[rowoff + jl] : 0.f;
-    const float zvec = valid ? ws.zp(g)[rowoff + jl] : 0.f;
-    float dsvec[G];
+    for (int v8 = 0; v8 < D / 8; ++v8) *reinterpret_cast<u32x4*>(&kch[lane][8 * v8]) = kv[v8];
+    const int dvec = dnext, wvec = wnext;
+    int dsvec[G];
 #pragma unroll
-    for (int h = 0; h < G; ++h) dsvec[h] = valid ? ws.ds(head0 + h)[rowoff + jl] : 0.f;
+    for (int h = 0; h < G; ++h) dsvec[h] = dsnext[h];
     __syncthreads();
-    float wvec = 0.f;
+    if (c + 1 < n_chunks) fetch(c + 1);
     const int n_here = min(kWave, i - j0 + 1);
     for (int jj = 0; jj < n_here; ++jj) {
-      const float delta = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, dvec), jj));
-      const float zp = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zvec), jj));
+      const float delta = __builtin_bit_cast(float, __builtin_amdgcn_readlane(dvec, jj));
+      const float wij = __builtin_bit_cast(float, __builtin_amdgcn_readlane(wvec, jj));
       const float k1 = bf16_to_f(kch[jj][dpair]), k2 = bf16_to_f(kch[jj][dpair + HALF]);
       const float x = __builtin_amdgcn_fractf(delta * w_turn);
       const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
       const float kt1 = __builtin_fmaf(cs, k1, sn * k2), kt2 = __builtin_fmaf(cs, k2, -(sn * k1));
-      float gacc = 0.f;
 #pragma unroll
       for (int h = 0; h < G; ++h) {
-        const float ds = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, dsvec[h]), jj));
-        dq1[h] = __builtin_fmaf(ds, kt1, dq1[h]);
-        dq2[h] = __builtin_fmaf(ds, kt2, dq2[h]);
-        gacc = __builtin_fmaf(ds, q1[h] * kt2 - q2[h] * kt1, gacc);
+        const float dsv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(dsvec[h], jj));
+        dq1[h] = __builtin_fmaf(dsv, kt1, dq1[h]);
+        dq2[h] = __builtin_fmaf(dsv, kt2, dq2[h]);
       }
-      const float gij = p.sm_scale * wave_sum(gacc * w_rad);   // G_ij: the one cross-lane reduction per (i, j)
-      const float wij = gprefix * zp;                          // dz_it z'(t) with the sum over keys j < t
-      gprefix += gij;
       dql1 = __builtin_fmaf(wij, k1, dql1);
       dql2 = __builtin_fmaf(wij, k2, dql2);
-      wvec = lane == jj ? wij : wvec;
     }
-    if (valid) ws.w(g)[rowoff + jl] = wvec;
   }
   if (act) {
 #pragma unroll
@@ -318,14 +374,16 @@ __global__ __launch_bounds__(kWave) void corope_bwd_dq_kernel(CoropeBwdParams p,
 
 // ---------------------------------------------------------------------------------------------------- dk, dv
 // One workgroup of 4 waves per (group, block of 32 keys); each wave owns 8 of the keys, lane = rotation pair.  Query
-// rows are visited 16 at a time: the 16 x 32 tiles of DELTA, W, DS^h, P^h and the 16 rows of q and dO of every head are
-// staged in LDS, so the column-wise access of the N x N matrices costs full 128-byte lines.
+// rows are visited 16 at a time: the 16 x 32 tiles of DELTA, W, DS^h, P^h (interleaved per element, so that one (row,
+// key) costs a few 16-byte broadcast reads) and the 16 rows of q and dO of every head are staged in LDS, so the
+// column-wise access of the N x N matrices costs full 128-byte lines.
 constexpr int kDkKeys = 32, kDkRows = 16, kDkWaves = 4, kDkKeysPerWave = kDkKeys / kDkWaves;
 
 template <int D, int G>
 struct CoropeDkCfg {
   static constexpr int kMats = 2 + 2 * G;                                   // DELTA, W, DS^h, P^h
-  static constexpr int kMatBytes = kMats * kDkRows * kDkKeys * 4;
+  static constexpr int kMS = (kMats + 3) / 4 * 4;                           // floats per (row, key) element
+  static constexpr int kMatBytes = kMS * kDkRows * kDkKeys * 4;
   static constexpr int kRowBytes = kDkRows * G * D * 2;                     // q rows (and as many dO rows), bf16
   static constexpr int kLdsBytes = kMatBytes + 2 * kRowBytes;
 };
@@ -334,13 +392,13 @@ template <int D, int G>
 __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(CoropeBwdParams p, CoropeBwdWs ws,
                                                                          CoropeBwdFreqs fr) {
   using Cfg = CoropeDkCfg<D, G>;
-  constexpr int HALF = D / 2, NT = kDkWaves * kWave;
+  constexpr int HALF = D / 2, NT = kDkWaves * kWave, MS = Cfg::kMS;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  float (*mats)[kDkRows][kDkKeys] = reinterpret_cast<float (*)[kDkRows][kDkKeys]>(smem);
+  float* mats = reinterpret_cast<float*>(smem);                                          // [row][key][MS]
   uint16_t (*qrows)[G][D] = reinterpret_cast<uint16_t (*)[G][D]>(smem + Cfg::kMatBytes);
   uint16_t (*dorows)[G][D] = reinterpret_cast<uint16_t (*)[G][D]>(smem + Cfg::kMatBytes + Cfg::kRowBytes);
 
-  const int jb = blockIdx.x * kDkKeys, g = blockIdx.y;
+  const int jb = blockIdx.x * kDkKeys, g = blockIdx.y;   // the first key blocks see the most rows and start first
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
   const int head0 = b * p.Hq + kvh * G;
@@ -353,30 +411,52 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(Corope
 #pragma unroll
   for (int kk = 0; kk < kDkKeysPerWave; ++kk) dk1[kk] = dk2[kk] = dv1[kk] = dv2[kk] = 0.f;
 
-  // rows i >= jb see at least one key of the block
-  for (int i0 = (jb / kDkRows) * kDkRows; i0 < N; i0 += kDkRows) {
-    __syncthreads();
-    // ---- stage the tiles: element (m, r, c) <- matrix m at [i0 + r][jb + c] (zero outside the causal triangle / N) ----
-    for (int e = threadIdx.x; e < Cfg::kMats * kDkRows * kDkKeys; e += NT) {
-      const int m = e / (kDkRows * kDkKeys), r = (e / kDkKeys) % kDkRows, c = e % kDkKeys;
-      const int i = i0 + r, j = jb + c;
-      float val = 0.f;
-      if (i < N && j <= i) {
-        const int64_t at = (int64_t)i * N + j;
-        const float* src = m == 0 ? ws.delta(g) : m == 1 ? ws.w(g) : m < 2 + G ? ws.ds(head0 + m - 2) : ws.p(head0 + m - 2 - G);
-        val = src[at];
+  // Staging: thread -> key column c and row r = rsub or rsub + 8 of the 16 x 32 tiles, plus its share of the 16-byte
+  // pieces of the q / dO rows.  The next tile's values are fetched into registers while the current tile is consumed.
+  constexpr int kRowItems = kDkRows * G * (D / 8), RI = (kRowItems + NT - 1) / NT;
+  const int sc = threadIdx.x % kDkKeys, rsub = threadIdx.x / kDkKeys;
+  float mv[2 * Cfg::kMats];
+  u32x4 qv[RI], ov[RI];
+  auto fetch = [&](int i0) __attribute__((always_inline)) {
+    static_for<2 * Cfg::kMats>([&](auto k_c) __attribute__((always_inline)) {
+      constexpr int k = decltype(k_c)::value, m = k / 2;
+      const int i = i0 + rsub + 8 * (k % 2), j = jb + sc;
+      const float* src = m == 0 ? ws.delta(g) : m == 1 ? ws.w(g) : m < 2 + G ? ws.ds(head0 + m - 2) : ws.p(head0 + m - 2 - G);
+      mv[k] = (i < N && j <= i) ? src[(int64_t)i * N + j] : 0.f;   // zero outside the causal triangle and past N
+    });
+    static_for<RI>([&](auto k_c) __attribute__((always_inline)) {
+      constexpr int k = decltype(k_c)::value;
+      const int e = threadIdx.x + k * NT;
+      if (kRowItems % NT == 0 || e < kRowItems) {
+        const int r = e / (G * (D / 8)), h = (e / (D / 8)) % G, v8 = e % (D / 8);
+        const int64_t off = ((int64_t)(head0 + h) * N + min(i0 + r, N - 1)) * D + 8 * v8;
+        qv[k] = *reinterpret_cast<const u32x4*>(p.q + off);
+        ov[k] = *reinterpret_cast<const u32x4*>(p.d_o + off);
       }
-      mats[m][r][c] = val;
-    }
-    for (int e = threadIdx.x; e < kDkRows * G * (D / 8); e += NT) {
-      const int r = e / (G * (D / 8)), h = (e / (D / 8)) % G, v8 = e % (D / 8);
-      const int i = min(i0 + r, N - 1);
-      const int64_t off = ((int64_t)(head0 + h) * N + i) * D + 8 * v8;
-      *reinterpret_cast<u32x4*>(&qrows[r][h][8 * v8]) = *reinterpret_cast<const u32x4*>(p.q + off);
-      *reinterpret_cast<u32x4*>(&dorows[r][h][8 * v8]) = *reinterpret_cast<const u32x4*>(p.d_o + off);
-    }
+    });
+  };
+  fetch(jb);
+  // rows i >= jb see at least one key of the block
+#pragma unroll 1
+  for (int i0 = jb; i0 < N; i0 += kDkRows) {
+    __syncthreads();   // the previous tile has been consumed
+    static_for<2 * Cfg::kMats>([&](auto k_c) __attribute__((always_inline)) {
+      constexpr int k = decltype(k_c)::value;
+      mats[((rsub + 8 * (k % 2)) * kDkKeys + sc) * MS + k / 2] = mv[k];
+    });
+    static_for<RI>([&](auto k_c) __attribute__((always_inline)) {
+      constexpr int k = decltype(k_c)::value;
+      const int e = threadIdx.x + k * NT;
+      if (kRowItems % NT == 0 || e < kRowItems) {
+        const int r = e / (G * (D / 8)), h = (e / (D / 8)) % G, v8 = e % (D / 8);
+        *reinterpret_cast<u32x4*>(&qrows[r][h][8 * v8]) = qv[k];
+        *reinterpret_cast<u32x4*>(&dorows[r][h][8 * v8]) = ov[k];
+      }
+    });
     __syncthreads();
+    if (i0 + kDkRows < N) fetch(i0 + kDkRows);
     const int n_rows = min(kDkRows, N - i0);
+#pragma unroll 1
     for (int r = 0; r < n_rows; ++r) {
       const int i = i0 + r;
       float q1[G], q2[G], o1[G], o2[G];
@@ -389,21 +469,26 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(Corope
       }
 #pragma unroll
       for (int kk = 0; kk < kDkKeysPerWave; ++kk) {
-        const int c = wave * kDkKeysPerWave + kk;
         if (jw + kk > i) continue;   // wave-uniform: keys above the diagonal of this row (their tiles are zero anyway)
-        const float delta = mats[0][r][c], wij = mats[1][r][c];
+        const f32x4* el = reinterpret_cast<const f32x4*>(mats + (r * kDkKeys + wave * kDkKeysPerWave + kk) * MS);
+        f32x4 ev[MS / 4];
+#pragma unroll
+        for (int u = 0; u < MS / 4; ++u) ev[u] = el[u];
+        const float delta = ev[0][0], wij = ev[0][1];
         const float x = __builtin_amdgcn_fractf(delta * w_turn);
         const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
+        float u1 = 0.f, u2 = 0.f;   // dS-weighted sum of the group's queries: rotating it once rotates them all
 #pragma unroll
         for (int h = 0; h < G; ++h) {
-          const float ds = mats[2 + h][r][c], pr = mats[2 + G + h][r][c];
-          const float qt1 = __builtin_fmaf(cs, q1[h], -(sn * q2[h])), qt2 = __builtin_fmaf(cs, q2[h], sn * q1[h]);
-          dk1[kk] = __builtin_fmaf(ds, qt1, dk1[kk]);
-          dk2[kk] = __builtin_fmaf(ds, qt2, dk2[kk]);
+          const float dsv = ev[(2 + h) / 4][(2 + h) % 4], pr = ev[(2 + G + h) / 4][(2 + G + h) % 4];
+          u1 = __builtin_fmaf(dsv, q1[h], u1);
+          u2 = __builtin_fmaf(dsv, q2[h], u2);
           dv1[kk] = __builtin_fmaf(pr, o1[h], dv1[kk]);
           dv2[kk] = __builtin_fmaf(pr, o2[h], dv2[kk]);
         }
-        dk1[kk] = __builtin_fmaf(wij, q1[0], dk1[kk]);   // the leader's logit path (unrotated q)
+        dk1[kk] = __builtin_fmaf(cs, u1, __builtin_fmaf(-sn, u2, dk1[kk]));
+        dk2[kk] = __builtin_fmaf(cs, u2, __builtin_fmaf(sn, u1, dk2[kk]));
+        dk1[kk] = __builtin_fmaf(wij, q1[0], dk1[kk]);   // the leader's gate path (unrotated q)
         dk2[kk] = __builtin_fmaf(wij, q2[0], dk2[kk]);
       }
     }
@@ -424,14 +509,13 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(Corope
 
 // ---------------------------------------------------------------------------------------------------- host side
 int64_t corope_gqa_bwd_workspace_floats(int B, int Hq, int Hkv, int N) {
-  return (int64_t)N * N * (3 * (int64_t)B * Hkv + 2 * (int64_t)B * Hq);
+  return (int64_t)N * N * (2 * (int64_t)B * Hkv + 3 * (int64_t)B * Hq);
 }
 
 template <int D, int G>
 static hipError_t launch_corope_bwd_cfg(const CoropeBwdParams& p, const CoropeBwdWs& ws, const CoropeBwdFreqs& fr,
                                         hipStream_t stream) {
   const dim3 rows(p.N, p.B * p.Hkv);
-  hipLaunchKernelGGL(corope_bwd_gates_kernel<D>, rows, dim3(kWave), 0, stream, p, ws);
   hipLaunchKernelGGL((corope_bwd_scores_kernel<D, G>), rows, dim3(kWave), 0, stream, p, ws, fr);
   hipLaunchKernelGGL((corope_bwd_dq_kernel<D, G>), rows, dim3(kWave), 0, stream, p, ws, fr);
   using Cfg = CoropeDkCfg<D, G>;

@@ -65,17 +65,6 @@ __device__ __forceinline__ void softmax_pair(int j, const f32x16& sacc, u32x4 (&
   pb[j / 4][j % 4] = w;
 }
 
-// f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
-// in the body, so register arrays indexed with it never look dynamically indexed to the optimiser.
-template <int... I, class F>
-__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
-}
-
 __device__ __forceinline__ float wave_reduce_max(float x) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) x = fmaxf(x, __shfl_xor(x, m));
