@@ -77,6 +77,41 @@ struct RowRegs {
 __device__ __forceinline__ float bf16_to_f(uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
 __device__ __forceinline__ uint16_t f_to_bf16(float x) { return (uint16_t)(pack_bf16(x, 0.f) & 0xffffu); }
 
+// ---------------------------------------------------------------------------------------------------- row dots
+// out[idx][i][j] = a[idx * a_mul][i] . b[idx / b_div][j] for the tiles that touch the causal triangle: the two plain
+// matrix products of the backward (leader logits qL K^T per group: a_mul = G, b_div = 1; dP = dO V^T per head: a_mul
+// = 1, b_div = G) on the matrix cores.  Both operands of a 32 x 32 x 16 step are 16-byte pieces of rows, so they are
+// loaded straight from global memory; one wave owns 32 rows of `a` and sweeps four 32-key tiles with them.
+template <int D>
+__global__ __launch_bounds__(4 * kWave) void corope_bwd_rowdot_kernel(const uint16_t* a, const uint16_t* b, float* out,
+                                                                      int64_t NN, int N, int a_mul, int b_div) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int r = lane % 32, hf = lane / 32;
+  const int idx = blockIdx.z;
+  const int i0 = blockIdx.y * 128 + wave * 32, j0 = blockIdx.x * 128;
+  if (j0 > i0 + 31 || i0 >= N) return;   // every key of the block lies beyond this wave's rows
+  const uint16_t* arow = a + ((int64_t)idx * a_mul * N + min(i0 + r, N - 1)) * D + 8 * hf;
+  u32x4 af[D / 16];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) af[ks] = *reinterpret_cast<const u32x4*>(arow + 16 * ks);
+  float* obase = out + (int64_t)idx * NN;
+#pragma unroll 1
+  for (int jt = 0; jt < 4; ++jt) {
+    const int jj0 = j0 + 32 * jt;
+    if (jj0 > i0 + 31 || jj0 >= N) break;
+    const uint16_t* brow = b + ((int64_t)(idx / b_div) * N + min(jj0 + r, N - 1)) * D + 8 * hf;
+    f32x16 c = f32x16{0};
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) c = mfma32(af[ks], *reinterpret_cast<const u32x4*>(brow + 16 * ks), c);
+    const int col = jj0 + r;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int row = i0 + acc_row(e, hf);
+      if (row < N && col < N) obase[(int64_t)row * N + col] = c[e];
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------- scores
 // One wave per (group, query row i), all G heads at once, lane = key.  The row's queries and upstream gradients sit in
 // LDS as fp32 and are read with broadcast loads, a few rotation pairs ahead of their use (the scheduling barriers keep
@@ -85,9 +120,7 @@ template <int D, int G>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void corope_bwd_scores_kernel(CoropeBwdParams p, CoropeBwdWs ws, CoropeBwdFreqs fr) {
   constexpr int HALF = D / 2, QW = 2 * G;
   constexpr int CH = G <= 4 ? 4 : 2;                                  // rotation pairs per look-ahead chunk
-  __shared__ __attribute__((aligned(16))) float ql[D];                // the leader's row
   __shared__ __attribute__((aligned(16))) float qs[HALF * QW];        // [pair d][head][q1, q2]
-  __shared__ __attribute__((aligned(16))) float dos[D * G];           // [column][head]
   __shared__ __attribute__((aligned(16))) float wsm[HALF * 2];        // [pair d][turns, radians]
   const int i = p.N - 1 - blockIdx.x, g = blockIdx.y, lane = threadIdx.x;   // longest rows first
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
@@ -96,10 +129,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   for (int h = 0; h < G; ++h) {
     const int64_t off = ((int64_t)(head0 + h) * N + i) * D;
     for (int d = lane; d < D; d += kWave) {
-      const float qv = bf16_to_f(p.q[off + d]);
-      qs[(d % HALF) * QW + 2 * h + d / HALF] = qv;
-      if (h == 0) ql[d] = qv;
-      dos[d * G + h] = bf16_to_f(p.d_o[off + d]);
+      qs[(d % HALF) * QW + 2 * h + d / HALF] = bf16_to_f(p.q[off + d]);
     }
   }
   if (lane < HALF) {
@@ -108,7 +138,6 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   }
   __syncthreads();
   const uint16_t* kbase = p.k + (int64_t)g * N * D;
-  const uint16_t* vbase = p.v + (int64_t)g * N * D;
   const int64_t rowoff = (int64_t)i * N;
   const int n_chunks = i / kWave + 1;
 
@@ -128,26 +157,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     asm volatile("" ::: "memory");   // the LDS operands are loop-invariant: keep their loads inside the iteration
     RowRegs<D> kr;
     kr.load(kbase + (int64_t)jc * D);
-    // leader logit
-    float logit = 0.f;
-    {
-      const f32x4* q4 = reinterpret_cast<const f32x4*>(ql);
-      f32x4 qa = q4[0], qb = q4[1], na = qa, nb = qb;
-      static_for<D / 8>([&](auto c8_c) __attribute__((always_inline)) {
-        constexpr int c8 = decltype(c8_c)::value;
-        if (c8 + 1 < D / 8) {
-          na = q4[2 * c8 + 2];
-          nb = q4[2 * c8 + 3];
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) logit = __builtin_fmaf(qa[e], kr.at(8 * c8 + e), logit);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) logit = __builtin_fmaf(qb[e], kr.at(8 * c8 + 4 + e), logit);
-        __builtin_amdgcn_sched_barrier(0);
-        qa = na;
-        qb = nb;
-      });
-    }
+    const float logit = ws.delta(g)[rowoff + jc];   // qL . k from the row-dot pass; replaced by delta below
     const float z = valid ? 1.f / (1.f + __expf(-logit * p.sm_scale)) : 0.f;
     float suf = z;   // inclusive suffix sum over the lanes (keys) at and to the right of this one
 #pragma unroll
@@ -207,36 +217,9 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     // from the loads that feed it
 #pragma unroll
     for (int h = 0; h < G; ++h) asm volatile("" : "+v"(acc[h]), "+v"(gacc[h]));
-    // dP = dO . v
-    float dpv[G];
+    float dpv[G];   // dP = dO . v from the row-dot pass
 #pragma unroll
-    for (int h = 0; h < G; ++h) dpv[h] = 0.f;
-    {
-      RowRegs<D> vr;
-      vr.load(vbase + (int64_t)jc * D);
-      const f32x4* d4 = reinterpret_cast<const f32x4*>(dos);   // 4 columns x G heads = G vectors per step
-      f32x4 dc[G], dn[G];
-#pragma unroll
-      for (int u = 0; u < G; ++u) dc[u] = dn[u] = d4[u];
-      static_for<D / 4>([&](auto step_c) __attribute__((always_inline)) {
-        constexpr int d0 = decltype(step_c)::value * 4;
-        if (d0 + 4 < D) {
-#pragma unroll
-          for (int u = 0; u < G; ++u) dn[u] = d4[(d0 + 4) / 4 * G + u];
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float vv = vr.at(d0 + e);
-#pragma unroll
-          for (int h = 0; h < G; ++h) dpv[h] = __builtin_fmaf(dc[(e * G + h) / 4][(e * G + h) % 4], vv, dpv[h]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int u = 0; u < G; ++u) dc[u] = dn[u];
-      });
-    }
-#pragma unroll
-    for (int h = 0; h < G; ++h) asm volatile("" : "+v"(dpv[h]));
+    for (int h = 0; h < G; ++h) dpv[h] = ws.dp(head0 + h)[rowoff + jc];
     if (valid) {
       ws.delta(g)[rowoff + j] = delta;
       ws.w(g)[rowoff + j] = z * (1.f - z);   // the sigmoid's slope; replaced by W in the second sweep
@@ -245,7 +228,6 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
         const float s = acc[h] * p.sm_scale;
         ws.p(head0 + h)[rowoff + j] = s;
         ws.ds(head0 + h)[rowoff + j] = gacc[h] * p.sm_scale;
-        ws.dp(head0 + h)[rowoff + j] = dpv[h];
         const float m_new = fmaxf(m_run[h], s);
         const float a = __expf(m_run[h] - m_new), e = __expf(s - m_new);
         l_run[h] = __builtin_fmaf(l_run[h], a, e);
@@ -516,6 +498,11 @@ template <int D, int G>
 static hipError_t launch_corope_bwd_cfg(const CoropeBwdParams& p, const CoropeBwdWs& ws, const CoropeBwdFreqs& fr,
                                         hipStream_t stream) {
   const dim3 rows(p.N, p.B * p.Hkv);
+  const int nt = (p.N + 127) / 128;
+  hipLaunchKernelGGL(corope_bwd_rowdot_kernel<D>, dim3(nt, nt, p.B * p.Hkv), dim3(4 * kWave), 0, stream, p.q, p.k,
+                     ws.delta(0), ws.NN, p.N, G, 1);
+  hipLaunchKernelGGL(corope_bwd_rowdot_kernel<D>, dim3(nt, nt, p.B * p.Hq), dim3(4 * kWave), 0, stream, p.d_o, p.v,
+                     ws.dp(0), ws.NN, p.N, 1, G);
   hipLaunchKernelGGL((corope_bwd_scores_kernel<D, G>), rows, dim3(kWave), 0, stream, p, ws, fr);
   hipLaunchKernelGGL((corope_bwd_dq_kernel<D, G>), rows, dim3(kWave), 0, stream, p, ws, fr);
   using Cfg = CoropeDkCfg<D, G>;
