@@ -287,6 +287,18 @@ __device__ __forceinline__ void store_unrotated(const f32x16 (&acc)[D / 32], uin
     }
 }
 
+// Natural-order variant of load_a_trans: slot j of lane-half h <-> k = kbase + 8*h + j.
+__device__ __forceinline__ u32x4 load_a_trans_natural(const uint16_t* tile, int stride, int kbase, int m0) {
+  typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+  const int l = threadIdx.x % kWave;
+  const int blk = l / 16, s = l % 16, h = blk / 2;
+  const uint16_t* p = tile + (kbase + 8 * h + s / 4) * stride + m0 + 16 * (blk % 2) + 4 * (s % 4);
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * stride));
+  u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
+  return u32x4{a[0], a[1], b[0], b[1]};
+}
+
 // f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
 // in the body, so register arrays indexed with it never look dynamically indexed to the optimiser.
 template <int... I, class F>

@@ -122,7 +122,11 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   constexpr int CH = G <= 4 ? 4 : 2;                                  // rotation pairs per look-ahead chunk
   __shared__ __attribute__((aligned(16))) float qs[HALF * QW];        // [pair d][head][q1, q2]
   __shared__ __attribute__((aligned(16))) float wsm[HALF * 2];        // [pair d][turns, radians]
+  constexpr int KS = D + 8, WS = kWave + 8, NVR = 2 * G + 1, NDB = D / 32;
+  __shared__ __attribute__((aligned(16))) uint16_t kt[kWave * KS];    // [key][d] bf16: rotated keys, later plain keys
+  __shared__ __attribute__((aligned(16))) uint16_t wts[NVR * WS];     // [virtual row][key] bf16 weights of the keys
   const int i = p.N - 1 - blockIdx.x, g = blockIdx.y, lane = threadIdx.x;   // longest rows first
+  const int vr = lane % 32, hf = lane / 32;                                  // matrix-core identity of this lane
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
   const int head0 = b * p.Hq + kvh * G;   // first head of the group, as a (batch, head) slab index
 #pragma unroll
@@ -142,7 +146,14 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   const int n_chunks = i / kWave + 1;
 
   // ---- right to left: gates, delta, raw scores, dS/ddelta, dP, lane-local softmax statistics -------------------------
-  float m_run[G], l_run[G], pd_run[G];   // per lane: largest score, sum of exp(s - m), sum of exp(s - m) dP
+  // dq^h = c sum_j dS_j kt_j = c (sum_j e_j dP_j kt_j - Delta sum_j e_j kt_j) / L with e_j = exp(s_j - m): both sums are
+  // accumulated on the matrix cores as rows 2h and 2h + 1 of W (virtual rows x keys) times Kt (keys x d), rescaled
+  // flash-attention style when the row's running maximum m moves.  dqa[db][4g + e] belongs to virtual row `vr` and
+  // column 32 db + 8 g + 4 hf + e.
+  f32x16 dqa[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db) dqa[db] = f32x16{0};
+  float m_run[G], l_run[G], pd_run[G];   // running maximum (wave-uniform); per lane: sum of exp(s - m), of exp(s - m) dP
 #pragma unroll
   for (int h = 0; h < G; ++h) {
     m_run[h] = -INFINITY;
@@ -190,6 +201,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
             for (int h = 0; h < G; ++h) qn[e][h] = *reinterpret_cast<const f32x2*>(qs + (d0 + CH + e) * QW + 2 * h);
           }
         }
+        float r1v[CH], r2v[CH];
 #pragma unroll
         for (int e = 0; e < CH; ++e) {
           const int d = d0 + e;
@@ -198,11 +210,21 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
           const float k1 = kr.at(d), k2 = kr.at(d + HALF);
           const float r1 = __builtin_fmaf(cs, k1, sn * k2), r2 = __builtin_fmaf(cs, k2, -(sn * k1));
           const float t1 = wc[e][1] * r2, t2 = wc[e][1] * r1;
+          r1v[e] = r1;
+          r2v[e] = r2;
 #pragma unroll
           for (int h = 0; h < G; ++h) {
             acc[h] = __builtin_fmaf(qc[e][h][0], r1, __builtin_fmaf(qc[e][h][1], r2, acc[h]));
             gacc[h] = __builtin_fmaf(qc[e][h][0], t1, __builtin_fmaf(-qc[e][h][1], t2, gacc[h]));
           }
+        }
+        // the rotated key goes to LDS as bf16, row = this lane's key: the A operand of the dq products is read from there
+        if constexpr (CH == 4) {
+          *reinterpret_cast<u32x2*>(kt + lane * KS + d0) = u32x2{pack_bf16(r1v[0], r1v[1]), pack_bf16(r1v[2], r1v[3])};
+          *reinterpret_cast<u32x2*>(kt + lane * KS + HALF + d0) = u32x2{pack_bf16(r2v[0], r2v[1]), pack_bf16(r2v[2], r2v[3])};
+        } else {
+          *reinterpret_cast<uint32_t*>(kt + lane * KS + d0) = pack_bf16(r1v[0], r1v[1]);
+          *reinterpret_cast<uint32_t*>(kt + lane * KS + HALF + d0) = pack_bf16(r2v[0], r2v[1]);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -223,31 +245,71 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     if (valid) {
       ws.delta(g)[rowoff + j] = delta;
       ws.w(g)[rowoff + j] = z * (1.f - z);   // the sigmoid's slope; replaced by W in the second sweep
-#pragma unroll
-      for (int h = 0; h < G; ++h) {
-        const float s = acc[h] * p.sm_scale;
-        ws.p(head0 + h)[rowoff + j] = s;
-        ws.ds(head0 + h)[rowoff + j] = gacc[h] * p.sm_scale;
-        const float m_new = fmaxf(m_run[h], s);
-        const float a = __expf(m_run[h] - m_new), e = __expf(s - m_new);
-        l_run[h] = __builtin_fmaf(l_run[h], a, e);
-        pd_run[h] = __builtin_fmaf(pd_run[h], a, e * dpv[h]);
-        m_run[h] = m_new;
-      }
     }
+    float al = 1.f;          // this lane's virtual row's rescale factor
+    bool moved = false;      // wave-uniform: some head's running maximum moved
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      const float sc = acc[h] * p.sm_scale;
+      if (valid) {
+        ws.p(head0 + h)[rowoff + j] = sc;
+        ws.ds(head0 + h)[rowoff + j] = gacc[h] * p.sm_scale;
+      }
+      const float m_new = fmaxf(m_run[h], wave_max(valid ? sc : -INFINITY));   // finite: the chunk holds a key <= i
+      const float a = __expf(m_run[h] - m_new), e = valid ? __expf(sc - m_new) : 0.f;
+      moved |= m_new != m_run[h];
+      m_run[h] = m_new;
+      l_run[h] = __builtin_fmaf(l_run[h], a, e);
+      pd_run[h] = __builtin_fmaf(pd_run[h], a, e * dpv[h]);
+      al = (vr / 2 == h && vr < 2 * G) ? a : al;
+      wts[(2 * h) * WS + lane] = f_to_bf16(e * dpv[h]);
+      wts[(2 * h + 1) * WS + lane] = f_to_bf16(e);
+    }
+    if (moved) {
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dqa[db][e] *= al;
+    }
+    __syncthreads();   // rotated keys and weights are in LDS
+#pragma unroll
+    for (int ks = 0; ks < kWave / 16; ++ks) {
+      u32x4 bop = u32x4{0, 0, 0, 0};
+      if (vr < 2 * G) bop = *reinterpret_cast<const u32x4*>(wts + vr * WS + 16 * ks + 8 * hf);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) dqa[db] = mfma32(load_a_trans_natural(kt, KS, 16 * ks, 32 * db), bop, dqa[db]);
+    }
+    __syncthreads();   // ... and consumed: the next chunk may overwrite them
   }
   // row statistics: largest score, 1 / sum of exponentials, rowsum(P o dP)
   float m_row[G], inv_l[G], dsum[G];
 #pragma unroll
   for (int h = 0; h < G; ++h) {
-    m_row[h] = wave_max(m_run[h]);   // finite: lane 0 of chunk 0 always holds a key
-    const float f = m_run[h] == -INFINITY ? 0.f : __expf(m_run[h] - m_row[h]);
-    const float l = wave_sum(l_run[h] * f), pd = wave_sum(pd_run[h] * f);
+    m_row[h] = m_run[h];
+    const float l = wave_sum(l_run[h]), pd = wave_sum(pd_run[h]);
     inv_l[h] = 1.f / l;
     dsum[h] = pd * inv_l[h];
   }
 
-  // ---- left to right: P, dS, G_ij = sum_h dS dS/ddelta, its running sum over the keys, W ------------------------------
+  // even virtual row 2h: (sum e dP kt - Delta sum e kt) / L, the second sum sitting in the neighbouring lane; the rows from
+  // 2G on are still zero and row 2G collects the leader's gate path below
+  {
+    float my_inv = 0.f, my_dsum = 0.f;
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      my_inv = vr / 2 == h ? inv_l[h] : my_inv;
+      my_dsum = vr / 2 == h ? dsum[h] : my_dsum;
+    }
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float other = __shfl_xor(dqa[db][e], 1);
+        if (vr < 2 * G) dqa[db][e] = (dqa[db][e] - my_dsum * other) * my_inv;
+      }
+  }
+
+  // ---- left to right: P, dS, G_ij = sum_h dS dS/ddelta, its running sum over the keys, W, and W K for the leader -------
   float gcarry = 0.f;
 #pragma unroll 1
   for (int c = 0; c < n_chunks; ++c) {
@@ -273,112 +335,126 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       const float t = __shfl_up(pre, off);
       if (lane >= off) pre += t;
     }
-    if (valid) ws.w(g)[rowoff + j] = (gcarry + pre - gij) * slope;   // (sum of G over the keys j < t) z'(t)
+    const float wij = valid ? (gcarry + pre - gij) * slope : 0.f;   // (sum of G over the keys j < t) z'(t)
+    if (valid) ws.w(g)[rowoff + j] = wij;
     gcarry += __shfl(pre, kWave - 1);
+    // leader's gate path: row 2G of the accumulators += W (1 x keys) K (keys x d)
+    {
+      const uint16_t* src = kbase + (int64_t)(valid ? j : i) * D;
+#pragma unroll
+      for (int v8 = 0; v8 < D / 8; ++v8)
+        *reinterpret_cast<u32x4*>(kt + lane * KS + 8 * v8) = *reinterpret_cast<const u32x4*>(src + 8 * v8);
+      wts[(2 * G) * WS + lane] = f_to_bf16(wij);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < kWave / 16; ++ks) {
+      u32x4 bop = u32x4{0, 0, 0, 0};
+      if (vr == 2 * G) bop = *reinterpret_cast<const u32x4*>(wts + vr * WS + 16 * ks + 8 * hf);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) dqa[db] = mfma32(load_a_trans_natural(kt, KS, 16 * ks, 32 * db), bop, dqa[db]);
+    }
+    __syncthreads();
+  }
+  // dq: even virtual rows hold the heads' gradients; the leader adds the gate path from row 2G of its lane half
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const float gate = __shfl(dqa[db][e], 32 * hf + 2 * G);
+      if (vr == 0) dqa[db][e] += gate;
+    }
+  if (vr < 2 * G && vr % 2 == 0) {
+    uint16_t* op = p.dq + ((int64_t)(head0 + vr / 2) * N + i) * D;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const u32x2 w = {pack_bf16(dqa[db][4 * g4] * p.sm_scale, dqa[db][4 * g4 + 1] * p.sm_scale),
+                         pack_bf16(dqa[db][4 * g4 + 2] * p.sm_scale, dqa[db][4 * g4 + 3] * p.sm_scale)};
+        *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
+      }
   }
 }
 
-// ---------------------------------------------------------------------------------------------------- dq
-// One wave per (group, query row i), lane = rotation pair (d, d + D/2).  The key chunk is staged in LDS; the row's
-// scalars (delta, W, dS per head) are loaded with lane = key and handed out with readlane.
+// ---------------------------------------------------------------------------------------------------- dv
+// dv_j = sum_{h, i} P^h_ij dO^h_i on the matrix cores: dv^T (d x keys) += dO^T (d x rows) P (rows x keys), 16 rows per
+// step.  One workgroup of 4 waves owns 128 keys (32 per wave) of one group; the 16 dO rows of every head are staged in
+// LDS and read transposed; P comes straight from the workspace (lane = key: 128-byte lines) and is rounded to bf16.
 template <int D, int G>
-__global__ __launch_bounds__(kWave) void corope_bwd_dq_kernel(CoropeBwdParams p, CoropeBwdWs ws, CoropeBwdFreqs fr) {
-  constexpr int HALF = D / 2;
-  __shared__ __attribute__((aligned(16))) uint16_t kch[kWave][D];   // 64 keys x D, bf16
-  const int i = p.N - 1 - blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+__global__ __launch_bounds__(4 * kWave) void corope_bwd_dv_kernel(CoropeBwdParams p, CoropeBwdWs ws) {
+  constexpr int TS = D + 16, NDB = D / 32, NT = 4 * kWave, ROWS = 16;
+  __shared__ __attribute__((aligned(16))) uint16_t tile[G * ROWS * TS];
+  const int jb = blockIdx.x * 128, g = blockIdx.y;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int r = lane % 32, hf = lane / 32;
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
   const int head0 = b * p.Hq + kvh * G;
-  const bool act = lane < HALF;           // D = 64 leaves the upper half of the wave without a pair
-  const int dpair = act ? lane : 0;
-  const float w_turn = fr.turns[dpair];
-  float dq1[G], dq2[G];
+  const int jw = jb + 32 * wave, j = jw + r;
+  f32x16 acc[NDB];
 #pragma unroll
-  for (int h = 0; h < G; ++h) dq1[h] = dq2[h] = 0.f;
-  float dql1 = 0.f, dql2 = 0.f;   // the leader's extra gradient through its gates
-  const uint16_t* kbase = p.k + (int64_t)g * N * D;
-  const int64_t rowoff = (int64_t)i * N;
-  const int n_chunks = i / kWave + 1;
-  // the next chunk's key row and scalars are fetched into registers while the current chunk is consumed
-  u32x4 kv[D / 8];
-  int dnext, wnext, dsnext[G];
-  auto fetch = [&](int c) __attribute__((always_inline)) {
-    const int jl = c * kWave + lane;
-    const bool valid = jl <= i;
-    const uint16_t* src = kbase + (int64_t)(valid ? jl : i) * D;
-#pragma unroll
-    for (int v8 = 0; v8 < D / 8; ++v8) kv[v8] = *reinterpret_cast<const u32x4*>(src + 8 * v8);
-    dnext = valid ? __builtin_bit_cast(int, ws.delta(g)[rowoff + jl]) : 0;
-    wnext = valid ? __builtin_bit_cast(int, ws.w(g)[rowoff + jl]) : 0;
-#pragma unroll
-    for (int h = 0; h < G; ++h) dsnext[h] = valid ? __builtin_bit_cast(int, ws.ds(head0 + h)[rowoff + jl]) : 0;
-  };
-  fetch(0);
+  for (int db = 0; db < NDB; ++db) acc[db] = f32x16{0};
 #pragma unroll 1
-  for (int c = 0; c < n_chunks; ++c) {
-    const int j0 = c * kWave;
-    __syncthreads();   // the previous chunk's keys are no longer needed
-#pragma unroll
-    for (int v8 = 0; v8 < D / 8; ++v8) *reinterpret_cast<u32x4*>(&kch[lane][8 * v8]) = kv[v8];
-    const int dvec = dnext, wvec = wnext;
-    int dsvec[G];
-#pragma unroll
-    for (int h = 0; h < G; ++h) dsvec[h] = dsnext[h];
+  for (int i0 = jb; i0 < N; i0 += ROWS) {
     __syncthreads();
-    if (c + 1 < n_chunks) fetch(c + 1);
-    const int n_here = min(kWave, i - j0 + 1);
-    for (int jj = 0; jj < n_here; ++jj) {
-      const float delta = __builtin_bit_cast(float, __builtin_amdgcn_readlane(dvec, jj));
-      const float wij = __builtin_bit_cast(float, __builtin_amdgcn_readlane(wvec, jj));
-      const float k1 = bf16_to_f(kch[jj][dpair]), k2 = bf16_to_f(kch[jj][dpair + HALF]);
-      const float x = __builtin_amdgcn_fractf(delta * w_turn);
-      const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
-      const float kt1 = __builtin_fmaf(cs, k1, sn * k2), kt2 = __builtin_fmaf(cs, k2, -(sn * k1));
+    for (int e = threadIdx.x; e < G * ROWS * (D / 8); e += NT) {
+      const int h = e / (ROWS * (D / 8)), rr = (e / (D / 8)) % ROWS, v8 = e % (D / 8);
+      const int64_t off = ((int64_t)(head0 + h) * N + min(i0 + rr, N - 1)) * D + 8 * v8;
+      *reinterpret_cast<u32x4*>(tile + (h * ROWS + rr) * TS + 8 * v8) = *reinterpret_cast<const u32x4*>(p.d_o + off);
+    }
+    __syncthreads();
+    if (i0 + ROWS - 1 >= jw && jw < N) {   // wave-uniform: some row of the step sees a key of this wave
 #pragma unroll
       for (int h = 0; h < G; ++h) {
-        const float dsv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(dsvec[h], jj));
-        dq1[h] = __builtin_fmaf(dsv, kt1, dq1[h]);
-        dq2[h] = __builtin_fmaf(dsv, kt2, dq2[h]);
+        float pv[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          const int i = i0 + 8 * hf + t;
+          pv[t] = (i < N && j <= i) ? ws.p(head0 + h)[(int64_t)i * N + j] : 0.f;   // nothing outside the triangle is defined
+        }
+        const u32x4 bop = {pack_bf16(pv[0], pv[1]), pack_bf16(pv[2], pv[3]), pack_bf16(pv[4], pv[5]), pack_bf16(pv[6], pv[7])};
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+          acc[db] = mfma32(load_a_trans_natural(tile + h * ROWS * TS, TS, 0, 32 * db), bop, acc[db]);
       }
-      dql1 = __builtin_fmaf(wij, k1, dql1);
-      dql2 = __builtin_fmaf(wij, k2, dql2);
     }
   }
-  if (act) {
+  if (j < N) {
+    uint16_t* op = p.dv + ((int64_t)g * N + j) * D;
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-      const int64_t off = ((int64_t)(head0 + h) * N + i) * D;
-      const float a1 = dq1[h] + (h == 0 ? dql1 : 0.f), a2 = dq2[h] + (h == 0 ? dql2 : 0.f);
-      p.dq[off + dpair] = f_to_bf16(a1 * p.sm_scale);
-      p.dq[off + dpair + HALF] = f_to_bf16(a2 * p.sm_scale);
-    }
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const u32x2 w = {pack_bf16(acc[db][4 * g4], acc[db][4 * g4 + 1]), pack_bf16(acc[db][4 * g4 + 2], acc[db][4 * g4 + 3])};
+        *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
+      }
   }
 }
 
-// ---------------------------------------------------------------------------------------------------- dk, dv
+// ---------------------------------------------------------------------------------------------------- dk
 // One workgroup of 4 waves per (group, block of 32 keys); each wave owns 8 of the keys, lane = rotation pair.  Query
-// rows are visited 16 at a time: the 16 x 32 tiles of DELTA, W, DS^h, P^h (interleaved per element, so that one (row,
-// key) costs a few 16-byte broadcast reads) and the 16 rows of q and dO of every head are staged in LDS, so the
-// column-wise access of the N x N matrices costs full 128-byte lines.
+// rows are visited 16 at a time: the 16 x 32 tiles of DELTA, W, DS^h (interleaved per element, so that one (row, key)
+// costs a few 16-byte broadcast reads) and the 16 rows of q of every head are staged in LDS, so the column-wise access
+// of the N x N matrices costs full 128-byte lines.
 constexpr int kDkKeys = 32, kDkRows = 16, kDkWaves = 4, kDkKeysPerWave = kDkKeys / kDkWaves;
 
 template <int D, int G>
 struct CoropeDkCfg {
-  static constexpr int kMats = 2 + 2 * G;                                   // DELTA, W, DS^h, P^h
+  static constexpr int kMats = 2 + G;                                       // DELTA, W, DS^h
   static constexpr int kMS = (kMats + 3) / 4 * 4;                           // floats per (row, key) element
   static constexpr int kMatBytes = kMS * kDkRows * kDkKeys * 4;
-  static constexpr int kRowBytes = kDkRows * G * D * 2;                     // q rows (and as many dO rows), bf16
-  static constexpr int kLdsBytes = kMatBytes + 2 * kRowBytes;
+  static constexpr int kRowBytes = kDkRows * G * D * 2;                     // q rows, bf16
+  static constexpr int kLdsBytes = kMatBytes + kRowBytes;
 };
 
 template <int D, int G>
-__global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(CoropeBwdParams p, CoropeBwdWs ws,
+__global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBwdParams p, CoropeBwdWs ws,
                                                                          CoropeBwdFreqs fr) {
   using Cfg = CoropeDkCfg<D, G>;
   constexpr int HALF = D / 2, NT = kDkWaves * kWave, MS = Cfg::kMS;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float* mats = reinterpret_cast<float*>(smem);                                          // [row][key][MS]
   uint16_t (*qrows)[G][D] = reinterpret_cast<uint16_t (*)[G][D]>(smem + Cfg::kMatBytes);
-  uint16_t (*dorows)[G][D] = reinterpret_cast<uint16_t (*)[G][D]>(smem + Cfg::kMatBytes + Cfg::kRowBytes);
 
   const int jb = blockIdx.x * kDkKeys, g = blockIdx.y;   // the first key blocks see the most rows and start first
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -389,21 +465,21 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(Corope
   const float w_turn = fr.turns[dpair];
   const int jw = jb + wave * kDkKeysPerWave;   // first key of this wave
 
-  float dk1[kDkKeysPerWave], dk2[kDkKeysPerWave], dv1[kDkKeysPerWave], dv2[kDkKeysPerWave];
+  float dk1[kDkKeysPerWave], dk2[kDkKeysPerWave];
 #pragma unroll
-  for (int kk = 0; kk < kDkKeysPerWave; ++kk) dk1[kk] = dk2[kk] = dv1[kk] = dv2[kk] = 0.f;
+  for (int kk = 0; kk < kDkKeysPerWave; ++kk) dk1[kk] = dk2[kk] = 0.f;
 
   // Staging: thread -> key column c and row r = rsub or rsub + 8 of the 16 x 32 tiles, plus its share of the 16-byte
-  // pieces of the q / dO rows.  The next tile's values are fetched into registers while the current tile is consumed.
+  // pieces of the q rows.  The next tile's values are fetched into registers while the current tile is consumed.
   constexpr int kRowItems = kDkRows * G * (D / 8), RI = (kRowItems + NT - 1) / NT;
   const int sc = threadIdx.x % kDkKeys, rsub = threadIdx.x / kDkKeys;
   float mv[2 * Cfg::kMats];
-  u32x4 qv[RI], ov[RI];
+  u32x4 qv[RI];
   auto fetch = [&](int i0) __attribute__((always_inline)) {
     static_for<2 * Cfg::kMats>([&](auto k_c) __attribute__((always_inline)) {
       constexpr int k = decltype(k_c)::value, m = k / 2;
       const int i = i0 + rsub + 8 * (k % 2), j = jb + sc;
-      const float* src = m == 0 ? ws.delta(g) : m == 1 ? ws.w(g) : m < 2 + G ? ws.ds(head0 + m - 2) : ws.p(head0 + m - 2 - G);
+      const float* src = m == 0 ? ws.delta(g) : m == 1 ? ws.w(g) : ws.ds(head0 + m - 2);
       mv[k] = (i < N && j <= i) ? src[(int64_t)i * N + j] : 0.f;   // zero outside the causal triangle and past N
     });
     static_for<RI>([&](auto k_c) __attribute__((always_inline)) {
@@ -413,7 +489,6 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(Corope
         const int r = e / (G * (D / 8)), h = (e / (D / 8)) % G, v8 = e % (D / 8);
         const int64_t off = ((int64_t)(head0 + h) * N + min(i0 + r, N - 1)) * D + 8 * v8;
         qv[k] = *reinterpret_cast<const u32x4*>(p.q + off);
-        ov[k] = *reinterpret_cast<const u32x4*>(p.d_o + off);
       }
     });
   };
@@ -432,7 +507,6 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(Corope
       if (kRowItems % NT == 0 || e < kRowItems) {
         const int r = e / (G * (D / 8)), h = (e / (D / 8)) % G, v8 = e % (D / 8);
         *reinterpret_cast<u32x4*>(&qrows[r][h][8 * v8]) = qv[k];
-        *reinterpret_cast<u32x4*>(&dorows[r][h][8 * v8]) = ov[k];
       }
     });
     __syncthreads();
@@ -441,13 +515,11 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(Corope
 #pragma unroll 1
     for (int r = 0; r < n_rows; ++r) {
       const int i = i0 + r;
-      float q1[G], q2[G], o1[G], o2[G];
+      float q1[G], q2[G];
 #pragma unroll
       for (int h = 0; h < G; ++h) {
         q1[h] = bf16_to_f(qrows[r][h][dpair]);
         q2[h] = bf16_to_f(qrows[r][h][dpair + HALF]);
-        o1[h] = bf16_to_f(dorows[r][h][dpair]);
-        o2[h] = bf16_to_f(dorows[r][h][dpair + HALF]);
       }
 #pragma unroll
       for (int kk = 0; kk < kDkKeysPerWave; ++kk) {
@@ -462,11 +534,9 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(Corope
         float u1 = 0.f, u2 = 0.f;   // dS-weighted sum of the group's queries: rotating it once rotates them all
 #pragma unroll
         for (int h = 0; h < G; ++h) {
-          const float dsv = ev[(2 + h) / 4][(2 + h) % 4], pr = ev[(2 + G + h) / 4][(2 + G + h) % 4];
+          const float dsv = ev[(2 + h) / 4][(2 + h) % 4];
           u1 = __builtin_fmaf(dsv, q1[h], u1);
           u2 = __builtin_fmaf(dsv, q2[h], u2);
-          dv1[kk] = __builtin_fmaf(pr, o1[h], dv1[kk]);
-          dv2[kk] = __builtin_fmaf(pr, o2[h], dv2[kk]);
         }
         dk1[kk] = __builtin_fmaf(cs, u1, __builtin_fmaf(-sn, u2, dk1[kk]));
         dk2[kk] = __builtin_fmaf(cs, u2, __builtin_fmaf(sn, u1, dk2[kk]));
@@ -483,8 +553,6 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dkdv_kernel(Corope
       const int64_t off = ((int64_t)g * N + j) * D;
       p.dk[off + dpair] = f_to_bf16(dk1[kk] * p.sm_scale);
       p.dk[off + dpair + HALF] = f_to_bf16(dk2[kk] * p.sm_scale);
-      p.dv[off + dpair] = f_to_bf16(dv1[kk]);
-      p.dv[off + dpair + HALF] = f_to_bf16(dv2[kk]);
     }
   }
 }
@@ -504,9 +572,9 @@ static hipError_t launch_corope_bwd_cfg(const CoropeBwdParams& p, const CoropeBw
   hipLaunchKernelGGL(corope_bwd_rowdot_kernel<D>, dim3(nt, nt, p.B * p.Hq), dim3(4 * kWave), 0, stream, p.d_o, p.v,
                      ws.dp(0), ws.NN, p.N, 1, G);
   hipLaunchKernelGGL((corope_bwd_scores_kernel<D, G>), rows, dim3(kWave), 0, stream, p, ws, fr);
-  hipLaunchKernelGGL((corope_bwd_dq_kernel<D, G>), rows, dim3(kWave), 0, stream, p, ws, fr);
   using Cfg = CoropeDkCfg<D, G>;
-  auto kern = corope_bwd_dkdv_kernel<D, G>;
+  hipLaunchKernelGGL((corope_bwd_dv_kernel<D, G>), dim3((p.N + 127) / 128, p.B * p.Hkv), dim3(4 * kWave), 0, stream, p, ws);
+  auto kern = corope_bwd_dk_kernel<D, G>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

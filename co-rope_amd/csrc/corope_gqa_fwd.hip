@@ -54,18 +54,6 @@ struct CoropeCfg {
   static constexpr int kLdsBytes = kOffW + kWBytes;
 };
 
-// Natural-order variant of load_a_trans: slot j of lane-half h <-> k = kbase + 8*h + j.
-__device__ __forceinline__ u32x4 load_a_trans_natural(const uint16_t* tile, int stride, int kbase, int m0) {
-  typedef __attribute__((address_space(3))) s16x4* lds_ptr;
-  const int l = threadIdx.x % kWave;
-  const int blk = l / 16, s = l % 16, h = blk / 2;
-  const uint16_t* p = tile + (kbase + 8 * h + s / 4) * stride + m0 + 16 * (blk % 2) + 4 * (s % 4);
-  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
-  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * stride));
-  u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
-  return u32x4{a[0], a[1], b[0], b[1]};
-}
-
 template <int D, int G>
 __global__ __launch_bounds__(kCoWaves* kWave) void corope_gqa_fwd_kernel(CoropeParams p, CoropeFreqs fr) {
   using Cfg = CoropeCfg<D, G>;
