@@ -113,16 +113,16 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_rowdot_kernel(const uint
 }
 
 // ---------------------------------------------------------------------------------------------------- scores
-// One wave per (group, query row i), all G heads at once, lane = key.  The row's queries and upstream gradients sit in
-// LDS as fp32 and are read with broadcast loads, a few rotation pairs ahead of their use (the scheduling barriers keep
-// the fully unrolled loops from pulling every LDS read to the top).
+// One wave per (group, query row i), all G heads at once, lane = key.  Per 64-key chunk the lanes rotate their keys
+// (the only place sines and cosines are evaluated) and park them in LDS as bf16; everything that is a dot product with
+// the rotated key then runs on the matrix cores: the raw scores q^h . kt and their derivatives with respect to delta
+// (rows [-w q2, w q1] . kt) as one (2G x D) x (D x 64 keys) product, and the dq sums as (weights x keys) x (keys x D).
 template <int D, int G>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void corope_bwd_scores_kernel(CoropeBwdParams p, CoropeBwdWs ws, CoropeBwdFreqs fr) {
-  constexpr int HALF = D / 2, QW = 2 * G;
-  constexpr int CH = G <= 4 ? 4 : 2;                                  // rotation pairs per look-ahead chunk
-  __shared__ __attribute__((aligned(16))) float qs[HALF * QW];        // [pair d][head][q1, q2]
-  __shared__ __attribute__((aligned(16))) float wsm[HALF * 2];        // [pair d][turns, radians]
+  constexpr int HALF = D / 2;
   constexpr int KS = D + 8, WS = kWave + 8, NVR = 2 * G + 1, NDB = D / 32;
+  constexpr int NI = 4 * ((2 * G - 1) / 8 + 1);                       // accumulator registers that hold rows < 2G
+  __shared__ __attribute__((aligned(16))) uint16_t qa[2 * G * KS];    // rows h: q^h; rows G + h: [-w q2^h, w q1^h]
   __shared__ __attribute__((aligned(16))) uint16_t kt[kWave * KS];    // [key][d] bf16: rotated keys, later plain keys
   __shared__ __attribute__((aligned(16))) uint16_t wts[NVR * WS];     // [virtual row][key] bf16 weights of the keys
   const int i = p.N - 1 - blockIdx.x, g = blockIdx.y, lane = threadIdx.x;   // longest rows first
@@ -131,21 +131,21 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   const int head0 = b * p.Hq + kvh * G;   // first head of the group, as a (batch, head) slab index
 #pragma unroll
   for (int h = 0; h < G; ++h) {
-    const int64_t off = ((int64_t)(head0 + h) * N + i) * D;
-    for (int d = lane; d < D; d += kWave) {
-      qs[(d % HALF) * QW + 2 * h + d / HALF] = bf16_to_f(p.q[off + d]);
+    const uint16_t* qrow = p.q + ((int64_t)(head0 + h) * N + i) * D;
+    for (int d = lane; d < HALF; d += kWave) {
+      const uint16_t a1 = qrow[d], a2 = qrow[d + HALF];
+      qa[h * KS + d] = a1;
+      qa[h * KS + d + HALF] = a2;
+      qa[(G + h) * KS + d] = f_to_bf16(-fr.rad[d] * bf16_to_f(a2));
+      qa[(G + h) * KS + d + HALF] = f_to_bf16(fr.rad[d] * bf16_to_f(a1));
     }
-  }
-  if (lane < HALF) {
-    wsm[2 * lane] = fr.turns[lane];
-    wsm[2 * lane + 1] = fr.rad[lane];
   }
   __syncthreads();
   const uint16_t* kbase = p.k + (int64_t)g * N * D;
   const int64_t rowoff = (int64_t)i * N;
   const int n_chunks = i / kWave + 1;
 
-  // ---- right to left: gates, delta, raw scores, dS/ddelta, dP, lane-local softmax statistics -------------------------
+  // ---- right to left: gates, delta, raw scores, dS/ddelta, softmax statistics, dq sums --------------------------------
   // dq^h = c sum_j dS_j kt_j = c (sum_j e_j dP_j kt_j - Delta sum_j e_j kt_j) / L with e_j = exp(s_j - m): both sums are
   // accumulated on the matrix cores as rows 2h and 2h + 1 of W (virtual rows x keys) times Kt (keys x d), rescaled
   // flash-attention style when the row's running maximum m moves.  dqa[db][4g + e] belongs to virtual row `vr` and
@@ -165,10 +165,9 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     const int j = c * kWave + lane;
     const bool valid = j <= i;
     const int jc = valid ? j : i;
-    asm volatile("" ::: "memory");   // the LDS operands are loop-invariant: keep their loads inside the iteration
+    const float logit = ws.delta(g)[rowoff + jc];   // qL . k from the row-dot pass; replaced by delta below
     RowRegs<D> kr;
     kr.load(kbase + (int64_t)jc * D);
-    const float logit = ws.delta(g)[rowoff + jc];   // qL . k from the row-dot pass; replaced by delta below
     const float z = valid ? 1.f / (1.f + __expf(-logit * p.sm_scale)) : 0.f;
     float suf = z;   // inclusive suffix sum over the lanes (keys) at and to the right of this one
 #pragma unroll
@@ -179,66 +178,50 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     const float delta = carry + suf - z;   // gates strictly to the right, up to and including the diagonal
     carry += __shfl(suf, 0);
 
-    // rotated dot products of every head, and their derivative with respect to delta
+    // the key rotated by -delta w_d goes to LDS as bf16, row = this lane's key
+    static_for<HALF / 4>([&](auto step_c) __attribute__((always_inline)) {
+      constexpr int d0 = decltype(step_c)::value * 4;
+      float r1v[4], r2v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float x = __builtin_amdgcn_fractf(delta * fr.turns[d0 + e]);
+        const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
+        const float k1 = kr.at(d0 + e), k2 = kr.at(d0 + e + HALF);
+        r1v[e] = __builtin_fmaf(cs, k1, sn * k2);
+        r2v[e] = __builtin_fmaf(cs, k2, -(sn * k1));
+      }
+      *reinterpret_cast<u32x2*>(kt + lane * KS + d0) = u32x2{pack_bf16(r1v[0], r1v[1]), pack_bf16(r1v[2], r1v[3])};
+      *reinterpret_cast<u32x2*>(kt + lane * KS + HALF + d0) = u32x2{pack_bf16(r2v[0], r2v[1]), pack_bf16(r2v[2], r2v[3])};
+    });
+    __syncthreads();   // rotated keys are in LDS
+
+    // (2G rows x D) x (D x 64 keys): lane = (row vr, half hf) for the A operand, (key vr [+ 32], half hf) for B
+    f32x16 c0 = f32x16{0}, c1 = f32x16{0};
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      u32x4 aop = u32x4{0, 0, 0, 0};
+      if (vr < 2 * G) aop = *reinterpret_cast<const u32x4*>(qa + vr * KS + 16 * ks + 8 * hf);
+      c0 = mfma32(aop, *reinterpret_cast<const u32x4*>(kt + vr * KS + 16 * ks + 8 * hf), c0);
+      c1 = mfma32(aop, *reinterpret_cast<const u32x4*>(kt + (32 + vr) * KS + 16 * ks + 8 * hf), c1);
+    }
+    // the results sit at lane = key % 32 with rows split over the lane halves; swapping the upper half of the keys-below-
+    // 32 result with the lower half of the keys-from-32 result puts every key's rows into its own lane
+    float lo_rows[NI], hi_rows[NI];   // rows 8 (n / 4) + n % 4 and the same + 4
+#pragma unroll
+    for (int n = 0; n < NI; ++n) {
+      const float x0 = c0[n], x1 = c1[n];   // (a bit_cast applied directly to a vector element reads element 0)
+      const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x0), __builtin_bit_cast(uint32_t, x1),
+                                                      false, false);
+      lo_rows[n] = __builtin_bit_cast(float, (uint32_t)r[0]);
+      hi_rows[n] = __builtin_bit_cast(float, (uint32_t)r[1]);
+    }
     float acc[G], gacc[G];
 #pragma unroll
-    for (int h = 0; h < G; ++h) acc[h] = gacc[h] = 0.f;
-    {
-      f32x2 qc[CH][G], qn[CH][G], wc[CH], wn[CH];
-#pragma unroll
-      for (int e = 0; e < CH; ++e) {
-        wc[e] = wn[e] = *reinterpret_cast<const f32x2*>(wsm + 2 * e);
-#pragma unroll
-        for (int h = 0; h < G; ++h) qc[e][h] = qn[e][h] = *reinterpret_cast<const f32x2*>(qs + e * QW + 2 * h);
-      }
-      static_for<HALF / CH>([&](auto step_c) __attribute__((always_inline)) {
-        constexpr int d0 = decltype(step_c)::value * CH;
-        if (d0 + CH < HALF) {
-#pragma unroll
-          for (int e = 0; e < CH; ++e) {
-            wn[e] = *reinterpret_cast<const f32x2*>(wsm + 2 * (d0 + CH + e));
-#pragma unroll
-            for (int h = 0; h < G; ++h) qn[e][h] = *reinterpret_cast<const f32x2*>(qs + (d0 + CH + e) * QW + 2 * h);
-          }
-        }
-        float r1v[CH], r2v[CH];
-#pragma unroll
-        for (int e = 0; e < CH; ++e) {
-          const int d = d0 + e;
-          const float x = __builtin_amdgcn_fractf(delta * wc[e][0]);
-          const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
-          const float k1 = kr.at(d), k2 = kr.at(d + HALF);
-          const float r1 = __builtin_fmaf(cs, k1, sn * k2), r2 = __builtin_fmaf(cs, k2, -(sn * k1));
-          const float t1 = wc[e][1] * r2, t2 = wc[e][1] * r1;
-          r1v[e] = r1;
-          r2v[e] = r2;
-#pragma unroll
-          for (int h = 0; h < G; ++h) {
-            acc[h] = __builtin_fmaf(qc[e][h][0], r1, __builtin_fmaf(qc[e][h][1], r2, acc[h]));
-            gacc[h] = __builtin_fmaf(qc[e][h][0], t1, __builtin_fmaf(-qc[e][h][1], t2, gacc[h]));
-          }
-        }
-        // the rotated key goes to LDS as bf16, row = this lane's key: the A operand of the dq products is read from there
-        if constexpr (CH == 4) {
-          *reinterpret_cast<u32x2*>(kt + lane * KS + d0) = u32x2{pack_bf16(r1v[0], r1v[1]), pack_bf16(r1v[2], r1v[3])};
-          *reinterpret_cast<u32x2*>(kt + lane * KS + HALF + d0) = u32x2{pack_bf16(r2v[0], r2v[1]), pack_bf16(r2v[2], r2v[3])};
-        } else {
-          *reinterpret_cast<uint32_t*>(kt + lane * KS + d0) = pack_bf16(r1v[0], r1v[1]);
-          *reinterpret_cast<uint32_t*>(kt + lane * KS + HALF + d0) = pack_bf16(r2v[0], r2v[1]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int e = 0; e < CH; ++e) {
-          wc[e] = wn[e];
-#pragma unroll
-          for (int h = 0; h < G; ++h) qc[e][h] = qn[e][h];
-        }
-      });
+    for (int h = 0; h < G; ++h) {
+      const int ra = h, rb = G + h;
+      acc[h] = (ra / 4) % 2 ? hi_rows[4 * (ra / 8) + ra % 4] : lo_rows[4 * (ra / 8) + ra % 4];
+      gacc[h] = (rb / 4) % 2 ? hi_rows[4 * (rb / 8) + rb % 4] : lo_rows[4 * (rb / 8) + rb % 4];
     }
-    // the sums are used only under `valid` below: pin them here, or the whole chain is sunk into that branch, away
-    // from the loads that feed it
-#pragma unroll
-    for (int h = 0; h < G; ++h) asm volatile("" : "+v"(acc[h]), "+v"(gacc[h]));
     float dpv[G];   // dP = dO . v from the row-dot pass
 #pragma unroll
     for (int h = 0; h < G; ++h) dpv[h] = ws.dp(head0 + h)[rowoff + jc];

@@ -58,9 +58,10 @@ def test_corope_backward_parity(pkg, B, Hq, Hkv, N, D):
 
 
 def test_corope_backward_unit_scale_small_theta(pkg):
-    """sm_scale = 1 and a small base: fast rotations make the path through the gates a large part of dQ and dK."""
+    """sm_scale = 1 and a small base: fast rotations make the path through the gates a large part of dQ and dK.
+    dO is halved so that the gradients stay below 4, where half a bf16 step of the result alone is under 8e-3."""
     q, k, v, d_o = _inputs(1, 4, 2, 48, 64, seed=7)
-    q, k = bf16_round(q * 0.3), bf16_round(k * 0.3)
+    q, k, d_o = bf16_round(q * 0.3), bf16_round(k * 0.3), d_o * 0.5
     _compare(_gpu_grads(pkg, q, k, v, d_o, 1.0, 100.0), _oracle_grads(q, k, v, d_o, 1.0, 100.0), 2)
 
 
@@ -69,7 +70,7 @@ def test_corope_backward_gate_path_is_material_and_right(pkg):
     position offsets cut out of the graph differs by far more than the bar), so parity here pins that path; a
     central finite difference through the dense forward pins the oracle's own gradient for one leader coordinate."""
     q, k, v, d_o = _inputs(1, 4, 2, 48, 64, seed=7)
-    q, k = bf16_round(q * 0.3), bf16_round(k * 0.3)
+    q, k, d_o = bf16_round(q * 0.3), bf16_round(k * 0.3), d_o * 0.5
     full = _oracle_grads(q, k, v, d_o, 1.0, 100.0)
     qd, kd, vd = (t.double().requires_grad_(True) for t in (q, k, v))
     o = C.corope_gqa_forward(qd, kd, vd, True, 1.0, 100.0, torch.float64, detach_gates=True)
