@@ -54,10 +54,34 @@ __device__ __forceinline__ float wave_sum(float x) {
   for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m);
   return x;
 }
-__device__ __forceinline__ float wave_max(float x) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) x = fmaxf(x, __shfl_xor(x, m));
+// Wave-wide scan and maximum with data-parallel-primitive moves (no LDS round trips): shifts by 1, 2, 4, 8 inside each
+// row of 16 lanes, then lane 15 of rows 0 and 2 is broadcast into rows 1 and 3, then lane 31 into rows 2 and 3.  Lanes
+// without a source take `identity`.  All 64 lanes must be active.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float identity, float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity), __builtin_bit_cast(int, x),
+                                                               CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_prefix_sum(float x) {   // inclusive: lane l gets the sum over lanes 0..l
+  x += dpp_move<0x111, 0xf>(0.f, x);
+  x += dpp_move<0x112, 0xf>(0.f, x);
+  x += dpp_move<0x114, 0xf>(0.f, x);
+  x += dpp_move<0x118, 0xf>(0.f, x);
+  x += dpp_move<0x142, 0xa>(0.f, x);
+  x += dpp_move<0x143, 0xc>(0.f, x);
   return x;
+}
+__device__ __forceinline__ float wave_last(float x) {          // lane 63's value, wave-uniform
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), kWave - 1));
+}
+__device__ __forceinline__ float wave_max(float x) {
+  x = fmaxf(x, dpp_move<0x111, 0xf>(-INFINITY, x));
+  x = fmaxf(x, dpp_move<0x112, 0xf>(-INFINITY, x));
+  x = fmaxf(x, dpp_move<0x114, 0xf>(-INFINITY, x));
+  x = fmaxf(x, dpp_move<0x118, 0xf>(-INFINITY, x));
+  x = fmaxf(x, dpp_move<0x142, 0xa>(-INFINITY, x));
+  x = fmaxf(x, dpp_move<0x143, 0xc>(-INFINITY, x));
+  return wave_last(x);
 }
 
 // One (N, D) bf16 row as D/8 16-byte words in registers; element e as float (one shift or mask per use).
@@ -160,23 +184,28 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     l_run[h] = pd_run[h] = 0.f;
   }
   float carry = 0.f;   // sum of z over the keys to the right of the current chunk (up to the diagonal)
+  // This chunk's key row, leader logit (from the row-dot pass; its slot then takes delta) and dP; the next chunk's are
+  // requested as soon as the rotation has consumed the key row, and arrive during the matrix-core phases.
+  RowRegs<D> kr;
+  float logit, dpv[G], logit_next = 0.f, dpv_next[G];
+  {
+    const int jc = min((n_chunks - 1) * kWave + lane, i);
+    kr.load(kbase + (int64_t)jc * D);
+    logit = ws.delta(g)[rowoff + jc];
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      dpv[h] = ws.dp(head0 + h)[rowoff + jc];
+      dpv_next[h] = 0.f;
+    }
+  }
 #pragma unroll 1
   for (int c = n_chunks - 1; c >= 0; --c) {
     const int j = c * kWave + lane;
     const bool valid = j <= i;
-    const int jc = valid ? j : i;
-    const float logit = ws.delta(g)[rowoff + jc];   // qL . k from the row-dot pass; replaced by delta below
-    RowRegs<D> kr;
-    kr.load(kbase + (int64_t)jc * D);
     const float z = valid ? 1.f / (1.f + __expf(-logit * p.sm_scale)) : 0.f;
-    float suf = z;   // inclusive suffix sum over the lanes (keys) at and to the right of this one
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      const float t = __shfl_down(suf, off);
-      if (lane + off < kWave) suf += t;
-    }
-    const float delta = carry + suf - z;   // gates strictly to the right, up to and including the diagonal
-    carry += __shfl(suf, 0);
+    const float zpre = wave_prefix_sum(z), ztot = wave_last(zpre);
+    const float delta = carry + (ztot - zpre);   // gates strictly to the right, up to and including the diagonal
+    carry += ztot;
 
     // the key rotated by -delta w_d goes to LDS as bf16, row = this lane's key
     static_for<HALF / 4>([&](auto step_c) __attribute__((always_inline)) {
@@ -193,6 +222,13 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       *reinterpret_cast<u32x2*>(kt + lane * KS + d0) = u32x2{pack_bf16(r1v[0], r1v[1]), pack_bf16(r1v[2], r1v[3])};
       *reinterpret_cast<u32x2*>(kt + lane * KS + HALF + d0) = u32x2{pack_bf16(r2v[0], r2v[1]), pack_bf16(r2v[2], r2v[3])};
     });
+    if (c > 0) {   // every key of the chunks to the left is at or below the diagonal
+      const int jn = j - kWave;
+      kr.load(kbase + (int64_t)jn * D);
+      logit_next = ws.delta(g)[rowoff + jn];
+#pragma unroll
+      for (int h = 0; h < G; ++h) dpv_next[h] = ws.dp(head0 + h)[rowoff + jn];
+    }
     __syncthreads();   // rotated keys are in LDS
 
     // (2G rows x D) x (D x 64 keys): lane = (row vr, half hf) for the A operand, (key vr [+ 32], half hf) for B
@@ -222,9 +258,6 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       acc[h] = (ra / 4) % 2 ? hi_rows[4 * (ra / 8) + ra % 4] : lo_rows[4 * (ra / 8) + ra % 4];
       gacc[h] = (rb / 4) % 2 ? hi_rows[4 * (rb / 8) + rb % 4] : lo_rows[4 * (rb / 8) + rb % 4];
     }
-    float dpv[G];   // dP = dO . v from the row-dot pass
-#pragma unroll
-    for (int h = 0; h < G; ++h) dpv[h] = ws.dp(head0 + h)[rowoff + jc];
     if (valid) {
       ws.delta(g)[rowoff + j] = delta;
       ws.w(g)[rowoff + j] = z * (1.f - z);   // the sigmoid's slope; replaced by W in the second sweep
@@ -263,6 +296,9 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       for (int db = 0; db < NDB; ++db) dqa[db] = mfma32(load_a_trans_natural(kt, KS, 16 * ks, 32 * db), bop, dqa[db]);
     }
     __syncthreads();   // ... and consumed: the next chunk may overwrite them
+    logit = logit_next;
+#pragma unroll
+    for (int h = 0; h < G; ++h) dpv[h] = dpv_next[h];
   }
   // row statistics: largest score, 1 / sum of exponentials, rowsum(P o dP)
   float m_row[G], inv_l[G], dsum[G];
@@ -294,41 +330,55 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
 
   // ---- left to right: P, dS, G_ij = sum_h dS dS/ddelta, its running sum over the keys, W, and W K for the leader -------
   float gcarry = 0.f;
+  // one chunk of look-ahead here too: the next chunk's S, dS/ddelta, dP, slope and key row are in flight during the
+  // matrix-core phase of the current one
+  float sl_n, sv_n[G], gv_n[G], dp_n[G];
+  u32x4 kv_n[D / 8];
+  auto fetch = [&](int c) __attribute__((always_inline)) {
+    const int j = c * kWave + lane;
+    const int jc = min(j, i);
+    sl_n = ws.w(g)[rowoff + jc];
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      sv_n[h] = ws.p(head0 + h)[rowoff + jc];
+      gv_n[h] = ws.ds(head0 + h)[rowoff + jc];
+      dp_n[h] = ws.dp(head0 + h)[rowoff + jc];
+    }
+    const uint16_t* src = kbase + (int64_t)jc * D;
+#pragma unroll
+    for (int v8 = 0; v8 < D / 8; ++v8) kv_n[v8] = *reinterpret_cast<const u32x4*>(src + 8 * v8);
+  };
+  fetch(0);
 #pragma unroll 1
   for (int c = 0; c < n_chunks; ++c) {
     const int j = c * kWave + lane;
     const bool valid = j <= i;
-    float gij = 0.f, slope = 0.f;
+    float gij = 0.f;
+    const float slope = sl_n;
+    float prv[G], dsv[G];
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      prv[h] = __expf(sv_n[h] - m_row[h]) * inv_l[h];
+      dsv[h] = prv[h] * (dp_n[h] - dsum[h]);
+      gij = __builtin_fmaf(dsv[h], gv_n[h], gij);
+    }
+    gij = valid ? gij : 0.f;
     if (valid) {
-      slope = ws.w(g)[rowoff + j];
 #pragma unroll
       for (int h = 0; h < G; ++h) {
-        float* pp = ws.p(head0 + h) + rowoff + j;
-        float* dd = ws.ds(head0 + h) + rowoff + j;
-        const float pr = __expf(*pp - m_row[h]) * inv_l[h];
-        const float dsv = pr * (ws.dp(head0 + h)[rowoff + j] - dsum[h]);
-        gij = __builtin_fmaf(dsv, *dd, gij);
-        *pp = pr;
-        *dd = dsv;
+        ws.p(head0 + h)[rowoff + j] = prv[h];
+        ws.ds(head0 + h)[rowoff + j] = dsv[h];
       }
     }
-    float pre = gij;   // inclusive prefix sum over the lanes (keys) at and to the left of this one
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      const float t = __shfl_up(pre, off);
-      if (lane >= off) pre += t;
-    }
+    const float pre = wave_prefix_sum(gij);   // over the keys at and to the left of this one
     const float wij = valid ? (gcarry + pre - gij) * slope : 0.f;   // (sum of G over the keys j < t) z'(t)
     if (valid) ws.w(g)[rowoff + j] = wij;
-    gcarry += __shfl(pre, kWave - 1);
+    gcarry += wave_last(pre);
     // leader's gate path: row 2G of the accumulators += W (1 x keys) K (keys x d)
-    {
-      const uint16_t* src = kbase + (int64_t)(valid ? j : i) * D;
 #pragma unroll
-      for (int v8 = 0; v8 < D / 8; ++v8)
-        *reinterpret_cast<u32x4*>(kt + lane * KS + 8 * v8) = *reinterpret_cast<const u32x4*>(src + 8 * v8);
-      wts[(2 * G) * WS + lane] = f_to_bf16(wij);
-    }
+    for (int v8 = 0; v8 < D / 8; ++v8) *reinterpret_cast<u32x4*>(kt + lane * KS + 8 * v8) = kv_n[v8];
+    wts[(2 * G) * WS + lane] = f_to_bf16(wij);
+    if (c + 1 < n_chunks) fetch(c + 1);
     __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < kWave / 16; ++ks) {
