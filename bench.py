@@ -9,7 +9,8 @@ oracle timed on the host cores as a baseline.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--no-cpu-baseline]
 
-(c3 is the metric shape and the default; c2/c4 are the other RoPE-attention shapes; c5 is the Co-RoPE GQA forward.)
+(c3 is the metric shape and the default; c2/c4 are the other RoPE-attention shapes; c5 is the Co-RoPE GQA forward,
+with its backward timed beside it.)
 """
 import argparse
 import importlib
@@ -192,6 +193,33 @@ def bench_corope(args):
     kms = sum(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps)) / args.steps
     flops = attention_flops(B, Hq, N, D, "fwd")
     pairs = B * Hkv * N * (N + 1) / 2 * D / 2
+
+    # backward (dq, dk, dv from q, k, v, dO): same shape, caller-owned workspace
+    do = torch.randn(B, Hq, N, D, generator=g).to(dev, torch.bfloat16)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    ws_bytes = lib.corope_gqa_bwd_workspace_bytes(B, Hq, Hkv, N, D)
+    wsp = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+    def bwd_step():
+        rc = lib.corope_gqa_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                dv.data_ptr(), B, Hq, Hkv, N, D, scale, 10000.0, wsp.data_ptr(), ws_bytes, stream)
+        if rc != 0:
+            sys.exit(pkg._lib.last_error())
+
+    bsteps = max(3, args.steps // 3)
+    for _ in range(2):
+        bwd_step()
+    bev = [torch.cuda.Event(enable_timing=True) for _ in range(bsteps + 1)]
+    bev[0].record()
+    for i in range(bsteps):
+        bwd_step()
+        bev[i + 1].record()
+    torch.cuda.synchronize()
+    bms = sum(bev[i].elapsed_time(bev[i + 1]) for i in range(bsteps)) / bsteps
+    G = Hq // Hkv
+    # lane-instructions per (sin, cos) pair: scores kernel 13 (phase 2, sin, cos, unpack 2, rotate 4, pack 1, LDS 1); dk
+    # kernel 9 + 2G (phase 2, sin, cos, rotate-accumulate 4, gate path 2, the dS-weighted query sum 2G)
+    bwd_instr = pairs * (13 + 9 + 2 * G)
     # VALU roofline: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz lane-instructions/s; per (sin, cos) pair the kernel issues
     # 14 + 2G full-rate instructions (2 of them transcendental, counted once here)
     out = {"metric": "Co-RoPE GQA fwd, B2 Hq32 Hkv8 N4096 D128 causal", "value": round(flops / (ms * 1e-3) * 1e-12, 2),
@@ -203,6 +231,13 @@ def bench_corope(args):
            "roofline": {"bound": "valu", "kernel": "corope_gqa_fwd", "achieved": round(pairs * 22 / (kms * 1e-3) * 1e-12, 3),
                         "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T lane-instr/s",
                         "frac": round(pairs * 22 / (kms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4), "traffic": None},
+           "backward": {"ms": round(bms, 4), "steps": bsteps, "workspace_gib": round(ws_bytes / 2**30, 2),
+                        "sincos_pairs_per_s": round(2 * pairs / (bms * 1e-3), 1),
+                        "tflops_attention_equivalent": round(2.5 * flops / (bms * 1e-3) * 1e-12, 2),
+                        "roofline": {"bound": "valu", "kernel": "corope_gqa_bwd (5 launches)",
+                                     "achieved": round(bwd_instr / (bms * 1e-3) * 1e-12, 3),
+                                     "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T lane-instr/s",
+                                     "frac": round(bwd_instr / (bms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4), "traffic": None}},
            "cpu_baseline": None}
     print(json.dumps(out))
 

@@ -17,16 +17,23 @@
 //                   dz_it = sum_{j < t} G_ij,   W_it = dz_it z_it (1 - z_it)   (gradient of the leader's logit),
 //                   dqL_i += c sum_t W_it k_t,   dk_t += c sum_i W_it qL_i.
 //
-// Three kernels, each a plain loop nest over (query row, key) pairs with one wave per row (or per few keys):
-//   scores  (lane = key):   right to left: z, delta by a suffix scan, S, dS/ddelta, dP and the row's softmax statistics;
-//                           left to right: P, dS, G and its prefix sum, W              -> DELTA, W [group][N][N]
-//                                                                                         P, DS, (DP) [head][N][N]
-//   dq      (lane = pair):  dq of every head, plus the leader's gate path
-//   dkdv    (lane = pair):  dk, dv for 32 keys per workgroup, tiles of the matrices staged through LDS
-// "lane = key" makes every dot product over d a per-lane loop and every sum over keys a lane-local accumulation that
-// is reduced once per row; "lane = pair" makes every sum over keys or queries a per-lane accumulation.  The angle
-// is shared by the group and rotation is linear, so sines and cosines are evaluated once per (i, j, d) in each kernel
-// and applied to one vector: the key (scores, dq) or the dS-weighted sum of the group's queries (dk).
+// Sines and cosines are evaluated in two places only, once per (i, j, d) each: where the key is rotated (scores kernel)
+// and where the dS-weighted sum of the group's queries is rotated (dk kernel) - the angle is shared by the group and
+// rotation is linear, so one vector is rotated per (i, j), not one per head.  Everything that is a dot product with an
+// already rotated or an unrotated row runs on the matrix cores.  Launches, in order:
+//   rowdot (x2)  leader logits qL K^T per group and dP = dO V^T per head, fp32 into the workspace (32x32x16 bf16 MFMA,
+//                operands straight from global memory)
+//   scores       one wave per (group, query row), lane = key:
+//                  right to left over 64-key chunks: z, delta by a scan, the rotated keys Kt -> LDS (bf16); on the matrix
+//                  cores S = q Kt^T and dS/ddelta = [-w q2, w q1] Kt^T for all heads at once, then - with running softmax
+//                  statistics, flash-attention style - the two sums that make dq: sum_j e_j dP_j kt_j and sum_j e_j kt_j;
+//                  left to right: P, dS, G and its running sum, W, and the leader's W K (matrix cores again);
+//                  writes dq and the workspace matrices DELTA, W [group][N][N] and P, DS [head][N][N]
+//   dv           dv^T += dO^T P on the matrix cores, 128 keys per workgroup
+//   dk           one workgroup per (group, 32 keys), lane = rotation pair: rotates sum_h dS^h q^h per (i, j) and adds the
+//                gate path W qL; tiles of DELTA, W, DS staged through LDS
+// Rounding: operands of the matrix products are bf16 (the rotated keys, the softmax weights e and e dP, W, P); sums,
+// statistics, delta, dS/ddelta and everything stored in the workspace are fp32.
 #include "common.hpp"
 #include "kernels.hpp"
 
