@@ -1,4 +1,4 @@
-"""Eager-PyTorch oracle for the Co-RoPE grouped-query attention forward.
+"""Eager-PyTorch oracle for the Co-RoPE grouped-query attention, forward and backward.
 
 TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke entry and by the
 benchmark's cpu_baseline leg, never by the shipped package.
@@ -19,7 +19,8 @@ Restates the reference's dense definition
 ``corope_gqa_forward_rows`` produces the same numbers for a chosen set of query
 rows per (batch, head) so that long sequences fit in memory.  The backward is
 obtained from torch.autograd through the dense forward, which is how the
-reference checks its own manual backward (:326-355).
+reference checks its own manual backward (:326-355); ``corope_gqa_backward_manual``
+restates that manual backward in closed form and is held against autograd by the tests.
 """
 from __future__ import annotations
 
@@ -121,6 +122,56 @@ def corope_gqa_forward_rows(q, k, v, causal, sm_scale, theta, rows, compute_dtyp
                 w, _ = _softmax_rows(sc, col > sel.unsqueeze(1))
                 out[b, hq, r0:r0 + row_block] = w @ vv
     return out
+
+
+def corope_gqa_backward_manual(q, k, v, grad_out, sm_scale, theta, compute_dtype=torch.float64):
+    """Dense closed-form backward: (dq, dk, dv) without autograd.
+
+    Restates the reference's manual backward (corope-exp/flash_attn_co_rope_gqa_triton.py:459-577, same as
+    corope-exp/corope_attn_gqa_pytorch.py:137-300) in the decomposition the GPU kernels use, so that a test can hold it
+    against autograd through ``corope_gqa_forward``:
+
+      kt[i,j]   = key j rotated by -delta[i,j] w_d;  S = c q . kt;  dS = P (dP - rowsum(P dP))         (:519-529)
+      dq        = c sum_j dS kt;   dk = c sum_{h,i} dS qt  (qt: the query rotated by +delta w_d)        (:541-547)
+      g[i,j]    = dS/ddelta = c sum_d w_d (q1 kt2 - q2 kt1);  G = sum_{h in group} dS g                (:531-539, :555)
+      dz[i,t]   = sum_{j<t} G[i,j]  (the reverse cumulative sum of d_a, :549-557);  W = dz z (1 - z)   (:559-560)
+      dq_leader += c W k;   dk += c W^T q_leader                                                       (:561-566)
+    """
+    G = _check_shapes(q, k, v, True)
+    cd = compute_dtype
+    q, k, v, go = q.to(cd), k.to(cd), v.to(cd), grad_out.to(cd)
+    B, Hq, N, D = q.shape
+    Hkv, h = k.shape[1], D // 2
+    w_d = corope_inv_freq(D, theta, q.device, cd)
+    kx, vx = k.repeat_interleave(G, dim=1), v.repeat_interleave(G, dim=1)
+    lead = q[:, ::G]
+    z = torch.sigmoid(torch.einsum("bhqd,bhkd->bhqk", lead, k) * sm_scale)          # (B, Hkv, N, N)
+    a = torch.cumsum(z, dim=-1)
+    delta_g = torch.diagonal(a, dim1=-2, dim2=-1).unsqueeze(-1) - a
+    delta = delta_g.repeat_interleave(G, dim=1)
+    phi = delta.unsqueeze(-1) * w_d                                                  # (B, Hq, N, N, h)
+    cs, sn = torch.cos(phi), torch.sin(phi)
+    k1, k2 = kx[..., :h].unsqueeze(2), kx[..., h:].unsqueeze(2)                      # (B, Hq, 1, N, h)
+    q1, q2 = q[..., :h].unsqueeze(3), q[..., h:].unsqueeze(3)                        # (B, Hq, N, 1, h)
+    kt1, kt2 = k1 * cs + k2 * sn, k2 * cs - k1 * sn
+    mask = _causal_mask(N, N, 0, q.device)[None, None]
+    scores = (q1 * kt1 + q2 * kt2).sum(-1) * sm_scale
+    p, _ = _softmax_rows(scores, mask)
+    dp = torch.einsum("bhqd,bhkd->bhqk", go, vx)
+    ds = p * (dp - (p * dp).sum(-1, keepdim=True))
+    dv = torch.einsum("bhqk,bhqd->bhkd", p, go).view(B, Hkv, G, N, D).sum(2)
+    dq = torch.cat([(ds.unsqueeze(-1) * kt1).sum(3), (ds.unsqueeze(-1) * kt2).sum(3)], dim=-1) * sm_scale
+    qt1, qt2 = q1 * cs - q2 * sn, q2 * cs + q1 * sn
+    dk = torch.cat([(ds.unsqueeze(-1) * qt1).sum(2), (ds.unsqueeze(-1) * qt2).sum(2)], dim=-1) * sm_scale
+    dk = dk.view(B, Hkv, G, N, D).sum(2)
+    g = ((q1 * kt2 - q2 * kt1) * w_d).sum(-1) * sm_scale
+    big_g = (ds * g).view(B, Hkv, G, N, N).sum(2)                                    # (B, Hkv, N, N), zero above the diagonal
+    dz = torch.cumsum(big_g, dim=-1) - big_g                                         # sum over j < t
+    wmat = (dz * z * (1 - z)).masked_fill(mask, 0.0)
+    dq = dq.clone()
+    dq[:, ::G] += torch.einsum("bhqk,bhkd->bhqd", wmat, k) * sm_scale
+    dk = dk + torch.einsum("bhqk,bhqd->bhkd", wmat, lead) * sm_scale
+    return dq, dk, dv
 
 
 class _CoRopeOracle(torch.autograd.Function):

@@ -106,6 +106,25 @@ def test_grouped_query_argument_checks(pkg):
     assert rc == -1 and "null" in pkg._lib.last_error()
 
 
+def test_corope_backward_argument_checks(pkg):
+    """Workspace size query and the checks corope_gqa_bwd makes before any launch (no GPU needed)."""
+    lib = pkg._lib.load()
+    assert lib.corope_gqa_bwd_workspace_bytes(2, 32, 8, 4096, 128) == 4 * 4096 * 4096 * (2 * 16 + 3 * 64)
+    assert lib.corope_gqa_bwd_workspace_bytes(1, 4, 2, 33, 64) == 4 * 33 * 33 * (2 * 2 + 3 * 4)
+    assert lib.corope_gqa_bwd_workspace_bytes(1, 5, 2, 33, 64) == -1      # Hq not a multiple of Hkv
+    assert lib.corope_gqa_bwd_workspace_bytes(1, 18, 2, 33, 64) == -1     # group size 9
+    assert lib.corope_gqa_bwd_workspace_bytes(1, 4, 2, 33, 96) == -1      # head dim not built
+    buf = ctypes.create_string_buffer(4096)
+    ok = (ctypes.addressof(buf) + 15) & ~15
+    need = lib.corope_gqa_bwd_workspace_bytes(1, 4, 2, 8, 64)
+    args = lambda ws, nbytes, dq=ok: (ok, ok, ok, ok, dq, ok, ok, 1, 4, 2, 8, 64, 0.125, 1e4, ws, nbytes, None)
+    assert lib.corope_gqa_bwd(*args(None, need)) == -1 and "null" in pkg._lib.last_error()
+    assert lib.corope_gqa_bwd(*args(ok, need, dq=ok + 2)) == -3 and "aligned" in pkg._lib.last_error()
+    assert lib.corope_gqa_bwd(*args(ok, need - 4)) == -1 and "workspace" in pkg._lib.last_error()
+    rc = lib.corope_gqa_bwd(ok, ok, ok, ok, ok, ok, ok, 1, 18, 2, 8, 64, 0.125, 1e4, ok, 1 << 40, None)
+    assert rc == -2 and "group size" in pkg._lib.last_error()
+
+
 def test_rope_freqs_argument_checks(pkg):
     lib = pkg._lib.load()
     buf = ctypes.create_string_buffer(4096)

@@ -116,3 +116,19 @@ def test_function_twin_backward_is_autograd():
     v = seeded((B, Hkv, N, D), 3, torch.float64).requires_grad_(True)
     assert torch.autograd.gradcheck(lambda a, b, c: C.attention_pytorch(a, b, c, True, 0.5, 100.0), (q, k, v),
                                     eps=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,N,D,scale,theta", [(1, 4, 2, 24, 16, 0.5, 100.0), (2, 3, 1, 17, 8, 1.0, 10.0),
+                                                     (1, 2, 2, 33, 32, 32 ** -0.5, 10000.0)])
+def test_closed_form_backward_matches_autograd(B, Hq, Hkv, N, D, scale, theta):
+    """The decomposition the GPU backward uses (rotated key / rotated query sums, the running sum of G over the keys for the
+    gate path) against autograd through the pinned dense forward, in fp64."""
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(B, Hq, N, D, generator=g, dtype=torch.float64)
+    k, v = (torch.randn(B, Hkv, N, D, generator=g, dtype=torch.float64) for _ in range(2))
+    go = torch.randn(B, Hq, N, D, generator=g, dtype=torch.float64)
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    ref = torch.autograd.grad(C.corope_gqa_forward(qa, ka, va, True, scale, theta, torch.float64), (qa, ka, va), go)
+    got = C.corope_gqa_backward_manual(q, k, v, go, scale, theta)
+    for name, a, b in zip(("dq", "dk", "dv"), got, ref):
+        assert (a - b).abs().max() <= 1e-10 * max(1.0, b.abs().max()), name
