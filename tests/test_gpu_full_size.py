@@ -91,3 +91,46 @@ def test_c5_corope_forward(pkg):
     print(f"  C5 O max-abs {err.max():.3e} mean-abs {err.mean():.3e} on {rows.numel()} rows x {B * Hq} heads", flush=True)
     assert torch.isfinite(o).all() and err.max() <= TOL
     assert torch.equal(o[:, :, 0], v.repeat_interleave(Hq // Hkv, 1)[:, :, 0])
+
+
+def test_c5_corope_backward(pkg):
+    """B2 Hq32 Hkv8 N4096 D128 Co-RoPE backward: dQ of sampled rows against autograd through the row-sampled oracle
+    (a query row's output depends on no other query row), and two size-independent identities for dK and dV:
+    sum_j dv_j = sum_{h,i} dO^h_i per group (softmax rows sum to one), and sum q.dq = sum k.dk per group (scores and
+    gates depend on q and k only through products q.k, so scaling q up and k down by the same factor changes nothing)."""
+    import importlib
+    mod = importlib.import_module("corope_amd.corope_gqa")
+    B, Hq, Hkv, N, D = 2, 32, 8, 4096, 128
+    G = Hq // Hkv
+    dev = torch.device("cuda:0")
+    q, d_o = bf16_round(seeded((B, Hq, N, D), 3)), bf16_round(seeded((B, Hq, N, D), 6))
+    k, v = bf16_round(seeded((B, Hkv, N, D), 4)), bf16_round(seeded((B, Hkv, N, D), 5))
+    scale = 1 / math.sqrt(D)
+    print("  C5 backward: launching", flush=True)
+    dq, dk, dv = (t.float().cpu() for t in mod.corope_gqa_backward(*(t.to(dev, torch.bfloat16) for t in (q, k, v, d_o)),
+                                                                     scale, 10000.0))
+    torch.cuda.synchronize()
+    assert all(torch.isfinite(t).all() for t in (dq, dk, dv))
+
+    rows = _rows(N, 3, 7)
+    qa = q.clone().requires_grad_(True)
+    out = C.corope_gqa_forward_rows(qa, k, v, True, scale, 10000.0, rows, torch.float32, row_block=16)
+    (ref_dq,) = torch.autograd.grad(out, qa, d_o[:, :, rows])
+    err = (dq[:, :, rows] - ref_dq[:, :, rows]).abs()
+    print(f"  C5 dQ max-abs {err.max():.3e} mean-abs {err.mean():.3e} on {rows.numel()} rows x {B * Hq} heads "
+          f"(max |ref| {ref_dq[:, :, rows].abs().max():.3f})", flush=True)
+    assert err.max() <= TOL
+
+    ulp = 2.0 ** -9
+    dv_sum, do_sum = dv.double().sum(2), d_o.double().view(B, Hkv, G, N, D).sum((2, 3))
+    bound = 8 * ulp * dv.double().pow(2).sum(2).sqrt()          # N independent roundings of dv rows
+    print(f"  C5 sum_j dv - sum dO: max {float((dv_sum - do_sum).abs().max()):.3e} (bound min {float(bound.min()):.3e})", flush=True)
+    assert ((dv_sum - do_sum).abs() <= bound + 1e-3 * do_sum.abs()).all()
+
+    qdq = (q.double() * dq.double()).view(B, Hkv, G, N, D)
+    kdk = k.double() * dk.double()
+    lhs, rhs = qdq.sum((2, 3, 4)), kdk.sum((2, 3))
+    bound = 8 * ulp * (qdq.pow(2).sum((2, 3, 4)) + kdk.pow(2).sum((2, 3))).sqrt()
+    print(f"  C5 sum q.dq vs sum k.dk per group: max diff {float((lhs - rhs).abs().max()):.3e}, "
+          f"|sum| up to {float(lhs.abs().max()):.3e}, bound min {float(bound.min()):.3e}", flush=True)
+    assert ((lhs - rhs).abs() <= bound + 2e-3 * lhs.abs()).all()
