@@ -144,6 +144,11 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_rowdot_kernel(const uint
 }
 
 // ---------------------------------------------------------------------------------------------------- scores
+// The scores kernel runs one wave per workgroup, and a wave's LDS instructions execute in program order, so LDS
+// written by the wave can be read back by it without a barrier or a wait; all that is needed is that the compiler keeps
+// the accesses in program order.  (A workgroup barrier would also wait for the global loads issued ahead of time.)
+__device__ __forceinline__ void lds_order() { asm volatile("" ::: "memory"); }
+
 // One wave per (group, query row i), all G heads at once, lane = key.  Per 64-key chunk the lanes rotate their keys
 // (the only place sines and cosines are evaluated) and park them in LDS as bf16; everything that is a dot product with
 // the rotated key then runs on the matrix cores: the raw scores q^h . kt and their derivatives with respect to delta
@@ -153,25 +158,39 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   constexpr int HALF = D / 2;
   constexpr int KS = D + 8, WS = kWave + 8, NVR = 2 * G + 1, NDB = D / 32;
   constexpr int NI = 4 * ((2 * G - 1) / 8 + 1);                       // accumulator registers that hold rows < 2G
-  __shared__ __attribute__((aligned(16))) uint16_t qa[2 * G * KS];    // rows h: q^h; rows G + h: [-w q2^h, w q1^h]
   __shared__ __attribute__((aligned(16))) uint16_t kt[kWave * KS];    // [key][d] bf16: rotated keys, later plain keys
   __shared__ __attribute__((aligned(16))) uint16_t wts[NVR * WS];     // [virtual row][key] bf16 weights of the keys
   const int i = p.N - 1 - blockIdx.x, g = blockIdx.y, lane = threadIdx.x;   // longest rows first
   const int vr = lane % 32, hf = lane / 32;                                  // matrix-core identity of this lane
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
   const int head0 = b * p.Hq + kvh * G;   // first head of the group, as a (batch, head) slab index
+  // A operand of the score products, constant over the row: lane (vr, hf) holds columns 16 ks + 8 hf .. + 7 of matrix row vr;
+  // rows h < G are q^h, rows G + h are [-w q2^h, w q1^h] (the derivative with respect to delta), the rest zero
+  u32x4 aop[D / 16];
+  {
+    const int h = vr < G ? vr : vr - G;
+    const uint16_t* qrow = p.q + ((int64_t)(head0 + (vr < 2 * G ? h : 0)) * N + i) * D;
 #pragma unroll
-  for (int h = 0; h < G; ++h) {
-    const uint16_t* qrow = p.q + ((int64_t)(head0 + h) * N + i) * D;
-    for (int d = lane; d < HALF; d += kWave) {
-      const uint16_t a1 = qrow[d], a2 = qrow[d + HALF];
-      qa[h * KS + d] = a1;
-      qa[h * KS + d + HALF] = a2;
-      qa[(G + h) * KS + d] = f_to_bf16(-fr.rad[d] * bf16_to_f(a2));
-      qa[(G + h) * KS + d + HALF] = f_to_bf16(fr.rad[d] * bf16_to_f(a1));
+    for (int ks = 0; ks < D / 16; ++ks) {
+      const int d0 = 16 * ks + 8 * hf;                      // first of this lane's 8 columns
+      u32x4 val = u32x4{0, 0, 0, 0};
+      if (vr < G) {
+        val = *reinterpret_cast<const u32x4*>(qrow + d0);
+      } else if (vr < 2 * G) {
+        const bool upper = d0 >= HALF;                       // columns of the second half take w q1, the first half -w q2
+        const u32x4 src = *reinterpret_cast<const u32x4*>(qrow + (upper ? d0 - HALF : d0 + HALF));
+        const float* wr = fr.rad + (upper ? d0 - HALF : d0);
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float qv = e % 2 ? bf16_hi(src[e / 2]) : bf16_lo(src[e / 2]);
+          x[e] = upper ? wr[e] * qv : -wr[e] * qv;
+        }
+        val = u32x4{pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7])};
+      }
+      aop[ks] = val;
     }
   }
-  __syncthreads();
   const uint16_t* kbase = p.k + (int64_t)g * N * D;
   const int64_t rowoff = (int64_t)i * N;
   const int n_chunks = i / kWave + 1;
@@ -191,61 +210,80 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     l_run[h] = pd_run[h] = 0.f;
   }
   float carry = 0.f;   // sum of z over the keys to the right of the current chunk (up to the diagonal)
-  // This chunk's key row, leader logit (from the row-dot pass; its slot then takes delta) and dP; the next chunk's are
-  // requested as soon as the rotation has consumed the key row, and arrive during the matrix-core phases.
-  RowRegs<D> kr;
-  float logit, dpv[G], logit_next = 0.f, dpv_next[G];
+  // A chunk's 64 key rows are one contiguous block of global memory: the wave fetches it with consecutive 16-byte pieces
+  // per lane (full cache lines per instruction) and parks it in the LDS tile, where each lane then finds its own key's
+  // row.  The block, the leader logits (from the row-dot pass; their slot then takes delta) and dP are each requested
+  // for the next chunk at the point where the current values have been used up.
+  constexpr int PIECES = D / 8;   // 16-byte pieces per row = fetch instructions per chunk
+  u32x4 kv[PIECES];
+  auto fetch_keys = [&](int c) __attribute__((always_inline)) {
+#pragma unroll
+    for (int it = 0; it < PIECES; ++it) {
+      const int row = (it * kWave + lane) / PIECES, piece = lane % PIECES;
+      kv[it] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)min(c * kWave + row, N - 1) * D + 8 * piece);
+    }
+  };
+  auto park_keys = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int it = 0; it < PIECES; ++it) {
+      const int row = (it * kWave + lane) / PIECES, piece = lane % PIECES;
+      *reinterpret_cast<u32x4*>(kt + row * KS + 8 * piece) = kv[it];
+    }
+  };
+  float logit, dpv[G];
   {
     const int jc = min((n_chunks - 1) * kWave + lane, i);
-    kr.load(kbase + (int64_t)jc * D);
+    fetch_keys(n_chunks - 1);
     logit = ws.delta(g)[rowoff + jc];
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-      dpv[h] = ws.dp(head0 + h)[rowoff + jc];
-      dpv_next[h] = 0.f;
-    }
+    for (int h = 0; h < G; ++h) dpv[h] = ws.dp(head0 + h)[rowoff + jc];
   }
 #pragma unroll 1
   for (int c = n_chunks - 1; c >= 0; --c) {
     const int j = c * kWave + lane;
     const bool valid = j <= i;
+    park_keys();
     const float z = valid ? 1.f / (1.f + __expf(-logit * p.sm_scale)) : 0.f;
+    const int jn = j - kWave;   // this lane's key in the next chunk: at or below the diagonal whenever that chunk exists
+    if (c > 0) logit = ws.delta(g)[rowoff + jn];
     const float zpre = wave_prefix_sum(z), ztot = wave_last(zpre);
     const float delta = carry + (ztot - zpre);   // gates strictly to the right, up to and including the diagonal
     carry += ztot;
 
-    // the key rotated by -delta w_d goes to LDS as bf16, row = this lane's key
+    // the key rotated by -delta w_d replaces the key in LDS (bf16, row = this lane's key)
+    lds_order();
+    u32x2 w1 = *reinterpret_cast<const u32x2*>(kt + lane * KS), w2 = *reinterpret_cast<const u32x2*>(kt + lane * KS + HALF);
+    u32x2 w1n = w1, w2n = w2;   // one step of look-ahead; the scheduling barriers keep the reads from all moving to the top
     static_for<HALF / 4>([&](auto step_c) __attribute__((always_inline)) {
       constexpr int d0 = decltype(step_c)::value * 4;
+      if (d0 + 4 < HALF) {
+        w1n = *reinterpret_cast<const u32x2*>(kt + lane * KS + d0 + 4);
+        w2n = *reinterpret_cast<const u32x2*>(kt + lane * KS + HALF + d0 + 4);
+      }
       float r1v[4], r2v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float x = __builtin_amdgcn_fractf(delta * fr.turns[d0 + e]);
         const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
-        const float k1 = kr.at(d0 + e), k2 = kr.at(d0 + e + HALF);
+        const float k1 = e % 2 ? bf16_hi(w1[e / 2]) : bf16_lo(w1[e / 2]);
+        const float k2 = e % 2 ? bf16_hi(w2[e / 2]) : bf16_lo(w2[e / 2]);
         r1v[e] = __builtin_fmaf(cs, k1, sn * k2);
         r2v[e] = __builtin_fmaf(cs, k2, -(sn * k1));
       }
       *reinterpret_cast<u32x2*>(kt + lane * KS + d0) = u32x2{pack_bf16(r1v[0], r1v[1]), pack_bf16(r1v[2], r1v[3])};
       *reinterpret_cast<u32x2*>(kt + lane * KS + HALF + d0) = u32x2{pack_bf16(r2v[0], r2v[1]), pack_bf16(r2v[2], r2v[3])};
+      __builtin_amdgcn_sched_barrier(0);
+      w1 = w1n;
+      w2 = w2n;
     });
-    if (c > 0) {   // every key of the chunks to the left is at or below the diagonal
-      const int jn = j - kWave;
-      kr.load(kbase + (int64_t)jn * D);
-      logit_next = ws.delta(g)[rowoff + jn];
-#pragma unroll
-      for (int h = 0; h < G; ++h) dpv_next[h] = ws.dp(head0 + h)[rowoff + jn];
-    }
-    __syncthreads();   // rotated keys are in LDS
+    lds_order();   // rotated keys are in LDS
 
     // (2G rows x D) x (D x 64 keys): lane = (row vr, half hf) for the A operand, (key vr [+ 32], half hf) for B
     f32x16 c0 = f32x16{0}, c1 = f32x16{0};
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
-      u32x4 aop = u32x4{0, 0, 0, 0};
-      if (vr < 2 * G) aop = *reinterpret_cast<const u32x4*>(qa + vr * KS + 16 * ks + 8 * hf);
-      c0 = mfma32(aop, *reinterpret_cast<const u32x4*>(kt + vr * KS + 16 * ks + 8 * hf), c0);
-      c1 = mfma32(aop, *reinterpret_cast<const u32x4*>(kt + (32 + vr) * KS + 16 * ks + 8 * hf), c1);
+      c0 = mfma32(aop[ks], *reinterpret_cast<const u32x4*>(kt + vr * KS + 16 * ks + 8 * hf), c0);
+      c1 = mfma32(aop[ks], *reinterpret_cast<const u32x4*>(kt + (32 + vr) * KS + 16 * ks + 8 * hf), c1);
     }
     // the results sit at lane = key % 32 with rows split over the lane halves; swapping the upper half of the keys-below-
     // 32 result with the lower half of the keys-from-32 result puts every key's rows into its own lane
@@ -258,6 +296,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       lo_rows[n] = __builtin_bit_cast(float, (uint32_t)r[0]);
       hi_rows[n] = __builtin_bit_cast(float, (uint32_t)r[1]);
     }
+    if (c > 0) fetch_keys(c - 1);   // the registers of the product are free again: request the next chunk's keys
     float acc[G], gacc[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) {
@@ -288,13 +327,17 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       wts[(2 * h) * WS + lane] = f_to_bf16(e * dpv[h]);
       wts[(2 * h + 1) * WS + lane] = f_to_bf16(e);
     }
+    if (c > 0) {
+#pragma unroll
+      for (int h = 0; h < G; ++h) dpv[h] = ws.dp(head0 + h)[rowoff + jn];
+    }
     if (moved) {
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int e = 0; e < 16; ++e) dqa[db][e] *= al;
     }
-    __syncthreads();   // rotated keys and weights are in LDS
+    lds_order();   // rotated keys and weights are in LDS
 #pragma unroll
     for (int ks = 0; ks < kWave / 16; ++ks) {
       u32x4 bop = u32x4{0, 0, 0, 0};
@@ -302,10 +345,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
 #pragma unroll
       for (int db = 0; db < NDB; ++db) dqa[db] = mfma32(load_a_trans_natural(kt, KS, 16 * ks, 32 * db), bop, dqa[db]);
     }
-    __syncthreads();   // ... and consumed: the next chunk may overwrite them
-    logit = logit_next;
-#pragma unroll
-    for (int h = 0; h < G; ++h) dpv[h] = dpv_next[h];
+    lds_order();   // ... and consumed: the next chunk may overwrite them
   }
   // row statistics: largest score, 1 / sum of exponentials, rowsum(P o dP)
   float m_row[G], inv_l[G], dsum[G];
@@ -340,7 +380,6 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   // one chunk of look-ahead here too: the next chunk's S, dS/ddelta, dP, slope and key row are in flight during the
   // matrix-core phase of the current one
   float sl_n, sv_n[G], gv_n[G], dp_n[G];
-  u32x4 kv_n[D / 8];
   auto fetch = [&](int c) __attribute__((always_inline)) {
     const int j = c * kWave + lane;
     const int jc = min(j, i);
@@ -351,42 +390,48 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       gv_n[h] = ws.ds(head0 + h)[rowoff + jc];
       dp_n[h] = ws.dp(head0 + h)[rowoff + jc];
     }
-    const uint16_t* src = kbase + (int64_t)jc * D;
-#pragma unroll
-    for (int v8 = 0; v8 < D / 8; ++v8) kv_n[v8] = *reinterpret_cast<const u32x4*>(src + 8 * v8);
+    fetch_keys(c);
   };
   fetch(0);
 #pragma unroll 1
   for (int c = 0; c < n_chunks; ++c) {
     const int j = c * kWave + lane;
     const bool valid = j <= i;
-    float gij = 0.f;
+    // take this chunk's values out of the look-ahead registers (the key row goes straight to LDS) and request the next
+    // chunk's before anything is stored, so that waiting for them never waits for this chunk's stores
     const float slope = sl_n;
+    float sv[G], gv[G], dpc[G];
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      sv[h] = sv_n[h];
+      gv[h] = gv_n[h];
+      dpc[h] = dp_n[h];
+    }
+    park_keys();
+    if (c + 1 < n_chunks) fetch(c + 1);
+    float gij = 0.f;
     float prv[G], dsv[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-      prv[h] = __expf(sv_n[h] - m_row[h]) * inv_l[h];
-      dsv[h] = prv[h] * (dp_n[h] - dsum[h]);
-      gij = __builtin_fmaf(dsv[h], gv_n[h], gij);
+      prv[h] = __expf(sv[h] - m_row[h]) * inv_l[h];
+      dsv[h] = prv[h] * (dpc[h] - dsum[h]);
+      gij = __builtin_fmaf(dsv[h], gv[h], gij);
     }
     gij = valid ? gij : 0.f;
+    const float pre = wave_prefix_sum(gij);   // over the keys at and to the left of this one
+    const float wij = valid ? (gcarry + pre - gij) * slope : 0.f;   // (sum of G over the keys j < t) z'(t)
+    gcarry += wave_last(pre);
+    wts[(2 * G) * WS + lane] = f_to_bf16(wij);
     if (valid) {
 #pragma unroll
       for (int h = 0; h < G; ++h) {
         ws.p(head0 + h)[rowoff + j] = prv[h];
         ws.ds(head0 + h)[rowoff + j] = dsv[h];
       }
+      ws.w(g)[rowoff + j] = wij;
     }
-    const float pre = wave_prefix_sum(gij);   // over the keys at and to the left of this one
-    const float wij = valid ? (gcarry + pre - gij) * slope : 0.f;   // (sum of G over the keys j < t) z'(t)
-    if (valid) ws.w(g)[rowoff + j] = wij;
-    gcarry += wave_last(pre);
+    lds_order();
     // leader's gate path: row 2G of the accumulators += W (1 x keys) K (keys x d)
-#pragma unroll
-    for (int v8 = 0; v8 < D / 8; ++v8) *reinterpret_cast<u32x4*>(kt + lane * KS + 8 * v8) = kv_n[v8];
-    wts[(2 * G) * WS + lane] = f_to_bf16(wij);
-    if (c + 1 < n_chunks) fetch(c + 1);
-    __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < kWave / 16; ++ks) {
       u32x4 bop = u32x4{0, 0, 0, 0};
@@ -394,7 +439,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
 #pragma unroll
       for (int db = 0; db < NDB; ++db) dqa[db] = mfma32(load_a_trans_natural(kt, KS, 16 * ks, 32 * db), bop, dqa[db]);
     }
-    __syncthreads();
+    lds_order();
   }
   // dq: even virtual rows hold the heads' gradients; the leader adds the gate path from row 2G of its lane half
 #pragma unroll
