@@ -69,6 +69,10 @@ template <typename T>
 __device__ __forceinline__ const T* byte_offset(const T* base, uint32_t bytes) {
   return reinterpret_cast<const T*>(reinterpret_cast<const char*>(base) + bytes);
 }
+template <typename T>
+__device__ __forceinline__ T* byte_offset(T* base, uint32_t bytes) {
+  return reinterpret_cast<T*>(reinterpret_cast<char*>(base) + bytes);
+}
 
 // Grouped-query attention: slab (batch, query head) -> slab (batch, key/value head) of tensors with Hkv heads.
 __device__ __forceinline__ int kv_slab(int bh, int H, int Hkv) {

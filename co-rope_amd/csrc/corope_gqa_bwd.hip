@@ -194,6 +194,17 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   const uint16_t* kbase = p.k + (int64_t)g * N * D;
   const int64_t rowoff = (int64_t)i * N;
   const int n_chunks = i / kWave + 1;
+  // this row of every workspace matrix: wave-uniform bases, addressed with 32-bit byte offsets of the key index
+  float* const d_row = ws.delta(g) + rowoff;
+  float* const w_row = ws.w(g) + rowoff;
+  float *p_row[G], *ds_row[G];
+  const float* dp_row[G];
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    p_row[h] = ws.p(head0 + h) + rowoff;
+    ds_row[h] = ws.ds(head0 + h) + rowoff;
+    dp_row[h] = ws.dp(head0 + h) + rowoff;
+  }
 
   // ---- right to left: gates, delta, raw scores, dS/ddelta, softmax statistics, dq sums --------------------------------
   // dq^h = c sum_j dS_j kt_j = c (sum_j e_j dP_j kt_j - Delta sum_j e_j kt_j) / L with e_j = exp(s_j - m): both sums are
@@ -217,10 +228,17 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   constexpr int PIECES = D / 8;   // 16-byte pieces per row = fetch instructions per chunk
   u32x4 kv[PIECES];
   auto fetch_keys = [&](int c) __attribute__((always_inline)) {
+    const uint16_t* block = kbase + (int64_t)c * kWave * D;   // wave-uniform
+    if (c * kWave + kWave <= N) {
 #pragma unroll
-    for (int it = 0; it < PIECES; ++it) {
-      const int row = (it * kWave + lane) / PIECES, piece = lane % PIECES;
-      kv[it] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)min(c * kWave + row, N - 1) * D + 8 * piece);
+      for (int it = 0; it < PIECES; ++it)
+        kv[it] = *reinterpret_cast<const u32x4*>(byte_offset(block, 16u * lane + 1024u * it));
+    } else {   // the block runs past the last key: clamp the rows (only the chunk on the diagonal can get here)
+#pragma unroll
+      for (int it = 0; it < PIECES; ++it) {
+        const int row = (it * kWave + lane) / PIECES, piece = lane % PIECES;
+        kv[it] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)min(c * kWave + row, N - 1) * D + 8 * piece);
+      }
     }
   };
   auto park_keys = [&]() __attribute__((always_inline)) {
@@ -234,9 +252,9 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   {
     const int jc = min((n_chunks - 1) * kWave + lane, i);
     fetch_keys(n_chunks - 1);
-    logit = ws.delta(g)[rowoff + jc];
+    logit = *byte_offset(d_row, 4u * jc);
 #pragma unroll
-    for (int h = 0; h < G; ++h) dpv[h] = ws.dp(head0 + h)[rowoff + jc];
+    for (int h = 0; h < G; ++h) dpv[h] = *byte_offset(dp_row[h], 4u * jc);
   }
 #pragma unroll 1
   for (int c = n_chunks - 1; c >= 0; --c) {
@@ -245,21 +263,24 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     park_keys();
     const float z = valid ? 1.f / (1.f + __expf(-logit * p.sm_scale)) : 0.f;
     const int jn = j - kWave;   // this lane's key in the next chunk: at or below the diagonal whenever that chunk exists
-    if (c > 0) logit = ws.delta(g)[rowoff + jn];
+    if (c > 0) logit = *byte_offset(d_row, 4u * jn);
     const float zpre = wave_prefix_sum(z), ztot = wave_last(zpre);
     const float delta = carry + (ztot - zpre);   // gates strictly to the right, up to and including the diagonal
     carry += ztot;
 
     // the key rotated by -delta w_d replaces the key in LDS (bf16, row = this lane's key)
     lds_order();
-    u32x2 w1 = *reinterpret_cast<const u32x2*>(kt + lane * KS), w2 = *reinterpret_cast<const u32x2*>(kt + lane * KS + HALF);
-    u32x2 w1n = w1, w2n = w2;   // one step of look-ahead; the scheduling barriers keep the reads from all moving to the top
+    // one step of look-ahead in two alternating register sets; the scheduling barriers keep the reads from all moving up
+    u32x2 wa[2][2];
+    wa[0][0] = *reinterpret_cast<const u32x2*>(kt + lane * KS);
+    wa[0][1] = *reinterpret_cast<const u32x2*>(kt + lane * KS + HALF);
     static_for<HALF / 4>([&](auto step_c) __attribute__((always_inline)) {
-      constexpr int d0 = decltype(step_c)::value * 4;
+      constexpr int step = decltype(step_c)::value, d0 = step * 4;
       if (d0 + 4 < HALF) {
-        w1n = *reinterpret_cast<const u32x2*>(kt + lane * KS + d0 + 4);
-        w2n = *reinterpret_cast<const u32x2*>(kt + lane * KS + HALF + d0 + 4);
+        wa[(step + 1) % 2][0] = *reinterpret_cast<const u32x2*>(kt + lane * KS + d0 + 4);
+        wa[(step + 1) % 2][1] = *reinterpret_cast<const u32x2*>(kt + lane * KS + HALF + d0 + 4);
       }
+      const u32x2 w1 = wa[step % 2][0], w2 = wa[step % 2][1];
       float r1v[4], r2v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -273,8 +294,6 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       *reinterpret_cast<u32x2*>(kt + lane * KS + d0) = u32x2{pack_bf16(r1v[0], r1v[1]), pack_bf16(r1v[2], r1v[3])};
       *reinterpret_cast<u32x2*>(kt + lane * KS + HALF + d0) = u32x2{pack_bf16(r2v[0], r2v[1]), pack_bf16(r2v[2], r2v[3])};
       __builtin_amdgcn_sched_barrier(0);
-      w1 = w1n;
-      w2 = w2n;
     });
     lds_order();   // rotated keys are in LDS
 
@@ -305,8 +324,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       gacc[h] = (rb / 4) % 2 ? hi_rows[4 * (rb / 8) + rb % 4] : lo_rows[4 * (rb / 8) + rb % 4];
     }
     if (valid) {
-      ws.delta(g)[rowoff + j] = delta;
-      ws.w(g)[rowoff + j] = z * (1.f - z);   // the sigmoid's slope; replaced by W in the second sweep
+      *byte_offset(d_row, 4u * j) = delta;
+      *byte_offset(w_row, 4u * j) = z * (1.f - z);   // the sigmoid's slope; replaced by W in the second sweep
     }
     float al = 1.f;          // this lane's virtual row's rescale factor
     bool moved = false;      // wave-uniform: some head's running maximum moved
@@ -314,8 +333,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     for (int h = 0; h < G; ++h) {
       const float sc = acc[h] * p.sm_scale;
       if (valid) {
-        ws.p(head0 + h)[rowoff + j] = sc;
-        ws.ds(head0 + h)[rowoff + j] = gacc[h] * p.sm_scale;
+        *byte_offset(p_row[h], 4u * j) = sc;
+        *byte_offset(ds_row[h], 4u * j) = gacc[h] * p.sm_scale;
       }
       const float m_new = fmaxf(m_run[h], wave_max(valid ? sc : -INFINITY));   // finite: the chunk holds a key <= i
       const float a = __expf(m_run[h] - m_new), e = valid ? __expf(sc - m_new) : 0.f;
@@ -329,7 +348,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     }
     if (c > 0) {
 #pragma unroll
-      for (int h = 0; h < G; ++h) dpv[h] = ws.dp(head0 + h)[rowoff + jn];
+      for (int h = 0; h < G; ++h) dpv[h] = *byte_offset(dp_row[h], 4u * jn);
     }
     if (moved) {
 #pragma unroll
@@ -383,12 +402,12 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   auto fetch = [&](int c) __attribute__((always_inline)) {
     const int j = c * kWave + lane;
     const int jc = min(j, i);
-    sl_n = ws.w(g)[rowoff + jc];
+    sl_n = *byte_offset(w_row, 4u * jc);
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-      sv_n[h] = ws.p(head0 + h)[rowoff + jc];
-      gv_n[h] = ws.ds(head0 + h)[rowoff + jc];
-      dp_n[h] = ws.dp(head0 + h)[rowoff + jc];
+      sv_n[h] = *byte_offset(p_row[h], 4u * jc);
+      gv_n[h] = *byte_offset(ds_row[h], 4u * jc);
+      dp_n[h] = *byte_offset(dp_row[h], 4u * jc);
     }
     fetch_keys(c);
   };
@@ -425,10 +444,10 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     if (valid) {
 #pragma unroll
       for (int h = 0; h < G; ++h) {
-        ws.p(head0 + h)[rowoff + j] = prv[h];
-        ws.ds(head0 + h)[rowoff + j] = dsv[h];
+        *byte_offset(p_row[h], 4u * j) = prv[h];
+        *byte_offset(ds_row[h], 4u * j) = dsv[h];
       }
-      ws.w(g)[rowoff + j] = wij;
+      *byte_offset(w_row, 4u * j) = wij;
     }
     lds_order();
     // leader's gate path: row 2G of the accumulators += W (1 x keys) K (keys x d)
