@@ -561,7 +561,7 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
   uint16_t (*qrows)[G][D] = reinterpret_cast<uint16_t (*)[G][D]>(smem + Cfg::kMatBytes);
 
   const int jb = blockIdx.x * kDkKeys, g = blockIdx.y;   // the first key blocks see the most rows and start first
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
   const int head0 = b * p.Hq + kvh * G;
   const bool act = lane < HALF;
@@ -627,7 +627,7 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
       }
 #pragma unroll
       for (int kk = 0; kk < kDkKeysPerWave; ++kk) {
-        if (jw + kk > i) continue;   // wave-uniform: keys above the diagonal of this row (their tiles are zero anyway)
+        // (keys above the diagonal of this row need no test: their tile entries were staged as zeros)
         const f32x4* el = reinterpret_cast<const f32x4*>(mats + (r * kDkKeys + wave * kDkKeysPerWave + kk) * MS);
         f32x4 ev[MS / 4];
 #pragma unroll
