@@ -217,9 +217,10 @@ def bench_corope(args):
     torch.cuda.synchronize()
     bms = sum(bev[i].elapsed_time(bev[i + 1]) for i in range(bsteps)) / bsteps
     G = Hq // Hkv
-    # lane-instructions per (sin, cos) pair: scores kernel 13 (phase 2, sin, cos, unpack 2, rotate 4, pack 1, LDS 1); dk
-    # kernel 9 + 2G (phase 2, sin, cos, rotate-accumulate 4, gate path 2, the dS-weighted query sum 2G)
-    bwd_instr = pairs * (13 + 9 + 2 * G)
+    # lane-instructions per (sin, cos) pair, counted as for the forward (a transcendental counts once): scores kernel 13
+    # (phase 2, sin, cos, unpack 2, rotate 4, pack 1, LDS 2); dk kernel 10 (phase 2, sin, cos, rotate-accumulate 4, gate
+    # path 2); the per-head sums run on the matrix cores
+    bwd_instr = pairs * (13 + 10)
     # VALU roofline: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz lane-instructions/s; per (sin, cos) pair the kernel issues
     # 14 + 2G full-rate instructions (2 of them transcendental, counted once here)
     out = {"metric": "Co-RoPE GQA fwd, B2 Hq32 Hkv8 N4096 D128 causal", "value": round(flops / (ms * 1e-3) * 1e-12, 2),

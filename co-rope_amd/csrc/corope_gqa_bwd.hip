@@ -536,127 +536,160 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_dv_kernel(CoropeBwdParam
 }
 
 // ---------------------------------------------------------------------------------------------------- dk
-// One workgroup of 4 waves per (group, block of 32 keys); each wave owns 8 of the keys, lane = rotation pair.  Query
-// rows are visited 16 at a time: the 16 x 32 tiles of DELTA, W, DS^h (interleaved per element, so that one (row, key)
-// costs a few 16-byte broadcast reads) and the 16 rows of q of every head are staged in LDS, so the column-wise access
-// of the N x N matrices costs full 128-byte lines.
-constexpr int kDkKeys = 32, kDkRows = 16, kDkWaves = 4, kDkKeysPerWave = kDkKeys / kDkWaves;
+// dk_j = c sum_i [ R(+delta_ij)(sum_h dS^h_ij q^h_i) + W_ij qL_i ].  One workgroup of 4 waves owns 128 keys of one group
+// (32 per wave) and walks the query rows from the block's first key to the end, 8 rows per staged tile.  Per row:
+//   u = sum_h dS^h q^h for the wave's 32 keys and all D columns: a (32 keys x heads) x (heads x D) product on the
+//       matrix cores - the contraction is only G long, but it takes 2G multiply-adds per (key, pair) off the vector
+//       units; the result lands as lane = column (mod 32), registers = 16 of the wave's keys;
+//   rotation and accumulation on the vector units: lane (c, half) owns pairs c and c + 32 (D = 128) for the 16 keys of
+//       its half: one (sin, cos) and six multiply-adds per (row, key, pair).
+// Work per key block falls linearly with the block index, so a workgroup takes blocks b and (last - b) in turn: every
+// workgroup sees the same number of rows.  Tiles of DELTA, W, DS^h ([row][matrix][key], fp32) and the rows' queries
+// ([row][column][head], bf16, heads padded to 8 with zeros: the B operand is then one 16-byte read) go through LDS,
+// fetched into registers one tile ahead.
+constexpr int kDkKeys = 128, kDkRows = 8, kDkWaves = 4;
 
 template <int D, int G>
 struct CoropeDkCfg {
   static constexpr int kMats = 2 + G;                                       // DELTA, W, DS^h
-  static constexpr int kMS = (kMats + 3) / 4 * 4;                           // floats per (row, key) element
-  static constexpr int kMatBytes = kMS * kDkRows * kDkKeys * 4;
-  static constexpr int kRowBytes = kDkRows * G * D * 2;                     // q rows, bf16
-  static constexpr int kLdsBytes = kMatBytes + kRowBytes;
+  static constexpr int kMatBytes = kDkRows * kMats * kDkKeys * 4;
+  static constexpr int kQBytes = kDkRows * D * 8 * 2;                       // [row][column][8 heads] bf16
+  static constexpr int kLdsBytes = kMatBytes + kQBytes;
 };
 
 template <int D, int G>
 __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBwdParams p, CoropeBwdWs ws,
-                                                                         CoropeBwdFreqs fr) {
+                                                                       CoropeBwdFreqs fr) {
   using Cfg = CoropeDkCfg<D, G>;
-  constexpr int HALF = D / 2, NT = kDkWaves * kWave, MS = Cfg::kMS;
+  constexpr int HALF = D / 2, NT = kDkWaves * kWave, MATS = Cfg::kMats, NB = D / 32, NP = D / 64;
+  static_assert(D == 64 || D == 128, "pairs per lane are laid out for these head dims");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  float* mats = reinterpret_cast<float*>(smem);                                          // [row][key][MS]
-  uint16_t (*qrows)[G][D] = reinterpret_cast<uint16_t (*)[G][D]>(smem + Cfg::kMatBytes);
+  float* tile = reinterpret_cast<float*>(smem);                                   // [row][matrix][key]
+  uint16_t* qT = reinterpret_cast<uint16_t*>(smem + Cfg::kMatBytes);             // [row][column][8 heads]
 
-  const int jb = blockIdx.x * kDkKeys, g = blockIdx.y;   // the first key blocks see the most rows and start first
+  const int g = blockIdx.y;
   const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int col = lane % 32, hf = lane / 32;
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
   const int head0 = b * p.Hq + kvh * G;
-  const bool act = lane < HALF;
-  const int dpair = act ? lane : 0;
-  const float w_turn = fr.turns[dpair];
-  const int jw = jb + wave * kDkKeysPerWave;   // first key of this wave
+  const int n_blocks = (N + kDkKeys - 1) / kDkKeys;
+  float w_turn[NP > 0 ? NP : 1];
+#pragma unroll
+  for (int np = 0; np < (NP > 0 ? NP : 1); ++np) w_turn[np] = fr.turns[min(32 * np + col, HALF - 1)];
 
-  float dk1[kDkKeysPerWave], dk2[kDkKeysPerWave];
-#pragma unroll
-  for (int kk = 0; kk < kDkKeysPerWave; ++kk) dk1[kk] = dk2[kk] = 0.f;
+  // heads G..7 of the query tile stay zero for the whole kernel
+  for (int e = threadIdx.x; e < Cfg::kQBytes / 16; e += NT) reinterpret_cast<u32x4*>(qT)[e] = u32x4{0, 0, 0, 0};
 
-  // Staging: thread -> key column c and row r = rsub or rsub + 8 of the 16 x 32 tiles, plus its share of the 16-byte
-  // pieces of the q rows.  The next tile's values are fetched into registers while the current tile is consumed.
-  constexpr int kRowItems = kDkRows * G * (D / 8), RI = (kRowItems + NT - 1) / NT;
-  const int sc = threadIdx.x % kDkKeys, rsub = threadIdx.x / kDkKeys;
-  float mv[2 * Cfg::kMats];
-  u32x4 qv[RI];
-  auto fetch = [&](int i0) __attribute__((always_inline)) {
-    static_for<2 * Cfg::kMats>([&](auto k_c) __attribute__((always_inline)) {
-      constexpr int k = decltype(k_c)::value, m = k / 2;
-      const int i = i0 + rsub + 8 * (k % 2), j = jb + sc;
-      const float* src = m == 0 ? ws.delta(g) : m == 1 ? ws.w(g) : ws.ds(head0 + m - 2);
-      mv[k] = (i < N && j <= i) ? src[(int64_t)i * N + j] : 0.f;   // zero outside the causal triangle and past N
-    });
-    static_for<RI>([&](auto k_c) __attribute__((always_inline)) {
-      constexpr int k = decltype(k_c)::value;
-      const int e = threadIdx.x + k * NT;
-      if (kRowItems % NT == 0 || e < kRowItems) {
-        const int r = e / (G * (D / 8)), h = (e / (D / 8)) % G, v8 = e % (D / 8);
-        const int64_t off = ((int64_t)(head0 + h) * N + min(i0 + r, N - 1)) * D + 8 * v8;
-        qv[k] = *reinterpret_cast<const u32x4*>(p.q + off);
-      }
-    });
-  };
-  fetch(jb);
-  // rows i >= jb see at least one key of the block
+  constexpr int kTileElems = kDkRows * MATS * kDkKeys, TI = kTileElems / NT;      // fp32 values per thread and tile
+  constexpr int kRowItems = kDkRows * G * (D / 8), RI = (kRowItems + NT - 1) / NT;  // 16-byte pieces of q rows
+  static_assert(kTileElems % NT == 0, "tile elements divide evenly over the threads");
+
 #pragma unroll 1
-  for (int i0 = jb; i0 < N; i0 += kDkRows) {
-    __syncthreads();   // the previous tile has been consumed
-    static_for<2 * Cfg::kMats>([&](auto k_c) __attribute__((always_inline)) {
-      constexpr int k = decltype(k_c)::value;
-      mats[((rsub + 8 * (k % 2)) * kDkKeys + sc) * MS + k / 2] = mv[k];
-    });
-    static_for<RI>([&](auto k_c) __attribute__((always_inline)) {
-      constexpr int k = decltype(k_c)::value;
-      const int e = threadIdx.x + k * NT;
-      if (kRowItems % NT == 0 || e < kRowItems) {
-        const int r = e / (G * (D / 8)), h = (e / (D / 8)) % G, v8 = e % (D / 8);
-        *reinterpret_cast<u32x4*>(&qrows[r][h][8 * v8]) = qv[k];
-      }
-    });
-    __syncthreads();
-    if (i0 + kDkRows < N) fetch(i0 + kDkRows);
-    const int n_rows = min(kDkRows, N - i0);
-#pragma unroll 1
-    for (int r = 0; r < n_rows; ++r) {
-      const int i = i0 + r;
-      float q1[G], q2[G];
-#pragma unroll
-      for (int h = 0; h < G; ++h) {
-        q1[h] = bf16_to_f(qrows[r][h][dpair]);
-        q2[h] = bf16_to_f(qrows[r][h][dpair + HALF]);
-      }
-#pragma unroll
-      for (int kk = 0; kk < kDkKeysPerWave; ++kk) {
-        // (keys above the diagonal of this row need no test: their tile entries were staged as zeros)
-        const f32x4* el = reinterpret_cast<const f32x4*>(mats + (r * kDkKeys + wave * kDkKeysPerWave + kk) * MS);
-        f32x4 ev[MS / 4];
-#pragma unroll
-        for (int u = 0; u < MS / 4; ++u) ev[u] = el[u];
-        const float delta = ev[0][0], wij = ev[0][1];
-        const float x = __builtin_amdgcn_fractf(delta * w_turn);
-        const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
-        float u1 = 0.f, u2 = 0.f;   // dS-weighted sum of the group's queries: rotating it once rotates them all
-#pragma unroll
-        for (int h = 0; h < G; ++h) {
-          const float dsv = ev[(2 + h) / 4][(2 + h) % 4];
-          u1 = __builtin_fmaf(dsv, q1[h], u1);
-          u2 = __builtin_fmaf(dsv, q2[h], u2);
+  for (int phase = 0; phase < 2; ++phase) {
+    const int kb = phase == 0 ? (int)blockIdx.x : n_blocks - 1 - (int)blockIdx.x;
+    if (phase == 1 && kb <= (int)blockIdx.x) break;   // odd number of blocks: the middle one has been done in phase 0
+    const int jb = kb * kDkKeys, jw = jb + 32 * wave;
+
+    float mv[TI];
+    u32x4 qv[RI];
+    auto fetch = [&](int i0) __attribute__((always_inline)) {
+      static_for<TI>([&](auto k_c) __attribute__((always_inline)) {
+        constexpr int k = decltype(k_c)::value;
+        const int e = threadIdx.x + k * NT;
+        const int key = e % kDkKeys, m = (e / kDkKeys) % MATS, r = e / (kDkKeys * MATS);
+        const int i = i0 + r, j = jb + key;
+        const float* src = m == 0 ? ws.delta(g) : m == 1 ? ws.w(g) : ws.ds(head0 + m - 2);
+        mv[k] = (i < N && j <= i) ? src[(int64_t)i * N + j] : 0.f;   // zero outside the causal triangle and past N
+      });
+      static_for<RI>([&](auto k_c) __attribute__((always_inline)) {
+        constexpr int k = decltype(k_c)::value;
+        const int e = threadIdx.x + k * NT;
+        if (kRowItems % NT == 0 || e < kRowItems) {
+          const int r = e / (G * (D / 8)), h = (e / (D / 8)) % G, v8 = e % (D / 8);
+          qv[k] = *reinterpret_cast<const u32x4*>(p.q + ((int64_t)(head0 + h) * N + min(i0 + r, N - 1)) * D + 8 * v8);
         }
-        dk1[kk] = __builtin_fmaf(cs, u1, __builtin_fmaf(-sn, u2, dk1[kk]));
-        dk2[kk] = __builtin_fmaf(cs, u2, __builtin_fmaf(sn, u1, dk2[kk]));
-        dk1[kk] = __builtin_fmaf(wij, q1[0], dk1[kk]);   // the leader's gate path (unrotated q)
-        dk2[kk] = __builtin_fmaf(wij, q2[0], dk2[kk]);
+      });
+    };
+    float dk1[NP][16], dk2[NP][16];
+#pragma unroll
+    for (int np = 0; np < NP; ++np)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) dk1[np][e] = dk2[np][e] = 0.f;
+
+    fetch(jb);
+#pragma unroll 1
+    for (int i0 = jb; i0 < N; i0 += kDkRows) {
+      __syncthreads();   // the previous tile has been consumed
+      static_for<TI>([&](auto k_c) __attribute__((always_inline)) {
+        constexpr int k = decltype(k_c)::value;
+        tile[threadIdx.x + k * NT] = mv[k];
+      });
+      static_for<RI>([&](auto k_c) __attribute__((always_inline)) {
+        constexpr int k = decltype(k_c)::value;
+        const int e = threadIdx.x + k * NT;
+        if (kRowItems % NT == 0 || e < kRowItems) {
+          const int r = e / (G * (D / 8)), h = (e / (D / 8)) % G, v8 = e % (D / 8);
+          uint16_t* dst = qT + ((r * D + 8 * v8) * 8 + h);
+#pragma unroll
+          for (int x = 0; x < 8; ++x) dst[8 * x] = (uint16_t)(x % 2 ? qv[k][x / 2] >> 16 : qv[k][x / 2] & 0xffffu);
+        }
+      });
+      __syncthreads();
+      if (i0 + kDkRows < N) fetch(i0 + kDkRows);
+      const int n_rows = min(kDkRows, N - i0);
+#pragma unroll 1
+      for (int r = 0; r < n_rows; ++r) {
+        if (i0 + r < jw) continue;   // wave-uniform: all keys of this wave lie above the diagonal of this row
+        const float* trow = tile + r * MATS * kDkKeys + 32 * wave;
+        // A: (32 keys x heads), lane (key, half 0) holds dS^h for h = 0..7; half 1 would be heads 8..15: zero
+        u32x4 aop = u32x4{0, 0, 0, 0};
+        if (hf == 0) {
+          float dsv[8];
+#pragma unroll
+          for (int h = 0; h < 8; ++h) dsv[h] = h < G ? trow[(2 + h) * kDkKeys + col] : 0.f;
+          aop = u32x4{pack_bf16(dsv[0], dsv[1]), pack_bf16(dsv[2], dsv[3]), pack_bf16(dsv[4], dsv[5]), pack_bf16(dsv[6], dsv[7])};
+        }
+        // B: (heads x 32 columns) per column block; the same read also carries the leader's (head 0) value of the column
+        f32x16 u[NB];
+        float ql[NB];
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk) {
+          const u32x4 bq = *reinterpret_cast<const u32x4*>(qT + (r * D + 32 * blk + col) * 8);
+          ql[blk] = bf16_lo(bq[0]);
+          u[blk] = mfma32(aop, hf == 0 ? bq : u32x4{0, 0, 0, 0}, f32x16{0});
+        }
+        // delta and W of this lane's 16 keys: keys 8 n + 4 half + 0..3 for n = 0..3, as the accumulator rows are laid out
+        f32x4 dl[4], wg[4];
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+          dl[n] = *reinterpret_cast<const f32x4*>(trow + 8 * n + 4 * hf);
+          wg[n] = *reinterpret_cast<const f32x4*>(trow + kDkKeys + 8 * n + 4 * hf);
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float delta = dl[e / 4][e % 4], wij = wg[e / 4][e % 4];
+#pragma unroll
+          for (int np = 0; np < NP; ++np) {
+            const float x = __builtin_amdgcn_fractf(delta * w_turn[np]);
+            const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
+            const float u1 = u[np][e], u2 = u[NP + np][e];
+            dk1[np][e] = __builtin_fmaf(cs, u1, __builtin_fmaf(-sn, u2, __builtin_fmaf(wij, ql[np], dk1[np][e])));
+            dk2[np][e] = __builtin_fmaf(cs, u2, __builtin_fmaf(sn, u1, __builtin_fmaf(wij, ql[NP + np], dk2[np][e])));
+          }
+        }
       }
     }
-  }
-  if (act) {
 #pragma unroll
-    for (int kk = 0; kk < kDkKeysPerWave; ++kk) {
-      const int j = jw + kk;
-      if (j >= N) continue;
-      const int64_t off = ((int64_t)g * N + j) * D;
-      p.dk[off + dpair] = f_to_bf16(dk1[kk] * p.sm_scale);
-      p.dk[off + dpair + HALF] = f_to_bf16(dk2[kk] * p.sm_scale);
+    for (int e = 0; e < 16; ++e) {
+      const int j = jw + acc_row(e, hf);
+      if (j < N) {
+        uint16_t* op = p.dk + ((int64_t)g * N + j) * D;
+#pragma unroll
+        for (int np = 0; np < NP; ++np) {
+          op[32 * np + col] = f_to_bf16(dk1[np][e] * p.sm_scale);
+          op[32 * np + col + HALF] = f_to_bf16(dk2[np][e] * p.sm_scale);
+        }
+      }
     }
   }
 }
@@ -686,8 +719,9 @@ static hipError_t launch_corope_bwd_cfg(const CoropeBwdParams& p, const CoropeBw
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3((p.N + kDkKeys - 1) / kDkKeys, p.B * p.Hkv), dim3(kDkWaves * kWave), Cfg::kLdsBytes, stream,
-                     p, ws, fr);
+  const int n_key_blocks = (p.N + kDkKeys - 1) / kDkKeys;
+  hipLaunchKernelGGL(kern, dim3((n_key_blocks + 1) / 2, p.B * p.Hkv), dim3(kDkWaves * kWave), Cfg::kLdsBytes, stream, p, ws,
+                     fr);
   return hipGetLastError();
 }
 
