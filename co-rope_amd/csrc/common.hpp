@@ -43,6 +43,16 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
                                                  0, 0, 0);
 }
 
+// The same tile shape with fp16 operands (11 significant bits instead of 8).
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+__device__ __forceinline__ f32x16 mfma32_f16(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+// Two floats -> packed fp16 (lo in bits 0..15), rounded toward zero by the one-instruction conversion.
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+}
+
 // Row index (0..31) held by accumulator register i of lane-half h in a 32x32 MFMA result.
 __device__ __forceinline__ constexpr int acc_row(int i, int h) { return 8 * (i / 4) + 4 * h + (i % 4); }
 
@@ -302,6 +312,50 @@ __device__ __forceinline__ u32x4 load_a_trans_natural(const uint16_t* tile, int 
   u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
   return u32x4{a[0], a[1], b[0], b[1]};
 }
+
+// ---- wave-wide reductions and scans ---------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m);
+  return x;
+}
+// Wave-wide scan and maximum with data-parallel-primitive moves (no LDS round trips): shifts by 1, 2, 4, 8 inside each
+// row of 16 lanes, then lane 15 of rows 0 and 2 is broadcast into rows 1 and 3, then lane 31 into rows 2 and 3.  Lanes
+// without a source take `identity`.  All 64 lanes must be active.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float identity, float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity), __builtin_bit_cast(int, x),
+                                                               CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_prefix_sum(float x) {   // inclusive: lane l gets the sum over lanes 0..l
+  x += dpp_move<0x111, 0xf>(0.f, x);
+  x += dpp_move<0x112, 0xf>(0.f, x);
+  x += dpp_move<0x114, 0xf>(0.f, x);
+  x += dpp_move<0x118, 0xf>(0.f, x);
+  x += dpp_move<0x142, 0xa>(0.f, x);
+  x += dpp_move<0x143, 0xc>(0.f, x);
+  return x;
+}
+__device__ __forceinline__ float wave_last(float x) {          // lane 63's value, wave-uniform
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), kWave - 1));
+}
+__device__ __forceinline__ float wave_max(float x) {
+  x = fmaxf(x, dpp_move<0x111, 0xf>(-INFINITY, x));
+  x = fmaxf(x, dpp_move<0x112, 0xf>(-INFINITY, x));
+  x = fmaxf(x, dpp_move<0x114, 0xf>(-INFINITY, x));
+  x = fmaxf(x, dpp_move<0x118, 0xf>(-INFINITY, x));
+  x = fmaxf(x, dpp_move<0x142, 0xa>(-INFINITY, x));
+  x = fmaxf(x, dpp_move<0x143, 0xc>(-INFINITY, x));
+  return wave_last(x);
+}
+
+__device__ __forceinline__ float bf16_to_f(uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
+__device__ __forceinline__ uint16_t f_to_bf16(float x) { return (uint16_t)(pack_bf16(x, 0.f) & 0xffffu); }
+
+// For kernels that run one wave per workgroup: a wave's LDS instructions execute in program order, so LDS written by
+// the wave can be read back by it without a barrier or a wait; all that is needed is that the compiler keeps the
+// accesses in program order.  (A workgroup barrier would also wait for the global loads issued ahead of time.)
+__device__ __forceinline__ void lds_order() { asm volatile("" ::: "memory"); }
 
 // f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
 // in the body, so register arrays indexed with it never look dynamically indexed to the optimiser.

@@ -56,58 +56,6 @@ struct CoropeBwdWs {
   __device__ __host__ float* dp(int h) const { return base + (int64_t)(2 * n_groups + 2 * n_heads + h) * NN; }
 };
 
-__device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m);
-  return x;
-}
-// Wave-wide scan and maximum with data-parallel-primitive moves (no LDS round trips): shifts by 1, 2, 4, 8 inside each
-// row of 16 lanes, then lane 15 of rows 0 and 2 is broadcast into rows 1 and 3, then lane 31 into rows 2 and 3.  Lanes
-// without a source take `identity`.  All 64 lanes must be active.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_move(float identity, float x) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, identity), __builtin_bit_cast(int, x),
-                                                               CTRL, ROW_MASK, 0xf, false));
-}
-__device__ __forceinline__ float wave_prefix_sum(float x) {   // inclusive: lane l gets the sum over lanes 0..l
-  x += dpp_move<0x111, 0xf>(0.f, x);
-  x += dpp_move<0x112, 0xf>(0.f, x);
-  x += dpp_move<0x114, 0xf>(0.f, x);
-  x += dpp_move<0x118, 0xf>(0.f, x);
-  x += dpp_move<0x142, 0xa>(0.f, x);
-  x += dpp_move<0x143, 0xc>(0.f, x);
-  return x;
-}
-__device__ __forceinline__ float wave_last(float x) {          // lane 63's value, wave-uniform
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), kWave - 1));
-}
-__device__ __forceinline__ float wave_max(float x) {
-  x = fmaxf(x, dpp_move<0x111, 0xf>(-INFINITY, x));
-  x = fmaxf(x, dpp_move<0x112, 0xf>(-INFINITY, x));
-  x = fmaxf(x, dpp_move<0x114, 0xf>(-INFINITY, x));
-  x = fmaxf(x, dpp_move<0x118, 0xf>(-INFINITY, x));
-  x = fmaxf(x, dpp_move<0x142, 0xa>(-INFINITY, x));
-  x = fmaxf(x, dpp_move<0x143, 0xc>(-INFINITY, x));
-  return wave_last(x);
-}
-
-// One (N, D) bf16 row as D/8 16-byte words in registers; element e as float (one shift or mask per use).
-template <int D>
-struct RowRegs {
-  u32x4 w[D / 8];
-  __device__ __forceinline__ void load(const uint16_t* row) {
-#pragma unroll
-    for (int i = 0; i < D / 8; ++i) w[i] = *reinterpret_cast<const u32x4*>(row + 8 * i);
-  }
-  __device__ __forceinline__ float at(int e) const {   // e: compile-time after unrolling
-    const uint32_t x = w[e / 8][(e % 8) / 2];
-    return (e % 2) ? bf16_hi(x) : bf16_lo(x);
-  }
-};
-
-__device__ __forceinline__ float bf16_to_f(uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
-__device__ __forceinline__ uint16_t f_to_bf16(float x) { return (uint16_t)(pack_bf16(x, 0.f) & 0xffffu); }
-
 // ---------------------------------------------------------------------------------------------------- row dots
 // out[idx][i][j] = a[idx * a_mul][i] . b[idx / b_div][j] for the tiles that touch the causal triangle: the two plain
 // matrix products of the backward (leader logits qL K^T per group: a_mul = G, b_div = 1; dP = dO V^T per head: a_mul
@@ -144,11 +92,6 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_rowdot_kernel(const uint
 }
 
 // ---------------------------------------------------------------------------------------------------- scores
-// The scores kernel runs one wave per workgroup, and a wave's LDS instructions execute in program order, so LDS
-// written by the wave can be read back by it without a barrier or a wait; all that is needed is that the compiler keeps
-// the accesses in program order.  (A workgroup barrier would also wait for the global loads issued ahead of time.)
-__device__ __forceinline__ void lds_order() { asm volatile("" ::: "memory"); }
-
 // One wave per (group, query row i), all G heads at once, lane = key.  Per 64-key chunk the lanes rotate their keys
 // (the only place sines and cosines are evaluated) and park them in LDS as bf16; everything that is a dot product with
 // the rotated key then runs on the matrix cores: the raw scores q^h . kt and their derivatives with respect to delta

@@ -9,310 +9,246 @@
 //   score[i,j] = s * sum_d ( (q1 k1 + q2 k2) cos(delta w_d) - (q2 k1 - q1 k2) sin(delta w_d) )
 //              = s * q[i] . R(delta[i,j]) k[j]      with R rotating each (k1, k2) pair by -delta w_d
 //
-// Two restatements keep the work down.  (1) delta is a suffix sum that starts at the diagonal, so key tiles are
-// swept right to left and delta accumulates directly: the reference's extra pass over all keys (:103-135) and
-// the cancellation in a[i,i] - a[i,j] disappear (online softmax does not care about tile order).  (2) The
-// angle is shared by the whole group, so the key pair is rotated once per (i, j, d) and every head of the
-// group is then a plain dot product with it: 4 + 2G multiply-adds instead of 6G.
+// Three restatements keep the work down.  (1) delta is a suffix sum that starts at the diagonal, so key chunks are
+// swept right to left and delta accumulates directly: the reference's extra pass over all keys (:103-135) and the
+// cancellation in a[i,i] - a[i,j] disappear (online softmax does not care about chunk order).  (2) The angle is
+// shared by the whole group, so the key is rotated once per (i, j, d) - the only place sines and cosines are evaluated.
+// (3) With the rotated keys parked in LDS, everything that is a dot product with a key row runs on the matrix cores:
+// the leader logits q_leader K^T (bf16 x bf16: exact products), the scores q^h Kt^T (one (G x D) x (D x 64 keys)
+// product per chunk, rows beyond G idle), and O^T += V^T P^T.  The rotated keys are rounded to fp16, not bf16, and the
+// score product runs in fp16 (the bf16 queries convert exactly): 11 significant bits keep the scores as accurate as the
+// bf16 rounding of P afterwards, also at sm_scale = 1 where a bf16 key would cost several percent of a weight.
 //
-// The kernel is bound by the D/2 sin/cos pairs per (query, key) and group, not by matrix math.  Mapping:
-// one workgroup = 4 waves = one (batch, kv head) x a block of query rows; each wave owns R = 32/G rows, i.e.
-// 32 (row, head) "virtual rows".  For one key tile (64 keys) a wave works in two domains:
-//   lane = key:   the key row sits in registers (fp32); query values are wave-uniform and come in through
-//                 scalar loads; per row: leader logit, gate, suffix scan across lanes, then the rotated dots
-//                 for the G heads; raw scores go to an LDS scratch [virtual row][key];
-//   lane = virtual row (MFMA layout): online softmax exactly as in the RoPE-attention forward, then
-//                 O^T += V^T P^T with 32x32x16 bf16 MFMAs (V tile read transposed from LDS).
+// Mapping: one wave (= one workgroup) per (batch, kv head, query row), longest rows first; lane = key inside a 64-key
+// chunk.  Per chunk: the contiguous 64 x D block of K is fetched with whole cache lines per instruction and parked in
+// the LDS tile -> logits (MFMA, results moved back to lane = key with v_permlane32_swap) -> gate, scan over the lanes,
+// delta -> each lane rotates its own key row in place -> scores (MFMA) -> online softmax with a wave-uniform running
+// maximum -> the block of V replaces the rotated keys in the tile -> O accumulation (MFMA).  A wave's LDS instructions
+// execute in order, so the kernel needs no barriers; global loads for the next step are issued one step ahead.
 #include "common.hpp"
 #include "kernels.hpp"
 
 namespace corope {
-
-constexpr int kCoBlockN = 64;   // keys per tile == lanes per wave
-constexpr int kCoWaves = 4;
 
 struct CoropeFreqs {
   float w[64];  // inverse frequencies divided by 2*pi (revolutions per unit of delta), D/2 entries used
 };
 
 template <int D, int G>
-struct CoropeCfg {
-  static constexpr int kR = 32 / G;                                    // query rows per wave
-  static constexpr int kRowsWg = kR * kCoWaves;                        // query rows per workgroup
-  static constexpr int kQW = 2 * G;                                    // floats per (row, rotation pair): (q1, q2) per head
-  static constexpr int kSStride = kCoBlockN + 4;                       // floats per scratch row
-  static constexpr int kKBytes = RowTile<D>::bytes(kCoBlockN);          // K tile, row-major bf16, read row-wise
-  static constexpr int kVPad = 32;                                     // V tile is read only through the transposing load
-  static constexpr int kVBytes = RowTile<D, kVPad>::bytes(kCoBlockN);
-  static constexpr int kSBytes = 32 * kSStride * 4;                     // score scratch, per wave
-  static constexpr int kQBytes = kRowsWg * (D / 2) * kQW * 4;           // the workgroup's queries as fp32, all heads
-  static constexpr int kWBytes = (D / 2) * 4;                           // inverse frequencies
-  static constexpr int kOffV = kKBytes;
-  static constexpr int kOffS = kOffV + kVBytes;
-  static constexpr int kOffQ = kOffS + kCoWaves * kSBytes;
-  static constexpr int kOffW = kOffQ + kQBytes;
-  static constexpr int kLdsBytes = kOffW + kWBytes;
-};
-
-template <int D, int G>
-__global__ __launch_bounds__(kCoWaves* kWave) void corope_gqa_fwd_kernel(CoropeParams p, CoropeFreqs fr) {
-  using Cfg = CoropeCfg<D, G>;
-  constexpr int R = Cfg::kR;             // query rows per wave
-  constexpr int VR = R * G;              // virtual rows in use (<= 32)
-  constexpr int ROWS_WG = Cfg::kRowsWg;  // query rows per workgroup
-  constexpr int HALF = D / 2, NDB = D / 32;
-  constexpr int LSV = RowTile<D, Cfg::kVPad>::kStride;
-  constexpr int NT = kCoWaves * kWave;
-  constexpr int QW = Cfg::kQW;
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint16_t* ks = reinterpret_cast<uint16_t*>(smem);
-  uint16_t* vs = reinterpret_cast<uint16_t*>(smem + Cfg::kOffV);
-  float* qs = reinterpret_cast<float*>(smem + Cfg::kOffQ);
-  float* ws = reinterpret_cast<float*>(smem + Cfg::kOffW);
-
-  const int lane = threadIdx.x % kWave;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  float* ss = reinterpret_cast<float*>(smem + Cfg::kOffS + wave * Cfg::kSBytes);
-
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void corope_gqa_fwd_kernel(CoropeParams p,
+                                                                                                       CoropeFreqs fr) {
+  constexpr int HALF = D / 2, KS = D + 8, WS = kWave + 8, NDB = D / 32, PIECES = D / 8;
+  constexpr int NI = 4 * ((G - 1) / 8 + 1);                            // accumulator registers that hold rows < G
+  __shared__ __attribute__((aligned(16))) uint16_t tile[kWave * KS];   // [key][d]: K (bf16), then rotated K (fp16), then V (bf16)
+  __shared__ __attribute__((aligned(16))) uint16_t ql[D];              // the leader's query row (bf16)
+  __shared__ __attribute__((aligned(16))) uint16_t wts[G * WS];        // [head][key] bf16 softmax weights of the chunk
   const int n_groups = p.B * p.Hkv;
-  const int grp = blockIdx.x % n_groups;                       // (batch, kv head)
-  const int mb = p.num_m_blocks - 1 - blockIdx.x / n_groups;   // heaviest row blocks first
+  const int grp = blockIdx.x % n_groups;
+  const int i = p.N - 1 - blockIdx.x / n_groups;                       // longest rows first
+  const int lane = threadIdx.x;
+  const int vr = lane % 32, hf = lane / 32;                            // matrix-core identity of this lane
   const int b = grp / p.Hkv, kvh = grp % p.Hkv;
   const int N = p.N;
-  const int m0 = mb * ROWS_WG;
-  const int row0 = m0 + wave * R;                              // first query row of this wave
-  const int row_hi = min(row0 + R - 1, N - 1);
+  const int head0 = b * p.Hq + kvh * G;
+  const uint16_t* kbase = p.k + (int64_t)grp * N * D;
+  const uint16_t* vbase = p.v + (int64_t)grp * N * D;
+  const int n_chunks = i / kWave + 1;
+  const float scale2 = p.sm_scale * 1.4426950408889634f;               // scores in the base-2 domain
 
-  const uint16_t* kg = p.k + ((int64_t)b * p.Hkv + kvh) * N * D;
-  const uint16_t* vg = p.v + ((int64_t)b * p.Hkv + kvh) * N * D;
-  const uint32_t* qg = reinterpret_cast<const uint32_t*>(p.q + ((int64_t)b * p.Hq + (int64_t)kvh * G) * N * D);
-  const int64_t q_head_words = (int64_t)N * D / 2;              // 32-bit words between consecutive heads
+  // A operand of the score product, constant over the row: lane (vr, hf) holds columns 16 ks + 8 hf .. + 7 of q^vr as fp16
+  // for vr < G, zeros otherwise.  The logit product takes the leader's row in bf16 from LDS (lanes with vr = 0).
+  u32x4 aop[D / 16];
+  {
+    const uint16_t* qrow = p.q + ((int64_t)(head0 + (vr < G ? vr : 0)) * N + i) * D + 8 * hf;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
+      u32x4 h16;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) h16[e] = pack_f16(bf16_lo(raw[e]), bf16_hi(raw[e]));
+      aop[ks] = vr < G ? h16 : u32x4{0, 0, 0, 0};
+    }
+    const uint16_t* lrow = p.q + ((int64_t)head0 * N + i) * D;
+    for (int d = lane; d < D; d += kWave) ql[d] = lrow[d];
+  }
 
-  // MFMA-domain identity of this lane
-  const int lv = lane % 32, lh = lane / 32;                    // virtual row, lane half
-  const int my_row = row0 + lv / G;                            // query row of the virtual row
-  const int my_head = lv % G;
+  // one 64 x D block of K or V: consecutive 16-byte pieces per lane, parked as rows of the tile
+  u32x4 blk[PIECES];
+  auto fetch_block = [&](const uint16_t* base, int c) __attribute__((always_inline)) {
+    const uint16_t* block = base + (int64_t)c * kWave * D;   // wave-uniform
+    if (c * kWave + kWave <= N) {
+#pragma unroll
+      for (int it = 0; it < PIECES; ++it)
+        blk[it] = *reinterpret_cast<const u32x4*>(byte_offset(block, 16u * lane + 1024u * it));
+    } else {   // the block runs past the last key: clamp the rows (only the chunk on the diagonal can get here)
+#pragma unroll
+      for (int it = 0; it < PIECES; ++it) {
+        const int row = (it * kWave + lane) / PIECES, piece = lane % PIECES;
+        blk[it] = *reinterpret_cast<const u32x4*>(base + (int64_t)min(c * kWave + row, N - 1) * D + 8 * piece);
+      }
+    }
+  };
+  auto park_block = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int it = 0; it < PIECES; ++it) {
+      const int row = (it * kWave + lane) / PIECES, piece = lane % PIECES;
+      *reinterpret_cast<u32x4*>(tile + row * KS + 8 * piece) = blk[it];
+    }
+  };
+  // (rows < G of a 64-key product) -> this lane's key: swapping the upper half of the keys-below-32 result with the lower
+  // half of the keys-from-32 result puts every key's rows into its own lane
+  auto rows_of_key = [&](const f32x16& c0, const f32x16& c1, float (&out)[G]) __attribute__((always_inline)) {
+    float lo_rows[NI], hi_rows[NI];   // rows 8 (n / 4) + n % 4 and the same + 4
+#pragma unroll
+    for (int n = 0; n < NI; ++n) {
+      const float x0 = c0[n], x1 = c1[n];   // (a bit_cast applied directly to a vector element reads element 0)
+      const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x0), __builtin_bit_cast(uint32_t, x1),
+                                                      false, false);
+      lo_rows[n] = __builtin_bit_cast(float, (uint32_t)r[0]);
+      hi_rows[n] = __builtin_bit_cast(float, (uint32_t)r[1]);
+    }
+#pragma unroll
+    for (int h = 0; h < G; ++h) out[h] = (h / 4) % 2 ? hi_rows[4 * (h / 8) + h % 4] : lo_rows[4 * (h / 8) + h % 4];
+  };
+  auto leader_times_tile = [&](f32x16& c0, f32x16& c1) __attribute__((always_inline)) {   // bf16: K as parked
+    c0 = f32x16{0};
+    c1 = f32x16{0};
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      u32x4 a = u32x4{0, 0, 0, 0};
+      if (vr == 0) a = *reinterpret_cast<const u32x4*>(ql + 16 * ks + 8 * hf);
+      c0 = mfma32(a, *reinterpret_cast<const u32x4*>(tile + vr * KS + 16 * ks + 8 * hf), c0);
+      c1 = mfma32(a, *reinterpret_cast<const u32x4*>(tile + (32 + vr) * KS + 16 * ks + 8 * hf), c1);
+    }
+  };
+  auto heads_times_tile = [&](f32x16& c0, f32x16& c1) __attribute__((always_inline)) {    // fp16: the rotated keys
+    c0 = f32x16{0};
+    c1 = f32x16{0};
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      c0 = mfma32_f16(aop[ks], *reinterpret_cast<const u32x4*>(tile + vr * KS + 16 * ks + 8 * hf), c0);
+      c1 = mfma32_f16(aop[ks], *reinterpret_cast<const u32x4*>(tile + (32 + vr) * KS + 16 * ks + 8 * hf), c1);
+    }
+  };
 
+  // oacc[db][4 g4 + e]: column 32 db + 8 g4 + 4 hf + e of head `vr`'s output row (lanes with vr >= G idle)
   f32x16 oacc[NDB];
 #pragma unroll
-  for (int i = 0; i < NDB; ++i) oacc[i] = f32x16{0};
-  float m_run = -INFINITY, l_run = 0.f;
-  float carry_v = 0.f;                                         // lane r holds the mileage carried by row r
-
-  const float scale2 = p.sm_scale * 1.4426950408889634f;
-  const int t_hi = min(m0 + ROWS_WG - 1, N - 1) / kCoBlockN;
-
-  // ---- the workgroup's query rows, all heads of the group, as fp32 in LDS: [row][pair d][head][q1, q2] -----------
-  // (wave-uniform operands of the lane = key domain are read from here with broadcast LDS loads)
-  for (int u = threadIdx.x; u < ROWS_WG * G * (HALF / 8); u += NT) {
-    const int ch = u % (HALF / 8), g = (u / (HALF / 8)) % G, row = u / ((HALF / 8) * G);
-    const uint32_t* src = qg + (int64_t)g * q_head_words + (int64_t)min(m0 + row, N - 1) * (D / 2) + ch * 4;
-    u32x4 x1 = *reinterpret_cast<const u32x4*>(src);
-    u32x4 x2 = *reinterpret_cast<const u32x4*>(src + HALF / 2);
+  for (int db = 0; db < NDB; ++db) oacc[db] = f32x16{0};
+  float m_run[G], l_run[G];   // running maximum (wave-uniform, base-2 domain) and this lane's sum of 2^(s - m)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float a = e % 2 ? bf16_hi(x1[e / 2]) : bf16_lo(x1[e / 2]);
-      float b2 = e % 2 ? bf16_hi(x2[e / 2]) : bf16_lo(x2[e / 2]);
-      *reinterpret_cast<f32x2*>(qs + ((row * HALF) + ch * 8 + e) * QW + 2 * g) = f32x2{a, b2};
-    }
+  for (int h = 0; h < G; ++h) {
+    m_run[h] = -INFINITY;
+    l_run[h] = 0.f;
   }
-  if (threadIdx.x < HALF) ws[threadIdx.x] = fr.w[threadIdx.x];
+  float carry = 0.f;          // sum of the gates of the chunks to the right (up to the diagonal)
 
-  CopyStage<D, kCoBlockN, NT> kst;
-  CopyStage<D, kCoBlockN, NT, Cfg::kVPad> vst;
-  for (int t = t_hi; t >= 0; --t) {
-    const int n0 = t * kCoBlockN;
-    kst.load(kg, n0, N);
-    vst.load(vg, n0, N);
-    __syncthreads();  // previous tile fully consumed
-    kst.store_rows(ks);
-    vst.store_rows(vs);
-    __syncthreads();
-
-    if (n0 <= row_hi) {
-      // ------------------------------------------------------------------ lane = key
-      float k1[HALF], k2[HALF];
-      {
-        const uint16_t* kr = ks + RowTile<D>::off(lane, 0);
-#pragma unroll
-        for (int c = 0; c < HALF / 8; ++c) {
-          u32x4 a = *reinterpret_cast<const u32x4*>(kr + 8 * c);
-          u32x4 bq = *reinterpret_cast<const u32x4*>(kr + HALF + 8 * c);
-#pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            k1[8 * c + 2 * w] = bf16_lo(a[w]);
-            k1[8 * c + 2 * w + 1] = bf16_hi(a[w]);
-            k2[8 * c + 2 * w] = bf16_lo(bq[w]);
-            k2[8 * c + 2 * w + 1] = bf16_hi(bq[w]);
-          }
-        }
-      }
-      const int key = n0 + lane;
+  fetch_block(kbase, n_chunks - 1);
 #pragma unroll 1
-      for (int r = 0; r < R; ++r) {
-        const int row = min(row0 + r, N - 1);                   // wave-uniform
-        const float* qrow = qs + (wave * R + r) * HALF * QW;     // fp32 (q1, q2) pairs of every head, broadcast reads
-        // leader logit (head 0 of the group)
-        float logit = 0.f;
-        {
-          // chunks of 8 pairs, fetched one chunk ahead; the scheduling barrier keeps the (fully unrolled) loop from
-          // hoisting every LDS read to the top and drowning in registers
-          f32x2 qc[8], qn[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) qc[e] = *reinterpret_cast<const f32x2*>(qrow + e * QW);
-#pragma unroll
-          for (int d8 = 0; d8 < HALF; d8 += 8) {
-            if (d8 + 8 < HALF) {
-#pragma unroll
-              for (int e = 0; e < 8; ++e) qn[e] = *reinterpret_cast<const f32x2*>(qrow + (d8 + 8 + e) * QW);
-            }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              logit = __builtin_fmaf(qc[e][0], k1[d8 + e], logit);
-              logit = __builtin_fmaf(qc[e][1], k2[d8 + e], logit);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) qc[e] = qn[e];
-          }
-        }
-        float z = 1.f / (1.f + __expf(-logit * p.sm_scale));
-        if (key > row) z = 0.f;                                  // gates beyond the diagonal do not count
-        // inclusive suffix sum over the lanes (keys to the right within the tile)
-        float suf = z;
-#pragma unroll
-        for (int off = 1; off < kWave; off <<= 1) {
-          float o = __shfl_down(suf, off);
-          if (lane + off < kWave) suf += o;
-        }
-        const float carry = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, carry_v), r));
-        const float delta = carry + (suf - z);
-        const float total = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, suf)));
-        if (lane == r) carry_v = carry + total;
+  for (int c = n_chunks - 1; c >= 0; --c) {
+    const int j = c * kWave + lane;
+    const bool valid = j <= i;
+    park_block();                 // K of this chunk
+    fetch_block(vbase, c);        // V of this chunk: needed after the scores
+    lds_order();                  // (also orders the one-time write of the leader's row before its first read)
 
-        float acc[G];
-#pragma unroll
-        for (int g = 0; g < G; ++g) acc[g] = 0.f;
-        {
-          constexpr int CH = G <= 4 ? 4 : 2;   // rotation pairs per chunk (bounds the registers of the look-ahead)
-          typedef float wvec __attribute__((ext_vector_type(CH)));
-          f32x2 qc[CH][G], qn[CH][G];
-          wvec wc = *reinterpret_cast<const wvec*>(ws), wn = wc;
-#pragma unroll
-          for (int e = 0; e < CH; ++e)
-#pragma unroll
-            for (int g = 0; g < G; ++g) qc[e][g] = *reinterpret_cast<const f32x2*>(qrow + e * QW + 2 * g);
-#pragma unroll
-          for (int d0 = 0; d0 < HALF; d0 += CH) {
-            if (d0 + CH < HALF) {
-              wn = *reinterpret_cast<const wvec*>(ws + d0 + CH);
-#pragma unroll
-              for (int e = 0; e < CH; ++e)
-#pragma unroll
-                for (int g = 0; g < G; ++g) qn[e][g] = *reinterpret_cast<const f32x2*>(qrow + (d0 + CH + e) * QW + 2 * g);
-            }
-#pragma unroll
-            for (int e = 0; e < CH; ++e) {
-              const int d = d0 + e;
-              float x = __builtin_amdgcn_fractf(delta * wc[e]);
-              float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
-              float r1 = __builtin_fmaf(cs, k1[d], sn * k2[d]);
-              float r2 = __builtin_fmaf(cs, k2[d], -(sn * k1[d]));
-#pragma unroll
-              for (int g = 0; g < G; ++g) {
-                acc[g] = __builtin_fmaf(qc[e][g][0], r1, acc[g]);
-                acc[g] = __builtin_fmaf(qc[e][g][1], r2, acc[g]);
-              }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            wc = wn;
-#pragma unroll
-            for (int e = 0; e < CH; ++e)
-#pragma unroll
-              for (int g = 0; g < G; ++g) qc[e][g] = qn[e][g];
-          }
-        }
-#pragma unroll
-        for (int g = 0; g < G; ++g) ss[(r * G + g) * Cfg::kSStride + lane] = acc[g] * scale2;
+    // leader logits (row 0 of the product), gates, delta
+    f32x16 c0, c1;
+    leader_times_tile(c0, c1);
+    float lg[G];
+    rows_of_key(c0, c1, lg);
+    const float z = valid ? 1.f / (1.f + __expf(-lg[0] * p.sm_scale)) : 0.f;   // gates beyond the diagonal do not count
+    const float zpre = wave_prefix_sum(z), ztot = wave_last(zpre);
+    const float delta = carry + (ztot - zpre);   // gates strictly to the right of this key, up to the diagonal
+    carry += ztot;
+
+    // each lane rotates its own key row in place: one step of look-ahead in two alternating register sets; the scheduling
+    // barriers keep the LDS reads from all moving to the top
+    u32x2 wa[2][2];
+    wa[0][0] = *reinterpret_cast<const u32x2*>(tile + lane * KS);
+    wa[0][1] = *reinterpret_cast<const u32x2*>(tile + lane * KS + HALF);
+    static_for<HALF / 4>([&](auto step_c) __attribute__((always_inline)) {
+      constexpr int step = decltype(step_c)::value, d0 = step * 4;
+      if (d0 + 4 < HALF) {
+        wa[(step + 1) % 2][0] = *reinterpret_cast<const u32x2*>(tile + lane * KS + d0 + 4);
+        wa[(step + 1) % 2][1] = *reinterpret_cast<const u32x2*>(tile + lane * KS + HALF + d0 + 4);
       }
+      const u32x2 w1 = wa[step % 2][0], w2 = wa[step % 2][1];
+      float r1v[4], r2v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float x = __builtin_amdgcn_fractf(delta * fr.w[d0 + e]);
+        const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
+        const float k1 = e % 2 ? bf16_hi(w1[e / 2]) : bf16_lo(w1[e / 2]);
+        const float k2 = e % 2 ? bf16_hi(w2[e / 2]) : bf16_lo(w2[e / 2]);
+        r1v[e] = __builtin_fmaf(cs, k1, sn * k2);
+        r2v[e] = __builtin_fmaf(cs, k2, -(sn * k1));
+      }
+      *reinterpret_cast<u32x2*>(tile + lane * KS + d0) = u32x2{pack_f16(r1v[0], r1v[1]), pack_f16(r1v[2], r1v[3])};
+      *reinterpret_cast<u32x2*>(tile + lane * KS + HALF + d0) = u32x2{pack_f16(r2v[0], r2v[1]), pack_f16(r2v[2], r2v[3])};
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    lds_order();
+
+    // scores of every head, online softmax
+    heads_times_tile(c0, c1);
+    float sc[G];
+    rows_of_key(c0, c1, sc);
+    float al = 1.f;          // this lane's head's rescale factor
+    bool moved = false;      // wave-uniform: some head's running maximum moved
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      const float s2 = sc[h] * scale2;
+      const float m_new = fmaxf(m_run[h], wave_max(valid ? s2 : -INFINITY));   // finite: the chunk holds a key <= i
+      const float a = fast_exp2(m_run[h] - m_new), e = valid ? fast_exp2(s2 - m_new) : 0.f;
+      moved |= m_new != m_run[h];
+      m_run[h] = m_new;
+      l_run[h] = __builtin_fmaf(l_run[h], a, e);
+      al = vr == h ? a : al;
+      wts[h * WS + lane] = f_to_bf16(e);
     }
-    __syncthreads();  // scratch written (each wave reads only its own scratch; the barrier orders LDS traffic)
-
-    if (n0 <= row_hi) {
-      // ------------------------------------------------------------------ lane = virtual row
-      float sv[kCoBlockN / 16][8];
-      const bool diag = n0 + kCoBlockN - 1 > row0;
-      float mt = -INFINITY;
-#pragma unroll
-      for (int c = 0; c < kCoBlockN / 16; ++c) {
-        const float* sp = ss + lv * Cfg::kSStride + 16 * c + 8 * lh;
-        f32x4 a = *reinterpret_cast<const f32x4*>(sp), bq = *reinterpret_cast<const f32x4*>(sp + 4);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          float x = j < 4 ? a[j] : bq[j - 4];
-          if (diag && (n0 + 16 * c + 8 * lh + j) > my_row) x = -INFINITY;
-          sv[c][j] = x;
-          mt = fmaxf(mt, x);
-        }
-      }
-      mt = half_max(mt);
-      // A wave's rows may straddle a tile boundary: a row below the tile sees no key of it yet (all -inf).
-      const float m_max = fmaxf(m_run, mt);
-      const float m_new = m_max == -INFINITY ? 0.f : m_max;
-      const float alpha = fast_exp2(m_run - m_new);
-      m_run = m_max;
-      float lsum = 0.f;
-      u32x4 pb[kCoBlockN / 16];
-#pragma unroll
-      for (int c = 0; c < kCoBlockN / 16; ++c)
-#pragma unroll
-        for (int j = 0; j < 8; j += 2) {
-          float p0 = fast_exp2(sv[c][j] - m_new), p1 = fast_exp2(sv[c][j + 1] - m_new);
-          lsum += p0 + p1;
-          pb[c][j / 2] = pack_bf16(p0, p1);
-        }
-      l_run = l_run * alpha + lsum;
+    if (moved) {
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
-#pragma unroll
-      for (int c = 0; c < kCoBlockN / 16; ++c)
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-          oacc[db] = mfma32(load_a_trans_natural(vs, LSV, 16 * c, db * 32), pb[c], oacc[db]);
+        for (int e = 0; e < 16; ++e) oacc[db][e] *= al;
     }
+    park_block();                          // V replaces the rotated keys
+    if (c > 0) fetch_block(kbase, c - 1);  // K of the next chunk
+    lds_order();
+#pragma unroll
+    for (int ks = 0; ks < kWave / 16; ++ks) {
+      u32x4 bop = u32x4{0, 0, 0, 0};
+      if (vr < G) bop = *reinterpret_cast<const u32x4*>(wts + vr * WS + 16 * ks + 8 * hf);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) oacc[db] = mfma32(load_a_trans_natural(tile, KS, 16 * ks, 32 * db), bop, oacc[db]);
+    }
+    lds_order();
   }
 
-  const float l_tot = half_sum(l_run);
-  const float inv_l = l_tot > 0.f ? 1.f / l_tot : 0.f;   // same guard as the reference's epilogue (:343-345)
-  if (lv < VR && my_row < N) {
-    uint16_t* op = p.o + (((int64_t)b * p.Hq + kvh * G + my_head) * N + my_row) * D;
+  float inv_l = 0.f;
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    const float l = wave_sum(l_run[h]);
+    inv_l = vr == h ? (l > 0.f ? 1.f / l : 0.f) : inv_l;   // same guard as the reference's epilogue (:343-345)
+  }
+  if (vr < G) {
+    uint16_t* op = p.o + ((int64_t)(head0 + vr) * N + i) * D;
 #pragma unroll
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w = {pack_bf16(oacc[db][4 * g] * inv_l, oacc[db][4 * g + 1] * inv_l),
-                   pack_bf16(oacc[db][4 * g + 2] * inv_l, oacc[db][4 * g + 3] * inv_l)};
-        *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g + 4 * lh) = w;
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const u32x2 w = {pack_bf16(oacc[db][4 * g4] * inv_l, oacc[db][4 * g4 + 1] * inv_l),
+                         pack_bf16(oacc[db][4 * g4 + 2] * inv_l, oacc[db][4 * g4 + 3] * inv_l)};
+        *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
       }
   }
 }
 
 template <int D, int G>
 static hipError_t launch_corope_cfg(CoropeParams p, const CoropeFreqs& fr, hipStream_t stream) {
-  using Cfg = CoropeCfg<D, G>;
-  auto kern = corope_gqa_fwd_kernel<D, G>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       Cfg::kLdsBytes);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
-  constexpr int rows_wg = Cfg::kRowsWg;
-  p.num_m_blocks = (p.N + rows_wg - 1) / rows_wg;
-  hipLaunchKernelGGL(kern, dim3(p.num_m_blocks * p.B * p.Hkv), dim3(kCoWaves * kWave), Cfg::kLdsBytes, stream, p, fr);
+  p.num_m_blocks = p.N;   // one query row per workgroup
+  hipLaunchKernelGGL((corope_gqa_fwd_kernel<D, G>), dim3(p.N * p.B * p.Hkv), dim3(kWave), 0, stream, p, fr);
   return hipGetLastError();
 }
 
