@@ -351,6 +351,7 @@ __device__ __forceinline__ float wave_max(float x) {
 
 __device__ __forceinline__ float bf16_to_f(uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
 __device__ __forceinline__ uint16_t f_to_bf16(float x) { return (uint16_t)(pack_bf16(x, 0.f) & 0xffffu); }
+__device__ __forceinline__ uint16_t f_to_f16(float x) { return (uint16_t)(pack_f16(x, 0.f) & 0xffffu); }
 
 // For kernels that run one wave per workgroup: a wave's LDS instructions execute in program order, so LDS written by
 // the wave can be read back by it without a barrier or a wait; all that is needed is that the compiler keeps the

@@ -32,8 +32,10 @@
 //   dv           dv^T += dO^T P on the matrix cores, 128 keys per workgroup
 //   dk           one workgroup per (group, 32 keys), lane = rotation pair: rotates sum_h dS^h q^h per (i, j) and adds the
 //                gate path W qL; tiles of DELTA, W, DS staged through LDS
-// Rounding: operands of the matrix products are bf16 (the rotated keys, the softmax weights e and e dP, W, P); sums,
-// statistics, delta, dS/ddelta and everything stored in the workspace are fp32.
+// Rounding: the rotated keys and what multiplies them (queries, the softmax weights e and e dP) are fp16 - the bf16
+// queries convert exactly, and 11 significant bits keep scores accurate at sm_scale = 1 too; the products on unrotated
+// rows (W K, P dO, the row dots) take bf16 operands; sums, statistics, delta, dS/ddelta and everything stored in the
+// workspace are fp32.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -101,8 +103,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   constexpr int HALF = D / 2;
   constexpr int KS = D + 8, WS = kWave + 8, NVR = 2 * G + 1, NDB = D / 32;
   constexpr int NI = 4 * ((2 * G - 1) / 8 + 1);                       // accumulator registers that hold rows < 2G
-  __shared__ __attribute__((aligned(16))) uint16_t kt[kWave * KS];    // [key][d] bf16: rotated keys, later plain keys
-  __shared__ __attribute__((aligned(16))) uint16_t wts[NVR * WS];     // [virtual row][key] bf16 weights of the keys
+  __shared__ __attribute__((aligned(16))) uint16_t kt[kWave * KS];    // [key][d]: keys (bf16), rotated in place (fp16)
+  __shared__ __attribute__((aligned(16))) uint16_t wts[NVR * WS];     // [virtual row][key] weights: fp16, row 2G (W) bf16
   const int i = p.N - 1 - blockIdx.x, g = blockIdx.y, lane = threadIdx.x;   // longest rows first
   const int vr = lane % 32, hf = lane / 32;                                  // matrix-core identity of this lane
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
@@ -118,7 +120,9 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       const int d0 = 16 * ks + 8 * hf;                      // first of this lane's 8 columns
       u32x4 val = u32x4{0, 0, 0, 0};
       if (vr < G) {
-        val = *reinterpret_cast<const u32x4*>(qrow + d0);
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + d0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) val[e] = pack_f16(bf16_lo(raw[e]), bf16_hi(raw[e]));   // exact
       } else if (vr < 2 * G) {
         const bool upper = d0 >= HALF;                       // columns of the second half take w q1, the first half -w q2
         const u32x4 src = *reinterpret_cast<const u32x4*>(qrow + (upper ? d0 - HALF : d0 + HALF));
@@ -129,7 +133,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
           const float qv = e % 2 ? bf16_hi(src[e / 2]) : bf16_lo(src[e / 2]);
           x[e] = upper ? wr[e] * qv : -wr[e] * qv;
         }
-        val = u32x4{pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7])};
+        val = u32x4{pack_f16(x[0], x[1]), pack_f16(x[2], x[3]), pack_f16(x[4], x[5]), pack_f16(x[6], x[7])};
       }
       aop[ks] = val;
     }
@@ -234,8 +238,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
         r1v[e] = __builtin_fmaf(cs, k1, sn * k2);
         r2v[e] = __builtin_fmaf(cs, k2, -(sn * k1));
       }
-      *reinterpret_cast<u32x2*>(kt + lane * KS + d0) = u32x2{pack_bf16(r1v[0], r1v[1]), pack_bf16(r1v[2], r1v[3])};
-      *reinterpret_cast<u32x2*>(kt + lane * KS + HALF + d0) = u32x2{pack_bf16(r2v[0], r2v[1]), pack_bf16(r2v[2], r2v[3])};
+      *reinterpret_cast<u32x2*>(kt + lane * KS + d0) = u32x2{pack_f16(r1v[0], r1v[1]), pack_f16(r1v[2], r1v[3])};
+      *reinterpret_cast<u32x2*>(kt + lane * KS + HALF + d0) = u32x2{pack_f16(r2v[0], r2v[1]), pack_f16(r2v[2], r2v[3])};
       __builtin_amdgcn_sched_barrier(0);
     });
     lds_order();   // rotated keys are in LDS
@@ -244,8 +248,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     f32x16 c0 = f32x16{0}, c1 = f32x16{0};
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
-      c0 = mfma32(aop[ks], *reinterpret_cast<const u32x4*>(kt + vr * KS + 16 * ks + 8 * hf), c0);
-      c1 = mfma32(aop[ks], *reinterpret_cast<const u32x4*>(kt + (32 + vr) * KS + 16 * ks + 8 * hf), c1);
+      c0 = mfma32_f16(aop[ks], *reinterpret_cast<const u32x4*>(kt + vr * KS + 16 * ks + 8 * hf), c0);
+      c1 = mfma32_f16(aop[ks], *reinterpret_cast<const u32x4*>(kt + (32 + vr) * KS + 16 * ks + 8 * hf), c1);
     }
     // the results sit at lane = key % 32 with rows split over the lane halves; swapping the upper half of the keys-below-
     // 32 result with the lower half of the keys-from-32 result puts every key's rows into its own lane
@@ -286,8 +290,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       l_run[h] = __builtin_fmaf(l_run[h], a, e);
       pd_run[h] = __builtin_fmaf(pd_run[h], a, e * dpv[h]);
       al = (vr / 2 == h && vr < 2 * G) ? a : al;
-      wts[(2 * h) * WS + lane] = f_to_bf16(e * dpv[h]);
-      wts[(2 * h + 1) * WS + lane] = f_to_bf16(e);
+      wts[(2 * h) * WS + lane] = f_to_f16(e * dpv[h]);
+      wts[(2 * h + 1) * WS + lane] = f_to_f16(e);
     }
     if (c > 0) {
 #pragma unroll
@@ -305,7 +309,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       u32x4 bop = u32x4{0, 0, 0, 0};
       if (vr < 2 * G) bop = *reinterpret_cast<const u32x4*>(wts + vr * WS + 16 * ks + 8 * hf);
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) dqa[db] = mfma32(load_a_trans_natural(kt, KS, 16 * ks, 32 * db), bop, dqa[db]);
+      for (int db = 0; db < NDB; ++db) dqa[db] = mfma32_f16(load_a_trans_natural(kt, KS, 16 * ks, 32 * db), bop, dqa[db]);
     }
     lds_order();   // ... and consumed: the next chunk may overwrite them
   }

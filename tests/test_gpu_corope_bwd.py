@@ -66,6 +66,14 @@ def test_corope_backward_unit_scale_small_theta(pkg):
     _compare(_gpu_grads(pkg, q, k, v, d_o, 1.0, 100.0), _oracle_grads(q, k, v, d_o, 1.0, 100.0), 2)
 
 
+def test_corope_backward_hot_softmax(pkg):
+    """sm_scale = 1 on unit-variance inputs (the reference's comparison script, compare_corope.py:23): scores of +-20, rows
+    dominated by one or two keys.  dO is scaled down so that the gradients stay of order one; the bar is the usual one."""
+    q, k, v, d_o = _inputs(1, 4, 2, 64, 64, seed=21)
+    d_o = bf16_round(d_o * 0.125)
+    _compare(_gpu_grads(pkg, q, k, v, d_o, 1.0, 10000.0), _oracle_grads(q, k, v, d_o, 1.0, 10000.0), 2)
+
+
 def test_corope_backward_gate_path_is_material_and_right(pkg):
     """On this input the gradient through the leader's gates is a large part of dQ and dK (the oracle with the
     position offsets cut out of the graph differs by far more than the bar), so parity here pins that path; a
