@@ -216,14 +216,14 @@ def bench_corope(args):
         bev[i + 1].record()
     torch.cuda.synchronize()
     bms = sum(bev[i].elapsed_time(bev[i + 1]) for i in range(bsteps)) / bsteps
-    # lane-instructions per (sin, cos) pair, counted as for the forward (a transcendental counts once): scores kernel 13
-    # (phase 2, sin, cos, unpack 2, rotate 4, pack 1, LDS 2); dk kernel 10 (phase 2, sin, cos, rotate-accumulate 4, gate
-    # path 2); the per-head sums run on the matrix cores
-    bwd_instr = pairs * (13 + 10)
-    # VALU roofline: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz lane-instructions/s.  Per (sin, cos) pair the forward issues 12
-    # of them (phase 2, sin, cos, unpack 2, rotate 4, pack 1, LDS 1; a transcendental counted once although it issues at a
-    # quarter of the rate); the per-head dot products run on the matrix cores
-    fwd_instr = pairs * 12
+    # issue slots per (sin, cos) pair, counted as for the forward (a transcendental = 4 slots): scores kernel 11 + 8 (phase
+    # 2, unpack 2, rotate 4, pack 1, LDS 2; sin, cos); dk kernel 8 + 8 (phase 2, rotate-accumulate 4, gate path 2; sin, cos);
+    # the per-head sums run on the matrix cores
+    bwd_instr = pairs * (19 + 16)
+    # VALU roofline: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz issue slots/s.  Per (sin, cos) pair the forward needs 18 slots:
+    # 10 full-rate instructions (phase 2, unpack 2, rotate 4, pack 1, LDS 1) and two transcendentals at a quarter of the
+    # rate (4 slots each); the per-head dot products run on the matrix cores
+    fwd_instr = pairs * 18
     out = {"metric": "Co-RoPE GQA fwd, B2 Hq32 Hkv8 N4096 D128 causal", "value": round(flops / (ms * 1e-3) * 1e-12, 2),
            "unit": "TFLOP/s (attention-equivalent)", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -231,14 +231,14 @@ def bench_corope(args):
            "config": {"workload": "C5: Co-RoPE GQA attention fwd B2 Hq32 Hkv8 N4096 D128 causal bf16", "theta": 10000.0},
            "sincos_pairs_per_s": round(pairs / (kms * 1e-3), 1), "kernel_ms": round(kms, 4),
            "roofline": {"bound": "valu", "kernel": "corope_gqa_fwd", "achieved": round(fwd_instr / (kms * 1e-3) * 1e-12, 3),
-                        "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T lane-instr/s",
+                        "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T issue slots/s",
                         "frac": round(fwd_instr / (kms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4), "traffic": None},
            "backward": {"ms": round(bms, 4), "steps": bsteps, "workspace_gib": round(ws_bytes / 2**30, 2),
                         "sincos_pairs_per_s": round(2 * pairs / (bms * 1e-3), 1),
                         "tflops_attention_equivalent": round(2.5 * flops / (bms * 1e-3) * 1e-12, 2),
                         "roofline": {"bound": "valu", "kernel": "corope_gqa_bwd (5 launches)",
                                      "achieved": round(bwd_instr / (bms * 1e-3) * 1e-12, 3),
-                                     "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T lane-instr/s",
+                                     "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T issue slots/s",
                                      "frac": round(bwd_instr / (bms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4), "traffic": None}},
            "cpu_baseline": None}
     print(json.dumps(out))
