@@ -659,13 +659,8 @@ static hipError_t launch_corope_bwd_cfg(const CoropeBwdParams& p, const CoropeBw
   using Cfg = CoropeDkCfg<D, G>;
   hipLaunchKernelGGL((corope_bwd_dv_kernel<D, G>), dim3((p.N + 127) / 128, p.B * p.Hkv), dim3(4 * kWave), 0, stream, p, ws);
   auto kern = corope_bwd_dk_kernel<D, G>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       Cfg::kLdsBytes);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
   const int n_key_blocks = (p.N + kDkKeys - 1) / kDkKeys;
   hipLaunchKernelGGL(kern, dim3((n_key_blocks + 1) / 2, p.B * p.Hkv), dim3(kDkWaves * kWave), Cfg::kLdsBytes, stream, p, ws,
                      fr);

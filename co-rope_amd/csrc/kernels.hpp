@@ -4,7 +4,23 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace corope {
+
+// Raises a kernel's dynamic-LDS limit once per (kernel, device): `done` is a per-kernel word, bit d set = device d has it.
+// Safe to call from several host threads (at worst the attribute is set twice to the same value).
+inline hipError_t allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
+
 
 struct FwdParams {
   const uint16_t* q;

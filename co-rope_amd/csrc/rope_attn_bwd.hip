@@ -366,11 +366,6 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdPara
 }
 
 // ===================================================================================== launchers
-template <typename K>
-static hipError_t set_lds(K kern, int bytes) {
-  return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-}
-
 // dK and dV are produced by two launches of the same kernel template: with both sets of accumulators resident a
 // wave needs more than 256 registers, which would halve the waves per SIMD.
 template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
@@ -378,12 +373,8 @@ static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
   constexpr int NWAVES = 8, BLOCK_M = (PREROT && !DO_DK) ? 128 : 64;   // the larger tile pays off (and fits) for dV on pre-rotated operands only
   using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? 8 : 32, DO_DV && DO_DK>;
   auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK, PREROT>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = set_lds(kern, Cfg::kLdsBytes);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
   p.num_blocks = (p.N + Cfg::kBlockN - 1) / Cfg::kBlockN;
   hipLaunchKernelGGL(kern, dim3(p.num_blocks * (p.BH / p.H * p.Hkv)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
@@ -394,12 +385,8 @@ static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
   constexpr int NWAVES = 8, BLOCK_N = 64;
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
   auto kern = rope_attn_bwd_dq_kernel<D, NWAVES, BLOCK_N, CAUSAL, PREROT>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = set_lds(kern, Cfg::kLdsBytes);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
   p.num_blocks = (p.N + Cfg::kBlockM - 1) / Cfg::kBlockM;
   hipLaunchKernelGGL(kern, dim3(p.num_blocks * p.BH), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();

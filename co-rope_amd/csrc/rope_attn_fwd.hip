@@ -290,13 +290,8 @@ template <int D, int BLOCK_N, bool CAUSAL>
 static hipError_t launch_fwd_cfg(FwdParams p, hipStream_t stream) {
   using Cfg = FwdCfg<D, BLOCK_N>;
   auto kern = rope_attn_fwd_kernel<D, BLOCK_N, CAUSAL>;
-  static bool attr_set = false;  // per instantiation; benign if raced (same value)
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       Cfg::kLdsBytes);
-    if (e != hipSuccess) return e;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
   p.num_m_blocks = (p.N + Cfg::kBlockM - 1) / Cfg::kBlockM;
   dim3 grid(p.num_m_blocks * p.BH);
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
