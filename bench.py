@@ -216,14 +216,15 @@ def bench_corope(args):
         bev[i + 1].record()
     torch.cuda.synchronize()
     bms = sum(bev[i].elapsed_time(bev[i + 1]) for i in range(bsteps)) / bsteps
-    # issue slots per (sin, cos) pair, counted as for the forward (a transcendental = 4 slots): scores kernel 11 + 8 (phase
-    # 2, unpack 2, rotate 4, pack 1, LDS 2; sin, cos); dk kernel 8 + 8 (phase 2, rotate-accumulate 4, gate path 2; sin, cos);
+    # issue slots per (sin, cos) pair, counted as for the forward (a transcendental = 2 slots): scores kernel 11 + 4 (phase
+    # 2, unpack 2, rotate 4, pack 1, LDS 2; sin, cos); dk kernel 8 + 4 (phase 2, rotate-accumulate 4, gate path 2; sin, cos);
     # the per-head sums run on the matrix cores
-    bwd_instr = pairs * (19 + 16)
-    # VALU roofline: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz issue slots/s.  Per (sin, cos) pair the forward needs 18 slots:
-    # 10 full-rate instructions (phase 2, unpack 2, rotate 4, pack 1, LDS 1) and two transcendentals at a quarter of the
-    # rate (4 slots each); the per-head dot products run on the matrix cores
-    fwd_instr = pairs * 18
+    bwd_instr = pairs * (15 + 12)
+    # VALU roofline: 256 CUs x 4 SIMDs x 16 lanes x 2.4 GHz issue slots/s.  Per (sin, cos) pair the forward needs 14 slots:
+    # 10 full-rate instructions (phase 2, unpack 2, rotate 4, pack 1, LDS 1) and two transcendentals, which issue at half
+    # the rate (measured on this chip: v_sin_f32 16.0 T lanes/s against 33.3 for v_fma_f32), so 2 slots each; the per-head
+    # dot products run on the matrix cores
+    fwd_instr = pairs * 14
     out = {"metric": "Co-RoPE GQA fwd, B2 Hq32 Hkv8 N4096 D128 causal", "value": round(flops / (ms * 1e-3) * 1e-12, 2),
            "unit": "TFLOP/s (attention-equivalent)", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

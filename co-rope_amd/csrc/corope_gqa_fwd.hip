@@ -56,7 +56,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   const float scale2 = p.sm_scale * 1.4426950408889634f;               // scores in the base-2 domain
 
   // A operand of the score product, constant over the row: lane (vr, hf) holds columns 16 ks + 8 hf .. + 7 of q^vr as fp16
-  // for vr < G, zeros otherwise.  The logit product takes the leader's row in bf16 from LDS (lanes with vr = 0).
+  // for vr < G, zeros otherwise.  The logit product takes the leader's row in bf16 from LDS.
   u32x4 aop[D / 16];
   {
     const uint16_t* qrow = p.q + ((int64_t)(head0 + (vr < G ? vr : 0)) * N + i) * D + 8 * hf;
@@ -115,8 +115,9 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     c1 = f32x16{0};
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
-      u32x4 a = u32x4{0, 0, 0, 0};
-      if (vr == 0) a = *reinterpret_cast<const u32x4*>(ql + 16 * ks + 8 * hf);
+      // every row of the A operand is the leader's row (a broadcast read): all result rows then hold the logits, and no
+      // lane needs a zero operand
+      const u32x4 a = *reinterpret_cast<const u32x4*>(ql + 16 * ks + 8 * hf);
       c0 = mfma32(a, *reinterpret_cast<const u32x4*>(tile + vr * KS + 16 * ks + 8 * hf), c0);
       c1 = mfma32(a, *reinterpret_cast<const u32x4*>(tile + (32 + vr) * KS + 16 * ks + 8 * hf), c1);
     }
