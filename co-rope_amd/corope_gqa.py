@@ -4,7 +4,7 @@
 ``_attention.apply`` (corope-exp/flash_attn_co_rope_gqa_triton.py:403-456, :580), including its validation
 errors (:407-425).  Forward and backward are hand-written gfx950 kernels reached through the C ABI.  The reference's
 own "fused" operator falls back to a dense PyTorch backward with (B, Hq, N, N, D/2) temporaries (:459-577); the
-backward here produces the same gradients from q, k, v and dO with N*N fp32 scalars per head of scratch memory
+backward here produces the same gradients from q, k, v and dO with N*N/2 fp32 scalars per matrix and head of scratch memory
 (``backward_workspace_bytes`` says how much)."""
 from __future__ import annotations
 
@@ -57,7 +57,8 @@ class _CoRopeGqaAttn(torch.autograd.Function):
 
 
 def backward_workspace_bytes(B, Hq, Hkv, N, D):
-    """Scratch memory the backward needs: (2 * B * Hkv + 3 * B * Hq) * N * N fp32 values."""
+    """Scratch memory the backward needs: (2 * B * Hkv + 3 * B * Hq) packed lower-triangular N x N fp32 matrices
+    (about N * N / 2 + 32 * N values each)."""
     n = _lib.load().corope_gqa_bwd_workspace_bytes(B, Hq, Hkv, N, D)
     if n < 0:
         raise ValueError(_lib.last_error() or "unsupported Co-RoPE shape")

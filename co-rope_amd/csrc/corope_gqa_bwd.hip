@@ -3,7 +3,7 @@
 // The reference's "fused" Co-RoPE operator falls back to a dense PyTorch backward that materialises (B, Hq, N, N, D/2)
 // temporaries (corope-exp/flash_attn_co_rope_gqa_triton.py:459-577; same mathematics as the manual backward of
 // corope-exp/corope_attn_gqa_pytorch.py:137-300).  This file computes the same gradients with O(N^2) scalars per head
-// in a caller-supplied workspace and no D-sized temporaries.
+// in a caller-supplied workspace (packed lower-triangular matrices) and no D-sized temporaries.
 //
 // Mathematics (group = the Hq/Hkv query heads sharing one key/value head; leader = first head of the group;
 // c = sm_scale; w_d = theta^(-2d/D); pairs (d, d + D/2) as in the forward):
@@ -46,7 +46,14 @@ struct CoropeBwdFreqs {
   float rad[64];     // w_d
 };
 
-// Workspace layout, in floats; NN = N * N.  Only the causal triangle of each matrix is written and read.
+// Row i of a workspace matrix holds the keys j <= i only: rows are packed, each padded to the 64-key chunk it ends in
+// (rows 64 c .. 64 c + 63 take 64 (c + 1) floats each), so every row starts on a 256-byte boundary.
+__device__ __host__ inline int64_t tri_row_start(int i) {
+  const int64_t c = i / 64, r = i % 64;
+  return 2048 * c * (c + 1) + 64 * (c + 1) * r;
+}
+
+// Workspace layout, in floats; NN = tri_row_start(N) is the size of one packed lower-triangular matrix.
 struct CoropeBwdWs {
   float* base;
   int64_t NN;
@@ -85,10 +92,12 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_rowdot_kernel(const uint
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) c = mfma32(af[ks], *reinterpret_cast<const u32x4*>(brow + 16 * ks), c);
     const int col = jj0 + r;
+    // the 32 rows of the tile lie in one 64-row band, so they share a row length; col <= i0 + 31 is inside the padded row
+    const int64_t row0 = tri_row_start(i0), row_len = 64 * (i0 / 64 + 1);
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const int row = i0 + acc_row(e, hf);
-      if (row < N && col < N) obase[(int64_t)row * N + col] = c[e];
+      const int dr = acc_row(e, hf);
+      if (i0 + dr < N && col < N) obase[row0 + row_len * dr + col] = c[e];
     }
   }
 }
@@ -139,7 +148,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     }
   }
   const uint16_t* kbase = p.k + (int64_t)g * N * D;
-  const int64_t rowoff = (int64_t)i * N;
+  const int64_t rowoff = tri_row_start(i);
   const int n_chunks = i / kWave + 1;
   // this row of every workspace matrix: wave-uniform bases, addressed with 32-bit byte offsets of the key index
   float* const d_row = ws.delta(g) + rowoff;
@@ -458,10 +467,12 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_dv_kernel(CoropeBwdParam
 #pragma unroll
       for (int h = 0; h < G; ++h) {
         float pv[8];
+        const float* prow = ws.p(head0 + h) + tri_row_start(i0) + j;   // the 16 rows of a step share a row length
+        const int64_t row_len = 64 * (i0 / 64 + 1);
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
           const int i = i0 + 8 * hf + t;
-          pv[t] = (i < N && j <= i) ? ws.p(head0 + h)[(int64_t)i * N + j] : 0.f;   // nothing outside the triangle is defined
+          pv[t] = (i < N && j <= i) ? prow[row_len * (8 * hf + t)] : 0.f;   // nothing outside the triangle is defined
         }
         const u32x4 bop = {pack_bf16(pv[0], pv[1]), pack_bf16(pv[2], pv[3]), pack_bf16(pv[4], pv[5]), pack_bf16(pv[6], pv[7])};
 #pragma unroll
@@ -540,13 +551,14 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
     float mv[TI];
     u32x4 qv[RI];
     auto fetch = [&](int i0) __attribute__((always_inline)) {
+      const int64_t tile0 = tri_row_start(i0), row_len = 64 * (i0 / 64 + 1);   // the 8 rows of a tile share a row length
       static_for<TI>([&](auto k_c) __attribute__((always_inline)) {
         constexpr int k = decltype(k_c)::value;
         const int e = threadIdx.x + k * NT;
         const int key = e % kDkKeys, m = (e / kDkKeys) % MATS, r = e / (kDkKeys * MATS);
         const int i = i0 + r, j = jb + key;
         const float* src = m == 0 ? ws.delta(g) : m == 1 ? ws.w(g) : ws.ds(head0 + m - 2);
-        mv[k] = (i < N && j <= i) ? src[(int64_t)i * N + j] : 0.f;   // zero outside the causal triangle and past N
+        mv[k] = (i < N && j <= i) ? src[tile0 + row_len * r + j] : 0.f;   // zero outside the causal triangle and past N
       });
       static_for<RI>([&](auto k_c) __attribute__((always_inline)) {
         constexpr int k = decltype(k_c)::value;
@@ -643,7 +655,7 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
 
 // ---------------------------------------------------------------------------------------------------- host side
 int64_t corope_gqa_bwd_workspace_floats(int B, int Hq, int Hkv, int N) {
-  return (int64_t)N * N * (2 * (int64_t)B * Hkv + 3 * (int64_t)B * Hq);
+  return tri_row_start(N) * (2 * (int64_t)B * Hkv + 3 * (int64_t)B * Hq);
 }
 
 template <int D, int G>
@@ -692,7 +704,7 @@ hipError_t launch_corope_gqa_bwd(const CoropeBwdParams& p, int D, float* workspa
     fr.rad[d] = inv;
     fr.turns[d] = (float)((double)inv / 6.283185307179586);
   }
-  CoropeBwdWs ws{workspace, (int64_t)p.N * p.N, p.B * p.Hkv, p.B * p.Hq};
+  CoropeBwdWs ws{workspace, tri_row_start(p.N), p.B * p.Hkv, p.B * p.Hq};
   return D == 128 ? launch_corope_bwd_d<128>(p, ws, fr, stream) : launch_corope_bwd_d<64>(p, ws, fr, stream);
 }
 

@@ -224,14 +224,14 @@ int corope_gqa_fwd(const void *q, const void *k, const void *v, void *o,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void *stream);
 
 /* Bytes of device workspace corope_gqa_bwd needs for these sizes (-1 for sizes corope_gqa_check rejects):
- * N*N floats per key/value head for the accumulated gates, the sigmoid slopes and the gate gradients, and per query
- * head for the attention weights and the score gradients. */
+ * packed lower-triangular N x N fp32 matrices (about N*N/2 + 32*N floats each): two per key/value head (accumulated
+ * gates; gate gradients) and three per query head (attention weights; score gradients; dO V^T). */
 int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D);
 
 /* Co-RoPE grouped-query attention backward (causal only): dq (B,Hq,N,D), dk/dv (B,Hkv,N,D) from q, k, v and dO.
  * Replaces _attention.backward (reference corope-exp/flash_attn_co_rope_gqa_triton.py:459-577), which recomputes the
  * forward densely in PyTorch with (B,Hq,N,N,D/2) temporaries; the same gradients (including the path through the
- * leader head's gates, :548-561) are produced here with N*N scalars per head in `workspace`.  Like the reference's, it
+ * leader head's gates, :548-561) are produced here with packed triangular N x N matrices of scalars in `workspace`.  Like the reference's, it
  * takes neither the forward's output nor its row statistics.  The workspace need not be initialised. */
 int corope_gqa_bwd(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta,
