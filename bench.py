@@ -201,7 +201,7 @@ def bench_corope(args):
     wsp = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
 
     def bwd_step():
-        rc = lib.corope_gqa_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+        rc = lib.corope_gqa_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(), dq.data_ptr(), dk.data_ptr(),
                                 dv.data_ptr(), B, Hq, Hkv, N, D, scale, 10000.0, wsp.data_ptr(), ws_bytes, stream)
         if rc != 0:
             sys.exit(pkg._lib.last_error())

@@ -42,7 +42,9 @@ class _CoRopeGqaAttn(torch.autograd.Function):
             rc = lib.corope_gqa_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, Hq, Hkv, N, D,
                                     float(sm_scale), float(theta), torch.cuda.current_stream(q.device).cuda_stream)
         _lib.check(rc, "corope_gqa_fwd")
-        ctx.save_for_backward(q, k, v)   # what the reference keeps (:451), minus inv_freq: theta is enough
+        # what the reference keeps (:451), minus inv_freq (theta is enough), plus the output: the backward takes a
+        # reference value for its row sums from it (accuracy of dQ on sharply peaked rows; not needed mathematically)
+        ctx.save_for_backward(q, k, v, o)
         ctx.group_size = Hq // Hkv
         ctx.sm_scale = sm_scale
         ctx.theta = theta
@@ -51,8 +53,8 @@ class _CoRopeGqaAttn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output):
-        q, k, v = ctx.saved_tensors
-        dq, dk, dv = corope_gqa_backward(q, k, v, grad_output, ctx.sm_scale, ctx.theta)
+        q, k, v, o = ctx.saved_tensors
+        dq, dk, dv = corope_gqa_backward(q, k, v, grad_output, ctx.sm_scale, ctx.theta, out=o)
         return dq, dk, dv, None, None, None, None
 
 
@@ -65,21 +67,24 @@ def backward_workspace_bytes(B, Hq, Hkv, N, D):
     return n
 
 
-def corope_gqa_backward(q, k, v, grad_output, sm_scale, theta, workspace=None):
+def corope_gqa_backward(q, k, v, grad_output, sm_scale, theta, workspace=None, out=None):
     """(dq, dk, dv) of the Co-RoPE GQA attention for upstream gradient ``grad_output`` (reference :459-577).
 
-    ``workspace`` may be a caller-owned uint8/float tensor of at least ``backward_workspace_bytes`` bytes."""
+    ``workspace`` may be a caller-owned uint8/float tensor of at least ``backward_workspace_bytes`` bytes; ``out`` the
+    forward's output for the same inputs (optional: it only steadies the rounding of dQ on sharply peaked rows)."""
     lib = _lib.load()
     B, Hq, N, D = q.shape
     Hkv = k.shape[1]
     q, k, v, d_o = q.contiguous(), k.contiguous(), v.contiguous(), grad_output.to(q.dtype).contiguous()
+    out_c = None if out is None else out.contiguous()
+    o_ptr = None if out_c is None else out_c.data_ptr()
     need = backward_workspace_bytes(B, Hq, Hkv, N, D)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
     have = workspace.numel() * workspace.element_size()
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     with torch.cuda.device(q.device):
-        rc = lib.corope_gqa_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), d_o.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+        rc = lib.corope_gqa_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o_ptr, d_o.data_ptr(), dq.data_ptr(), dk.data_ptr(),
                                 dv.data_ptr(), B, Hq, Hkv, N, D, float(sm_scale), float(theta), workspace.data_ptr(),
                                 have, torch.cuda.current_stream(q.device).cuda_stream)
     _lib.check(rc, "corope_gqa_bwd")

@@ -503,13 +503,14 @@ int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D) {
   return 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N);
 }
 
-int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* d_o, void* dq, void* dk, void* dv, int B,
-                   int Hq, int Hkv, int N, int D, float sm_scale, float theta, void* workspace, int64_t workspace_bytes,
-                   void* stream) {
+int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk, void* dv,
+                   int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void* workspace,
+                   int64_t workspace_bytes, void* stream) {
   int rc = corope_gqa_check(B, Hq, Hkv, N, D, sm_scale, theta);
   if (rc) return rc;
   rc = check_ptrs("corope_gqa_bwd", {q, k, v, d_o, dq, dk, dv, workspace});
   if (rc) return rc;
+  if (o != nullptr && !aligned16(o)) return fail(COROPE_E_ALIGN, "corope_gqa_bwd: pointer %p is not 16-byte aligned", o);
   if ((int64_t)B * Hkv > 65535) return fail(COROPE_E_UNSUPPORTED, "corope_gqa_bwd: B * Hkv = %lld exceeds 65535", (long long)B * Hkv);
   const int64_t need = 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N);
   if (workspace_bytes < need)
@@ -518,6 +519,7 @@ int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* d_o,
   p.q = static_cast<const uint16_t*>(q);
   p.k = static_cast<const uint16_t*>(k);
   p.v = static_cast<const uint16_t*>(v);
+  p.o = static_cast<const uint16_t*>(o);
   p.d_o = static_cast<const uint16_t*>(d_o);
   p.dq = static_cast<uint16_t*>(dq);
   p.dk = static_cast<uint16_t*>(dk);

@@ -48,9 +48,10 @@ typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 __device__ __forceinline__ f32x16 mfma32_f16(u32x4 a, u32x4 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
-// Two floats -> packed fp16 (lo in bits 0..15), rounded toward zero by the one-instruction conversion.
+// Two floats -> packed fp16 (lo in bits 0..15), round to nearest even (v_cvt_pk_f16_f32).
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 __device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
-  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, f16x2));
 }
 
 // Row index (0..31) held by accumulator register i of lane-half h in a 32x32 MFMA result.

@@ -110,7 +110,7 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_rowdot_kernel(const uint
 template <int D, int G>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void corope_bwd_scores_kernel(CoropeBwdParams p, CoropeBwdWs ws, CoropeBwdFreqs fr) {
   constexpr int HALF = D / 2;
-  constexpr int KS = D + 8, WS = kWave + 8, NVR = 2 * G + 1, NDB = D / 32;
+  constexpr int KS = D + 8, WS = kWave + 8, NVR = 2 * G + 2, NDB = D / 32;
   constexpr int NI = 4 * ((2 * G - 1) / 8 + 1);                       // accumulator registers that hold rows < 2G
   __shared__ __attribute__((aligned(16))) uint16_t kt[kWave * KS];    // [key][d]: keys (bf16), rotated in place (fp16)
   __shared__ __attribute__((aligned(16))) uint16_t wts[NVR * WS];     // [virtual row][key] weights: fp16, row 2G (W) bf16
@@ -177,6 +177,20 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     l_run[h] = pd_run[h] = 0.f;
   }
   float carry = 0.f;   // sum of z over the keys to the right of the current chunk (up to the diagonal)
+  // Reference value for Delta = rowsum(P o dP), which is only known at the end of the row: the dq sums take e (dP - ref)
+  // as weights and are corrected by (Delta - ref) afterwards, which is exact for any ref; the closer ref is to Delta, the
+  // less the two sums cancel (rows dominated by one key would otherwise lose the 11 bits of the weights).  With the forward
+  // output at hand ref = rowsum(O o dO), equal to Delta up to O's rounding; without it ref = 0.
+  float dref[G];
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    float acc = 0.f;
+    if (p.o != nullptr) {
+      const int64_t off = ((int64_t)(head0 + h) * N + i) * D;
+      for (int d = lane; d < D; d += kWave) acc = __builtin_fmaf(bf16_to_f(p.o[off + d]), bf16_to_f(p.d_o[off + d]), acc);
+    }
+    dref[h] = wave_sum(acc);
+  }
   // A chunk's 64 key rows are one contiguous block of global memory: the wave fetches it with consecutive 16-byte pieces
   // per lane (full cache lines per instruction) and parks it in the LDS tile, where each lane then finds its own key's
   // row.  The block, the leader logits (from the row-dot pass; their slot then takes delta) and dP are each requested
@@ -299,7 +313,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       l_run[h] = __builtin_fmaf(l_run[h], a, e);
       pd_run[h] = __builtin_fmaf(pd_run[h], a, e * dpv[h]);
       al = (vr / 2 == h && vr < 2 * G) ? a : al;
-      wts[(2 * h) * WS + lane] = f_to_f16(e * dpv[h]);
+      wts[(2 * h) * WS + lane] = f_to_f16(e * (dpv[h] - dref[h]));
       wts[(2 * h + 1) * WS + lane] = f_to_f16(e);
     }
     if (c > 0) {
@@ -332,14 +346,14 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     dsum[h] = pd * inv_l[h];
   }
 
-  // even virtual row 2h: (sum e dP kt - Delta sum e kt) / L, the second sum sitting in the neighbouring lane; the rows from
-  // 2G on are still zero and row 2G collects the leader's gate path below
+  // even virtual row 2h: (sum e (dP - ref) kt - (Delta - ref) sum e kt) / L, the second sum sitting in the neighbouring lane; the rows from
+  // 2G on are still zero and rows 2G, 2G + 1 collect the leader's gate path below
   {
     float my_inv = 0.f, my_dsum = 0.f;
 #pragma unroll
     for (int h = 0; h < G; ++h) {
       my_inv = vr / 2 == h ? inv_l[h] : my_inv;
-      my_dsum = vr / 2 == h ? dsum[h] : my_dsum;
+      my_dsum = vr / 2 == h ? dsum[h] - dref[h] : my_dsum;
     }
 #pragma unroll
     for (int db = 0; db < NDB; ++db)
@@ -396,7 +410,11 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     const float pre = wave_prefix_sum(gij);   // over the keys at and to the left of this one
     const float wij = valid ? (gcarry + pre - gij) * slope : 0.f;   // (sum of G over the keys j < t) z'(t)
     gcarry += wave_last(pre);
-    wts[(2 * G) * WS + lane] = f_to_bf16(wij);
+    {   // W as the sum of two bf16 values (the keys it multiplies are exact), in virtual rows 2G and 2G + 1
+      const uint16_t w_hi = f_to_bf16(wij);
+      wts[(2 * G) * WS + lane] = w_hi;
+      wts[(2 * G + 1) * WS + lane] = f_to_bf16(wij - bf16_to_f(w_hi));
+    }
     if (valid) {
 #pragma unroll
       for (int h = 0; h < G; ++h) {
@@ -406,22 +424,22 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       *byte_offset(w_row, 4u * j) = wij;
     }
     lds_order();
-    // leader's gate path: row 2G of the accumulators += W (1 x keys) K (keys x d)
+    // leader's gate path: rows 2G and 2G + 1 of the accumulators += W (high and low part, 1 x keys each) K (keys x d)
 #pragma unroll
     for (int ks = 0; ks < kWave / 16; ++ks) {
       u32x4 bop = u32x4{0, 0, 0, 0};
-      if (vr == 2 * G) bop = *reinterpret_cast<const u32x4*>(wts + vr * WS + 16 * ks + 8 * hf);
+      if (vr == 2 * G || vr == 2 * G + 1) bop = *reinterpret_cast<const u32x4*>(wts + vr * WS + 16 * ks + 8 * hf);
 #pragma unroll
       for (int db = 0; db < NDB; ++db) dqa[db] = mfma32(load_a_trans_natural(kt, KS, 16 * ks, 32 * db), bop, dqa[db]);
     }
     lds_order();
   }
-  // dq: even virtual rows hold the heads' gradients; the leader adds the gate path from row 2G of its lane half
+  // dq: even virtual rows hold the heads' gradients; the leader adds the gate path from rows 2G and 2G + 1 of its lane half
 #pragma unroll
   for (int db = 0; db < NDB; ++db)
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const float gate = __shfl(dqa[db][e], 32 * hf + 2 * G);
+      const float gate = __shfl(dqa[db][e], 32 * hf + 2 * G) + __shfl(dqa[db][e], 32 * hf + 2 * G + 1);
       if (vr == 0) dqa[db][e] += gate;
     }
   if (vr < 2 * G && vr % 2 == 0) {
@@ -600,12 +618,17 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
       for (int r = 0; r < n_rows; ++r) {
         if (i0 + r < jw) continue;   // wave-uniform: all keys of this wave lie above the diagonal of this row
         const float* trow = tile + r * MATS * kDkKeys + 32 * wave;
-        // A: (32 keys x heads), lane (key, half 0) holds dS^h for h = 0..7; half 1 would be heads 8..15: zero
-        u32x4 aop = u32x4{0, 0, 0, 0};
-        if (hf == 0) {
+        // A: (32 keys x 16 contraction slots): lane (key, half 0) holds dS^h for h = 0..7 rounded to bf16, half 1 what the
+        // rounding left over (again as bf16); with the queries of heads 0..7 in both halves of B the product carries dS to
+        // about 16 bits
+        u32x4 aop;
+        {
           float dsv[8];
 #pragma unroll
-          for (int h = 0; h < 8; ++h) dsv[h] = h < G ? trow[(2 + h) * kDkKeys + col] : 0.f;
+          for (int h = 0; h < 8; ++h) {
+            const float x = h < G ? trow[(2 + h) * kDkKeys + col] : 0.f;
+            dsv[h] = hf == 0 ? x : x - bf16_to_f(f_to_bf16(x));
+          }
           aop = u32x4{pack_bf16(dsv[0], dsv[1]), pack_bf16(dsv[2], dsv[3]), pack_bf16(dsv[4], dsv[5]), pack_bf16(dsv[6], dsv[7])};
         }
         // B: (heads x 32 columns) per column block; the same read also carries the leader's (head 0) value of the column
@@ -615,7 +638,7 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
         for (int blk = 0; blk < NB; ++blk) {
           const u32x4 bq = *reinterpret_cast<const u32x4*>(qT + (r * D + 32 * blk + col) * 8);
           ql[blk] = bf16_lo(bq[0]);
-          u[blk] = mfma32(aop, hf == 0 ? bq : u32x4{0, 0, 0, 0}, f32x16{0});
+          u[blk] = mfma32(aop, bq, f32x16{0});
         }
         // delta and W of this lane's 16 keys: keys 8 n + 4 half + 0..3 for n = 0..3, as the accumulator rows are laid out
         f32x4 dl[4], wg[4];

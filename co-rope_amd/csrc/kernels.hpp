@@ -81,6 +81,7 @@ struct CoropeBwdParams {
   const uint16_t* q;    // (B, Hq, N, D)
   const uint16_t* k;    // (B, Hkv, N, D)
   const uint16_t* v;
+  const uint16_t* o;    // (B, Hq, N, D) forward output, or null: only a reference value for rowsum(P o dP) is taken from it
   const uint16_t* d_o;  // (B, Hq, N, D)
   uint16_t* dq;
   uint16_t* dk;

@@ -231,9 +231,12 @@ int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D);
 /* Co-RoPE grouped-query attention backward (causal only): dq (B,Hq,N,D), dk/dv (B,Hkv,N,D) from q, k, v and dO.
  * Replaces _attention.backward (reference corope-exp/flash_attn_co_rope_gqa_triton.py:459-577), which recomputes the
  * forward densely in PyTorch with (B,Hq,N,N,D/2) temporaries; the same gradients (including the path through the
- * leader head's gates, :548-561) are produced here with packed triangular N x N matrices of scalars in `workspace`.  Like the reference's, it
- * takes neither the forward's output nor its row statistics.  The workspace need not be initialised. */
-int corope_gqa_bwd(const void *q, const void *k, const void *v, const void *d_o, void *dq, void *dk, void *dv,
+ * leader head's gates, :548-561) are produced here with packed triangular N x N matrices of scalars in `workspace`.
+ * Like the reference's, it needs neither the forward's output nor its row statistics; `o` may be NULL.  When the forward's output is
+ * passed, rowsum(O o dO) serves as a reference value that keeps dQ accurate for rows dominated by a single key (the
+ * result is mathematically the same with or without it).  The workspace need not be initialised. */
+int corope_gqa_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                   void *dq, void *dk, void *dv,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta,
                    void *workspace, int64_t workspace_bytes, void *stream);
 

@@ -119,11 +119,12 @@ def test_corope_backward_argument_checks(pkg):
     buf = ctypes.create_string_buffer(4096)
     ok = (ctypes.addressof(buf) + 15) & ~15
     need = lib.corope_gqa_bwd_workspace_bytes(1, 4, 2, 8, 64)
-    args = lambda ws, nbytes, dq=ok: (ok, ok, ok, ok, dq, ok, ok, 1, 4, 2, 8, 64, 0.125, 1e4, ws, nbytes, None)
+    args = lambda ws, nbytes, dq=ok, o=None: (ok, ok, ok, o, ok, dq, ok, ok, 1, 4, 2, 8, 64, 0.125, 1e4, ws, nbytes, None)
     assert lib.corope_gqa_bwd(*args(None, need)) == -1 and "null" in pkg._lib.last_error()
     assert lib.corope_gqa_bwd(*args(ok, need, dq=ok + 2)) == -3 and "aligned" in pkg._lib.last_error()
     assert lib.corope_gqa_bwd(*args(ok, need - 4)) == -1 and "workspace" in pkg._lib.last_error()
-    rc = lib.corope_gqa_bwd(ok, ok, ok, ok, ok, ok, ok, 1, 18, 2, 8, 64, 0.125, 1e4, ok, 1 << 40, None)
+    assert lib.corope_gqa_bwd(*args(ok, need, o=ok + 2)) == -3 and "aligned" in pkg._lib.last_error()   # o is optional, not sloppy
+    rc = lib.corope_gqa_bwd(ok, ok, ok, None, ok, ok, ok, ok, 1, 18, 2, 8, 64, 0.125, 1e4, ok, 1 << 40, None)
     assert rc == -2 and "group size" in pkg._lib.last_error()
 
 

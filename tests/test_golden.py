@@ -52,6 +52,16 @@ def test_oracle_reproduces_corope_fixture(path):
     rows = torch.arange(q.shape[2])
     o_rows = C.corope_gqa_forward_rows(q.float(), k.float(), v.float(), True, float(z["sm_scale"]), float(z["theta"]), rows)
     assert (o_rows.double() - _t(z["o"]).double()).abs().max() < 1e-4
+    # gradients: the fixture's come from finite differences of the brute-force program (see make_golden.py)
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    do = _t(z["do"]).double()
+    auto = torch.autograd.grad(C.corope_gqa_forward(qa, ka, va, True, float(z["sm_scale"]), float(z["theta"]), torch.float64),
+                               (qa, ka, va), do)
+    manual = C.corope_gqa_backward_manual(q, k, v, do, float(z["sm_scale"]), float(z["theta"]))
+    for name, a, m in zip(("dq", "dk", "dv"), auto, manual):
+        ref = _t(z[name]).double()
+        tol = 1e-5 * max(1.0, float(ref.abs().max()))     # the fixture is stored in fp32
+        assert (a - ref).abs().max() <= tol and (m - ref).abs().max() <= tol, name
 
 
 @pytest.mark.gpu
@@ -75,9 +85,15 @@ def test_kernels_reproduce_rope_fixture(pkg, path):
 def test_kernel_reproduces_corope_fixture(pkg, path):
     z = np.load(path)
     dev = torch.device("cuda:0")
-    q, k, v = (_t(z[n]).to(dev, torch.bfloat16) for n in ("q", "k", "v"))
+    q, k, v = (_t(z[n]).to(dev, torch.bfloat16).requires_grad_(True) for n in ("q", "k", "v"))
     o = pkg.corope_attention(q, k, v, True, float(z["sm_scale"]), float(z["theta"]))
+    o.backward(_t(z["do"]).to(dev, torch.bfloat16))
     torch.cuda.synchronize()
-    err = (o.float().cpu() - _t(z["o"])).abs().max().item()
+    err = (o.detach().float().cpu() - _t(z["o"])).abs().max().item()
     print(f"  {os.path.basename(path)} o: max-abs {err:.3e}")
     assert err <= 2e-2
+    group = q.shape[1] // k.shape[1]
+    for name, got in (("dq", q.grad), ("dk", k.grad), ("dv", v.grad)):
+        ok, err = within_bar(got.float().cpu(), _t(z[name]), 2e-2 * (1.0 if name == "dq" else group ** 0.5))
+        print(f"  {os.path.basename(path)} {name}: max-abs {err:.3e}")
+        assert ok, name
