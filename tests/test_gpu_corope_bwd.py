@@ -22,7 +22,7 @@ def _inputs(B, Hq, Hkv, N, D, seed=42):
 
 def _oracle_grads(q, k, v, d_o, scale, theta):
     cd = torch.float64 if q.shape[2] <= 160 else torch.float32   # the dense form holds (B, Hq, N, N, D/2) temporaries
-    q, k, v = (t.to(cd).requires_grad_(True) for t in (q, k, v))
+    q, k, v = (t.to(cd).clone().requires_grad_(True) for t in (q, k, v))   # (.to is a no-op for fp32 inputs: never mark the caller's tensor)
     o = C.corope_gqa_forward(q, k, v, True, scale, theta, cd)
     return [g.float() for g in torch.autograd.grad(o, (q, k, v), d_o.to(cd))]
 
@@ -120,3 +120,34 @@ def test_corope_backward_caller_workspace_and_reuse(pkg):
         assert torch.equal(x, y)
     with pytest.raises(ValueError):
         mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4, workspace=ws[: need // 4 - 1])
+
+
+def test_corope_random_shapes_forward_and_backward(pkg):
+    """A seeded sweep over batch, group size, head dim, ragged lengths, temperature and rotation base: forward and
+    backward in one go, each tensor against the dense oracle with the bar of conftest.within_bar (2e-2, or one bf16 step
+    of the value where it exceeds 2.56; dK and dV scaled by sqrt(G) as above)."""
+    import random
+    from conftest import within_bar
+    rnd = random.Random(5)
+    dev = torch.device("cuda:0")
+    for case in range(16):
+        B, Hkv, G, D = rnd.choice([1, 2]), rnd.choice([1, 2, 3]), rnd.randint(1, 8), rnd.choice([64, 128])
+        N = rnd.choice([1, 2, 31, 63, 64, 65, 100, 127, 128, 129, 190])
+        scale, theta = rnd.choice([1 / math.sqrt(D), 0.25, 0.05]), rnd.choice([100.0, 10000.0, 500000.0])
+        Hq = Hkv * G
+        print(f"case {case}: B={B} Hq={Hq} Hkv={Hkv} N={N} D={D} scale={scale:.3f} theta={theta}", flush=True)
+        q, k, v, d_o = _inputs(B, Hq, Hkv, N, D, seed=1000 + 4 * case)
+        d_o = bf16_round(d_o * 0.5)
+        cd = torch.float64 if N <= 130 else torch.float32
+        qr, kr, vr = (t.to(cd).clone().requires_grad_(True) for t in (q, k, v))
+        o_ref = C.corope_gqa_forward(qr, kr, vr, True, scale, theta, cd)
+        g_ref = torch.autograd.grad(o_ref, (qr, kr, vr), d_o.to(cd))
+        qg, kg, vg = (t.to(dev, torch.bfloat16).requires_grad_(True) for t in (q, k, v))
+        o = pkg.corope_attention(qg, kg, vg, True, scale, theta)
+        o.backward(d_o.to(dev, torch.bfloat16))
+        torch.cuda.synchronize()
+        checks = [("O", o.detach(), o_ref.detach(), TOL)]
+        checks += [(n, t.grad, r, TOL * (1.0 if n == "dQ" else math.sqrt(G))) for n, t, r in zip(("dQ", "dK", "dV"), (qg, kg, vg), g_ref)]
+        for name, got, ref, tol in checks:
+            ok, err = within_bar(got.float().cpu(), ref.float(), tol)
+            assert torch.isfinite(got).all() and ok, (case, name, err)
