@@ -237,7 +237,7 @@ def bench_corope(args):
            "backward": {"ms": round(bms, 4), "steps": bsteps, "workspace_gib": round(ws_bytes / 2**30, 2),
                         "sincos_pairs_per_s": round(2 * pairs / (bms * 1e-3), 1),
                         "tflops_attention_equivalent": round(2.5 * flops / (bms * 1e-3) * 1e-12, 2),
-                        "roofline": {"bound": "valu", "kernel": "corope_gqa_bwd (5 launches)",
+                        "roofline": {"bound": "valu", "kernel": "corope_gqa_bwd (6 launches)",
                                      "achieved": round(bwd_instr / (bms * 1e-3) * 1e-12, 3),
                                      "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T issue slots/s",
                                      "frac": round(bwd_instr / (bms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4), "traffic": None}},

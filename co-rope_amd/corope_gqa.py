@@ -60,7 +60,7 @@ class _CoRopeGqaAttn(torch.autograd.Function):
 
 def backward_workspace_bytes(B, Hq, Hkv, N, D):
     """Scratch memory the backward needs: (2 * B * Hkv + 3 * B * Hq) packed lower-triangular N x N fp32 matrices
-    (about N * N / 2 + 32 * N values each)."""
+    (about N * N / 2 + 32 * N values each), plus B * Hkv * N * D values."""
     n = _lib.load().corope_gqa_bwd_workspace_bytes(B, Hq, Hkv, N, D)
     if n < 0:
         raise ValueError(_lib.last_error() or "unsupported Co-RoPE shape")

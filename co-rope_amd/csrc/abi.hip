@@ -500,7 +500,7 @@ int corope_gqa_fwd(const void* q, const void* k, const void* v, void* o, int B, 
 
 int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D) {
   if (corope_gqa_check(B, Hq, Hkv, N, D, 1.f, 2.f)) return -1;
-  return 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N);
+  return 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N, D);
 }
 
 int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk, void* dv,
@@ -512,7 +512,7 @@ int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* o, c
   if (rc) return rc;
   if (o != nullptr && !aligned16(o)) return fail(COROPE_E_ALIGN, "corope_gqa_bwd: pointer %p is not 16-byte aligned", o);
   if ((int64_t)B * Hkv > 65535) return fail(COROPE_E_UNSUPPORTED, "corope_gqa_bwd: B * Hkv = %lld exceeds 65535", (long long)B * Hkv);
-  const int64_t need = 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N);
+  const int64_t need = 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N, D);
   if (workspace_bytes < need)
     return fail(COROPE_E_BADARG, "corope_gqa_bwd: workspace of %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
   corope::CoropeBwdParams p{};

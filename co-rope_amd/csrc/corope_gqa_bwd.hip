@@ -27,11 +27,13 @@
 //                  right to left over 64-key chunks: z, delta by a scan, the rotated keys Kt -> LDS (bf16); on the matrix
 //                  cores S = q Kt^T and dS/ddelta = [-w q2, w q1] Kt^T for all heads at once, then - with running softmax
 //                  statistics, flash-attention style - the two sums that make dq: sum_j e_j dP_j kt_j and sum_j e_j kt_j;
-//                  left to right: P, dS, G and its running sum, W, and the leader's W K (matrix cores again);
-//                  writes dq and the workspace matrices DELTA, W [group][N][N] and P, DS [head][N][N]
+//                  left to right: P, dS, G and its running sum, W;
+//                  writes dq of the heads 1..G-1, the leader's dq without its gate path (fp32, workspace) and the workspace
+//                  matrices DELTA, W [group] and P, DS [head] (packed lower triangles)
+//   dq_leader    dq_leader = c (partial + W K): a plain product on the matrix cores, 128 rows per workgroup
 //   dv           dv^T += dO^T P on the matrix cores, 128 keys per workgroup
-//   dk           one workgroup per (group, 32 keys), lane = rotation pair: rotates sum_h dS^h q^h per (i, j) and adds the
-//                gate path W qL; tiles of DELTA, W, DS staged through LDS
+//   dk           one workgroup per (group, 128 keys): sum_h dS^h q^h on the matrix cores, then lane = rotation pair x 16
+//                keys rotates it per (i, j) and adds the gate path W qL; tiles of DELTA, W, DS staged through LDS
 // Rounding: the rotated keys and what multiplies them (queries, the softmax weights e and e dP) are fp16 - the bf16
 // queries convert exactly, and 11 significant bits keep scores accurate at sm_scale = 1 too; the products on unrotated
 // rows (W K, P dO, the row dots) take bf16 operands; sums, statistics, delta, dS/ddelta and everything stored in the
@@ -63,6 +65,10 @@ struct CoropeBwdWs {
   __device__ __host__ float* p(int h) const { return base + (int64_t)(2 * n_groups + h) * NN; }               // S, then P
   __device__ __host__ float* ds(int h) const { return base + (int64_t)(2 * n_groups + n_heads + h) * NN; }    // dS/ddelta, then dS
   __device__ __host__ float* dp(int h) const { return base + (int64_t)(2 * n_groups + 2 * n_heads + h) * NN; }
+  // (N, D) per group: the leader head's dq without the gate path and without the factor sm_scale
+  __device__ __host__ float* dql(int g, int N, int D) const {
+    return base + (int64_t)(2 * n_groups + 3 * n_heads) * NN + (int64_t)g * N * D;
+  }
 };
 
 // ---------------------------------------------------------------------------------------------------- row dots
@@ -110,10 +116,10 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_rowdot_kernel(const uint
 template <int D, int G>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void corope_bwd_scores_kernel(CoropeBwdParams p, CoropeBwdWs ws, CoropeBwdFreqs fr) {
   constexpr int HALF = D / 2;
-  constexpr int KS = D + 8, WS = kWave + 8, NVR = 2 * G + 2, NDB = D / 32;
+  constexpr int KS = D + 8, WS = kWave + 8, NVR = 2 * G, NDB = D / 32;
   constexpr int NI = 4 * ((2 * G - 1) / 8 + 1);                       // accumulator registers that hold rows < 2G
   __shared__ __attribute__((aligned(16))) uint16_t kt[kWave * KS];    // [key][d]: keys (bf16), rotated in place (fp16)
-  __shared__ __attribute__((aligned(16))) uint16_t wts[NVR * WS];     // [virtual row][key] weights: fp16, row 2G (W) bf16
+  __shared__ __attribute__((aligned(16))) uint16_t wts[NVR * WS];     // [virtual row][key] fp16 weights of the keys
   const int i = p.N - 1 - blockIdx.x, g = blockIdx.y, lane = threadIdx.x;   // longest rows first
   const int vr = lane % 32, hf = lane / 32;                                  // matrix-core identity of this lane
   const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv;
@@ -347,7 +353,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   }
 
   // even virtual row 2h: (sum e (dP - ref) kt - (Delta - ref) sum e kt) / L, the second sum sitting in the neighbouring lane; the rows from
-  // 2G on are still zero and rows 2G, 2G + 1 collect the leader's gate path below
+  // 2G on are idle
   {
     float my_inv = 0.f, my_dsum = 0.f;
 #pragma unroll
@@ -363,11 +369,33 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
         if (vr < 2 * G) dqa[db][e] = (dqa[db][e] - my_dsum * other) * my_inv;
       }
   }
+  // dq of the heads 1..G-1 is final; the leader's still lacks the gate path W K, which a separate plain matrix product
+  // adds (corope_bwd_dq_leader_kernel): its row goes to the workspace in fp32, unscaled
+  if (vr < 2 * G && vr % 2 == 0) {
+    if (vr == 0) {
+      float* op = ws.dql(g, N, D) + (int64_t)i * D;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4)
+          *reinterpret_cast<f32x4*>(op + db * 32 + 8 * g4 + 4 * hf) =
+              f32x4{dqa[db][4 * g4], dqa[db][4 * g4 + 1], dqa[db][4 * g4 + 2], dqa[db][4 * g4 + 3]};
+    } else {
+      uint16_t* op = p.dq + ((int64_t)(head0 + vr / 2) * N + i) * D;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const u32x2 w = {pack_bf16(dqa[db][4 * g4] * p.sm_scale, dqa[db][4 * g4 + 1] * p.sm_scale),
+                           pack_bf16(dqa[db][4 * g4 + 2] * p.sm_scale, dqa[db][4 * g4 + 3] * p.sm_scale)};
+          *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
+        }
+    }
+  }
 
-  // ---- left to right: P, dS, G_ij = sum_h dS dS/ddelta, its running sum over the keys, W, and W K for the leader -------
+  // ---- left to right: P, dS, G_ij = sum_h dS dS/ddelta, its running sum over the keys, W ------------------------------
   float gcarry = 0.f;
-  // one chunk of look-ahead here too: the next chunk's S, dS/ddelta, dP, slope and key row are in flight during the
-  // matrix-core phase of the current one
+  // one chunk of look-ahead here too
   float sl_n, sv_n[G], gv_n[G], dp_n[G];
   auto fetch = [&](int c) __attribute__((always_inline)) {
     const int j = c * kWave + lane;
@@ -379,15 +407,14 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       gv_n[h] = *byte_offset(ds_row[h], 4u * jc);
       dp_n[h] = *byte_offset(dp_row[h], 4u * jc);
     }
-    fetch_keys(c);
   };
   fetch(0);
 #pragma unroll 1
   for (int c = 0; c < n_chunks; ++c) {
     const int j = c * kWave + lane;
     const bool valid = j <= i;
-    // take this chunk's values out of the look-ahead registers (the key row goes straight to LDS) and request the next
-    // chunk's before anything is stored, so that waiting for them never waits for this chunk's stores
+    // take this chunk's values out of the look-ahead registers and request the next chunk's before anything is stored,
+    // so that waiting for them never waits for this chunk's stores
     const float slope = sl_n;
     float sv[G], gv[G], dpc[G];
 #pragma unroll
@@ -396,7 +423,6 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       gv[h] = gv_n[h];
       dpc[h] = dp_n[h];
     }
-    park_keys();
     if (c + 1 < n_chunks) fetch(c + 1);
     float gij = 0.f;
     float prv[G], dsv[G];
@@ -410,11 +436,6 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     const float pre = wave_prefix_sum(gij);   // over the keys at and to the left of this one
     const float wij = valid ? (gcarry + pre - gij) * slope : 0.f;   // (sum of G over the keys j < t) z'(t)
     gcarry += wave_last(pre);
-    {   // W as the sum of two bf16 values (the keys it multiplies are exact), in virtual rows 2G and 2G + 1
-      const uint16_t w_hi = f_to_bf16(wij);
-      wts[(2 * G) * WS + lane] = w_hi;
-      wts[(2 * G + 1) * WS + lane] = f_to_bf16(wij - bf16_to_f(w_hi));
-    }
     if (valid) {
 #pragma unroll
       for (int h = 0; h < G; ++h) {
@@ -423,33 +444,74 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       }
       *byte_offset(w_row, 4u * j) = wij;
     }
-    lds_order();
-    // leader's gate path: rows 2G and 2G + 1 of the accumulators += W (high and low part, 1 x keys each) K (keys x d)
-#pragma unroll
-    for (int ks = 0; ks < kWave / 16; ++ks) {
-      u32x4 bop = u32x4{0, 0, 0, 0};
-      if (vr == 2 * G || vr == 2 * G + 1) bop = *reinterpret_cast<const u32x4*>(wts + vr * WS + 16 * ks + 8 * hf);
-#pragma unroll
-      for (int db = 0; db < NDB; ++db) dqa[db] = mfma32(load_a_trans_natural(kt, KS, 16 * ks, 32 * db), bop, dqa[db]);
-    }
-    lds_order();
   }
-  // dq: even virtual rows hold the heads' gradients; the leader adds the gate path from rows 2G and 2G + 1 of its lane half
+}
+
+// ---------------------------------------------------------------------------------------------------- leader's dq
+// dq_leader_i = c (partial_i + sum_{t <= i} W_it k_t): a plain (rows x keys) x (keys x D) product on the matrix cores,
+// computed transposed (dq^T += K^T W^T) so that W is read along its packed rows: lane = query row, 8 consecutive keys per
+// step, each value split into two bf16 parts (the keys are exact, so the product carries W to about 16 bits).  One
+// workgroup of 4 waves owns 128 rows (32 per wave) of one group; the 16 key rows of a step are staged in LDS and read
+// transposed.
+template <int D>
+__global__ __launch_bounds__(4 * kWave) void corope_bwd_dq_leader_kernel(CoropeBwdParams p, CoropeBwdWs ws) {
+  constexpr int TS = D + 16, NDB = D / 32, NT = 4 * kWave, STEP = 16;
+  __shared__ __attribute__((aligned(16))) uint16_t tile[STEP * TS];
+  const int g = blockIdx.y;
+  const int rb = (int)gridDim.x - 1 - (int)blockIdx.x;            // the last row blocks see the most keys: first
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int r = lane % 32, hf = lane / 32;
+  const int N = p.N, b = g / p.Hkv, kvh = g % p.Hkv, G = p.Hq / p.Hkv;
+  const int iw = rb * 128 + 32 * wave, i = iw + r;                // this wave's first row, this lane's row
+  const uint16_t* kbase = p.k + (int64_t)g * N * D;
+  const float* wrow = ws.w(g) + tri_row_start(min(i, N - 1));
+  f32x16 acc[NDB];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const float gate = __shfl(dqa[db][e], 32 * hf + 2 * G) + __shfl(dqa[db][e], 32 * hf + 2 * G + 1);
-      if (vr == 0) dqa[db][e] += gate;
+  for (int db = 0; db < NDB; ++db) acc[db] = f32x16{0};
+  const int t_end = min(N, rb * 128 + 128);                       // keys up to the block's last row
+#pragma unroll 1
+  for (int t0 = 0; t0 < t_end; t0 += STEP) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < STEP * (D / 8); e += NT) {
+      const int rr = e / (D / 8), v8 = e % (D / 8);
+      *reinterpret_cast<u32x4*>(tile + rr * TS + 8 * v8) =
+          *reinterpret_cast<const u32x4*>(kbase + (int64_t)min(t0 + rr, N - 1) * D + 8 * v8);
     }
-  if (vr < 2 * G && vr % 2 == 0) {
-    uint16_t* op = p.dq + ((int64_t)(head0 + vr / 2) * N + i) * D;
+    __syncthreads();
+    if (t0 <= iw + 31 && iw < N) {   // wave-uniform: some row of this wave sees a key of the step
+      const int t = t0 + 8 * hf;     // first of this lane's 8 keys; t <= i keeps the 32-byte read inside the padded row
+      f32x4 w0 = f32x4{0.f, 0.f, 0.f, 0.f}, w1 = w0;
+      if (i < N && t <= i) {
+        w0 = *reinterpret_cast<const f32x4*>(wrow + t);
+        w1 = *reinterpret_cast<const f32x4*>(wrow + t + 4);
+      }
+      float hi[8], lo[8];
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        const float wv = (i < N && t + x <= i) ? (x < 4 ? w0[x] : w1[x - 4]) : 0.f;   // nothing beyond the diagonal is defined
+        hi[x] = bf16_to_f(f_to_bf16(wv));
+        lo[x] = wv - hi[x];
+      }
+      const u32x4 bhi = {pack_bf16(hi[0], hi[1]), pack_bf16(hi[2], hi[3]), pack_bf16(hi[4], hi[5]), pack_bf16(hi[6], hi[7])};
+      const u32x4 blo = {pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]), pack_bf16(lo[4], lo[5]), pack_bf16(lo[6], lo[7])};
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        const u32x4 a = load_a_trans_natural(tile, TS, 0, 32 * db);
+        acc[db] = mfma32(a, bhi, acc[db]);
+        acc[db] = mfma32(a, blo, acc[db]);
+      }
+    }
+  }
+  if (i < N) {
+    const float* part = ws.dql(g, N, D) + (int64_t)i * D;
+    uint16_t* op = p.dq + ((int64_t)(b * p.Hq + kvh * G) * N + i) * D;
 #pragma unroll
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
-        const u32x2 w = {pack_bf16(dqa[db][4 * g4] * p.sm_scale, dqa[db][4 * g4 + 1] * p.sm_scale),
-                         pack_bf16(dqa[db][4 * g4 + 2] * p.sm_scale, dqa[db][4 * g4 + 3] * p.sm_scale)};
+        const f32x4 pv = *reinterpret_cast<const f32x4*>(part + db * 32 + 8 * g4 + 4 * hf);
+        const u32x2 w = {pack_bf16((acc[db][4 * g4] + pv[0]) * p.sm_scale, (acc[db][4 * g4 + 1] + pv[1]) * p.sm_scale),
+                         pack_bf16((acc[db][4 * g4 + 2] + pv[2]) * p.sm_scale, (acc[db][4 * g4 + 3] + pv[3]) * p.sm_scale)};
         *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
       }
   }
@@ -677,8 +739,8 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
 }
 
 // ---------------------------------------------------------------------------------------------------- host side
-int64_t corope_gqa_bwd_workspace_floats(int B, int Hq, int Hkv, int N) {
-  return tri_row_start(N) * (2 * (int64_t)B * Hkv + 3 * (int64_t)B * Hq);
+int64_t corope_gqa_bwd_workspace_floats(int B, int Hq, int Hkv, int N, int D) {
+  return tri_row_start(N) * (2 * (int64_t)B * Hkv + 3 * (int64_t)B * Hq) + (int64_t)B * Hkv * N * D;
 }
 
 template <int D, int G>
@@ -691,6 +753,7 @@ static hipError_t launch_corope_bwd_cfg(const CoropeBwdParams& p, const CoropeBw
   hipLaunchKernelGGL(corope_bwd_rowdot_kernel<D>, dim3(nt, nt, p.B * p.Hq), dim3(4 * kWave), 0, stream, p.d_o, p.v,
                      ws.dp(0), ws.NN, p.N, 1, G);
   hipLaunchKernelGGL((corope_bwd_scores_kernel<D, G>), rows, dim3(kWave), 0, stream, p, ws, fr);
+  hipLaunchKernelGGL(corope_bwd_dq_leader_kernel<D>, dim3((p.N + 127) / 128, p.B * p.Hkv), dim3(4 * kWave), 0, stream, p, ws);
   using Cfg = CoropeDkCfg<D, G>;
   hipLaunchKernelGGL((corope_bwd_dv_kernel<D, G>), dim3((p.N + 127) / 128, p.B * p.Hkv), dim3(4 * kWave), 0, stream, p, ws);
   auto kern = corope_bwd_dk_kernel<D, G>;

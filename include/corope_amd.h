@@ -225,7 +225,8 @@ int corope_gqa_fwd(const void *q, const void *k, const void *v, void *o,
 
 /* Bytes of device workspace corope_gqa_bwd needs for these sizes (-1 for sizes corope_gqa_check rejects):
  * packed lower-triangular N x N fp32 matrices (about N*N/2 + 32*N floats each): two per key/value head (accumulated
- * gates; gate gradients) and three per query head (attention weights; score gradients; dO V^T). */
+ * gates; gate gradients) and three per query head (attention weights; score gradients; dO V^T), plus N*D floats per
+ * key/value head (the leader head's dq before its gate-path term is added). */
 int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D);
 
 /* Co-RoPE grouped-query attention backward (causal only): dq (B,Hq,N,D), dk/dv (B,Hkv,N,D) from q, k, v and dO.

@@ -110,8 +110,8 @@ def test_corope_backward_argument_checks(pkg):
     """Workspace size query and the checks corope_gqa_bwd makes before any launch (no GPU needed)."""
     lib = pkg._lib.load()
     packed = lambda n: sum(64 * (i // 64 + 1) for i in range(n))   # one lower-triangular matrix, rows padded to 64 keys
-    assert lib.corope_gqa_bwd_workspace_bytes(2, 32, 8, 4096, 128) == 4 * packed(4096) * (2 * 16 + 3 * 64)
-    assert lib.corope_gqa_bwd_workspace_bytes(1, 4, 2, 33, 64) == 4 * packed(33) * (2 * 2 + 3 * 4)
+    assert lib.corope_gqa_bwd_workspace_bytes(2, 32, 8, 4096, 128) == 4 * (packed(4096) * (2 * 16 + 3 * 64) + 16 * 4096 * 128)
+    assert lib.corope_gqa_bwd_workspace_bytes(1, 4, 2, 33, 64) == 4 * (packed(33) * (2 * 2 + 3 * 4) + 2 * 33 * 64)
     assert packed(4096) == 4096 * 4096 // 2 + 32 * 4096
     assert lib.corope_gqa_bwd_workspace_bytes(1, 5, 2, 33, 64) == -1      # Hq not a multiple of Hkv
     assert lib.corope_gqa_bwd_workspace_bytes(1, 18, 2, 33, 64) == -1     # group size 9

@@ -111,7 +111,7 @@ def test_corope_backward_caller_workspace_and_reuse(pkg):
     q, k, v, d_o = (t.to(dev, torch.bfloat16) for t in _inputs(B, Hq, Hkv, N, D, seed=3))
     need = mod.backward_workspace_bytes(B, Hq, Hkv, N, D)
     packed = sum(64 * (i // 64 + 1) for i in range(N))          # rows hold the keys j <= i, padded to 64-key chunks
-    assert need == 4 * packed * (2 * B * Hkv + 3 * B * Hq)
+    assert need == 4 * (packed * (2 * B * Hkv + 3 * B * Hq) + B * Hkv * N * D)   # + the leader's fp32 dq rows
     a = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4)
     ws = torch.full((need // 4 + 64,), float("nan"), device=dev)
     b = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4, workspace=ws)
