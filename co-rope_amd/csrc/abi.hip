@@ -91,6 +91,10 @@ int corope_gqa_check(int B, int Hq, int Hkv, int N, int D, float sm_scale, float
   if (D != 64 && D != 128) return fail(COROPE_E_UNSUPPORTED, "corope_gqa: head dim %d not built (64 and 128 are)", D);
   if (!std::isfinite(sm_scale)) return fail(COROPE_E_BADARG, "corope_gqa: sm_scale must be finite");
   if (!(theta > 0.f) || !std::isfinite(theta)) return fail(COROPE_E_BADARG, "corope_gqa: theta must be positive and finite");
+  // one workgroup per (batch, kv head, query row) on a single grid axis; slabs addressed with 32-bit byte offsets
+  if ((int64_t)B * Hkv * N >= ((int64_t)1 << 31) || (int64_t)N * D * 2 >= ((int64_t)1 << 32))
+    return fail(COROPE_E_UNSUPPORTED, "corope_gqa: B * Hkv * N = %lld rows exceed the grid, or one slab exceeds 4 GiB",
+                (long long)B * Hkv * N);
   g_err[0] = 0;
   return COROPE_OK;
 }
@@ -511,7 +515,7 @@ int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* o, c
   rc = check_ptrs("corope_gqa_bwd", {q, k, v, d_o, dq, dk, dv, workspace});
   if (rc) return rc;
   if (o != nullptr && !aligned16(o)) return fail(COROPE_E_ALIGN, "corope_gqa_bwd: pointer %p is not 16-byte aligned", o);
-  if ((int64_t)B * Hkv > 65535) return fail(COROPE_E_UNSUPPORTED, "corope_gqa_bwd: B * Hkv = %lld exceeds 65535", (long long)B * Hkv);
+  if ((int64_t)B * Hq > 65535) return fail(COROPE_E_UNSUPPORTED, "corope_gqa_bwd: B * Hq = %lld exceeds 65535", (long long)B * Hq);
   const int64_t need = 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N, D);
   if (workspace_bytes < need)
     return fail(COROPE_E_BADARG, "corope_gqa_bwd: workspace of %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);

@@ -27,7 +27,7 @@ __global__ __launch_bounds__(kRotThreads) void rope_rotate_kernel(const uint16_t
   using Stage = RotStage<D, kRotRows, kRotThreads>;
   constexpr int kChunks = Stage::kChunks;
   __shared__ float wave_max[kRotThreads / kWave];
-  const int tile = blockIdx.x, bh = blockIdx.y;
+  const int tile = blockIdx.x % n_tiles, bh = blockIdx.x / n_tiles;
   const int row0 = tile * kRotRows;
   const uint16_t* xg = x + (int64_t)bh * N * D;
   uint16_t* yg = y + (int64_t)bh * N * D;
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(kRotThreads) void rope_rotate_kernel(const uint16_t
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
                               float* tile_max, int BH, int N, int D, hipStream_t stream) {
   const int n_tiles = (N + kRotRows - 1) / kRotRows;
-  dim3 grid(n_tiles, BH);
+  dim3 grid((unsigned)n_tiles * BH);   // one axis: the second grid axis stops at 65535 slabs
   if (D == 128)
     hipLaunchKernelGGL(rope_rotate_kernel<128>, grid, dim3(kRotThreads), 0, stream, x, cosp, sinp, fstride, y, tile_max,
                        N, n_tiles);

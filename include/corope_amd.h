@@ -219,7 +219,7 @@ int corope_rope_attn_bwd_gqa(const void *q, const void *k, int prerotated, const
  * Replaces the launch of _corope_fwd_backbone in _attention.forward
  * (reference corope-exp/flash_attn_co_rope_gqa_triton.py:48-400 kernel, :428-450 launch);
  * the inverse frequencies theta^(-2d/D) the reference builds with torch (:428) are computed
- * on the host here and passed to the kernel by value. */
+ * on the host here and passed to the kernel by value.  Limits: B*Hkv*N < 2^31, N*D*2 bytes < 4 GiB. */
 int corope_gqa_fwd(const void *q, const void *k, const void *v, void *o,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void *stream);
 
@@ -235,7 +235,7 @@ int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D);
  * leader head's gates, :548-561) are produced here with packed triangular N x N matrices of scalars in `workspace`.
  * Like the reference's, it needs neither the forward's output nor its row statistics; `o` may be NULL.  When the forward's output is
  * passed, rowsum(O o dO) serves as a reference value that keeps dQ accurate for rows dominated by a single key (the
- * result is mathematically the same with or without it).  The workspace need not be initialised. */
+ * result is mathematically the same with or without it).  The workspace need not be initialised.  Limit: B*Hq <= 65535. */
 int corope_gqa_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,
                    void *dq, void *dk, void *dv,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta,

@@ -68,6 +68,8 @@ def test_rope_attn_check_codes(pkg, args, code):
     ((1, 4, 2, 64, 32, 1.0, 1e4), -2),
     ((1, 4, 2, 64, 64, 1.0, 0.0), -1),
     ((1, 4, 2, 0, 64, 1.0, 1e4), -1),
+    ((64, 64, 64, 1 << 19, 64, 1.0, 1e4), -2),   # B * Hkv * N rows do not fit one grid axis
+    ((1, 1, 1, 1 << 24, 128, 1.0, 1e4), -2),     # a slab beyond 32-bit byte offsets
 ])
 def test_corope_check_codes(pkg, args, code):
     assert pkg._lib.load().corope_gqa_check(*args) == code
@@ -126,6 +128,8 @@ def test_corope_backward_argument_checks(pkg):
     assert lib.corope_gqa_bwd(*args(ok, need, o=ok + 2)) == -3 and "aligned" in pkg._lib.last_error()   # o is optional, not sloppy
     rc = lib.corope_gqa_bwd(ok, ok, ok, None, ok, ok, ok, ok, 1, 18, 2, 8, 64, 0.125, 1e4, ok, 1 << 40, None)
     assert rc == -2 and "group size" in pkg._lib.last_error()
+    rc = lib.corope_gqa_bwd(ok, ok, ok, None, ok, ok, ok, ok, 16384, 8, 1, 8, 64, 0.125, 1e4, ok, 1 << 50, None)
+    assert rc == -2 and "B * Hq" in pkg._lib.last_error()
 
 
 def test_rope_freqs_argument_checks(pkg):

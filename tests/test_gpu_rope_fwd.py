@@ -144,6 +144,21 @@ def test_rotate_pass_matches_the_oracle(pkg):
         assert torch.equal(y_only.float().cpu(), y)
 
 
+def test_rotate_pass_with_more_slabs_than_a_grid_axis(pkg):
+    """70000 (batch, head) slabs of 3 rows: every slab is rotated (the launch does not put slabs on a 65535-limited axis)."""
+    dev = torch.device("cuda:0")
+    B, H, N, D = 70, 1000, 3, 64
+    print(f"case rotate B={B} H={H} N={N} D={D}", flush=True)
+    x = bf16_round(seeded((B, H, N, D), 5))
+    c, s = O.precompute_freqs_cis(D, N)
+    y, tm = pkg.rope_rotate(x.to(dev, torch.bfloat16), c.to(dev), s.to(dev), with_tile_max=True)
+    y = y.float().cpu()
+    ref = O.apply_rotary_emb(x, c, s)
+    # one bf16 ulp, plus the fp32 rounding of the two products where they cancel (13 M elements: some do)
+    assert ((y - ref).abs() <= ref.abs() / 128 + 1e-6).all()
+    assert torch.allclose(tm.cpu()[..., 0], y.norm(dim=-1).amax(-1), rtol=1e-5, atol=0)
+
+
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("case", ["large_norms", "outlier_keys", "growing_scores", "tiny_scores", "huge_norms_hot"])
 def test_two_launch_softmax_modes(pkg, case, causal):
