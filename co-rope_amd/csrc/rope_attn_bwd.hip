@@ -127,6 +127,14 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
     load_tile(0);
     store_tile(0);
   }
+  // The wave's K_r (and V) rows must have landed on EVERY path into the loop: left to the first product that reads them,
+  // the wait for them is placed inside the loop, where each time round it also waits for the next tile's loads issued
+  // a few instructions earlier, and the prefetch hides less.
+#pragma unroll
+  for (int kc = 0; kc < KC; ++kc) {
+    asm volatile("" ::"v"(kb[kc]));
+    if constexpr (DO_DK && !V_LDS) asm volatile("" ::"v"(vb[kc]));
+  }
   __syncthreads();
 
   const float scale2 = p.qk_scale;
