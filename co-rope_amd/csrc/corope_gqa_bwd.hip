@@ -74,37 +74,81 @@ struct CoropeBwdWs {
 // ---------------------------------------------------------------------------------------------------- row dots
 // out[idx][i][j] = a[idx * a_mul][i] . b[idx / b_div][j] for the tiles that touch the causal triangle: the two plain
 // matrix products of the backward (leader logits qL K^T per group: a_mul = G, b_div = 1; dP = dO V^T per head: a_mul
-// = 1, b_div = G) on the matrix cores.  Both operands of a 32 x 32 x 16 step are 16-byte pieces of rows, so they are
-// loaded straight from global memory; one wave owns 32 rows of `a` and sweeps four 32-key tiles with them.
+// = 1, b_div = G) on the matrix cores.  A workgroup of 4 waves owns 128 rows x 128 keys; the rows of both operands are
+// fetched with whole cache lines and parked in LDS (an operand piece read straight from global memory is 16 bytes of a
+// row per lane: every instruction would touch 64 different lines); one wave owns 32 rows and sweeps the keys in two
+// halves of 64, the second half fetched while the first is multiplied.
+constexpr int kRowdotRows = 128, kRowdotKeys = 64;
+
 template <int D>
 __global__ __launch_bounds__(4 * kWave) void corope_bwd_rowdot_kernel(const uint16_t* a, const uint16_t* b, float* out,
                                                                       int64_t NN, int N, int a_mul, int b_div) {
+  constexpr int TS = D + 8, NT = 4 * kWave, PIECES = D / 8;
+  constexpr int A_PER = kRowdotRows * PIECES / NT, B_PER = kRowdotKeys * PIECES / NT;
+  __shared__ __attribute__((aligned(16))) uint16_t atile[kRowdotRows * TS];
+  __shared__ __attribute__((aligned(16))) uint16_t btile[kRowdotKeys * TS];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int r = lane % 32, hf = lane / 32;
   const int idx = blockIdx.z;
-  const int i0 = blockIdx.y * 128 + wave * 32, j0 = blockIdx.x * 128;
-  if (j0 > i0 + 31 || i0 >= N) return;   // every key of the block lies beyond this wave's rows
-  const uint16_t* arow = a + ((int64_t)idx * a_mul * N + min(i0 + r, N - 1)) * D + 8 * hf;
+  const int ib = blockIdx.y * kRowdotRows, j0 = blockIdx.x * 128;
+  if (j0 > ib + kRowdotRows - 1 || ib >= N) return;   // every key of the block lies beyond its rows (workgroup-uniform)
+  const int i0 = ib + wave * 32;
+  const uint16_t* arows = a + (int64_t)idx * a_mul * N * D;
+  const uint16_t* brows = b + (int64_t)(idx / b_div) * N * D;
+  u32x4 breg[B_PER];
+  auto fetch_b = [&](int jh) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < B_PER; ++u) {
+      const int e = threadIdx.x + u * NT;
+      breg[u] = *reinterpret_cast<const u32x4*>(brows + (int64_t)min(jh + e / PIECES, N - 1) * D + 8 * (e % PIECES));
+    }
+  };
+  auto park_b = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < B_PER; ++u) {
+      const int e = threadIdx.x + u * NT;
+      *reinterpret_cast<u32x4*>(btile + (e / PIECES) * TS + 8 * (e % PIECES)) = breg[u];
+    }
+  };
+  fetch_b(j0);
+#pragma unroll
+  for (int u = 0; u < A_PER; ++u) {
+    const int e = threadIdx.x + u * NT;
+    *reinterpret_cast<u32x4*>(atile + (e / PIECES) * TS + 8 * (e % PIECES)) =
+        *reinterpret_cast<const u32x4*>(arows + (int64_t)min(ib + e / PIECES, N - 1) * D + 8 * (e % PIECES));
+  }
+  park_b();
+  __syncthreads();
   u32x4 af[D / 16];
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) af[ks] = *reinterpret_cast<const u32x4*>(arow + 16 * ks);
+  for (int ks = 0; ks < D / 16; ++ks) af[ks] = *reinterpret_cast<const u32x4*>(atile + (wave * 32 + r) * TS + 16 * ks + 8 * hf);
   float* obase = out + (int64_t)idx * NN;
+  // the 32 rows of the wave lie in one 64-row band, so they share a row length; a column <= i0 + 31 is inside the padded row
+  const int64_t row0 = tri_row_start(min(i0, N - 1)), row_len = 64 * (i0 / 64 + 1);
 #pragma unroll 1
-  for (int jt = 0; jt < 4; ++jt) {
-    const int jj0 = j0 + 32 * jt;
-    if (jj0 > i0 + 31 || jj0 >= N) break;
-    const uint16_t* brow = b + ((int64_t)(idx / b_div) * N + min(jj0 + r, N - 1)) * D + 8 * hf;
-    f32x16 c = f32x16{0};
+  for (int half = 0; half < 2; ++half) {
+    const int jh = j0 + kRowdotKeys * half;
+    const bool more = half == 0 && jh + kRowdotKeys <= ib + kRowdotRows - 1 && jh + kRowdotKeys < N;   // workgroup-uniform
+    if (more) fetch_b(jh + kRowdotKeys);
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) c = mfma32(af[ks], *reinterpret_cast<const u32x4*>(brow + 16 * ks), c);
-    const int col = jj0 + r;
-    // the 32 rows of the tile lie in one 64-row band, so they share a row length; col <= i0 + 31 is inside the padded row
-    const int64_t row0 = tri_row_start(i0), row_len = 64 * (i0 / 64 + 1);
+    for (int jt = 0; jt < kRowdotKeys / 32; ++jt) {
+      const int jj0 = jh + 32 * jt;
+      if (jj0 > i0 + 31 || jj0 >= N || i0 >= N) continue;   // wave-uniform
+      f32x16 c = f32x16{0};
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int dr = acc_row(e, hf);
-      if (i0 + dr < N && col < N) obase[row0 + row_len * dr + col] = c[e];
+      for (int ks = 0; ks < D / 16; ++ks)
+        c = mfma32(af[ks], *reinterpret_cast<const u32x4*>(btile + (32 * jt + r) * TS + 16 * ks + 8 * hf), c);
+      const int col = jj0 + r;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int dr = acc_row(e, hf);
+        if (i0 + dr < N && col < N) obase[row0 + row_len * dr + col] = c[e];
+      }
     }
+    if (!more) break;
+    __syncthreads();   // every wave is done with the first half of the keys
+    park_b();
+    __syncthreads();
   }
 }
 
@@ -469,31 +513,46 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_dq_leader_kernel(CoropeB
 #pragma unroll
   for (int db = 0; db < NDB; ++db) acc[db] = f32x16{0};
   const int t_end = min(N, rb * 128 + 128);                       // keys up to the block's last row
+  // the key rows and this lane's W values of a step are fetched into registers one step ahead (the workgroup of the last
+  // row block walks N / 16 steps one after the other)
+  constexpr int UNITS = STEP * (D / 8), PER = (UNITS + NT - 1) / NT;
+  u32x4 kreg[PER];
+  f32x4 w0 = f32x4{0.f, 0.f, 0.f, 0.f}, w1 = w0;
+  auto fetch = [&](int t0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int e = min((int)threadIdx.x + u * NT, UNITS - 1);
+      kreg[u] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)min(t0 + e / (D / 8), N - 1) * D + 8 * (e % (D / 8)));
+    }
+    const int t = t0 + 8 * hf;     // first of this lane's 8 keys; t <= i keeps the 32-byte read inside the padded row
+    w0 = w1 = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (t0 <= iw + 31 && iw < N && i < N && t <= i) {
+      w0 = *reinterpret_cast<const f32x4*>(wrow + t);
+      w1 = *reinterpret_cast<const f32x4*>(wrow + t + 4);
+    }
+  };
+  if (t_end > 0) fetch(0);
 #pragma unroll 1
   for (int t0 = 0; t0 < t_end; t0 += STEP) {
-    __syncthreads();
-    for (int e = threadIdx.x; e < STEP * (D / 8); e += NT) {
-      const int rr = e / (D / 8), v8 = e % (D / 8);
-      *reinterpret_cast<u32x4*>(tile + rr * TS + 8 * v8) =
-          *reinterpret_cast<const u32x4*>(kbase + (int64_t)min(t0 + rr, N - 1) * D + 8 * v8);
+    __syncthreads();   // the previous step's reads of the tile are done
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int e = threadIdx.x + u * NT;
+      if (UNITS % NT == 0 || e < UNITS) *reinterpret_cast<u32x4*>(tile + (e / (D / 8)) * TS + 8 * (e % (D / 8))) = kreg[u];
     }
+    const int t = t0 + 8 * hf;
+    float hi[8], lo[8];
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      const float wv = (i < N && t + x <= i) ? (x < 4 ? w0[x] : w1[x - 4]) : 0.f;   // nothing beyond the diagonal is defined
+      hi[x] = bf16_to_f(f_to_bf16(wv));
+      lo[x] = wv - hi[x];
+    }
+    const u32x4 bhi = {pack_bf16(hi[0], hi[1]), pack_bf16(hi[2], hi[3]), pack_bf16(hi[4], hi[5]), pack_bf16(hi[6], hi[7])};
+    const u32x4 blo = {pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]), pack_bf16(lo[4], lo[5]), pack_bf16(lo[6], lo[7])};
+    if (t0 + STEP < t_end) fetch(t0 + STEP);
     __syncthreads();
     if (t0 <= iw + 31 && iw < N) {   // wave-uniform: some row of this wave sees a key of the step
-      const int t = t0 + 8 * hf;     // first of this lane's 8 keys; t <= i keeps the 32-byte read inside the padded row
-      f32x4 w0 = f32x4{0.f, 0.f, 0.f, 0.f}, w1 = w0;
-      if (i < N && t <= i) {
-        w0 = *reinterpret_cast<const f32x4*>(wrow + t);
-        w1 = *reinterpret_cast<const f32x4*>(wrow + t + 4);
-      }
-      float hi[8], lo[8];
-#pragma unroll
-      for (int x = 0; x < 8; ++x) {
-        const float wv = (i < N && t + x <= i) ? (x < 4 ? w0[x] : w1[x - 4]) : 0.f;   // nothing beyond the diagonal is defined
-        hi[x] = bf16_to_f(f_to_bf16(wv));
-        lo[x] = wv - hi[x];
-      }
-      const u32x4 bhi = {pack_bf16(hi[0], hi[1]), pack_bf16(hi[2], hi[3]), pack_bf16(hi[4], hi[5]), pack_bf16(hi[6], hi[7])};
-      const u32x4 blo = {pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]), pack_bf16(lo[4], lo[5]), pack_bf16(lo[6], lo[7])};
 #pragma unroll
       for (int db = 0; db < NDB; ++db) {
         const u32x4 a = load_a_trans_natural(tile, TS, 0, 32 * db);
@@ -524,6 +583,7 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_dq_leader_kernel(CoropeB
 template <int D, int G>
 __global__ __launch_bounds__(4 * kWave) void corope_bwd_dv_kernel(CoropeBwdParams p, CoropeBwdWs ws) {
   constexpr int TS = D + 16, NDB = D / 32, NT = 4 * kWave, ROWS = 16;
+  constexpr int UNITS = G * ROWS * (D / 8), PER = (UNITS + NT - 1) / NT;   // 16-byte pieces of a dO tile, per thread
   __shared__ __attribute__((aligned(16))) uint16_t tile[G * ROWS * TS];
   const int jb = blockIdx.x * 128, g = blockIdx.y;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -534,31 +594,54 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_dv_kernel(CoropeBwdParam
   f32x16 acc[NDB];
 #pragma unroll
   for (int db = 0; db < NDB; ++db) acc[db] = f32x16{0};
+
+  // Both streams run one step ahead in registers: the workgroup of the first key block walks N / 16 steps one after the
+  // other, and with a step's loads issued only when the step begins its time is N / 16 memory latencies.
+  u32x4 dreg[PER];
+  float pnext[G][8];
+  auto fetch = [&](int i0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int e = min((int)threadIdx.x + u * NT, UNITS - 1);
+      const int h = e / (ROWS * (D / 8)), rr = (e / (D / 8)) % ROWS, v8 = e % (D / 8);
+      dreg[u] = *reinterpret_cast<const u32x4*>(p.d_o + ((int64_t)(head0 + h) * N + min(i0 + rr, N - 1)) * D + 8 * v8);
+    }
+    const bool wave_on = i0 + ROWS - 1 >= jw && jw < N;   // wave-uniform: some row of the step sees a key of this wave
+    const int64_t row_len = 64 * (i0 / 64 + 1);           // the 16 rows of a step share a row length
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      const float* prow = ws.p(head0 + h) + tri_row_start(min(i0, N - 1)) + j;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const int i = i0 + 8 * hf + t;
+        pnext[h][t] = (wave_on && i < N && j <= i) ? prow[row_len * (8 * hf + t)] : 0.f;   // nothing outside the triangle is defined
+      }
+    }
+  };
+  if (jb < N) fetch(jb);
 #pragma unroll 1
   for (int i0 = jb; i0 < N; i0 += ROWS) {
-    __syncthreads();
-    for (int e = threadIdx.x; e < G * ROWS * (D / 8); e += NT) {
-      const int h = e / (ROWS * (D / 8)), rr = (e / (D / 8)) % ROWS, v8 = e % (D / 8);
-      const int64_t off = ((int64_t)(head0 + h) * N + min(i0 + rr, N - 1)) * D + 8 * v8;
-      *reinterpret_cast<u32x4*>(tile + (h * ROWS + rr) * TS + 8 * v8) = *reinterpret_cast<const u32x4*>(p.d_o + off);
+    __syncthreads();   // the previous step's reads of the tile are done
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int e = threadIdx.x + u * NT;
+      if (UNITS % NT == 0 || e < UNITS)
+        *reinterpret_cast<u32x4*>(tile + (e / (D / 8)) * TS + 8 * (e % (D / 8))) = dreg[u];   // rows are (head, row) pairs
     }
+    u32x4 bop[G];
+#pragma unroll
+    for (int h = 0; h < G; ++h)
+      bop[h] = u32x4{pack_bf16(pnext[h][0], pnext[h][1]), pack_bf16(pnext[h][2], pnext[h][3]),
+                     pack_bf16(pnext[h][4], pnext[h][5]), pack_bf16(pnext[h][6], pnext[h][7])};
+    const bool wave_on = i0 + ROWS - 1 >= jw && jw < N;
+    if (i0 + ROWS < N) fetch(i0 + ROWS);
     __syncthreads();
-    if (i0 + ROWS - 1 >= jw && jw < N) {   // wave-uniform: some row of the step sees a key of this wave
+    if (wave_on) {
 #pragma unroll
-      for (int h = 0; h < G; ++h) {
-        float pv[8];
-        const float* prow = ws.p(head0 + h) + tri_row_start(i0) + j;   // the 16 rows of a step share a row length
-        const int64_t row_len = 64 * (i0 / 64 + 1);
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-          const int i = i0 + 8 * hf + t;
-          pv[t] = (i < N && j <= i) ? prow[row_len * (8 * hf + t)] : 0.f;   // nothing outside the triangle is defined
-        }
-        const u32x4 bop = {pack_bf16(pv[0], pv[1]), pack_bf16(pv[2], pv[3]), pack_bf16(pv[4], pv[5]), pack_bf16(pv[6], pv[7])};
+      for (int h = 0; h < G; ++h)
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
-          acc[db] = mfma32(load_a_trans_natural(tile + h * ROWS * TS, TS, 0, 32 * db), bop, acc[db]);
-      }
+          acc[db] = mfma32(load_a_trans_natural(tile + h * ROWS * TS, TS, 0, 32 * db), bop[h], acc[db]);
     }
   }
   if (j < N) {

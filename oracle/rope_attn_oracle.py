@@ -204,7 +204,7 @@ class _AttentionOracle(torch.autograd.Function):
 attention_pytorch = _AttentionOracle.apply
 
 
-# ------------------------------------------------------------------- FLOP model (§ bench)
+# ------------------------------------------------------------------- FLOP model (used by bench.py)
 def attention_flops(B, H, N, D, mode="fwd", causal=False):
     """The reference's FLOP model (fused-rope/bench_compare.py:61-86): two N x N x D
     matmuls, halved when causal, x2.5 for the backward; rotation FLOPs are not counted."""
