@@ -247,9 +247,11 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   // for the next chunk at the point where the current values have been used up.
   constexpr int PIECES = D / 8;   // 16-byte pieces per row = fetch instructions per chunk
   u32x4 kv[PIECES];
-  auto fetch_keys = [&](int c) __attribute__((always_inline)) {
+  // may_run_past_end: only the chunk on the diagonal can; the form without the clamped variant keeps one address per
+  // lane (with both forms present the compiler merges them into loads behind sixteen selected 64-bit addresses)
+  auto fetch_keys = [&](int c, auto may_run_past_end) __attribute__((always_inline)) {
     const uint16_t* block = kbase + (int64_t)c * kWave * D;   // wave-uniform
-    if (c * kWave + kWave <= N) {
+    if (!decltype(may_run_past_end)::value || c * kWave + kWave <= N) {
 #pragma unroll
       for (int it = 0; it < PIECES; ++it)
         kv[it] = *reinterpret_cast<const u32x4*>(byte_offset(block, 16u * lane + 1024u * it));
@@ -271,7 +273,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   float logit, dpv[G];
   {
     const int jc = min((n_chunks - 1) * kWave + lane, i);
-    fetch_keys(n_chunks - 1);
+    fetch_keys(n_chunks - 1, std::true_type{});
     logit = *byte_offset(d_row, 4u * jc);
 #pragma unroll
     for (int h = 0; h < G; ++h) dpv[h] = *byte_offset(dp_row[h], 4u * jc);
@@ -335,7 +337,9 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       lo_rows[n] = __builtin_bit_cast(float, (uint32_t)r[0]);
       hi_rows[n] = __builtin_bit_cast(float, (uint32_t)r[1]);
     }
-    if (c > 0) fetch_keys(c - 1);   // the registers of the product are free again: request the next chunk's keys
+    // the registers of the product are free again: request the next chunk's keys (a chunk left of the diagonal one lies
+    // inside the sequence)
+    if (c > 0) fetch_keys(c - 1, std::false_type{});
     float acc[G], gacc[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) {
