@@ -74,9 +74,11 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
 
   // one 64 x D block of K or V: consecutive 16-byte pieces per lane, parked as rows of the tile
   u32x4 blk[PIECES];
-  auto fetch_block = [&](const uint16_t* base, int c) __attribute__((always_inline)) {
+  // may_run_past_end: only the chunk on the diagonal can; the form without the clamped variant keeps one address per
+  // lane (with both forms present the compiler merges them into loads behind sixteen selected 64-bit addresses)
+  auto fetch_block = [&](const uint16_t* base, int c, auto may_run_past_end) __attribute__((always_inline)) {
     const uint16_t* block = base + (int64_t)c * kWave * D;   // wave-uniform
-    if (c * kWave + kWave <= N) {
+    if (!decltype(may_run_past_end)::value || c * kWave + kWave <= N) {
 #pragma unroll
       for (int it = 0; it < PIECES; ++it)
         blk[it] = *reinterpret_cast<const u32x4*>(byte_offset(block, 16u * lane + 1024u * it));
@@ -144,13 +146,19 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   }
   float carry = 0.f;          // sum of the gates of the chunks to the right (up to the diagonal)
 
-  fetch_block(kbase, n_chunks - 1);
+  // the chunk on the diagonal, the only one that can run past the last key, is fetched here; the loop's own fetches
+  // are for chunks inside the sequence
+  fetch_block(kbase, n_chunks - 1, std::true_type{});
+  park_block();
+  fetch_block(vbase, n_chunks - 1, std::true_type{});
 #pragma unroll 1
   for (int c = n_chunks - 1; c >= 0; --c) {
     const int j = c * kWave + lane;
     const bool valid = j <= i;
-    park_block();                 // K of this chunk
-    fetch_block(vbase, c);        // V of this chunk: needed after the scores
+    if (c != n_chunks - 1) {
+      park_block();                                  // K of this chunk
+      fetch_block(vbase, c, std::false_type{});      // V of this chunk: needed after the scores
+    }
     lds_order();                  // (also orders the one-time write of the leader's row before its first read)
 
     // leader logits (row 0 of the product), gates, delta
@@ -215,7 +223,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
         for (int e = 0; e < 16; ++e) oacc[db][e] *= al;
     }
     park_block();                          // V replaces the rotated keys
-    if (c > 0) fetch_block(kbase, c - 1);  // K of the next chunk
+    if (c > 0) fetch_block(kbase, c - 1, std::false_type{});  // K of the next chunk
     lds_order();
 #pragma unroll
     for (int ks = 0; ks < kWave / 16; ++ks) {
