@@ -707,7 +707,7 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
 
   constexpr int kTileElems = kDkRows * MATS * kDkKeys, TI = kTileElems / NT;      // fp32 values per thread and tile
   constexpr int kRowItems = kDkRows * G * (D / 8), RI = (kRowItems + NT - 1) / NT;  // 16-byte pieces of q rows
-  static_assert(kTileElems % NT == 0, "tile elements divide evenly over the threads");
+  static_assert(kTileElems % (4 * NT) == 0, "tile elements divide evenly over the threads, four keys at a time");
 
 #pragma unroll 1
   for (int phase = 0; phase < 2; ++phase) {
@@ -715,17 +715,23 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
     if (phase == 1 && kb <= (int)blockIdx.x) break;   // odd number of blocks: the middle one has been done in phase 0
     const int jb = kb * kDkKeys, jw = jb + 32 * wave;
 
-    float mv[TI];
+    f32x4 mv[TI / 4];
     u32x4 qv[RI];
     auto fetch = [&](int i0) __attribute__((always_inline)) {
-      const int64_t tile0 = tri_row_start(i0), row_len = 64 * (i0 / 64 + 1);   // the 8 rows of a tile share a row length
-      static_for<TI>([&](auto k_c) __attribute__((always_inline)) {
+      // the 8 rows of a tile share a row length; rows past the end repeat the last one (and are zeroed below)
+      const int64_t tile0 = tri_row_start(i0);
+      const int row_len = 64 * (i0 / 64 + 1);
+      static_for<TI / 4>([&](auto k_c) __attribute__((always_inline)) {
         constexpr int k = decltype(k_c)::value;
-        const int e = threadIdx.x + k * NT;
+        const int e = 4 * (threadIdx.x + k * NT);
         const int key = e % kDkKeys, m = (e / kDkKeys) % MATS, r = e / (kDkKeys * MATS);
         const int i = i0 + r, j = jb + key;
         const float* src = m == 0 ? ws.delta(g) : m == 1 ? ws.w(g) : ws.ds(head0 + m - 2);
-        mv[k] = (i < N && j <= i) ? src[tile0 + row_len * r + j] : 0.f;   // zero outside the causal triangle and past N
+        // four keys with one load, always inside the padded row (no branch); what lies outside the causal triangle or
+        // past N is not defined there and becomes zero
+        const f32x4 v = *reinterpret_cast<const f32x4*>(src + tile0 + (int64_t)row_len * min(r, N - 1 - i0) + min(j, row_len - 4));
+#pragma unroll
+        for (int x = 0; x < 4; ++x) mv[k][x] = (i < N && j + x <= i) ? v[x] : 0.f;
       });
       static_for<RI>([&](auto k_c) __attribute__((always_inline)) {
         constexpr int k = decltype(k_c)::value;
@@ -746,9 +752,9 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
 #pragma unroll 1
     for (int i0 = jb; i0 < N; i0 += kDkRows) {
       __syncthreads();   // the previous tile has been consumed
-      static_for<TI>([&](auto k_c) __attribute__((always_inline)) {
+      static_for<TI / 4>([&](auto k_c) __attribute__((always_inline)) {
         constexpr int k = decltype(k_c)::value;
-        tile[threadIdx.x + k * NT] = mv[k];
+        *reinterpret_cast<f32x4*>(tile + 4 * (threadIdx.x + k * NT)) = mv[k];
       });
       static_for<RI>([&](auto k_c) __attribute__((always_inline)) {
         constexpr int k = decltype(k_c)::value;
