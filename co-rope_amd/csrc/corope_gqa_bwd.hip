@@ -683,10 +683,10 @@ struct CoropeDkCfg {
 };
 
 template <int D, int G>
-__global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBwdParams p, CoropeBwdWs ws,
+__global__ __launch_bounds__(kDkWaves* kWave) __attribute__((amdgpu_waves_per_eu(2))) void corope_bwd_dk_kernel(CoropeBwdParams p, CoropeBwdWs ws,
                                                                        CoropeBwdFreqs fr) {
   using Cfg = CoropeDkCfg<D, G>;
-  constexpr int HALF = D / 2, NT = kDkWaves * kWave, MATS = Cfg::kMats, NB = D / 32, NP = D / 64;
+  constexpr int HALF = D / 2, NT = kDkWaves * kWave, MATS = Cfg::kMats, NP = D / 64;
   static_assert(D == 64 || D == 128, "pairs per lane are laid out for these head dims");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float* tile = reinterpret_cast<float*>(smem);                                   // [row][matrix][key]
@@ -786,15 +786,6 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
           }
           aop = u32x4{pack_bf16(dsv[0], dsv[1]), pack_bf16(dsv[2], dsv[3]), pack_bf16(dsv[4], dsv[5]), pack_bf16(dsv[6], dsv[7])};
         }
-        // B: (heads x 32 columns) per column block; the same read also carries the leader's (head 0) value of the column
-        f32x16 u[NB];
-        float ql[NB];
-#pragma unroll
-        for (int blk = 0; blk < NB; ++blk) {
-          const u32x4 bq = *reinterpret_cast<const u32x4*>(qT + (r * D + 32 * blk + col) * 8);
-          ql[blk] = bf16_lo(bq[0]);
-          u[blk] = mfma32(aop, bq, f32x16{0});
-        }
         // delta and W of this lane's 16 keys: keys 8 n + 4 half + 0..3 for n = 0..3, as the accumulator rows are laid out
         f32x4 dl[4], wg[4];
 #pragma unroll
@@ -802,16 +793,21 @@ __global__ __launch_bounds__(kDkWaves* kWave) void corope_bwd_dk_kernel(CoropeBw
           dl[n] = *reinterpret_cast<const f32x4*>(trow + 8 * n + 4 * hf);
           wg[n] = *reinterpret_cast<const f32x4*>(trow + kDkKeys + 8 * n + 4 * hf);
         }
+        // B: (heads x 32 columns) per column block; the same read also carries the leader's (head 0) value of the column.
+        // One rotation pair per pass (columns 32 np + col and the same + D/2), so that only two product blocks are live.
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const float delta = dl[e / 4][e % 4], wij = wg[e / 4][e % 4];
+        for (int np = 0; np < NP; ++np) {
+          const u32x4 bq1 = *reinterpret_cast<const u32x4*>(qT + (r * D + 32 * np + col) * 8);
+          const u32x4 bq2 = *reinterpret_cast<const u32x4*>(qT + (r * D + 32 * (NP + np) + col) * 8);
+          const float ql1 = bf16_lo(bq1[0]), ql2 = bf16_lo(bq2[0]);
+          const f32x16 u1 = mfma32(aop, bq1, f32x16{0}), u2 = mfma32(aop, bq2, f32x16{0});
 #pragma unroll
-          for (int np = 0; np < NP; ++np) {
+          for (int e = 0; e < 16; ++e) {
+            const float delta = dl[e / 4][e % 4], wij = wg[e / 4][e % 4];
             const float x = __builtin_amdgcn_fractf(delta * w_turn[np]);
             const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
-            const float u1 = u[np][e], u2 = u[NP + np][e];
-            dk1[np][e] = __builtin_fmaf(cs, u1, __builtin_fmaf(-sn, u2, __builtin_fmaf(wij, ql[np], dk1[np][e])));
-            dk2[np][e] = __builtin_fmaf(cs, u2, __builtin_fmaf(sn, u1, __builtin_fmaf(wij, ql[NP + np], dk2[np][e])));
+            dk1[np][e] = __builtin_fmaf(cs, u1[e], __builtin_fmaf(-sn, u2[e], __builtin_fmaf(wij, ql1, dk1[np][e])));
+            dk2[np][e] = __builtin_fmaf(cs, u2[e], __builtin_fmaf(sn, u1[e], __builtin_fmaf(wij, ql2, dk2[np][e])));
           }
         }
       }
