@@ -203,24 +203,38 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     heads_times_tile(c0, c1);
     float sc[G];
     rows_of_key(c0, c1, sc);
-    float al = 1.f;          // this lane's head's rescale factor
-    bool moved = false;      // wave-uniform: some head's running maximum moved
+    // The reference value m_run[h] of the exponentials only has to keep them in range, it need not be the running
+    // maximum: it moves (to the exact maximum so far, with the usual rescaling) only when some score of the chunk lies
+    // more than kLazyMargin above it, which after the first chunks of a row is rare.  The common case then costs one
+    // comparison per head instead of a cross-lane maximum.
+    constexpr float kLazyMargin = 8.f;   // base-2 units: weights stay below 2^8
+    float (&s2)[G] = sc;   // scaled in place
+    bool exceeds = false;
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-      const float s2 = sc[h] * scale2;
-      const float m_new = fmaxf(m_run[h], wave_max(valid ? s2 : -INFINITY));   // finite: the chunk holds a key <= i
-      const float a = fast_exp2(m_run[h] - m_new), e = valid ? fast_exp2(s2 - m_new) : 0.f;
-      moved |= m_new != m_run[h];
-      m_run[h] = m_new;
-      l_run[h] = __builtin_fmaf(l_run[h], a, e);
-      al = vr == h ? a : al;
-      wts[h * WS + lane] = f_to_bf16(e);
+      s2[h] = valid ? sc[h] * scale2 : -INFINITY;
+      exceeds |= s2[h] > m_run[h] + kLazyMargin;   // m_run starts at -inf: the first chunk always moves it
     }
-    if (moved) {
+    if (__builtin_amdgcn_ballot_w64(exceeds) != 0) {   // wave-uniform
+      float al = 1.f;          // this lane's head's rescale factor
+#pragma unroll
+      for (int h = 0; h < G; ++h) {
+        const float m_new = fmaxf(m_run[h], wave_max(s2[h]));   // finite: the chunk holds a key <= i
+        const float a = fast_exp2(m_run[h] - m_new);
+        m_run[h] = m_new;
+        l_run[h] *= a;
+        al = vr == h ? a : al;
+      }
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int e = 0; e < 16; ++e) oacc[db][e] *= al;
+    }
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      const float e = fast_exp2(s2[h] - m_run[h]);   // 0 for the keys beyond the diagonal
+      l_run[h] += e;
+      wts[h * WS + lane] = f_to_bf16(e);
     }
     park_block();                          // V replaces the rotated keys
     if (c > 0) fetch_block(kbase, c - 1, std::false_type{});  // K of the next chunk
