@@ -351,8 +351,13 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       *byte_offset(d_row, 4u * j) = delta;
       *byte_offset(w_row, 4u * j) = z * (1.f - z);   // the sigmoid's slope; replaced by W in the second sweep
     }
-    float al = 1.f;          // this lane's virtual row's rescale factor
-    bool moved = false;      // wave-uniform: some head's running maximum moved
+    // The reference value m_run[h] of the exponentials only has to keep them in range, it need not be the running
+    // maximum (any value gives the same P once the row is normalised): it moves, to the exact maximum so far and with the
+    // usual rescaling, only when some score of the chunk lies more than kLazyMargin above it -- rare after the first
+    // chunks of a row -- and the common case costs one comparison per head instead of a cross-lane maximum.  The margin
+    // bounds the weights e (dP - ref) that go to the matrix cores as fp16.
+    constexpr float kLazyMargin = 4.f;
+    bool exceeds = false;
 #pragma unroll
     for (int h = 0; h < G; ++h) {
       const float sc = acc[h] * p.sm_scale;
@@ -360,25 +365,36 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
         *byte_offset(p_row[h], 4u * j) = sc;
         *byte_offset(ds_row[h], 4u * j) = gacc[h] * p.sm_scale;
       }
-      const float m_new = fmaxf(m_run[h], wave_max(valid ? sc : -INFINITY));   // finite: the chunk holds a key <= i
-      const float a = __expf(m_run[h] - m_new), e = valid ? __expf(sc - m_new) : 0.f;
-      moved |= m_new != m_run[h];
-      m_run[h] = m_new;
-      l_run[h] = __builtin_fmaf(l_run[h], a, e);
-      pd_run[h] = __builtin_fmaf(pd_run[h], a, e * dpv[h]);
-      al = (vr / 2 == h && vr < 2 * G) ? a : al;
+      acc[h] = valid ? sc : -INFINITY;
+      exceeds |= acc[h] > m_run[h] + kLazyMargin;   // m_run starts at -inf: the first chunk always moves it
+    }
+    if (__builtin_amdgcn_ballot_w64(exceeds) != 0) {   // wave-uniform
+      float al = 1.f;          // this lane's virtual row's rescale factor
+#pragma unroll
+      for (int h = 0; h < G; ++h) {
+        const float m_new = fmaxf(m_run[h], wave_max(acc[h]));   // finite: the chunk holds a key <= i
+        const float a = __expf(m_run[h] - m_new);
+        m_run[h] = m_new;
+        l_run[h] *= a;
+        pd_run[h] *= a;
+        al = (vr / 2 == h && vr < 2 * G) ? a : al;
+      }
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) dqa[db][e] *= al;
+    }
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      const float e = __expf(acc[h] - m_run[h]);   // 0 for the keys beyond the diagonal
+      l_run[h] += e;
+      pd_run[h] = __builtin_fmaf(e, dpv[h], pd_run[h]);
       wts[(2 * h) * WS + lane] = f_to_f16(e * (dpv[h] - dref[h]));
       wts[(2 * h + 1) * WS + lane] = f_to_f16(e);
     }
     if (c > 0) {
 #pragma unroll
       for (int h = 0; h < G; ++h) dpv[h] = *byte_offset(dp_row[h], 4u * jn);
-    }
-    if (moved) {
-#pragma unroll
-      for (int db = 0; db < NDB; ++db)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) dqa[db][e] *= al;
     }
     lds_order();   // rotated keys and weights are in LDS
 #pragma unroll
