@@ -74,6 +74,27 @@ def test_corope_backward_hot_softmax(pkg):
     _compare(_gpu_grads(pkg, q, k, v, d_o, 1.0, 10000.0), _oracle_grads(q, k, v, d_o, 1.0, 10000.0), 2)
 
 
+@pytest.mark.parametrize("trend", ["growing", "shrinking"])
+def test_corope_score_trend_along_the_sweep(pkg, trend):
+    """The kernels sweep a row's keys from the diagonal towards key 0 and move the reference value of their exponentials
+    only when a score rises well above it.  Key norms that grow (resp. shrink) towards key 0 make the scores rise chunk
+    after chunk (the reference moves again and again) or fall away (it stays at the first chunk's maximum while the
+    weights become tiny): forward and all gradients against the oracle in both regimes."""
+    B, Hq, Hkv, N, D = 1, 4, 2, 320, 64
+    q, k, v, d_o = _inputs(B, Hq, Hkv, N, D, seed=33)
+    ramp = torch.linspace(3.0, 0.5, N) if trend == "growing" else torch.linspace(0.3, 2.0, N)
+    k = bf16_round(k * ramp[None, None, :, None])
+    d_o = bf16_round(d_o * 0.25)
+    scale = 1 / math.sqrt(D)
+    print(f"case trend={trend}", flush=True)
+    dev = torch.device("cuda:0")
+    o = pkg.corope_attention(*(t.to(dev, torch.bfloat16) for t in (q, k, v)), True, scale, 10000.0).float().cpu()
+    ro = C.corope_gqa_forward(q.double(), k.double(), v.double(), True, scale, 10000.0, torch.float64).float()
+    print(f"  O max-abs {(o - ro).abs().max():.3e}", flush=True)
+    assert torch.isfinite(o).all() and (o - ro).abs().max() <= TOL
+    _compare(_gpu_grads(pkg, q, k, v, d_o, scale, 10000.0), _oracle_grads(q, k, v, d_o, scale, 10000.0), Hq // Hkv)
+
+
 def test_corope_backward_gate_path_is_material_and_right(pkg):
     """On this input the gradient through the leader's gates is a large part of dQ and dK (the oracle with the
     position offsets cut out of the graph differs by far more than the bar), so parity here pins that path; a
