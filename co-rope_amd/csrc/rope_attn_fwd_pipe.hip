@@ -220,6 +220,8 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
     for (int i = 0; i < M; ++i) oacc[i % NDB] = mfma32(v_operand(vp_lane, 1, i), pb1[i / NDB], oacc[i % NDB]);
   };
 
+  // (the first 64 key-norm maxima have landed before the loop on every path, for the same reason as in the reload below)
+  asm volatile("" ::"v"(kvec));
   // ---- tiles this wave's rows can see ------------------------------------------------------------------------------
   for (int t = 0; t <= t_last; ++t) {
     const int n0 = t * BLOCK_N;
@@ -283,6 +285,9 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
     if (t - kvec_base == kWave) {
       kvec_base = t;
       kvec = tile_kmax_bits[min(t + lane, n_k_tiles - 1)];
+      // waited for here, once in 64 tiles: left to the first use below, the wait would sit on the common path too and
+      // there also wait for the next tile's loads, half a tile after they were issued instead of a whole one
+      asm volatile("" ::"v"(kvec));
     }
     const uint32_t kmax_bits = __builtin_amdgcn_readlane(kvec, t - kvec_base);
     if (t == 0 || kmax_bits > thr_bits) {
