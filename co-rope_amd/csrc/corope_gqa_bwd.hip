@@ -22,9 +22,9 @@
 // rotation is linear, so one vector is rotated per (i, j), not one per head.  Everything that is a dot product with an
 // already rotated or an unrotated row runs on the matrix cores.  Launches, in order:
 //   rowdot (x2)  leader logits qL K^T per group and dP = dO V^T per head, fp32 into the workspace (32x32x16 bf16 MFMA,
-//                operands straight from global memory)
+//                128 rows x 128 keys per workgroup, operands fetched with whole cache lines and parked in LDS)
 //   scores       one wave per (group, query row), lane = key:
-//                  right to left over 64-key chunks: z, delta by a scan, the rotated keys Kt -> LDS (bf16); on the matrix
+//                  right to left over 64-key chunks: z, delta by a scan, the rotated keys Kt -> LDS (fp16); on the matrix
 //                  cores S = q Kt^T and dS/ddelta = [-w q2, w q1] Kt^T for all heads at once, then - with running softmax
 //                  statistics, flash-attention style - the two sums that make dq: sum_j e_j dP_j kt_j and sum_j e_j kt_j;
 //                  left to right: P, dS, G and its running sum, W;
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_rowdot_kernel(const uint
 
 // ---------------------------------------------------------------------------------------------------- scores
 // One wave per (group, query row i), all G heads at once, lane = key.  Per 64-key chunk the lanes rotate their keys
-// (the only place sines and cosines are evaluated) and park them in LDS as bf16; everything that is a dot product with
+// (the only place sines and cosines are evaluated) and park them in LDS as fp16; everything that is a dot product with
 // the rotated key then runs on the matrix cores: the raw scores q^h . kt and their derivatives with respect to delta
 // (rows [-w q2, w q1] . kt) as one (2G x D) x (D x 64 keys) product, and the dq sums as (weights x keys) x (keys x D).
 template <int D, int G>
