@@ -248,8 +248,9 @@ def bench_corope(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    # defaults long enough for the clocks to settle: the first ~50 ms of sustained load run 3-10 % slower than what follows
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--config", default="c3", choices=sorted(CONFIGS) + ["c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sweep", action="store_true",
@@ -349,19 +350,23 @@ def main():
                 ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq(qp, kp, vp, dop, M.data_ptr(), delta.data_ptr(),
                                                                         cp, sp, fs, dq.data_ptr(), B, H, N, D, scale, 1, stream)),
             ]
+    # the launches of a step in step order, back to back over all iterations with no host synchronisation in between: the
+    # matrix pipes run at a power-limited clock, and a pause per iteration lets every kernel run 4-7 % faster than it
+    # does inside a training step
     durs = {n: [] for n, _ in launches}
-    for it in range(args.warmup + args.steps):
-        evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(launches) + 1)]
+    all_evs = [[torch.cuda.Event(enable_timing=True) for _ in range(len(launches) + 1)]
+               for _ in range(args.warmup + args.steps)]
+    for evs in all_evs:
         evs[0].record()
         for i, (name, fn) in enumerate(launches):
             rc = fn()
             if rc != 0:
                 sys.exit(f"{name} failed: {pkg._lib.last_error()}")
             evs[i + 1].record()
-        torch.cuda.synchronize()
-        if it >= args.warmup:
-            for i, (name, _) in enumerate(launches):
-                durs[name].append(evs[i].elapsed_time(evs[i + 1]))
+    torch.cuda.synchronize()
+    for evs in all_evs[args.warmup:]:
+        for i, (name, _) in enumerate(launches):
+            durs[name].append(evs[i].elapsed_time(evs[i + 1]))
     avg = {n: sum(d) / len(d) for n, d in durs.items()}
     # algorithmic FLOPs per launch (the reference's model: forward 2 matmul units, backward 5): fused dK+dV kernel 4 units
     # (the counted S recompute, dP, dV, dK) -- as two launches: dV 2 units, dK 2 units (its own S recompute is overhead on
