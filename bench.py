@@ -48,6 +48,24 @@ CONFIGS = {
 }
 
 
+SETTLE_SECONDS = 0.1
+
+
+def settle_clocks(step, torch):
+    """Untimed: keeps running `step` until SETTLE_SECONDS of sustained load have passed.  The first ~50 ms after an idle
+    period run at other clocks than what follows (the matrix kernels 3-10 % slower, the vector-bound ones a little faster),
+    so a short --warmup alone would time the transient.  Returns the number of extra steps."""
+    step()                       # first call: library load, kernel attributes, allocator growth
+    torch.cuda.synchronize()
+    n, t0 = 1, time.perf_counter()
+    while time.perf_counter() - t0 < SETTLE_SECONDS:
+        for _ in range(16):
+            step()
+        torch.cuda.synchronize()
+        n += 16
+    return n
+
+
 def attention_flops(B, H, N, D, mode, causal=True):
     total = 4.0 * B * H * N * N * D * (0.5 if causal else 1.0)
     return total * (2.5 if mode == "bwd" else 1.0)
@@ -176,6 +194,7 @@ def bench_corope(args):
         if rc != 0:
             sys.exit(pkg._lib.last_error())
 
+    settle_steps = settle_clocks(step, torch)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -228,6 +247,7 @@ def bench_corope(args):
     out = {"metric": "Co-RoPE GQA fwd, B2 Hq32 Hkv8 N4096 D128 causal", "value": round(flops / (ms * 1e-3) * 1e-12, 2),
            "unit": "TFLOP/s (attention-equivalent)", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "settle_steps": settle_steps,
            "dtype": "bf16", "data": "synthetic",
            "config": {"workload": "C5: Co-RoPE GQA attention fwd B2 Hq32 Hkv8 N4096 D128 causal bf16", "theta": 10000.0},
            "sincos_pairs_per_s": round(pairs / (kms * 1e-3), 1), "kernel_ms": round(kms, 4),
@@ -296,6 +316,7 @@ def main():
             q.grad = k.grad = v.grad = None
         return o
 
+    settle_steps = settle_clocks(step, torch)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -396,6 +417,7 @@ def main():
         "metric": "RoPE-attn fwd+bwd TFLOPS & % bf16 MFMA peak, B2 H32 N4096 D128 causal",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "settle_steps": settle_steps,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": cfg["name"], "B": B, "H": H, "N": N, "D": D, "causal": True,
                    "sm_scale": "1/sqrt(D)", "rope_base": 10000.0},
