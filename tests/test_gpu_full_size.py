@@ -93,6 +93,26 @@ def test_c5_corope_forward(pkg):
     assert torch.equal(o[:, :, 0], v.repeat_interleave(Hq // Hkv, 1)[:, :, 0])
 
 
+def test_corope_long_hot_rows(pkg):
+    """2048 keys at sm_scale = 0.5 (scores of +-15) with key norms rising towards key 0: over a row's 32 chunks the
+    reference value of the exponentials has to move again and again.  Sampled rows against the oracle; mean-abs bar as for
+    the other hot cases (bf16 inputs at this temperature), finite everywhere."""
+    B, Hq, Hkv, N, D = 1, 4, 2, 2048, 64
+    dev = torch.device("cuda:0")
+    q = bf16_round(seeded((B, Hq, N, D), 13))
+    k, v = bf16_round(seeded((B, Hkv, N, D), 14)), bf16_round(seeded((B, Hkv, N, D), 15))
+    k = bf16_round(k * torch.linspace(1.6, 0.6, N)[None, None, :, None])
+    o = pkg.corope_attention(q.to(dev, torch.bfloat16), k.to(dev, torch.bfloat16), v.to(dev, torch.bfloat16), True, 0.5, 10000.0)
+    torch.cuda.synchronize()
+    o = o.float().cpu()
+    rows = _rows(N, 12, 5)
+    ref = C.corope_gqa_forward_rows(q, k, v, True, 0.5, 10000.0, rows, torch.float32, row_block=16)
+    err = (o[:, :, rows] - ref).abs()
+    print(f"  long hot rows: O max-abs {err.max():.3e} mean-abs {err.mean():.3e}", flush=True)
+    assert torch.isfinite(o).all()
+    assert err.max() <= 0.15 and err.mean() <= 5e-3
+
+
 def test_c5_corope_backward(pkg):
     """B2 Hq32 Hkv8 N4096 D128 Co-RoPE backward: dQ of sampled rows against autograd through the row-sampled oracle
     (a query row's output depends on no other query row), and two size-independent identities for dK and dV:
