@@ -77,6 +77,10 @@ int corope_rope_attn_check(int B, int H, int N, int D, int64_t freq_row_stride, 
     return fail(COROPE_E_BADARG, "rope_attn: freq_row_stride %lld must be >= D/2 and a multiple of 4", (long long)freq_row_stride);
   if (!(sm_scale > 0.f) || !std::isfinite(sm_scale)) return fail(COROPE_E_BADARG, "rope_attn: sm_scale must be positive and finite");
   if ((int64_t)B * H * N * D >= ((int64_t)1 << 40)) return fail(COROPE_E_UNSUPPORTED, "rope_attn: tensor too large");
+  // one workgroup per (batch, head, 64-row tile) on a single grid axis in the rotation pass, fewer in the other kernels
+  if ((int64_t)B * H * ((N + 63) / 64) >= ((int64_t)1 << 31))
+    return fail(COROPE_E_UNSUPPORTED, "rope_attn: B * H * ceil(N / 64) = %lld workgroups exceed the grid",
+                (long long)B * H * ((N + 63) / 64));
   // staging loads address a (batch, head) slab and the tables with 32-bit byte offsets
   if ((int64_t)N * D * 2 >= ((int64_t)1 << 32) || (int64_t)N * freq_row_stride * 4 >= ((int64_t)1 << 32))
     return fail(COROPE_E_UNSUPPORTED, "rope_attn: one (batch, head) slab or a cos/sin table exceeds 4 GiB");

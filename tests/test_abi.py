@@ -53,6 +53,7 @@ def test_header_cites_reference_for_each_entry_point():
     ((1, 1, 1 << 24, 128, 64, 1.0, 0), -2),   # one (batch, head) slab of 4 GiB: past the 32-bit staging offsets
     ((1, 1, 1 << 22, 128, 256, 1.0, 0), -2),  # cos/sin table of 4 GiB
     ((1, 1, 1 << 22, 128, 64, 1.0, 0), 0),
+    ((1 << 16, 1 << 15, 1, 64, 32, 1.0, 0), -2),    # 2^31 (batch, head) slabs of one row: more workgroups than a grid axis takes
 ])
 def test_rope_attn_check_codes(pkg, args, code):
     lib = pkg._lib.load()
