@@ -22,8 +22,9 @@
 // Mapping: one wave (= one workgroup) per (batch, kv head, query row), longest rows first; lane = key inside a 64-key
 // chunk.  Per chunk: the contiguous 64 x D block of K is fetched with whole cache lines per instruction and parked in
 // the LDS tile -> logits (MFMA, results moved back to lane = key with v_permlane32_swap) -> gate, scan over the lanes,
-// delta -> each lane rotates its own key row in place -> scores (MFMA) -> online softmax with a wave-uniform running
-// maximum -> the block of V replaces the rotated keys in the tile -> O accumulation (MFMA).  A wave's LDS instructions
+// delta -> each lane rotates its own key row in place -> scores (MFMA) -> online softmax against a wave-uniform
+// reference value per head (moved to the running maximum only when a score rises well above it) -> the block of V
+// replaces the rotated keys in the tile -> O accumulation (MFMA).  A wave's LDS instructions
 // execute in order, so the kernel needs no barriers; global loads for the next step are issued one step ahead.
 #include "common.hpp"
 #include "kernels.hpp"
