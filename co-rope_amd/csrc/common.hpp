@@ -274,32 +274,167 @@ __device__ __forceinline__ void load_b_rows(u32x4 (&out)[D / 16], const uint16_t
   }
 }
 
-// Epilogue for gradients held as a transposed accumulator (lane = row of the output matrix, registers =
-// columns): undoes the rotation, d1 = d1r c + d2r s, d2 = d2r c - d1r s, scales, rounds and stores.
-// acc[db][i] holds column db*32 + 8*(i/4) + 4*h + (i%4) of the lane's row.
+// A wave's LDS instructions execute in program order, so LDS bytes that only this wave touches can be written and read
+// back by it without a barrier or a wait; all that is needed is that the compiler keeps the accesses in program order.
+// (A workgroup barrier would also wait for the global loads issued ahead of time.)
+__device__ __forceinline__ void lds_order() { asm volatile("" ::: "memory"); }
+
+// ---- a wave's 32 rows through LDS: coalesced global accesses on one side, lane = row on the other ---------------------
+// The MFMA layouts make a lane own a row (a query or a key), so loading B operands or storing transposed accumulators
+// straight from / to global memory touches 32 different rows per instruction, 16 or 32 bytes of each.  These helpers go
+// through a wave-private LDS tile instead: global memory sees whole 128- or 256-byte row segments per instruction.  A wave's
+// LDS instructions execute in program order, so no barrier is needed between the two halves of a helper; the caller only
+// has to make sure that no other wave uses the same LDS bytes at the same time.
+
+// B operand chunks (as load_b_rows) of rows row0 .. row0 + 31 of a (n_rows, D) bf16 matrix, rows clamped to n_rows - 1,
+// in two steps so that a kernel can issue all its prologue loads before it waits for any of them: load() starts the
+// global loads, park() writes the rows (ROTATE: after the half-layout rotation, fp32, one rounding) into the wave's LDS
+// tile and reads them back as B operands; rot_out (may be null) receives the rotated rows that lie inside the matrix.
+// wave_tile: 32 * RowTile<D>::kStride elements of LDS.
+template <int D, bool ROTATE>
+struct WaveRows;
+
 template <int D>
-__device__ __forceinline__ void store_unrotated(const f32x16 (&acc)[D / 32], uint16_t* __restrict__ dst_row,
-                                                const float* __restrict__ cos_row, const float* __restrict__ sin_row,
-                                                float scale) {
-  constexpr int NDB = D / 32;
-  const int lh = (threadIdx.x % kWave) / 32;
+struct WaveRows<D, false> {
+  static constexpr int CPR = D / 8;            // 16-byte chunks per row
+  static constexpr int RPI = kWave / CPR;      // rows per load instruction
+  static constexpr int IT = 32 / RPI;
+  u32x4 x[IT];
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float*, const float*, int64_t, int row0,
+                                       int n_rows) {
+    const int l = threadIdx.x % kWave;
 #pragma unroll
-  for (int db = 0; db < NDB / 2; ++db)
+    for (int i = 0; i < IT; ++i)
+      x[i] = *reinterpret_cast<const u32x4*>(
+          byte_offset(src, (uint32_t)min(row0 + RPI * i + l / CPR, n_rows - 1) * (D * 2) + (l % CPR) * 16));
+  }
+  __device__ __forceinline__ void park(u32x4 (&out)[D / 16], uint16_t* wave_tile, uint16_t* = nullptr, int = 0, int = 0) {
+    const int l = threadIdx.x % kWave;
+    lds_order();
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int col = db * 32 + 8 * g + 4 * lh;
-      f32x4 c = *reinterpret_cast<const f32x4*>(cos_row + col);
-      f32x4 s = *reinterpret_cast<const f32x4*>(sin_row + col);
-      float o1[4], o2[4];
+    for (int i = 0; i < IT; ++i)
+      *reinterpret_cast<u32x4*>(wave_tile + RowTile<D>::off(RPI * i + l / CPR, (l % CPR) * 8)) = x[i];
+    lds_order();
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float r1 = acc[db][4 * g + e] * scale, r2 = acc[db + NDB / 2][4 * g + e] * scale;
-        o1[e] = r1 * c[e] + r2 * s[e];
-        o2[e] = r2 * c[e] - r1 * s[e];
-      }
-      *reinterpret_cast<u32x2*>(dst_row + col) = u32x2{pack_bf16(o1[0], o1[1]), pack_bf16(o1[2], o1[3])};
-      *reinterpret_cast<u32x2*>(dst_row + D / 2 + col) = u32x2{pack_bf16(o2[0], o2[1]), pack_bf16(o2[2], o2[3])};
+    for (int kc = 0; kc < D / 16; ++kc)
+      out[kc] = *reinterpret_cast<const u32x4*>(wave_tile + RowTile<D>::off(l % 32, 16 * kc + 8 * (l / 32)));
+    lds_order();
+  }
+};
+
+template <int D>
+struct WaveRows<D, true> {
+  static constexpr int UPR = D / 16;           // units (8 rotation pairs) per row
+  static constexpr int RPI = kWave / UPR;
+  static constexpr int IT = 32 / RPI;
+  u32x4 x1[IT], x2[IT];
+  f32x4 c[IT][2], s[IT][2];
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float* __restrict__ cosp,
+                                       const float* __restrict__ sinp, int64_t fstride, int row0, int n_rows) {
+    const int l = threadIdx.x % kWave;
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+      const int row = min(row0 + RPI * i + l / UPR, n_rows - 1), u = l % UPR;
+      const uint16_t* xp = byte_offset(src, (uint32_t)row * (D * 2) + u * 16);
+      x1[i] = *reinterpret_cast<const u32x4*>(xp);
+      x2[i] = *reinterpret_cast<const u32x4*>(xp + D / 2);
+      const uint32_t foff = ((uint32_t)row * (uint32_t)fstride + u * 8) * 4;
+      const float* cp = byte_offset(cosp, foff);
+      const float* sp = byte_offset(sinp, foff);
+      c[i][0] = *reinterpret_cast<const f32x4*>(cp);
+      c[i][1] = *reinterpret_cast<const f32x4*>(cp + 4);
+      s[i][0] = *reinterpret_cast<const f32x4*>(sp);
+      s[i][1] = *reinterpret_cast<const f32x4*>(sp + 4);
     }
+  }
+  __device__ __forceinline__ void park(u32x4 (&out)[D / 16], uint16_t* wave_tile, uint16_t* __restrict__ rot_out = nullptr,
+                                       int row0 = 0, int n_rows = 0) {
+    const int l = threadIdx.x % kWave;
+    lds_order();
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+      const int r = RPI * i + l / UPR, u = l % UPR;
+      u32x4 y1, y2;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        float a0 = bf16_lo(x1[i][w]), a1 = bf16_hi(x1[i][w]), b0 = bf16_lo(x2[i][w]), b1 = bf16_hi(x2[i][w]);
+        float c0 = c[i][w / 2][(2 * w) % 4], c1 = c[i][w / 2][(2 * w) % 4 + 1];
+        float s0 = s[i][w / 2][(2 * w) % 4], s1 = s[i][w / 2][(2 * w) % 4 + 1];
+        y1[w] = pack_bf16(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+        y2[w] = pack_bf16(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+      }
+      *reinterpret_cast<u32x4*>(wave_tile + RowTile<D>::off(r, u * 8)) = y1;
+      *reinterpret_cast<u32x4*>(wave_tile + RowTile<D>::off(r, D / 2 + u * 8)) = y2;
+      if (rot_out != nullptr && row0 + r < n_rows) {
+        uint16_t* dst = byte_offset(rot_out, (uint32_t)(row0 + r) * (D * 2) + u * 16);
+        *reinterpret_cast<u32x4*>(dst) = y1;
+        *reinterpret_cast<u32x4*>(dst + D / 2) = y2;
+      }
+    }
+    lds_order();
+#pragma unroll
+    for (int kc = 0; kc < D / 16; ++kc)
+      out[kc] = *reinterpret_cast<const u32x4*>(wave_tile + RowTile<D>::off(l % 32, 16 * kc + 8 * (l / 32)));
+    lds_order();
+  }
+};
+
+// Rows row0 .. row0 + 31 of a (n_rows, D) bf16 matrix from transposed fp32 accumulators (lane = row l % 32, acc[db][i] =
+// column db*32 + 8*(i/4) + 4*(l/32) + i%4): every value is multiplied by `scale` (which may
+// differ from lane to lane, i.e. from row to row), UNROTATE undoes the half-layout rotation in fp32 (d1 = d1r c + d2r s,
+// d2 = d2r c - d1r s), one rounding to bf16, 16-byte stores that cover whole 128-byte row segments.
+// wave_tile: 32 * kAccTileStride<D> floats of LDS.
+template <int D>
+constexpr int kAccTileStride = D + 4;
+template <int D, bool UNROTATE>
+__device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], uint16_t* __restrict__ dst, int row0,
+                                                   int n_rows, const float* __restrict__ cosp,
+                                                   const float* __restrict__ sinp, int64_t fstride, float scale,
+                                                   float* wave_tile) {
+  constexpr int LS = kAccTileStride<D>;
+  const int l = threadIdx.x % kWave, lq = l % 32, lh = l / 32;
+  lds_order();
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      *reinterpret_cast<f32x4*>(wave_tile + lq * LS + db * 32 + 8 * g + 4 * lh) =
+          f32x4{acc[db][4 * g] * scale, acc[db][4 * g + 1] * scale, acc[db][4 * g + 2] * scale, acc[db][4 * g + 3] * scale};
+  lds_order();
+  constexpr int UPR = D / 16, RPI = kWave / UPR;
+#pragma unroll
+  for (int i = 0; i < 32 / RPI; ++i) {
+    const int r = RPI * i + l / UPR, u = l % UPR, row = row0 + r;
+    const float* t = wave_tile + r * LS + u * 8;
+    f32x4 a[2] = {*reinterpret_cast<const f32x4*>(t), *reinterpret_cast<const f32x4*>(t + 4)};
+    f32x4 b[2] = {*reinterpret_cast<const f32x4*>(t + D / 2), *reinterpret_cast<const f32x4*>(t + D / 2 + 4)};
+    if (row < n_rows) {
+      float o1[8], o2[8];
+      if constexpr (UNROTATE) {
+        const uint32_t foff = ((uint32_t)row * (uint32_t)fstride + u * 8) * 4;
+        const float* cp = byte_offset(cosp, foff);
+        const float* sp = byte_offset(sinp, foff);
+        f32x4 c[2] = {*reinterpret_cast<const f32x4*>(cp), *reinterpret_cast<const f32x4*>(cp + 4)};
+        f32x4 s[2] = {*reinterpret_cast<const f32x4*>(sp), *reinterpret_cast<const f32x4*>(sp + 4)};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float r1 = a[e / 4][e % 4], r2 = b[e / 4][e % 4], ce = c[e / 4][e % 4], se = s[e / 4][e % 4];
+          o1[e] = r1 * ce + r2 * se;
+          o2[e] = r2 * ce - r1 * se;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          o1[e] = a[e / 4][e % 4];
+          o2[e] = b[e / 4][e % 4];
+        }
+      }
+      uint16_t* d = byte_offset(dst, (uint32_t)row * (D * 2) + u * 16);
+      *reinterpret_cast<u32x4*>(d) = u32x4{pack_bf16(o1[0], o1[1]), pack_bf16(o1[2], o1[3]), pack_bf16(o1[4], o1[5]), pack_bf16(o1[6], o1[7])};
+      *reinterpret_cast<u32x4*>(d + D / 2) = u32x4{pack_bf16(o2[0], o2[1]), pack_bf16(o2[2], o2[3]), pack_bf16(o2[4], o2[5]), pack_bf16(o2[6], o2[7])};
+    }
+  }
+  lds_order();
 }
 
 // Natural-order variant of load_a_trans: slot j of lane-half h <-> k = kbase + 8*h + j.
@@ -353,11 +488,6 @@ __device__ __forceinline__ float wave_max(float x) {
 __device__ __forceinline__ float bf16_to_f(uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
 __device__ __forceinline__ uint16_t f_to_bf16(float x) { return (uint16_t)(pack_bf16(x, 0.f) & 0xffffu); }
 __device__ __forceinline__ uint16_t f_to_f16(float x) { return (uint16_t)(pack_f16(x, 0.f) & 0xffffu); }
-
-// For kernels that run one wave per workgroup: a wave's LDS instructions execute in program order, so LDS written by
-// the wave can be read back by it without a barrier or a wait; all that is needed is that the compiler keeps the
-// accesses in program order.  (A workgroup barrier would also wait for the global loads issued ahead of time.)
-__device__ __forceinline__ void lds_order() { asm volatile("" ::: "memory"); }
 
 // f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
 // in the body, so register arrays indexed with it never look dynamically indexed to the optimiser.

@@ -22,7 +22,29 @@ inline hipError_t allow_dynamic_lds(const void* kernel, int bytes, std::atomic<u
 }
 
 
+#ifdef COROPE_TRACE
+// Experiment builds only: per-workgroup time stamps (100 MHz counter) for splitting a launch into its phases.
+extern uint64_t* g_trace_buf;
+#define COROPE_TRACE_FIELD uint64_t* trace;
+#define COROPE_STAMP(slot, tid)                                                                              \
+  do {                                                                                                       \
+    if (p.trace != nullptr && threadIdx.x == (tid)) p.trace[(int64_t)blockIdx.x * 16 + (slot)] = __builtin_amdgcn_s_memrealtime(); \
+  } while (0)
+#define COROPE_STAMP_ID(tid, extra)                                                                          \
+  do {                                                                                                       \
+    if (p.trace != nullptr && threadIdx.x == (tid)) {                                                        \
+      p.trace[(int64_t)blockIdx.x * 16 + 14] = (uint64_t)__builtin_amdgcn_s_getreg(63492) | ((uint64_t)__builtin_amdgcn_s_getreg(63508) << 32); \
+      p.trace[(int64_t)blockIdx.x * 16 + 15] = (uint64_t)(extra);                                              \
+    }                                                                                                        \
+  } while (0)
+#else
+#define COROPE_TRACE_FIELD
+#define COROPE_STAMP(slot, tid) do {} while (0)
+#define COROPE_STAMP_ID(tid, extra) do {} while (0)
+#endif
+
 struct FwdParams {
+  COROPE_TRACE_FIELD
   const uint16_t* q;
   const uint16_t* k;
   const uint16_t* v;
@@ -43,6 +65,7 @@ struct FwdParams {
 };
 
 struct BwdParams {
+  COROPE_TRACE_FIELD
   const uint16_t* q;
   const uint16_t* k;
   const uint16_t* v;

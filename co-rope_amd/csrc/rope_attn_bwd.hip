@@ -39,12 +39,16 @@ struct DkdvCfg {
   static constexpr int kStatBytes = BLOCK_M * 4;
   static constexpr int kStageBytes = kTileBytes + kDoTileBytes + 2 * kStatBytes;
   static constexpr int kVRowsBytes = V_LDS ? RowTile<D>::bytes(kBlockN) : 0;
-  static constexpr int kLdsBytes = 2 * kStageBytes + kVRowsBytes;
+  static constexpr int kLoopBytes = 2 * kStageBytes + kVRowsBytes;
+  static constexpr int kEpilogueBytes = NWAVES * 32 * kAccTileStride<D> * 4;   // fp32 rows of all waves on their way out
+  static constexpr int kLdsBytes = kLoopBytes > kEpilogueBytes ? kLoopBytes : kEpilogueBytes;
+  // the prologue parks each wave's 32 operand rows in the two tile stages, next to (not on) the V rows
+  static_assert(NWAVES * RowTile<D>::bytes(32) <= 2 * kStageBytes, "prologue tiles do not fit the tile stages");
 };
 
 // PREROT: Q and K come from copies that rope_rotate_kernel rotated beforehand (no table reads in the loop).
 template <int D, int NWAVES, int BLOCK_M, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
-__global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
+__global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
   constexpr int DO_PAD = DO_DK ? 8 : 32;
   constexpr bool V_LDS = DO_DV && DO_DK;
   using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_PAD, V_LDS>;
@@ -55,6 +59,7 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
 
   // The workgroup owns a key block of one key/value slab and sweeps the query tiles of every query head of its group
   // (one head without grouped-query attention), accumulating dK and dV over all of them.
+  COROPE_STAMP(0, 0);
   const int BHkv = p.BH / p.H * p.Hkv, GQ = p.H / p.Hkv;
   const int bkv = blockIdx.x % BHkv;
   const int nb = blockIdx.x / BHkv;  // key block; for causal the low blocks are the heavy ones and start first
@@ -67,18 +72,19 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
   const uint16_t* q_all = PREROT ? p.q_rot : p.q;
 
   const int key = n0 + wave * 32 + lq;
-  const int key_c = min(key, N - 1);
   const int wk_lo = n0 + wave * 32, wk_hi = wk_lo + 31;
 
+  // The wave's K_r (and V) rows as B operands, through a wave-private LDS tile (whole row segments per global load).
+  // Every load of the prologue is issued before the first of them is waited for.
   u32x4 kb[KC], vb[(DO_DK && !V_LDS) ? KC : 1];
-  load_b_rows<D, !PREROT>(kb, (PREROT ? p.k_rot : p.k) + base, p.cos, p.sin, p.fstride, key_c);
-  if constexpr (DO_DK && !V_LDS) load_b_rows<D, false>(vb, p.v + base, nullptr, nullptr, 0, key_c);
+  uint16_t* wave_rows = reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride;
   uint16_t* vrows = reinterpret_cast<uint16_t*>(smem + 2 * Cfg::kStageBytes);   // V_LDS: the block's V rows, row-major
-  if constexpr (V_LDS) {
-    CopyStage<D, Cfg::kBlockN, NT> vcp;
-    vcp.load(p.v + base, n0, N);
-    vcp.store_rows(vrows);    // visible after the barrier that ends the prologue
-  }
+  WaveRows<D, !PREROT> krows;
+  krows.load((PREROT ? p.k_rot : p.k) + base, p.cos, p.sin, p.fstride, wk_lo, N);
+  WaveRows<D, false> vrows_regs;
+  if constexpr (DO_DK && !V_LDS) vrows_regs.load(p.v + base, nullptr, nullptr, 0, wk_lo, N);
+  CopyStage<D, Cfg::kBlockN, NT> vcp;
+  if constexpr (V_LDS) vcp.load(p.v + base, n0, N);
 
   RopeStage<D, BLOCK_M, NT, PREROT> qst;
   CopyStage<D, BLOCK_M, NT, DO_PAD> dst;
@@ -123,10 +129,12 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
     if constexpr (DO_DK) dkacc[i] = f32x16{0};
   }
 
-  if (n_iter > 0) {
-    load_tile(0);
-    store_tile(0);
-  }
+  if (n_iter > 0) load_tile(0);
+  krows.park(kb, wave_rows);
+  if constexpr (DO_DK && !V_LDS) vrows_regs.park(vb, wave_rows);
+  if constexpr (V_LDS) vcp.store_rows(vrows);    // visible after the barrier that ends the prologue
+  __syncthreads();   // the tile stages overlap the tiles the waves parked their rows in
+  if (n_iter > 0) store_tile(0);
   // The wave's K_r (and V) rows must have landed on EVERY path into the loop: left to the first product that reads them,
   // the wait for them is placed inside the loop, where each time round it also waits for the next tile's loads issued
   // a few instructions earlier, and the prefetch hides less.
@@ -136,10 +144,16 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
     if constexpr (DO_DK && !V_LDS) asm volatile("" ::"v"(vb[kc]));
   }
   __syncthreads();
+  COROPE_STAMP(1, 0);
+  COROPE_STAMP_ID(0, n_iter);
 
   const float scale2 = p.qk_scale;
   for (int it = 0; it < n_iter; ++it) {
     const int m0 = tile_m0(it);
+#ifdef COROPE_TRACE
+    if (it == 1) COROPE_STAMP(3, 0);
+    if (it == Cfg::kBlockN / BLOCK_M) COROPE_STAMP(4, 0);   // first tile past the diagonal block
+#endif
     const int cur = it & 1;
     if (it + 1 < n_iter) load_tile(it + 1);
 
@@ -211,22 +225,16 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dkdv_kernel(BwdPa
     __syncthreads();
   }
 
-  if (key < N) {
-    if constexpr (DO_DV) {
-      uint16_t* dvp = p.dv + base + (int64_t)key * D;
-#pragma unroll
-      for (int db = 0; db < NDB; ++db)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          u32x2 w = {pack_bf16(dvacc[db][4 * g], dvacc[db][4 * g + 1]),
-                     pack_bf16(dvacc[db][4 * g + 2], dvacc[db][4 * g + 3])};
-          *reinterpret_cast<u32x2*>(dvp + db * 32 + 8 * g + 4 * lh) = w;
-        }
-    }
-    if constexpr (DO_DK)
-      store_unrotated<D>(dkacc, p.dk + base + (int64_t)key * D, p.cos + (int64_t)key * p.fstride,
-                         p.sin + (int64_t)key * p.fstride, p.sm_scale);
-  }
+  COROPE_STAMP(5, 0);
+  // every wave is past its last read of the tiles (the loop ends with a barrier): their LDS now carries the accumulators
+  // to a row-major order, so that dV and dK leave in whole row segments and the tables are read the same way
+  float* wave_out = reinterpret_cast<float*>(smem) + wave * 32 * kAccTileStride<D>;
+  if constexpr (DO_DV) store_rows_via_lds<D, false>(dvacc, p.dv + base, wk_lo, N, nullptr, nullptr, 0, 1.f, wave_out);
+  if constexpr (DO_DK) store_rows_via_lds<D, true>(dkacc, p.dk + base, wk_lo, N, p.cos, p.sin, p.fstride, p.sm_scale, wave_out);
+#ifdef COROPE_TRACE
+  __builtin_amdgcn_s_waitcnt(0);
+  COROPE_STAMP(6, 0);
+#endif
 }
 
 // ===================================================================================== dQ
@@ -242,17 +250,24 @@ struct DqCfg {
   static constexpr int kBlockM = NWAVES * 32;
   static constexpr int kTileBytes = RowTile<D>::bytes(BLOCK_N);
   static constexpr int kStageBytes = 2 * kTileBytes;
-  static constexpr int kLdsBytes = 2 * kStageBytes;
+  static constexpr int kLoopBytes = 2 * kStageBytes;
+  static constexpr int kEpilogueBytes = NWAVES * 32 * kAccTileStride<D> * 4;   // fp32 dQ rows of all waves on their way out
+  // prologue: each wave's 32 operand rows (bf16) and their 32 delta values
+  static constexpr int kPrologueBytes = NWAVES * (RowTile<D>::bytes(32) + 32 * 4);
+  static constexpr int kLdsBytes = kLoopBytes > kEpilogueBytes ? (kLoopBytes > kPrologueBytes ? kLoopBytes : kPrologueBytes)
+                                                               : (kEpilogueBytes > kPrologueBytes ? kEpilogueBytes : kPrologueBytes);
 };
 
 template <int D, int NWAVES, int BLOCK_N, bool CAUSAL, bool PREROT>
-__global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_bwd_dq_kernel(BwdParams p) {
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
   constexpr int NT = Cfg::kThreads;
   constexpr int KC = D / 16, NDB = D / 32, NKB = BLOCK_N / 32;
   constexpr int LS = RowTile<D>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
+  [[maybe_unused]] constexpr int TT = NT - kWave;   // stamping thread: first lane of the last wave (it sees every tile)
+  COROPE_STAMP(0, TT);
   const int bh = blockIdx.x % p.BH;
   const int mb = p.num_blocks - 1 - blockIdx.x / p.BH;  // heaviest (last) query blocks first
   const int m0 = mb * Cfg::kBlockM;
@@ -276,27 +291,42 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdPara
   kst.load(kg, p.cos, p.sin, p.fstride, 0, N);
   vst.load(vg, 0, N);
 
+  // Q_r and dO rows of the wave as B operands, through a wave-private LDS tile (whole row segments per global load).
+  // Every load of the prologue is issued before the first of them is waited for.
   u32x4 qb[KC], dob[KC];
-  load_b_rows<D, !PREROT>(qb, (PREROT ? p.q_rot : p.q) + base, p.cos, p.sin, p.fstride, q_c);
-  load_b_rows<D, false>(dob, p.d_o + base, nullptr, nullptr, 0, q_c);
+  uint16_t* wave_rows = reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride;
+  WaveRows<D, !PREROT> qrows;
+  WaveRows<D, false> dorows, orows;
+  qrows.load((PREROT ? p.q_rot : p.q) + base, p.cos, p.sin, p.fstride, wq_lo, N);
+  dorows.load(p.d_o + base, nullptr, nullptr, 0, wq_lo, N);
+  if (p.o != nullptr) orows.load(p.o + base, nullptr, nullptr, 0, wq_lo, N);
   const float lse_q = p.lse[(int64_t)bh * N + q_c];
   // delta_i = sum_d o_id * do_id (reference _attn_bwd_preprocess, :324-337): read from the preprocess pass, or -- when the
   // caller hands over O instead -- computed here for the rows this workgroup owns and written out for the dK kernel,
   // which then has to run after this one.
-  float delta_q;
+  float delta_q = 0.f;
+  if (p.o == nullptr) delta_q = p.delta[(int64_t)bh * N + q_c];
+  qrows.park(qb, wave_rows);
+  dorows.park(dob, wave_rows);
   if (p.o != nullptr) {
-    u32x4 ob[KC];
-    load_b_rows<D, false>(ob, p.o + base, nullptr, nullptr, 0, q_c);
-    float acc = 0.f;
+    // 16 lanes per row: O in registers (same chunk order as dO went into the tile), dO from the tile
+    constexpr int CPR = D / 8, RPI = kWave / CPR;
+    float* wave_delta = reinterpret_cast<float*>(smem + NWAVES * RowTile<D>::bytes(32)) + wave * 32;
 #pragma unroll
-    for (int kc = 0; kc < KC; ++kc)
+    for (int i = 0; i < 32 / RPI; ++i) {
+      const int r = RPI * i + lane / CPR, ch = lane % CPR;
+      const u32x4 ow = orows.x[i], dw = dorows.x[i];
+      float acc = 0.f;
 #pragma unroll
-      for (int w = 0; w < 4; ++w)
-        acc += bf16_lo(ob[kc][w]) * bf16_lo(dob[kc][w]) + bf16_hi(ob[kc][w]) * bf16_hi(dob[kc][w]);
-    delta_q = half_sum(acc);
+      for (int w = 0; w < 4; ++w) acc += bf16_lo(ow[w]) * bf16_lo(dw[w]) + bf16_hi(ow[w]) * bf16_hi(dw[w]);
+#pragma unroll
+      for (int m = CPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m);
+      if (ch == 0) wave_delta[r] = acc;
+    }
+    lds_order();
+    delta_q = wave_delta[lq];
+    lds_order();
     if (lh == 0 && q_row < N) p.delta[(int64_t)bh * N + q_row] = delta_q;
-  } else {
-    delta_q = p.delta[(int64_t)bh * N + q_c];
   }
 
   auto k_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
@@ -306,13 +336,20 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdPara
 #pragma unroll
   for (int i = 0; i < NDB; ++i) dqacc[i] = f32x16{0};
 
+  __syncthreads();   // the tile stages overlap the tiles the waves parked their rows in
   kst.store_rows(k_tile(0));
   vst.store_rows(v_tile(0));
   __syncthreads();
+  COROPE_STAMP(1, TT);
+  COROPE_STAMP_ID(TT, n_tiles);
 
   const float scale2 = p.qk_scale;
   for (int t = 0; t < n_tiles; ++t) {
     const int n0 = t * BLOCK_N;
+#ifdef COROPE_TRACE
+    if (t == 1) COROPE_STAMP(3, TT);
+    if (n0 == m0) COROPE_STAMP(4, TT);
+#endif
     const int cur = t & 1;
     if (t + 1 < n_tiles) {
       kst.load(kg, p.cos, p.sin, p.fstride, n0 + BLOCK_N, N);
@@ -368,14 +405,20 @@ __global__ __launch_bounds__(NWAVES* kWave) void rope_attn_bwd_dq_kernel(BwdPara
     __syncthreads();
   }
 
-  if (q_row < N)
-    store_unrotated<D>(dqacc, p.dq + base + (int64_t)q_row * D, p.cos + (int64_t)q_row * p.fstride,
-                       p.sin + (int64_t)q_row * p.fstride, p.sm_scale);
+  COROPE_STAMP(5, TT);
+  // every wave is past its last read of the tiles (the loop ends with a barrier): their LDS now carries dQ_r to a
+  // row-major order, so that the tables are read and dQ is written in whole row segments
+  store_rows_via_lds<D, true>(dqacc, p.dq + base, wq_lo, N, p.cos, p.sin, p.fstride, p.sm_scale,
+                              reinterpret_cast<float*>(smem) + wave * 32 * kAccTileStride<D>);
+#ifdef COROPE_TRACE
+  __builtin_amdgcn_s_waitcnt(0);
+  COROPE_STAMP(6, TT);
+#endif
 }
 
 // ===================================================================================== launchers
-// dK and dV are produced by two launches of the same kernel template: with both sets of accumulators resident a
-// wave needs more than 256 registers, which would halve the waves per SIMD.
+// The fused dK+dV kernel sits at 246 of the 256 registers that two waves per SIMD leave each of them; dV alone is
+// small enough for a 128-row tile on pre-rotated operands.
 template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
 static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
   constexpr int NWAVES = 8, BLOCK_M = (PREROT && !DO_DK) ? 128 : 64;   // the larger tile pays off (and fits) for dV on pre-rotated operands only
@@ -384,6 +427,9 @@ static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
   static std::atomic<uint64_t> lds_ok{0};
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
   p.num_blocks = (p.N + Cfg::kBlockN - 1) / Cfg::kBlockN;
+#ifdef COROPE_TRACE
+  p.trace = g_trace_buf;
+#endif
   hipLaunchKernelGGL(kern, dim3(p.num_blocks * (p.BH / p.H * p.Hkv)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
 }
@@ -396,6 +442,9 @@ static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
   static std::atomic<uint64_t> lds_ok{0};
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
   p.num_blocks = (p.N + Cfg::kBlockM - 1) / Cfg::kBlockM;
+#ifdef COROPE_TRACE
+  p.trace = g_trace_buf;
+#endif
   hipLaunchKernelGGL(kern, dim3(p.num_blocks * p.BH), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
 }

@@ -43,7 +43,9 @@ struct FwdCfg {
   static constexpr int kKBytes = RowTile<D>::bytes(BLOCK_N);             // K tile, row-major, read row-wise
   static constexpr int kVBytes = RowTile<D, kVPad>::bytes(BLOCK_N);      // V tile, row-major, read transposed
   static constexpr int kStageBytes = kKBytes + kVBytes;
-  static constexpr int kLdsBytes = kFwdStages * kStageBytes;
+  static constexpr int kLoopBytes = kFwdStages * kStageBytes;
+  static constexpr int kEpilogueBytes = kFwdWaves * 32 * kAccTileStride<D> * 4;   // fp32 O rows of all waves on their way out
+  static constexpr int kLdsBytes = kLoopBytes > kEpilogueBytes ? kLoopBytes : kEpilogueBytes;
 };
 
 // ---- online softmax with a lazily updated reference maximum -------------------------------------------------------
@@ -134,10 +136,16 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
   kst.load(kg, p.cos, p.sin, p.fstride, 0, N);
   vst.load(vg, 0, N);
 
-  // ---- Q rows of this wave: load, rotate, keep as the B operand ------------------------------------------
+  // ---- Q rows of this wave: load, rotate, keep as the B operand (through a wave-private LDS tile, so that the
+  // global loads touch whole row segments) ---------------------------------------------------------------------
   const int q_row = m0 + wave * 32 + lq;           // absolute query index of this lane
   u32x4 qb[KC];
-  load_b_rows<D, true>(qb, qg, p.cos, p.sin, p.fstride, min(q_row, N - 1));
+  {
+    WaveRows<D, true> qrows;
+    qrows.load(qg, p.cos, p.sin, p.fstride, m0 + wave * 32, N);
+    qrows.park(qb, reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride);
+  }
+  __syncthreads();   // the K and V buffers below overlap the tiles the waves just used
 
   const float scale = p.qk_scale;
   f32x16 oacc[NDB];
@@ -267,22 +275,13 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
     __syncthreads();
   }
 
-  // ---- epilogue: normalise, write O and the base-2 log-sum-exp ----------------------------------------------
+  // ---- epilogue: normalise, write O (through LDS, whole row segments per store) and the base-2 log-sum-exp ------------
+  // (the loop ends with a barrier: every wave is done with the K and V buffers)
   const float l_tot = half_sum(l_run);
   const float inv_l = 1.f / l_tot;
-  if (q_row < N) {
-    uint16_t* op = p.o + ((int64_t)bh * N + q_row) * D;
-#pragma unroll
-    for (int db = 0; db < NDB; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = pack_bf16(oacc[db][4 * g] * inv_l, oacc[db][4 * g + 1] * inv_l);
-        w[1] = pack_bf16(oacc[db][4 * g + 2] * inv_l, oacc[db][4 * g + 3] * inv_l);
-        *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g + 4 * lh) = w;
-      }
-    if (lh == 0) p.lse[(int64_t)bh * N + q_row] = m_run * scale + fast_log2(l_tot);
-  }
+  store_rows_via_lds<D, false>(oacc, p.o + (int64_t)bh * N * D, m0 + wave * 32, N, nullptr, nullptr, 0, inv_l,
+                               reinterpret_cast<float*>(smem) + wave * 32 * kAccTileStride<D>);
+  if (q_row < N && lh == 0) p.lse[(int64_t)bh * N + q_row] = m_run * scale + fast_log2(l_tot);
 }
 
 // ---- host-side launch -----------------------------------------------------------------------------------------

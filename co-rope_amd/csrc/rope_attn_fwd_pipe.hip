@@ -53,7 +53,9 @@ struct FwdPipeCfg {
   static constexpr int kKBytes = RowTile<D>::bytes(kPipeBlockN);          // K tile, row-major, read row-wise
   static constexpr int kVBytes = RowTile<D, kVPad>::bytes(kPipeBlockN);   // V tile, row-major, read transposed
   static constexpr int kKStages = 2, kVStages = 3;
-  static constexpr int kLdsBytes = kKStages * kKBytes + kVStages * kVBytes;
+  static constexpr int kLoopBytes = kKStages * kKBytes + kVStages * kVBytes;
+  static constexpr int kEpilogueBytes = kPipeWaves * 32 * kAccTileStride<D> * 4;   // fp32 O rows of all waves
+  static constexpr int kLdsBytes = kLoopBytes > kEpilogueBytes ? kLoopBytes : kEpilogueBytes;
 };
 
 // One exponential pair of a 32-key half: scores 2j, 2j+1 of the lane -> one bf16x2 word of the P^T operand.
@@ -93,6 +95,8 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int lq = lane % 32, lh = lane / 32;
   const int N = p.N;
+  [[maybe_unused]] constexpr int TT = NT - kWave;   // stamping thread: first lane of the last wave (it sees every tile)
+  COROPE_STAMP(0, TT);
 
   const uint16_t* qg = p.q + (int64_t)bh * N * D;
   const int kvs = kv_slab(bh, p.H, p.Hkv);   // key/value slab of this query head
@@ -107,15 +111,24 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
   kst.load(kg, 0, N);
   vst.load(vg, 0, N);
 
-  // ---- Q rows of this wave: load, rotate, keep as the B operand ------------------------------------------
+  // ---- Q rows of this wave: load, rotate, keep as the B operand (through a wave-private LDS tile: the global loads and
+  // the copy of the rotated rows kept for the backward then touch whole row segments) ----------------------------------
   const int q_row = m0 + wave * 32 + lq;           // absolute query index of this lane
   u32x4 qb[M];
-  load_b_rows<D, true>(qb, qg, p.cos, p.sin, p.fstride, min(q_row, N - 1));
-  if (p.q_rot_out != nullptr && q_row < N) {   // the rotated rows, exactly as the MFMAs see them
-    uint16_t* dst = p.q_rot_out + ((int64_t)bh * N + q_row) * D + 8 * lh;
-#pragma unroll
-    for (int kc = 0; kc < M; ++kc) *reinterpret_cast<u32x4*>(dst + 16 * kc) = qb[kc];
+  {
+    WaveRows<D, true> qrows;
+    qrows.load(qg, p.cos, p.sin, p.fstride, m0 + wave * 32, N);
+    COROPE_STAMP(8, TT);
+#ifdef COROPE_TRACE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    COROPE_STAMP(9, TT);
+#endif
+    qrows.park(qb, reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride,
+               p.q_rot_out != nullptr ? p.q_rot_out + (int64_t)bh * N * D : nullptr, m0 + wave * 32, N);
   }
+  COROPE_STAMP(10, TT);
+  __syncthreads();   // the K and V buffers below overlap the tiles the waves just used
+  COROPE_STAMP(11, TT);
 
   const float scale = p.qk_scale;
   // Largest |q_r| * scale of the wave's rows (a little generous): times a tile's largest key norm it bounds the
@@ -170,7 +183,9 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
     reinterpret_cast<u32x4*>(smem + voff_prev)[i] = u32x4{0, 0, 0, 0};
   kst.load(kg, BLOCK_N, N);
   vst.load(vg, BLOCK_N, N);
+  COROPE_STAMP(12, TT);
   __syncthreads();
+  COROPE_STAMP(1, TT);
 
   const int wave_q_lo = m0 + wave * 32, wave_q_hi = wave_q_lo + 31;
   const int key_limit = CAUSAL ? q_row : N - 1;   // last key this lane's query attends to
@@ -222,9 +237,18 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
 
   // (the first 64 key-norm maxima have landed before the loop on every path, for the same reason as in the reload below)
   asm volatile("" ::"v"(kvec));
+  COROPE_STAMP(2, TT);
+  COROPE_STAMP_ID(TT, n_tiles);
+#ifdef COROPE_TRACE
+  const uint64_t clk0 = __builtin_readcyclecounter();
+#endif
   // ---- tiles this wave's rows can see ------------------------------------------------------------------------------
   for (int t = 0; t <= t_last; ++t) {
     const int n0 = t * BLOCK_N;
+#ifdef COROPE_TRACE
+    if (t == 1) COROPE_STAMP(3, TT);
+    if (n0 == m0) COROPE_STAMP(4, TT);
+#endif
     uint32_t k_lane = k_lane_off + koff_cur, vt = v_lane_off + voff_cur, vprev = v_lane_off + voff_prev;   // K(t), V(t), V(t-1)
     asm volatile("" : "+v"(k_lane), "+v"(vt), "+v"(vprev));
     auto k_operand = [&](int half, int kc) {
@@ -333,6 +357,10 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
     __syncthreads();
   }
   drain();
+  COROPE_STAMP(5, TT);
+#ifdef COROPE_TRACE
+  if (p.trace != nullptr && threadIdx.x == TT) p.trace[(int64_t)blockIdx.x * 16 + 7] = __builtin_readcyclecounter() - clk0;
+#endif
   // ---- tiles entirely above this wave's diagonal: it only stages its share ------------------------------------------
   for (int t = t_last + 1; t < n_tiles; ++t) {
     stage_next(t);
@@ -340,22 +368,17 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
     __syncthreads();
   }
 
-  // ---- epilogue: normalise, write O and the base-2 log-sum-exp ----------------------------------------------
+  // ---- epilogue: normalise, write O (through LDS, whole row segments per store) and the base-2 log-sum-exp ------------
   const float l_tot = half_sum(l_run + lsum);
   const float inv_l = 1.f / l_tot;
-  if (q_row < N) {
-    uint16_t* op = p.o + ((int64_t)bh * N + q_row) * D;
-#pragma unroll
-    for (int db = 0; db < NDB; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = pack_bf16(oacc[db][4 * g] * inv_l, oacc[db][4 * g + 1] * inv_l);
-        w[1] = pack_bf16(oacc[db][4 * g + 2] * inv_l, oacc[db][4 * g + 3] * inv_l);
-        *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g + 4 * lh) = w;
-      }
-    if (lh == 0) p.lse[(int64_t)bh * N + q_row] = m_run * scale + fast_log2(l_tot);
-  }
+  __syncthreads();   // every wave is done with the K and V buffers
+  store_rows_via_lds<D, false>(oacc, p.o + (int64_t)bh * N * D, m0 + wave * 32, N, nullptr, nullptr, 0, inv_l,
+                               reinterpret_cast<float*>(smem) + wave * 32 * kAccTileStride<D>);
+  if (q_row < N && lh == 0) p.lse[(int64_t)bh * N + q_row] = m_run * scale + fast_log2(l_tot);
+#ifdef COROPE_TRACE
+  __builtin_amdgcn_s_waitcnt(0);
+  COROPE_STAMP(6, TT);
+#endif
 }
 
 // ---- host-side launch -----------------------------------------------------------------------------------------
@@ -366,6 +389,9 @@ static hipError_t launch_pipe_cfg(FwdParams p, hipStream_t stream) {
   static std::atomic<uint64_t> lds_ok{0};
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
   p.num_m_blocks = (p.N + Cfg::kBlockM - 1) / Cfg::kBlockM;
+#ifdef COROPE_TRACE
+  p.trace = g_trace_buf;
+#endif
   dim3 grid(p.num_m_blocks * p.BH);
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
