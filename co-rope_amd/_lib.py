@@ -27,6 +27,8 @@ SIGNATURES = {
     "corope_rope_attn_fwd": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_fwd_workspace_bytes": (_L, [_I, _I, _I, _I]),
     "corope_rope_attn_fwd_ws": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P, _L, _P]),
+    "corope_rope_attn_fwd_noalloc_max_bytes": (_L, []),
+    "corope_rope_attn_fwd_noalloc": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_fwd_prerotated": (_I, [_P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_fwd_train": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_rotate": (_I, [_P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _P]),

@@ -168,6 +168,67 @@ int corope_rope_attn_fwd(const void* q, const void* k, const void* v, const floa
                             causal, nullptr, nullptr, nullptr, nullptr, 0, stream);
 }
 
+// ---- the forward for callers that cannot allocate -------------------------------------------------------------------
+// Scratch of corope_rope_attn_fwd_noalloc: the rotated K and the per-tile key norms that corope_rope_attn_fwd_ws keeps in
+// a caller-supplied workspace.  One copy per GPU the library is loaded on, held until the process ends.  In host code the
+// array's name only stands for the symbol: the device address comes from hipGetSymbolAddress, once per device.
+}  // extern "C" (reopened below)
+
+#define COROPE_NOALLOC_MAX_BYTES (65ll << 20)
+static __device__ __align__(256) unsigned char scratch[COROPE_NOALLOC_MAX_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];   // per device: address of that device's copy of `scratch`
+
+// Device address of the current device's scratch array (null + error text on failure).
+void* scratch_address(const char* what) {
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) {
+    launch_status(what, e);
+    return nullptr;
+  }
+  if (dev < 0 || dev >= kMaxDevices) {
+    fail(COROPE_E_UNSUPPORTED, "%s: device ordinal %d outside [0, %d)", what, dev, kMaxDevices);
+    return nullptr;
+  }
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr != nullptr) return ptr;
+  if (hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)); e != hipSuccess || ptr == nullptr) {
+    launch_status(what, e != hipSuccess ? e : hipErrorInvalidSymbol);
+    return nullptr;
+  }
+  g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // two threads racing here store the same address
+  return ptr;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t corope_rope_attn_fwd_noalloc_max_bytes(void) { return COROPE_NOALLOC_MAX_BYTES; }
+
+int corope_rope_attn_fwd_noalloc(const void* q, const void* k, const void* v, const float* freqs_cos, const float* freqs_sin,
+                                 int64_t freq_row_stride, void* o, float* lse, int B, int H, int N, int D, float sm_scale,
+                                 int causal, void* stream) {
+  const char* what = "rope_attn_fwd_noalloc";
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
+  if (rc) return rc;
+  const int64_t need = fwd_ws_bytes(B, H, N, D);
+  if (need > COROPE_NOALLOC_MAX_BYTES)
+    return fail(COROPE_E_UNSUPPORTED,
+                "%s: B*H*N*D = %lld needs %lld bytes of scratch, the built-in buffer holds %lld; use corope_rope_attn_fwd_ws "
+                "with a workspace of your own",
+                what, (long long)B * H * N * D, (long long)need, (long long)COROPE_NOALLOC_MAX_BYTES);
+  rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse});
+  if (rc) return rc;
+  void* ptr = scratch_address(what);
+  if (ptr == nullptr) return COROPE_E_LAUNCH;
+  return rope_attn_fwd_impl(what, q, k, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, H, N, D, sm_scale, causal,
+                            nullptr, nullptr, nullptr, ptr, COROPE_NOALLOC_MAX_BYTES, stream);
+}
+
 int64_t corope_rope_attn_fwd_workspace_bytes(int B, int H, int N, int D) {
   if (corope_rope_attn_check(B, H, N, D, D, 1.f, 0)) return -1;
   return fwd_ws_bytes(B, H, N, D);

@@ -76,6 +76,22 @@ int corope_rope_attn_fwd_ws(const void *q, const void *k, const void *v,
                             int B, int H, int N, int D, float sm_scale, int causal,
                             void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The two-launch forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose forward allocates its outputs and
+ * lets Triton allocate the rest.  Same kernels and same results, bit for bit, as corope_rope_attn_fwd_ws; the rotated
+ * K and the per-tile key norms live in a buffer built into the library (one copy per GPU, held until the process ends,
+ * corope_rope_attn_fwd_noalloc_max_bytes() = 65 MiB of it), so the call itself allocates and frees nothing.  Sizes whose
+ * scratch (corope_rope_attn_fwd_workspace_bytes) exceeds that limit are refused with COROPE_E_UNSUPPORTED: the metric
+ * shape B2 H32 N4096 D128 fits, B*H*N*D may reach about 34 million elements.  Nothing in the buffer has to start at zero
+ * (the rotation pass writes every byte the attention kernel reads).  All calls on one GPU share that GPU's buffer:
+ * calls that overlap in time on one GPU (different streams, or a captured graph replayed beside another call) race;
+ * calls on one stream, or otherwise ordered, are safe. */
+int64_t corope_rope_attn_fwd_noalloc_max_bytes(void);
+int corope_rope_attn_fwd_noalloc(const void *q, const void *k, const void *v,
+                                 const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                                 void *o, float *lse,
+                                 int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
 /* y = half-layout rotation of x (B,H,N,D) bf16, fp32 arithmetic, rounded to bf16; tile_max (may be NULL) receives
  * [B*H][ceil(N/64)] floats, the largest norm of a rotated row in every 64-row tile.
  * Replaces apply_rotary_emb (reference fused-rope/rope_attn_pytorch.py:60-91). */
