@@ -8,9 +8,13 @@ rotation FLOPs not counted), the roofline of the dominant kernel from per-launch
 oracle timed on the host cores as a baseline.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--no-cpu-baseline]
+                    [--parity] [--data normal|sink] [--phase-trace] [--sweep [--lanes]]
 
 (c3 is the metric shape and the default; c2/c4 are the other RoPE-attention shapes; c5 is the Co-RoPE GQA forward,
-with its backward timed beside it.)
+with its backward timed beside it.)  --parity adds per-tensor errors against the CPU oracle to the line (outside the
+timed region); --data sink times the same shape on attention-sink-like keys; --phase-trace splits the three attention
+kernels into prologue / steady state / diagonal / epilogue from time stamps taken inside the kernels (needs the
+trace build of the library that co-rope_amd/build.py makes beside the shipped one).
 """
 import argparse
 import importlib
@@ -27,10 +31,6 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak used for every "fraction of peak" below
 PEAK_HBM_GBS = 8000.0
-# What a loop of nothing but independent 32x32x16 bf16 MFMAs on random operands sustains on this part (the clock drops by
-# a third under the switching activity of real data; all-zero operands reach 2.1-2.3 PFLOP/s).  Reported next to the
-# published peak, never instead of it.
-SUSTAINED_BF16_TFLOPS = 1520.0
 
 # HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE on this
 # benchmark (summary and commands: profiles/rope_attn_c3_hbm_traffic.md); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE
@@ -64,6 +64,109 @@ def settle_clocks(step, torch):
         torch.cuda.synchronize()
         n += 16
     return n
+
+
+def calc_sim(x, y):
+    """The reference's similarity measure, 2 sum(xy) / sum(x^2 + y^2) in fp64 (utils.py:12-19): 1 for equal tensors."""
+    x, y = x.double(), y.double()
+    den = (x * x + y * y).sum()
+    return 1.0 if float(den) == 0.0 else float(2 * (x * y).sum() / den)
+
+
+def make_inputs(B, H, N, D, data, torch, seed=42):
+    """q, k, v, dO (bf16-representable fp32, on the host).  "normal": N(0,1).  "sink": the same with an attention-sink
+    first key (x8), one outlier key in 1000 (x16) and key norms growing 0.5 -> 2 along the sequence -- the per-tile norm
+    bounds of the two-launch forward are then far above the scores that occur, and rise tile after tile."""
+    g = torch.Generator().manual_seed(seed)
+    q, k, v, do = (torch.randn(B, H, N, D, generator=g) for _ in range(4))
+    if data == "sink":
+        k = k * torch.linspace(0.5, 2.0, N).reshape(1, 1, N, 1)
+        k[:, :, 0] *= 8
+        k[:, :, 7::1000] *= 16
+    elif data != "normal":
+        sys.exit(f"bench.py: unknown --data {data}")
+    return tuple(t.to(torch.bfloat16).float() for t in (q, k, v, do))
+
+
+def err_stats(got, ref, torch):
+    """max / mean / percentiles of |got - ref| as the reference's verification script prints them (verification.py:91-114)."""
+    d = (got.float() - ref.float()).abs().flatten()
+    if d.numel() > (1 << 24):        # torch.quantile refuses more than 2^24 elements: a fixed stride sample for the percentiles
+        dq = d[:: d.numel() // (1 << 24) + 1]
+    else:
+        dq = d
+    qs = torch.quantile(dq, torch.tensor([0.5, 0.95, 0.99]))
+    return {"max_abs": float(d.max()), "mean_abs": float(d.mean()), "p50": float(qs[0]), "p95": float(qs[1]),
+            "p99": float(qs[2]), "max_abs_ref": float(ref.abs().max()), "calc_sim": round(calc_sim(got, ref), 8),
+            "n": int(d.numel())}
+
+
+def sample_rows(N, n, torch, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    r = torch.randperm(N, generator=g)[:n]
+    return torch.unique(torch.cat([r, torch.tensor([0, 1, 63, 64, N // 2, N - 2, N - 1]).clamp(0, N - 1)]))
+
+
+def rope_parity(pkg, cfg_name, q, k, v, do, cos, sin, scale, fwd_only, torch):
+    """Per-tensor errors of the HIP path against the fp32 CPU oracle on the same bf16-rounded inputs: O (and the row
+    statistic) on sampled rows of every head, dQ / dK / dV on whole heads (all of them at C2, 8 at C3)."""
+    from oracle import rope_attn_oracle as O
+    B, H, N, D = q.shape
+    dev = torch.device("cuda:0")
+    qd, kd, vd = (t.to(dev, torch.bfloat16).requires_grad_(not fwd_only) for t in (q, k, v))
+    o = pkg.attention(qd, kd, vd, True, scale, cos, sin)
+    if not fwd_only:
+        o.backward(do.to(dev, torch.bfloat16))
+    torch.cuda.synchronize()
+    o = o.detach().float().cpu()
+    rows = sample_rows(N, 128 if N <= 8192 else 48, torch)
+    c, s = cos.float().cpu(), sin.float().cpu()
+    ro, _ = O.rope_attn_forward_blocked(q, k, v, True, scale, c, s, rows=rows)
+    out = {"bar": "max-abs <= 2e-2 against the fp32 oracle (one bf16 ulp of the reference value where that is larger)",
+           "O": dict(err_stats(o[:, :, rows], ro, torch), sample=f"{rows.numel()} rows x {B * H} heads")}
+    if not fwd_only:
+        heads = [(b, h) for b in range(B) for h in range(H)]
+        if len(heads) > 32:
+            heads = heads[:: len(heads) // 8][:8]
+        acc = {n: ([], []) for n in ("dQ", "dK", "dV")}
+        for (b, h) in heads:
+            sl = (slice(b, b + 1), slice(h, h + 1))
+            _, _, rdq, rdk, rdv, _ = O.rope_attn_fwd_bwd_blocked(q[sl], k[sl], v[sl], do[sl], True, scale, c, s)
+            for n, t, r in (("dQ", qd, rdq), ("dK", kd, rdk), ("dV", vd, rdv)):
+                acc[n][0].append(t.grad[sl].float().cpu())
+                acc[n][1].append(r)
+        for n, (got, ref) in acc.items():
+            out[n] = dict(err_stats(torch.cat(got), torch.cat(ref), torch), sample=f"{len(heads)} whole heads of {B * H}")
+    return out
+
+
+def corope_parity(pkg, q, k, v, do, o_gpu, grads_gpu, scale, theta, torch):
+    """Per-tensor errors of the Co-RoPE kernels against the fp32 CPU oracle: O and dQ on sampled query rows of every head
+    (a query row's output depends on no other query row, so autograd through the row-sampled oracle gives its dQ), dK and
+    dV of one whole (batch, key/value head) group, accumulated by autograd over all its query rows, 64 at a time."""
+    from oracle import corope_gqa_oracle as C
+    B, Hq, N, D = q.shape
+    Hkv = k.shape[1]
+    G = Hq // Hkv
+    dq_g, dk_g, dv_g = grads_gpu
+    rows = sample_rows(N, 9, torch, seed=3)
+    qa = q.clone().requires_grad_(True)
+    ref = C.corope_gqa_forward_rows(qa, k, v, True, scale, theta, rows, torch.float32, row_block=16)
+    (ref_dq,) = torch.autograd.grad(ref, qa, do[:, :, rows])
+    out = {"bar": "max-abs <= 2e-2 against the fp32 oracle (dK, dV: x sqrt(group size), sums over the group's heads)",
+           "O": dict(err_stats(o_gpu[:, :, rows], ref.detach(), torch), sample=f"{rows.numel()} rows x {B * Hq} heads"),
+           "dQ": dict(err_stats(dq_g[:, :, rows], ref_dq[:, :, rows], torch), sample=f"{rows.numel()} rows x {B * Hq} heads")}
+    b, kv = B - 1, Hkv // 2                       # one whole group
+    qs, dos = q[b:b + 1, kv * G:(kv + 1) * G], do[b:b + 1, kv * G:(kv + 1) * G]
+    kx, vx = (t[b:b + 1, kv:kv + 1].clone().requires_grad_(True) for t in (k, v))
+    for r0 in range(0, N, 64):
+        hi = min(r0 + 64, N)
+        blk = C.corope_gqa_forward_rows(qs[:, :, :hi], kx[:, :, :hi], vx[:, :, :hi], True, scale, theta,
+                                        torch.arange(r0, hi), torch.float32, row_block=64)
+        blk.backward(dos[:, :, r0:hi])
+    out["dK"] = dict(err_stats(dk_g[b:b + 1, kv:kv + 1], kx.grad, torch), sample=f"group (batch {b}, kv head {kv}), all {N} keys")
+    out["dV"] = dict(err_stats(dv_g[b:b + 1, kv:kv + 1], vx.grad, torch), sample=f"group (batch {b}, kv head {kv}), all {N} keys")
+    return out
 
 
 def attention_flops(B, H, N, D, mode, causal=True):
@@ -157,8 +260,7 @@ def bench_sweep(args):
             ub_ms = rot_ms + timed(lambda: ou.backward(do, retain_graph=True))
             row.update({"unfused_fwd_ms": round(uf_ms, 4), "unfused_bwd_ms": round(ub_ms, 4),
                         "fwd_speedup_vs_unfused": round(uf_ms / f_ms, 3), "bwd_speedup_vs_unfused": round(ub_ms / b_ms, 3),
-                        "cos_sim_vs_unfused": round(float(torch.nn.functional.cosine_similarity(
-                            o.detach().float().flatten(), ou.detach().float().flatten(), dim=0)), 6)})
+                        "calc_sim_vs_unfused": round(calc_sim(o.detach(), ou.detach()), 8)})
             try:
                 sdpa = torch.nn.functional.scaled_dot_product_attention
                 sf_ms = rot_ms + timed(lambda: sdpa(qr, kr, v, is_causal=True, scale=0.5))
@@ -262,7 +364,128 @@ def bench_corope(args):
                                      "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T issue slots/s",
                                      "frac": round(bwd_instr / (bms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4), "traffic": None}},
            "cpu_baseline": None}
+    if args.parity:
+        torch.cuda.synchronize()
+        out["parity"] = corope_parity(pkg, q.float().cpu(), k.float().cpu(), v.float().cpu(), do.float().cpu(), o.float().cpu(),
+                                      tuple(t.float().cpu() for t in (dq, dk, dv)), scale, 10000.0, torch)
     print(json.dumps(out))
+
+
+def forward_ms(pkg, q, k, v, cos, sin, scale, torch, reps=100):
+    """Average duration of the operator's forward (all its launches) over `reps` back-to-back calls, HIP events."""
+    for _ in range(20):
+        pkg.rope_attn_forward_with_lse(q, k, v, True, scale, cos, sin)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        pkg.rope_attn_forward_with_lse(q, k, v, True, scale, cos, sin)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def bench_phase_trace(args):
+    """Where the time of the forward, dQ and dK+dV kernels goes at the chosen shape: every workgroup of the trace build
+    stamps the constant 100 MHz counter at its phase boundaries (one lane of the wave that sees every tile) and the
+    core-clock counter around its tile loop.  Prints a markdown table (one traced step in the middle of a run of steps)."""
+    import ctypes
+    import numpy as np
+    import torch
+    pkg = importlib.import_module("corope_amd")
+    path = os.path.join(os.path.dirname(pkg._lib.LIB_PATH), "libcorope_amd_trace.so")
+    if not os.path.exists(path):
+        sys.exit(f"bench.py: {path} not found (python co-rope_amd/build.py makes it)")
+    lib = ctypes.CDLL(path)
+    for n, (r, a) in pkg._lib.SIGNATURES.items():
+        getattr(lib, n).restype, getattr(lib, n).argtypes = r, a
+    lib.corope_debug_trace.argtypes, lib.corope_debug_trace.restype = [ctypes.c_void_p], None
+    dev = torch.device("cuda:0")
+    cfg = CONFIGS[args.config]
+    B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
+    scale = 1 / math.sqrt(D)
+    q, k, v, do = (t.to(dev, torch.bfloat16) for t in make_inputs(B, H, N, D, args.data, torch))
+    c, s = pkg.precompute_freqs_cis(D, N, 10000.0, device=dev)
+    st, fs = torch.cuda.current_stream().cuda_stream, c.stride(0)
+    o, qr, kr, dq, dk, dv = (torch.empty_like(q) for _ in range(6))
+    M = torch.empty(B, H, N, device=dev, dtype=torch.float32)
+    delta = torch.empty_like(M)
+    kmax = torch.empty(B, H, (N + 63) // 64, device=dev, dtype=torch.float32)
+    P = lambda t: t.data_ptr()
+    launches = [
+        ("rope_rotate_k", lambda: lib.corope_rope_rotate(P(k), P(c), P(s), fs, P(kr), P(kmax), B, H, N, D, st)),
+        ("rope_attn_fwd", lambda: lib.corope_rope_attn_fwd_prerotated(P(q), P(kr), P(kmax), P(v), P(c), P(s), fs, P(o), P(M), P(qr),
+                                                                      B, H, N, D, scale, 1, st)),
+        ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq_prerotated(P(qr), P(kr), P(v), P(o), P(do), P(M), P(delta), P(c),
+                                                                            P(s), fs, P(dq), B, H, N, D, scale, 1, st)),
+        ("rope_attn_bwd_dkdv", lambda: lib.corope_rope_attn_bwd_dkdv_prerotated(P(qr), P(kr), P(v), P(do), P(M), P(delta), P(c), P(s),
+                                                                                fs, P(dk), P(dv), B, H, N, D, scale, 1, st)),
+    ]
+    lib.corope_debug_trace(None)
+    for _ in range(60):          # settle the clocks
+        for n, f in launches:
+            assert f() == 0, n
+    torch.cuda.synchronize()
+    n_wg = B * H * ((N + 255) // 256)
+    bufs = {n: torch.zeros(n_wg * 16, dtype=torch.int64, device=dev) for n, _ in launches[1:]}
+    for rep in range(3):         # the traced step sits between untraced ones
+        for n, f in launches:
+            lib.corope_debug_trace(bufs[n].data_ptr() if (n in bufs and rep == 1) else None)
+            assert f() == 0, n
+    torch.cuda.synchronize()
+    lib.corope_debug_trace(None)
+
+    def row(label, x):
+        x = np.asarray(x, dtype=float)
+        return f"| {label} | {x.mean():.2f} | {np.percentile(x, 10):.2f} | {np.percentile(x, 50):.2f} | {np.percentile(x, 90):.2f} | {x.max():.2f} |"
+
+    print(f"Workload: {cfg['name']}, data {args.data}; times in microseconds per workgroup (256 rows) unless said otherwise.\n")
+    for name, buf in bufs.items():
+        a = buf.cpu().numpy().reshape(-1, 16)
+        a = a[a[:, 0] != 0]
+        t = a[:, :14].astype(np.float64) * 0.01
+        t = np.where(a[:, :14] != 0, t - t[:, 0].min(), np.nan)
+        hw, xcc = a[:, 14] & 0xffffffff, (a[:, 14] >> 32) & 0xf
+        cu_key = xcc * 1000 + ((hw >> 13) & 7) * 100 + ((hw >> 12) & 1) * 16 + ((hw >> 8) & 0xf)
+        ntile = a[:, 15].astype(float)
+        dkdv = name.endswith("dkdv")
+        gaps, busy = [], []
+        for kk in set(cu_key):
+            idx = np.where(cu_key == kk)[0]
+            idx = idx[np.argsort(t[idx, 0])]
+            gaps += [t[j, 0] - t[i, 6] for i, j in zip(idx[:-1], idx[1:])]
+            busy.append(sum(t[i, 6] - t[i, 0] for i in idx))
+        span = np.nanmax(t[:, 6])
+        ghz = a[:, 7] / ((a[:, 5] - (a[:, 1] if name != "rope_attn_fwd" else a[:, 2])) * 10.0)
+        print(f"### {name}: {len(a)} workgroups on {len(set(cu_key))} CUs, {len(a) / len(set(cu_key)):.1f} per CU, "
+              f"launch span {span:.1f} us, mean busy time per CU {np.mean(busy):.1f} us\n")
+        print("| phase | mean | p10 | p50 | p90 | max |\n|---|---|---|---|---|---|")
+        print(row("whole workgroup", t[:, 6] - t[:, 0]))
+        print(row("gap to the next workgroup on the same CU", gaps))
+        print(row("prologue (entry -> first tile staged)", t[:, 1] - t[:, 0]))
+        big = ntile > 5
+        if dkdv:      # the key block's diagonal query tiles come first
+            print(row("first tile", t[:, 3] - t[:, 1]))
+            print(row("diagonal tiles 2-4, per tile", (t[big, 4] - t[big, 3]) / 3))
+            print(row("steady state, per tile (64 queries x 256 keys)", (t[big, 5] - t[big, 4]) / (ntile[big] - 4)))
+        else:
+            if name == "rope_attn_fwd":
+                print(row("  of which: loads issued", t[:, 8] - t[:, 0]))
+                print(row("  of which: loads landed", t[:, 9] - t[:, 8]))
+                print(row("  of which: rotate Q, through LDS, rotated copy stored", t[:, 10] - t[:, 9]))
+                print(row("  of which: K/V tile 0 to LDS, tile 1 requested, barriers", t[:, 1] - t[:, 10]))
+                print(row("key-norm bounds of the wave's tiles", t[:, 2] - t[:, 1]))
+                print(row("first tile (with its exact pass)", t[:, 3] - t[:, 2]))
+                print(row("tiles examined twice, fraction of the wave's tiles", a[:, 13] / ntile))
+            else:
+                print(row("first tile", t[:, 3] - t[:, 1]))
+            print(row("steady state, per tile (256 queries x 64 keys)", (t[big, 4] - t[big, 3]) / (ntile[big] - 5)))
+            print(row("diagonal block, per tile (4 tiles, waves drop out)", (t[:, 5] - t[:, 4]) / 4))
+        print(row("epilogue (last tile -> stores done)", t[:, 6] - t[:, 5]))
+        print(row("shader clock in the tile loop [GHz]", ghz))
+        per_cu = len(a) / len(set(cu_key))
+        edge = np.nanmean(t[:, 1] - t[:, 0]) + np.nanmean(t[:, 6] - t[:, 5]) + np.mean(gaps)
+        print(f"\nPer CU: {per_cu:.0f} workgroups x {edge:.1f} us of prologue + epilogue + gap = {per_cu * edge:.0f} us "
+              f"of {np.mean(busy):.0f} us ({100 * per_cu * edge / np.mean(busy):.0f} %).\n")
 
 
 def main():
@@ -277,6 +500,12 @@ def main():
                     help="time the reference harness's 19 shapes instead (one JSON line per shape)")
     ap.add_argument("--lanes", action="store_true",
                     help="with --sweep: also time the unfused lanes (separate rotation + identity-table attention, PyTorch SDPA)")
+    ap.add_argument("--parity", action="store_true",
+                    help="after the timed region, add per-tensor errors against the CPU oracle to the line")
+    ap.add_argument("--data", default="normal", choices=["normal", "sink"],
+                    help="synthetic inputs: N(0,1), or attention-sink-like keys (see make_inputs)")
+    ap.add_argument("--phase-trace", action="store_true",
+                    help="split the attention kernels of the chosen RoPE config into phases (trace build of the library)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
@@ -296,6 +525,8 @@ def main():
         return bench_sweep(args)
     if args.config == "c5":
         return bench_corope(args)
+    if args.phase_trace:
+        return bench_phase_trace(args)
     import torch
     pkg = importlib.import_module("corope_amd")
     lib = pkg._lib.load()
@@ -304,8 +535,8 @@ def main():
     B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
     fwd_only = args.config == "c4"
     scale = 1 / math.sqrt(D)
-    g = torch.Generator().manual_seed(42)
-    q, k, v, do = (torch.randn(B, H, N, D, generator=g).to(dev, torch.bfloat16) for _ in range(4))
+    host = make_inputs(B, H, N, D, args.data, torch)
+    q, k, v, do = (t.to(dev, torch.bfloat16) for t in host)
     cos, sin = pkg.precompute_freqs_cis(D, N, 10000.0, device=dev)
     q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
 
@@ -409,7 +640,6 @@ def main():
     traffic = HBM_TRAFFIC_BYTES.get((args.config, dom))
     roofline = {"bound": "mfma", "kernel": dom, "achieved": round(dom_tf, 1), "peak": PEAK_BF16_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(dom_tf / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
-                "frac_of_sustained_mfma_rate": round(dom_tf / SUSTAINED_BF16_TFLOPS, 4),
                 "avg_launch_ms": round(avg[dom], 4)}
     fwd_ms = avg["rope_attn_fwd"] + avg.get("rope_rotate_k", 0.0)
     fwd_tf = alg["rope_attn_fwd"] / (fwd_ms * 1e-3) * 1e-12
@@ -418,7 +648,7 @@ def main():
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "settle_steps": settle_steps,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "bf16", "data": "synthetic" if args.data == "normal" else "synthetic (attention-sink keys)",
         "config": {"workload": cfg["name"], "B": B, "H": H, "N": N, "D": D, "causal": True,
                    "sm_scale": "1/sqrt(D)", "rope_base": 10000.0},
         "frac_of_bf16_peak": round(value / PEAK_BF16_TFLOPS, 4),
@@ -430,6 +660,27 @@ def main():
         bwd_ms = sum(ms for n, ms in avg.items() if n not in ("rope_rotate_k", "rope_attn_fwd"))
         bwd_tf = f_bwd / (bwd_ms * 1e-3) * 1e-12
         out["bwd"] = {"ms": round(bwd_ms, 4), "tflops": round(bwd_tf, 1), "frac_of_peak": round(bwd_tf / PEAK_BF16_TFLOPS, 4)}
+    # the dO.O pass (delta = rowsum(O o dO)) on its own: at this shape the dQ kernel computes delta on its way, so the pass is
+    # not one of the step's launches; timed here for its HBM rate (two (B,H,N,D) bf16 tensors read, (B,H,N) fp32 written)
+    if not fwd_only and "rope_attn_bwd_preprocess" not in kernels:
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(51)]
+        for i in range(-5, 50):
+            lib.corope_rope_attn_bwd_preprocess(o.data_ptr(), dop, delta.data_ptr(), B, H, N, D, stream)
+            if i >= -1:
+                evs[i + 1].record()
+        torch.cuda.synchronize()
+        ms = sum(evs[i].elapsed_time(evs[i + 1]) for i in range(50)) / 50
+        by = 2.0 * B * H * N * D * 2 + B * H * N * 4
+        kernels["rope_attn_bwd_preprocess (standalone: not a launch of the step at this shape)"] = {
+            "ms": round(ms, 4), "gbs": round(by / (ms * 1e-3) * 1e-9, 1), "frac_of_hbm_peak": round(by / (ms * 1e-3) * 1e-9 / PEAK_HBM_GBS, 4)}
+    if args.data != "normal":
+        # the same forward on N(0,1) inputs, timed the same way, beside the line's own
+        hq, hk, hv, _ = make_inputs(B, H, N, D, "normal", torch)
+        out["fwd_ms_by_data"] = {args.data: round(forward_ms(pkg, q.detach(), k.detach(), v.detach(), cos, sin, scale, torch), 4),
+                                 "normal": round(forward_ms(pkg, *(t.to(dev, torch.bfloat16) for t in (hq, hk, hv)), cos, sin,
+                                                            scale, torch), 4)}
+    if args.parity:
+        out["parity"] = rope_parity(pkg, args.config, host[0], host[1], host[2], host[3], cos, sin, scale, fwd_only, torch)
     out["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline()
     print(json.dumps(out))
 

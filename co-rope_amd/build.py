@@ -1,7 +1,10 @@
 """Builds libcorope_amd.so (gfx950 HIP kernels + C ABI) in-tree with hipcc.
 
 Run as ``python co-rope_amd/build.py`` or call ``build()``; the result lands in
-``co-rope_amd/lib/libcorope_amd.so`` and is what ``_lib.load()`` opens."""
+``co-rope_amd/lib/libcorope_amd.so`` and is what ``_lib.load()`` opens.  Beside it, for measurement only:
+``libcorope_amd_trace.so`` (the same sources with -DCOROPE_TRACE: the attention kernels stamp a clock at their phase
+boundaries into a buffer ``bench.py --phase-trace`` hands them) and the stand-alone program ``mfma_rate``
+(``csrc/mfma_rate.hip``: what the matrix pipes sustain on this machine)."""
 from __future__ import annotations
 
 import os
@@ -13,6 +16,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libcorope_amd.so")
+TRACE_LIB = os.path.join(LIBDIR, "libcorope_amd_trace.so")
+MFMA_RATE = os.path.join(LIBDIR, "mfma_rate")
 
 SOURCES = ["abi.hip", "rope_freqs.hip", "rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_fwd_pipe.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip", "corope_gqa_bwd.hip"]
 
@@ -29,8 +34,8 @@ def _hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def _compile(src, extra):
-    obj = os.path.join(LIBDIR, os.path.splitext(src)[0] + ".o")
+def _compile(src, extra, suffix=""):
+    obj = os.path.join(LIBDIR, os.path.splitext(src)[0] + suffix + ".o")
     cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
@@ -40,19 +45,32 @@ def _compile(src, extra):
     return obj, err
 
 
-def build(verbose=False, extra_flags=()):
-    os.makedirs(LIBDIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
-        results = list(ex.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
-    if verbose:
-        for (_, err), s in zip(results, SOURCES):
-            if err.strip():
-                print(f"--- {s}\n{err}", file=sys.stderr)
-    objs = [o for o, _ in results]
-    r = subprocess.run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB],
+def _link(objs, out, shared=True):
+    r = subprocess.run([_hipcc(), "--offload-arch=gfx950", *(["-shared", "-fPIC"] if shared else []), *objs, "-o", out],
                        capture_output=True, text=True)
     if r.returncode != 0:
-        raise RuntimeError(f"link failed:\n{r.stderr}")
+        raise RuntimeError(f"link of {out} failed:\n{r.stderr}")
+    return out
+
+
+def build(verbose=False, extra_flags=(), extras=True):
+    """Compiles every source.  ``extras``: also the trace variant of the library and the mfma_rate program."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    jobs = [(s, list(extra_flags), "") for s in SOURCES]
+    if extras:
+        jobs += [(s, list(extra_flags) + ["-DCOROPE_TRACE"], ".trace") for s in SOURCES]
+        jobs += [("mfma_rate.hip", [], "")]
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        results = list(ex.map(lambda j: _compile(*j), jobs))
+    if verbose:
+        for (_, err), j in zip(results, jobs):
+            if err.strip():
+                print(f"--- {j[0]}{j[2]}\n{err}", file=sys.stderr)
+    n = len(SOURCES)
+    _link([o for o, _ in results[:n]], LIB)
+    if extras:
+        _link([o for o, _ in results[n:2 * n]], TRACE_LIB)
+        _link([results[2 * n][0]], MFMA_RATE, shared=False)
     return LIB
 
 

@@ -7,6 +7,12 @@
 
 #include "kernels.hpp"
 
+#ifdef COROPE_TRACE
+// Measurement builds only (libcorope_amd_trace.so): where the attention kernels write their time stamps, or null.
+namespace corope { uint64_t* g_trace_buf = nullptr; }
+extern "C" void corope_debug_trace(void* buf) { corope::g_trace_buf = static_cast<uint64_t*>(buf); }
+#endif
+
 namespace {
 
 thread_local char g_err[256] = "";
@@ -260,7 +266,9 @@ int corope_rope_attn_fwd_prerotated(const void* q, const void* k_rot, const floa
 int corope_rope_attn_fwd_train(const void* q, const void* k, const void* v, const float* freqs_cos, const float* freqs_sin,
                                int64_t freq_row_stride, void* o, float* lse, void* q_rot, void* k_rot, float* tile_kmax,
                                int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
-  int rc = check_ptrs("rope_attn_fwd_train", {q_rot, k_rot});
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
+  if (rc) return rc;
+  rc = check_ptrs("rope_attn_fwd_train", {q, k, v, freqs_cos, freqs_sin, o, lse, q_rot, k_rot});
   if (rc) return rc;
   if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
     return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "rope_attn_fwd_train: tile_kmax %p is null or misaligned",
@@ -308,6 +316,15 @@ void mark_prerotated(corope::BwdParams& p, bool prerot) {
     p.q_rot = p.q;
     p.k_rot = p.k;
   }
+}
+
+// Everything a whole backward takes, checked before the first launch of a composite entry point: sizes, then every
+// pointer (null and alignment).  `o` may be null only where the caller says so.
+int validate_bwd(const char* what, int B, int H, int N, int D, int64_t freq_row_stride, float sm_scale,
+                 std::initializer_list<const void*> ptrs) {
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
+  if (rc) return rc;
+  return check_ptrs(what, ptrs);
 }
 
 int bwd_dv_impl(const char* what, bool prerot, const void* q, const void* k, const void* d_o, const float* lse,
@@ -375,7 +392,8 @@ int corope_rope_attn_bwd_dkdv(const void* q, const void* k, const void* v, const
                               const float* delta, const float* freqs_cos, const float* freqs_sin,
                               int64_t freq_row_stride, void* dk, void* dv, int B, int H, int N, int D, float sm_scale,
                               int causal, void* stream) {
-  int rc = check_ptrs("rope_attn_bwd_dkdv", {v, delta, dk, dv});
+  int rc = validate_bwd("rope_attn_bwd_dkdv", B, H, N, D, freq_row_stride, sm_scale,
+                        {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dk, dv});
   if (rc) return rc;
   rc = corope_rope_attn_bwd_dv(q, k, d_o, lse, freqs_cos, freqs_sin, freq_row_stride, dv, B, H, N, D, sm_scale, causal,
                                stream);
@@ -434,7 +452,10 @@ int corope_rope_attn_bwd(const void* q, const void* k, const void* v, const void
                          float* delta, const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride,
                          void* dq, void* dk, void* dv, int B, int H, int N, int D, float sm_scale, int causal,
                          void* stream) {
-  int rc = corope_rope_attn_bwd_preprocess(o, d_o, delta, B, H, N, D, stream);
+  int rc = validate_bwd("rope_attn_bwd", B, H, N, D, freq_row_stride, sm_scale,
+                        {q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv});
+  if (rc) return rc;
+  rc = corope_rope_attn_bwd_preprocess(o, d_o, delta, B, H, N, D, stream);
   if (rc) return rc;
   rc = corope_rope_attn_bwd_dkdv(q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dk, dv, B, H, N, D,
                                  sm_scale, causal, stream);
@@ -449,7 +470,8 @@ int corope_rope_attn_bwd_prerotated(const void* q_rot, const void* k_rot, const 
                                     float sm_scale, int causal, void* stream) {
   // two launches: the dQ kernel computes delta for the rows it owns on its way (no separate pass over o and dO), the
   // fused dK+dV kernel reads it afterwards
-  int rc = check_ptrs("rope_attn_bwd_prerotated", {o});
+  int rc = validate_bwd("rope_attn_bwd_prerotated", B, H, N, D, freq_row_stride, sm_scale,
+                        {q_rot, k_rot, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv});
   if (rc) return rc;
   rc = corope_rope_attn_bwd_dq_prerotated(q_rot, k_rot, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, B,
                                           H, N, D, sm_scale, causal, stream);
@@ -467,9 +489,8 @@ int corope_rope_attn_bwd_ws(const void* q, const void* k, const void* v, const v
                             const float* lse, float* delta, const float* freqs_cos, const float* freqs_sin,
                             int64_t freq_row_stride, void* dq, void* dk, void* dv, int B, int H, int N, int D,
                             float sm_scale, int causal, void* workspace, int64_t workspace_bytes, void* stream) {
-  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
-  if (rc) return rc;
-  rc = check_ptrs("rope_attn_bwd_ws", {workspace});
+  int rc = validate_bwd("rope_attn_bwd_ws", B, H, N, D, freq_row_stride, sm_scale,
+                        {q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv, workspace});
   if (rc) return rc;
   if (workspace_bytes < 2 * bwd_ws_tensor_bytes(B, H, N, D))
     return fail(COROPE_E_BADARG, "rope_attn_bwd_ws: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
@@ -494,7 +515,9 @@ int corope_rope_attn_fwd_gqa(const void* q, const void* k, const void* v, const 
     return rope_attn_fwd_impl(what, q, k, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, Hq, N, D, sm_scale, causal,
                               nullptr, nullptr, nullptr, nullptr, 0, stream, Hkv);
   }
-  int rc = check_ptrs(what, {k_rot});
+  int rc = corope_rope_attn_check(B, Hq, N, D, freq_row_stride, sm_scale, 0);
+  if (rc) return rc;
+  rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse, k_rot});
   if (rc) return rc;
   if (q_rot != nullptr && !aligned16(q_rot)) return fail(COROPE_E_ALIGN, "%s: q_rot %p is not 16-byte aligned", what, q_rot);
   if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))

@@ -146,6 +146,9 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   __syncthreads();
   COROPE_STAMP(1, 0);
   COROPE_STAMP_ID(0, n_iter);
+#ifdef COROPE_TRACE
+  const uint64_t clk0 = __builtin_readcyclecounter();
+#endif
 
   const float scale2 = p.qk_scale;
   for (int it = 0; it < n_iter; ++it) {
@@ -226,6 +229,9 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   }
 
   COROPE_STAMP(5, 0);
+#ifdef COROPE_TRACE
+  if (p.trace != nullptr && threadIdx.x == 0) p.trace[(int64_t)blockIdx.x * 16 + 7] = __builtin_readcyclecounter() - clk0;
+#endif
   // every wave is past its last read of the tiles (the loop ends with a barrier): their LDS now carries the accumulators
   // to a row-major order, so that dV and dK leave in whole row segments and the tables are read the same way
   float* wave_out = reinterpret_cast<float*>(smem) + wave * 32 * kAccTileStride<D>;
@@ -342,6 +348,9 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   __syncthreads();
   COROPE_STAMP(1, TT);
   COROPE_STAMP_ID(TT, n_tiles);
+#ifdef COROPE_TRACE
+  const uint64_t clk0 = __builtin_readcyclecounter();
+#endif
 
   const float scale2 = p.qk_scale;
   for (int t = 0; t < n_tiles; ++t) {
@@ -406,6 +415,9 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   }
 
   COROPE_STAMP(5, TT);
+#ifdef COROPE_TRACE
+  if (p.trace != nullptr && threadIdx.x == TT) p.trace[(int64_t)blockIdx.x * 16 + 7] = __builtin_readcyclecounter() - clk0;
+#endif
   // every wave is past its last read of the tiles (the loop ends with a barrier): their LDS now carries dQ_r to a
   // row-major order, so that the tables are read and dQ is written in whole row segments
   store_rows_via_lds<D, true>(dqacc, p.dq + base, wq_lo, N, p.cos, p.sin, p.fstride, p.sm_scale,

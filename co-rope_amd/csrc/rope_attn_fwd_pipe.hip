@@ -241,6 +241,7 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
   COROPE_STAMP_ID(TT, n_tiles);
 #ifdef COROPE_TRACE
   const uint64_t clk0 = __builtin_readcyclecounter();
+  uint64_t exact_passes = 0;   // tiles of this wave that were examined a second time to move the reference
 #endif
   // ---- tiles this wave's rows can see ------------------------------------------------------------------------------
   for (int t = 0; t <= t_last; ++t) {
@@ -315,6 +316,9 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
     }
     const uint32_t kmax_bits = __builtin_amdgcn_readlane(kvec, t - kvec_base);
     if (t == 0 || kmax_bits > thr_bits) {
+#ifdef COROPE_TRACE
+      ++exact_passes;
+#endif
       if (t > 0) drain();
       f32x16 r0 = f32x16{0}, r1 = f32x16{0};
 #pragma unroll
@@ -359,7 +363,10 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
   drain();
   COROPE_STAMP(5, TT);
 #ifdef COROPE_TRACE
-  if (p.trace != nullptr && threadIdx.x == TT) p.trace[(int64_t)blockIdx.x * 16 + 7] = __builtin_readcyclecounter() - clk0;
+  if (p.trace != nullptr && threadIdx.x == TT) {
+    p.trace[(int64_t)blockIdx.x * 16 + 7] = __builtin_readcyclecounter() - clk0;
+    p.trace[(int64_t)blockIdx.x * 16 + 13] = exact_passes;
+  }
 #endif
   // ---- tiles entirely above this wave's diagonal: it only stages its share ------------------------------------------
   for (int t = t_last + 1; t < n_tiles; ++t) {

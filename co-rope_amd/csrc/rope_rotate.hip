@@ -1,7 +1,7 @@
 // Half-layout rotation of a whole (B*H, N, D) bf16 tensor, written back as bf16, plus the largest row norm of
 // every 64-row tile.
 //
-// The rotation is the reference's apply_rotary_emb (fused-rope/rope_attn_pytorch.py:60-91; in-kernel form
+// The rotation is the reference's apply_rotary_emb (fused-rope/rope_attn_pytorch.py:71-84, rotate_half :52-68; in-kernel form
 // fused-rope/fused_rope_attn.py:82-99): y1 = x1 cos - x2 sin, y2 = x2 cos + x1 sin on the two halves of a row,
 // evaluated in fp32 and rounded to bf16 once -- bit for bit what the attention kernels produce when they rotate a
 // tile themselves.  A K tile is needed by every query block of its head, so for long sequences rotating K once

@@ -94,7 +94,7 @@ int corope_rope_attn_fwd_noalloc(const void *q, const void *k, const void *v,
 
 /* y = half-layout rotation of x (B,H,N,D) bf16, fp32 arithmetic, rounded to bf16; tile_max (may be NULL) receives
  * [B*H][ceil(N/64)] floats, the largest norm of a rotated row in every 64-row tile.
- * Replaces apply_rotary_emb (reference fused-rope/rope_attn_pytorch.py:60-91). */
+ * Replaces apply_rotary_emb (reference fused-rope/rope_attn_pytorch.py:71-84, rotate_half :52-68). */
 int corope_rope_rotate(const void *x, const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
                        void *y, float *tile_max, int B, int H, int N, int D, void *stream);
 

@@ -93,6 +93,48 @@ def test_null_and_misaligned_pointers_are_rejected_before_any_launch(pkg):
         pkg._lib.check(rc, "corope_gqa_fwd")
 
 
+def test_composite_entry_points_check_every_argument_before_the_first_launch(pkg):
+    """The entry points that make several launches look at ALL their arguments first: a null or misaligned pointer that
+    only the last launch would use is refused with a BADARG / ALIGN status (a launch attempted here, without a GPU, would
+    come back as a LAUNCH status instead)."""
+    lib = pkg._lib.load()
+    buf = ctypes.create_string_buffer(4096)
+    ok = (ctypes.addressof(buf) + 15) & ~15
+    tail = (1, 1, 8, 64, 1.0, 1)
+    # corope_rope_attn_bwd(q, k, v, o, d_o, lse, delta, cos, sin, stride, dq, dk, dv, ...): dq is used by the last launch
+    rc = lib.corope_rope_attn_bwd(ok, ok, ok, ok, ok, ok, ok, ok, ok, 64, None, ok, ok, *tail, None)
+    assert rc == -1 and "null" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_bwd(ok, ok, ok, ok, ok, ok, ok, ok, ok, 64, ok + 2, ok, ok, *tail, None)
+    assert rc == -3 and "aligned" in pkg._lib.last_error()
+    # the same on rotated operands: dk / dv belong to the second launch
+    rc = lib.corope_rope_attn_bwd_prerotated(ok, ok, ok, ok, ok, ok, ok, ok, ok, 64, ok, ok, None, *tail, None)
+    assert rc == -1 and "null" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_bwd_prerotated(ok, ok, ok, ok, ok, ok, ok, ok, ok, 64, ok, ok + 4, ok, *tail, None)
+    assert rc == -3
+    # with a workspace: the rotation passes come first, dq last
+    need = lib.corope_rope_attn_bwd_workspace_bytes(1, 1, 8, 64)
+    rc = lib.corope_rope_attn_bwd_ws(ok, ok, ok, ok, ok, ok, ok, ok, ok, 64, None, ok, ok, *tail, ok, need, None)
+    assert rc == -1 and "null" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_bwd_ws(ok, ok, ok, ok, ok, ok, ok, ok, ok, 64, ok, ok, ok, *tail, ok, need - 1, None)
+    assert rc == -1 and "workspace" in pkg._lib.last_error()
+    # dK+dV as two launches: v and dk belong to the second
+    rc = lib.corope_rope_attn_bwd_dkdv(ok, ok, None, ok, ok, ok, ok, ok, 64, ok, ok, *tail, None)
+    assert rc == -1 and "null" in pkg._lib.last_error()
+    # training forward: o and lse belong to the second launch (the first rotates K)
+    rc = lib.corope_rope_attn_fwd_train(ok, ok, ok, ok, ok, 64, None, ok, ok, ok, ok, *tail, None)
+    assert rc == -1 and "null" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_fwd_train(ok, ok, ok, ok, ok, 64, ok, ok + 8, ok, ok, ok, *tail, None)
+    assert rc == -3
+    # grouped-query forward with a rotation pass: q belongs to the second launch
+    rc = lib.corope_rope_attn_fwd_gqa(None, ok, ok, ok, ok, 64, ok, ok, None, ok, ok, 1, 4, 2, 8, 64, 1.0, 1, None)
+    assert rc == -1 and "null" in pkg._lib.last_error()
+    # the forward that allocates nothing refuses oversized shapes and bad pointers alike without a launch
+    rc = lib.corope_rope_attn_fwd_noalloc(ok, ok, ok, ok, ok, 64, ok, None, *tail, None)
+    assert rc == -1 and "null" in pkg._lib.last_error()
+    rc = lib.corope_rope_attn_fwd_noalloc(ok, ok, ok, ok, ok, 128, ok, ok, 4, 32, 4096, 128, 1.0, 1, None)
+    assert rc == -2 and "scratch" in pkg._lib.last_error()
+
+
 def test_grouped_query_argument_checks(pkg):
     """Head-count and pointer checks of the grouped-query entry points happen before any launch."""
     lib = pkg._lib.load()
