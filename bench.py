@@ -328,15 +328,26 @@ def bench_corope(args):
             sys.exit(pkg._lib.last_error())
 
     bsteps = max(3, args.steps // 3)
-    for _ in range(2):
-        bwd_step()
-    bev = [torch.cuda.Event(enable_timing=True) for _ in range(bsteps + 1)]
-    bev[0].record()
-    for i in range(bsteps):
-        bwd_step()
-        bev[i + 1].record()
-    torch.cuda.synchronize()
-    bms = sum(bev[i].elapsed_time(bev[i + 1]) for i in range(bsteps)) / bsteps
+
+    def time_bwd():
+        for _ in range(2):
+            bwd_step()
+        bev = [torch.cuda.Event(enable_timing=True) for _ in range(bsteps + 1)]
+        bev[0].record()
+        for i in range(bsteps):
+            bwd_step()
+            bev[i + 1].record()
+        torch.cuda.synchronize()
+        return sum(bev[i].elapsed_time(bev[i + 1]) for i in range(bsteps)) / bsteps
+
+    bms = time_bwd()
+    # the same backward with less scratch: the groups are then walked in passes of as many as fit
+    full_bytes, one = ws_bytes, lib.corope_gqa_bwd_min_workspace_bytes(B, Hq, Hkv, N, D)
+    by_workspace = {}
+    for groups in (4, 1):
+        ws_bytes = groups * one
+        by_workspace[f"{groups} of {B * Hkv} groups per pass, {ws_bytes / 2**30:.2f} GiB"] = round(time_bwd(), 4)
+    ws_bytes = full_bytes
     # issue slots per (sin, cos) pair, counted as for the forward (a transcendental = 2 slots): scores kernel 11 + 4 (phase
     # 2, unpack 2, rotate 4, pack 1, LDS 2; sin, cos); dk kernel 8 + 4 (phase 2, rotate-accumulate 4, gate path 2; sin, cos);
     # the per-head sums run on the matrix cores
@@ -356,7 +367,7 @@ def bench_corope(args):
            "roofline": {"bound": "valu", "kernel": "corope_gqa_fwd", "achieved": round(fwd_instr / (kms * 1e-3) * 1e-12, 3),
                         "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T issue slots/s",
                         "frac": round(fwd_instr / (kms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4), "traffic": None},
-           "backward": {"ms": round(bms, 4), "steps": bsteps, "workspace_gib": round(ws_bytes / 2**30, 2),
+           "backward": {"ms": round(bms, 4), "steps": bsteps, "workspace_gib": round(ws_bytes / 2**30, 2), "ms_by_workspace": by_workspace,
                         "sincos_pairs_per_s": round(2 * pairs / (bms * 1e-3), 1),
                         "tflops_attention_equivalent": round(2.5 * flops / (bms * 1e-3) * 1e-12, 2),
                         "roofline": {"bound": "valu", "kernel": "corope_gqa_bwd (6 launches)",

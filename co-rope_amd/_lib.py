@@ -49,6 +49,7 @@ SIGNATURES = {
     "corope_rope_attn_bwd_gqa": (_I, [_P, _P, _I] + [_P] * 7 + [_L, _P, _P, _P] + [_I] * 5 + [_F, _I, _P]),
     "corope_gqa_fwd": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P]),
     "corope_gqa_bwd_workspace_bytes": (_L, [_I, _I, _I, _I, _I]),
+    "corope_gqa_bwd_min_workspace_bytes": (_L, [_I, _I, _I, _I, _I]),
     "corope_gqa_bwd": (_I, [_P] * 8 + [_I] * 5 + [_F, _F, _P, _L, _P]),
 }
 

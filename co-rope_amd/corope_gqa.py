@@ -59,18 +59,32 @@ class _CoRopeGqaAttn(torch.autograd.Function):
 
 
 def backward_workspace_bytes(B, Hq, Hkv, N, D):
-    """Scratch memory the backward needs: (2 * B * Hkv + 3 * B * Hq) packed lower-triangular N x N fp32 matrices
-    (about N * N / 2 + 32 * N values each), plus B * Hkv * N * D values."""
+    """Scratch memory for a backward that handles all groups in one pass: (2 * B * Hkv + 3 * B * Hq) packed
+    lower-triangular N x N fp32 matrices (about N * N / 2 + 32 * N values each), plus B * Hkv * N * D values."""
     n = _lib.load().corope_gqa_bwd_workspace_bytes(B, Hq, Hkv, N, D)
     if n < 0:
         raise ValueError(_lib.last_error() or "unsupported Co-RoPE shape")
     return n
 
 
+def backward_min_workspace_bytes(B, Hq, Hkv, N, D):
+    """The smallest scratch the backward accepts: one (batch, key/value head) group's matrices."""
+    n = _lib.load().corope_gqa_bwd_min_workspace_bytes(B, Hq, Hkv, N, D)
+    if n < 0:
+        raise ValueError(_lib.last_error() or "unsupported Co-RoPE shape")
+    return n
+
+
+# The backward's scratch when the caller brings none: as many groups per pass as fit this share of the free device memory
+# (at least one group; all of them in one pass is fastest, see include/corope_amd.h).
+WORKSPACE_FREE_SHARE = 0.6
+
+
 def corope_gqa_backward(q, k, v, grad_output, sm_scale, theta, workspace=None, out=None):
     """(dq, dk, dv) of the Co-RoPE GQA attention for upstream gradient ``grad_output`` (reference :459-577).
 
-    ``workspace`` may be a caller-owned uint8/float tensor of at least ``backward_workspace_bytes`` bytes; ``out`` the
+    ``workspace`` may be a caller-owned uint8/float tensor of at least ``backward_min_workspace_bytes`` bytes (the groups
+    are then processed in passes of as many as fit; ``backward_workspace_bytes`` holds them all); ``out`` the
     forward's output for the same inputs (optional: it only steadies the rounding of dQ on sharply peaked rows)."""
     lib = _lib.load()
     B, Hq, N, D = q.shape
@@ -78,9 +92,16 @@ def corope_gqa_backward(q, k, v, grad_output, sm_scale, theta, workspace=None, o
     q, k, v, d_o = q.contiguous(), k.contiguous(), v.contiguous(), grad_output.to(q.dtype).contiguous()
     out_c = None if out is None else out.contiguous()
     o_ptr = None if out_c is None else out_c.data_ptr()
-    need = backward_workspace_bytes(B, Hq, Hkv, N, D)
     if workspace is None:
-        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        one, full = backward_min_workspace_bytes(B, Hq, Hkv, N, D), backward_workspace_bytes(B, Hq, Hkv, N, D)
+        free, _ = torch.cuda.mem_get_info(q.device)
+        free += torch.cuda.memory_reserved(q.device) - torch.cuda.memory_allocated(q.device)   # what torch's cache holds idle
+        if one > free:
+            raise MemoryError(f"Co-RoPE backward at B={B} Hq={Hq} Hkv={Hkv} N={N} D={D} needs at least {one} bytes of "
+                              f"scratch (one key/value group; {full} for all groups in one pass); {free} bytes are free "
+                              f"on {q.device}")
+        groups = max(1, int(free * WORKSPACE_FREE_SHARE) // one)
+        workspace = torch.empty(min(full, groups * one), dtype=torch.uint8, device=q.device)
     have = workspace.numel() * workspace.element_size()
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     with torch.cuda.device(q.device):

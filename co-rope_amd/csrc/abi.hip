@@ -595,6 +595,11 @@ int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D) {
   return 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N, D);
 }
 
+int64_t corope_gqa_bwd_min_workspace_bytes(int B, int Hq, int Hkv, int N, int D) {
+  if (corope_gqa_check(B, Hq, Hkv, N, D, 1.f, 2.f)) return -1;
+  return 4 * corope::corope_gqa_bwd_workspace_floats(1, Hq / Hkv, 1, N, D);
+}
+
 int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk, void* dv,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void* workspace,
                    int64_t workspace_bytes, void* stream) {
@@ -604,9 +609,10 @@ int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* o, c
   if (rc) return rc;
   if (o != nullptr && !aligned16(o)) return fail(COROPE_E_ALIGN, "corope_gqa_bwd: pointer %p is not 16-byte aligned", o);
   if ((int64_t)B * Hq > 65535) return fail(COROPE_E_UNSUPPORTED, "corope_gqa_bwd: B * Hq = %lld exceeds 65535", (long long)B * Hq);
-  const int64_t need = 4 * corope::corope_gqa_bwd_workspace_floats(B, Hq, Hkv, N, D);
+  const int64_t need = 4 * corope::corope_gqa_bwd_workspace_floats(1, Hq / Hkv, 1, N, D);
   if (workspace_bytes < need)
-    return fail(COROPE_E_BADARG, "corope_gqa_bwd: workspace of %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
+    return fail(COROPE_E_BADARG, "corope_gqa_bwd: workspace of %lld bytes, at least %lld needed (one group's matrices)",
+                (long long)workspace_bytes, (long long)need);
   corope::CoropeBwdParams p{};
   p.q = static_cast<const uint16_t*>(q);
   p.k = static_cast<const uint16_t*>(k);
@@ -622,7 +628,7 @@ int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* o, c
   p.Hq = Hq;
   p.Hkv = Hkv;
   p.N = N;
-  return launch_status("corope_gqa_bwd", corope::launch_corope_gqa_bwd(p, D, static_cast<float*>(workspace),
+  return launch_status("corope_gqa_bwd", corope::launch_corope_gqa_bwd(p, D, static_cast<float*>(workspace), workspace_bytes / 4,
                                                                        static_cast<hipStream_t>(stream)));
 }
 

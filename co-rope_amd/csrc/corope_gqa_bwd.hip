@@ -38,6 +38,8 @@
 // queries convert exactly, and 11 significant bits keep scores accurate at sm_scale = 1 too; the products on unrotated
 // rows (W K, P dO, the row dots) take bf16 operands; sums, statistics, delta, dS/ddelta and everything stored in the
 // workspace are fp32.
+#include <algorithm>
+
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -231,15 +233,25 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
   // as weights and are corrected by (Delta - ref) afterwards, which is exact for any ref; the closer ref is to Delta, the
   // less the two sums cancel (rows dominated by one key would otherwise lose the 11 bits of the weights).  With the forward
   // output at hand ref = rowsum(O o dO), equal to Delta up to O's rounding; without it ref = 0.
+  // The weights e (dP - ref) go to the matrix cores as fp16, whose 5 exponent bits would tie the result to the scale of
+  // dO (overflow from |dP - ref| ~ 1e3 on, nothing left of a mean-reduced loss's 1e-7): they are divided by a power of two
+  // w_scale >= 4 |dO_i| first (|dP_ij| <= |dO_i| |v_j|, so the scaled weights are at most e^4 |v_j| / 4 whatever dO is)
+  // and the sum is multiplied back afterwards -- exact both ways.
   float dref[G];
+  int w_exp[G];   // w_scale = 2^w_exp, wave-uniform (scalar registers)
 #pragma unroll
   for (int h = 0; h < G; ++h) {
-    float acc = 0.f;
-    if (p.o != nullptr) {
-      const int64_t off = ((int64_t)(head0 + h) * N + i) * D;
-      for (int d = lane; d < D; d += kWave) acc = __builtin_fmaf(bf16_to_f(p.o[off + d]), bf16_to_f(p.d_o[off + d]), acc);
+    float acc = 0.f, sq = 0.f;
+    const int64_t off = ((int64_t)(head0 + h) * N + i) * D;
+    for (int d = lane; d < D; d += kWave) {
+      const float g_d = bf16_to_f(p.d_o[off + d]);
+      sq = __builtin_fmaf(g_d, g_d, sq);
+      if (p.o != nullptr) acc = __builtin_fmaf(bf16_to_f(p.o[off + d]), g_d, acc);
     }
     dref[h] = wave_sum(acc);
+    int ex = 0;
+    (void)frexpf(__builtin_sqrtf(wave_sum(sq)), &ex);       // |dO_i| = m 2^ex with m in [0.5, 1); 0 gives ex = 0
+    w_exp[h] = __builtin_amdgcn_readfirstlane(max(-100, min(100, ex + 2)));
   }
   // A chunk's 64 key rows are one contiguous block of global memory: the wave fetches it with consecutive 16-byte pieces
   // per lane (full cache lines per instruction) and parks it in the LDS tile, where each lane then finds its own key's
@@ -389,7 +401,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
       const float e = __expf(acc[h] - m_run[h]);   // 0 for the keys beyond the diagonal
       l_run[h] += e;
       pd_run[h] = __builtin_fmaf(e, dpv[h], pd_run[h]);
-      wts[(2 * h) * WS + lane] = f_to_f16(e * (dpv[h] - dref[h]));
+      // (clamped to fp16's range: a value row |v_j| in the thousands saturates instead of turning into infinity)
+      wts[(2 * h) * WS + lane] = f_to_f16(fminf(fmaxf(e * ldexpf(dpv[h] - dref[h], -w_exp[h]), -65504.f), 65504.f));
       wts[(2 * h + 1) * WS + lane] = f_to_f16(e);
     }
     if (c > 0) {
@@ -420,17 +433,19 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
   // 2G on are idle
   {
     float my_inv = 0.f, my_dsum = 0.f;
+    int my_exp = 0;
 #pragma unroll
     for (int h = 0; h < G; ++h) {
       my_inv = vr / 2 == h ? inv_l[h] : my_inv;
       my_dsum = vr / 2 == h ? dsum[h] - dref[h] : my_dsum;
+      my_exp = vr / 2 == h ? w_exp[h] : my_exp;
     }
 #pragma unroll
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const float other = __shfl_xor(dqa[db][e], 1);
-        if (vr < 2 * G) dqa[db][e] = (dqa[db][e] - my_dsum * other) * my_inv;
+        if (vr < 2 * G) dqa[db][e] = (ldexpf(dqa[db][e], my_exp) - my_dsum * other) * my_inv;
       }
   }
   // dq of the heads 1..G-1 is final; the leader's still lacks the gate path W K, which a separate plain matrix product
@@ -886,7 +901,11 @@ static hipError_t launch_corope_bwd_d(const CoropeBwdParams& p, const CoropeBwdW
   }
 }
 
-hipError_t launch_corope_gqa_bwd(const CoropeBwdParams& p, int D, float* workspace, hipStream_t stream) {
+// One pass of the launch sequence handles `gc` (batch, key/value head) groups with gc * (2 + 3 G) packed matrices; a
+// workspace smaller than the whole problem's is walked in passes of as many groups as fit (every group is independent:
+// its queries' heads, its key/value head, its slices of dq, dk, dv).
+hipError_t launch_corope_gqa_bwd(const CoropeBwdParams& p, int D, float* workspace, int64_t workspace_floats,
+                                 hipStream_t stream) {
   CoropeBwdFreqs fr{};
   // theta^(-2d/D) evaluated like the reference's torch expression (fp32 exponent, fp32 power), as in the forward
   for (int d = 0; d < D / 2; ++d) {
@@ -895,8 +914,30 @@ hipError_t launch_corope_gqa_bwd(const CoropeBwdParams& p, int D, float* workspa
     fr.rad[d] = inv;
     fr.turns[d] = (float)((double)inv / 6.283185307179586);
   }
-  CoropeBwdWs ws{workspace, tri_row_start(p.N), p.B * p.Hkv, p.B * p.Hq};
-  return D == 128 ? launch_corope_bwd_d<128>(p, ws, fr, stream) : launch_corope_bwd_d<64>(p, ws, fr, stream);
+  const int G = p.Hq / p.Hkv, n_groups = p.B * p.Hkv;
+  const int64_t per_group = corope_gqa_bwd_workspace_floats(1, G, 1, p.N, D);
+  const int per_pass = (int)std::min<int64_t>(n_groups, workspace_floats / per_group);
+  if (per_pass < 1) return hipErrorInvalidValue;
+  for (int g0 = 0; g0 < n_groups; g0 += per_pass) {
+    const int gc = std::min(per_pass, n_groups - g0);
+    CoropeBwdParams c = p;
+    const int64_t qoff = (int64_t)g0 * G * p.N * D, koff = (int64_t)g0 * p.N * D;
+    c.q += qoff;
+    c.d_o += qoff;
+    c.dq += qoff;
+    if (c.o != nullptr) c.o += qoff;
+    c.k += koff;
+    c.v += koff;
+    c.dk += koff;
+    c.dv += koff;
+    c.B = 1;
+    c.Hkv = gc;
+    c.Hq = gc * G;
+    CoropeBwdWs ws{workspace, tri_row_start(p.N), gc, gc * G};
+    const hipError_t e = D == 128 ? launch_corope_bwd_d<128>(c, ws, fr, stream) : launch_corope_bwd_d<64>(c, ws, fr, stream);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 }  // namespace corope

@@ -126,7 +126,8 @@ hipError_t launch_bwd_dkdv_fused(const BwdParams& p, int D, bool causal, hipStre
 hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_corope_gqa_fwd(const CoropeParams& p, int D, hipStream_t stream);
 int64_t corope_gqa_bwd_workspace_floats(int B, int Hq, int Hkv, int N, int D);
-hipError_t launch_corope_gqa_bwd(const CoropeBwdParams& p, int D, float* workspace, hipStream_t stream);
+hipError_t launch_corope_gqa_bwd(const CoropeBwdParams& p, int D, float* workspace, int64_t workspace_floats,
+                                 hipStream_t stream);   // any workspace that holds at least one group's matrices
 hipError_t launch_rope_freqs(float* cosp, float* sinp, int n_pos, int D, int width, int64_t row_stride, int pos0,
                              float theta, hipStream_t stream);
 

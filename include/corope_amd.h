@@ -245,13 +245,21 @@ int corope_gqa_fwd(const void *q, const void *k, const void *v, void *o,
  * key/value head (the leader head's dq before its gate-path term is added). */
 int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D);
 
+/* The smallest workspace corope_gqa_bwd accepts: the matrices of ONE (batch, key/value head) group, i.e. the figure above
+ * divided by B*Hkv.  Groups are independent, so with a workspace between the two sizes the launch sequence runs once per
+ * batch of as many groups as fit.  Fewer, larger passes are much faster, because two of the kernels spread over key blocks
+ * x groups only: at B2 Hq32 Hkv8 N4096 D128 on MI355X 14.3 ms with all 16 groups in one pass (7.1 GiB), 31 ms with 4 per
+ * pass (1.8 GiB), 94 ms with 1 (0.45 GiB) -- give it what memory allows.  -1 for sizes corope_gqa_check rejects. */
+int64_t corope_gqa_bwd_min_workspace_bytes(int B, int Hq, int Hkv, int N, int D);
+
 /* Co-RoPE grouped-query attention backward (causal only): dq (B,Hq,N,D), dk/dv (B,Hkv,N,D) from q, k, v and dO.
  * Replaces _attention.backward (reference corope-exp/flash_attn_co_rope_gqa_triton.py:459-577), which recomputes the
  * forward densely in PyTorch with (B,Hq,N,N,D/2) temporaries; the same gradients (including the path through the
  * leader head's gates, :548-561) are produced here with packed triangular N x N matrices of scalars in `workspace`.
  * Like the reference's, it needs neither the forward's output nor its row statistics; `o` may be NULL.  When the forward's output is
  * passed, rowsum(O o dO) serves as a reference value that keeps dQ accurate for rows dominated by a single key (the
- * result is mathematically the same with or without it).  The workspace need not be initialised.  Limit: B*Hq <= 65535. */
+ * result is mathematically the same with or without it).  The workspace need not be initialised and may be any size from
+ * corope_gqa_bwd_min_workspace_bytes up (see there).  Limit: B*Hq <= 65535. */
 int corope_gqa_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,
                    void *dq, void *dk, void *dv,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta,

@@ -163,7 +163,11 @@ def test_corope_backward_argument_checks(pkg):
     assert lib.corope_gqa_bwd_workspace_bytes(1, 4, 2, 33, 96) == -1      # head dim not built
     buf = ctypes.create_string_buffer(4096)
     ok = (ctypes.addressof(buf) + 15) & ~15
-    need = lib.corope_gqa_bwd_workspace_bytes(1, 4, 2, 8, 64)
+    # the smallest accepted workspace holds one (batch, kv head) group: the full figure divided by the number of groups
+    assert lib.corope_gqa_bwd_min_workspace_bytes(2, 32, 8, 4096, 128) * 16 == lib.corope_gqa_bwd_workspace_bytes(2, 32, 8, 4096, 128)
+    assert lib.corope_gqa_bwd_min_workspace_bytes(1, 5, 2, 33, 64) == -1
+    need = lib.corope_gqa_bwd_min_workspace_bytes(1, 4, 2, 8, 64)
+    assert 2 * need == lib.corope_gqa_bwd_workspace_bytes(1, 4, 2, 8, 64)
     args = lambda ws, nbytes, dq=ok, o=None: (ok, ok, ok, o, ok, dq, ok, ok, 1, 4, 2, 8, 64, 0.125, 1e4, ws, nbytes, None)
     assert lib.corope_gqa_bwd(*args(None, need)) == -1 and "null" in pkg._lib.last_error()
     assert lib.corope_gqa_bwd(*args(ok, need, dq=ok + 2)) == -3 and "aligned" in pkg._lib.last_error()

@@ -124,11 +124,13 @@ def test_corope_backward_gate_path_is_material_and_right(pkg):
 
 
 def test_corope_backward_caller_workspace_and_reuse(pkg):
-    """A caller-owned workspace filled with garbage gives the same gradients; a short one is refused."""
+    """A caller-owned workspace filled with garbage gives the same gradients, whether it holds every group's matrices
+    (one pass), some of them (the groups are walked in passes of as many as fit) or a single group's; one that cannot
+    hold a single group's is refused."""
     import importlib
     mod = importlib.import_module("corope_amd.corope_gqa")
     dev = torch.device("cuda:0")
-    B, Hq, Hkv, N, D = 1, 4, 2, 70, 64
+    B, Hq, Hkv, N, D = 2, 6, 3, 70, 64
     q, k, v, d_o = (t.to(dev, torch.bfloat16) for t in _inputs(B, Hq, Hkv, N, D, seed=3))
     need = mod.backward_workspace_bytes(B, Hq, Hkv, N, D)
     packed = sum(64 * (i // 64 + 1) for i in range(N))          # rows hold the keys j <= i, padded to 64-key chunks
@@ -139,8 +141,16 @@ def test_corope_backward_caller_workspace_and_reuse(pkg):
     torch.cuda.synchronize()
     for x, y in zip(a, b):
         assert torch.equal(x, y)
+    one = mod.backward_min_workspace_bytes(B, Hq, Hkv, N, D)
+    assert one * B * Hkv == need
+    for groups in (1, 2, 4):              # 6 groups in passes of 1, of 2, and of 4 + 2
+        ws.fill_(float("nan"))
+        c = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4, workspace=ws[: groups * one // 4 + 3])
+        torch.cuda.synchronize()
+        for x, y in zip(a, c):
+            assert torch.equal(x, y), groups
     with pytest.raises(ValueError):
-        mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4, workspace=ws[: need // 4 - 1])
+        mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4, workspace=ws[: one // 4 - 1])
 
 
 def test_corope_random_shapes_forward_and_backward(pkg):
@@ -172,3 +182,28 @@ def test_corope_random_shapes_forward_and_backward(pkg):
         for name, got, ref, tol in checks:
             ok, err = within_bar(got.float().cpu(), ref.float(), tol)
             assert torch.isfinite(got).all() and ok, (case, name, err)
+
+
+@pytest.mark.parametrize("with_o", [True, False])
+@pytest.mark.parametrize("B,Hq,Hkv,N,D", [(1, 4, 2, 130, 64), (1, 8, 2, 100, 128)])
+def test_corope_backward_does_not_depend_on_the_scale_of_dO(pkg, B, Hq, Hkv, N, D, with_o):
+    """Upstream gradients of a mean-reduced loss (1e-6 and below) and unnormalised ones (1e3): the backward is linear in
+    dO, and a power-of-two factor commutes with every rounding in it (the fp16 weights of the dQ sums are normalised per
+    row by a power of two of |dO_i|), so grad(2^k dO) == 2^k grad(dO) bit for bit -- and both match the oracle."""
+    import importlib
+    mod = importlib.import_module("corope_amd.corope_gqa")
+    dev = torch.device("cuda:0")
+    q, k, v, d_o = _inputs(B, Hq, Hkv, N, D, seed=11)
+    scale = 1 / math.sqrt(D)
+    qd, kd, vd, gd = (t.to(dev, torch.bfloat16) for t in (q, k, v, d_o))
+    out = pkg.corope_attention(qd, kd, vd, True, scale, 10000.0) if with_o else None
+    base = [t.float().cpu() for t in mod.corope_gqa_backward(qd, kd, vd, gd, scale, 10000.0, out=out)]
+    _compare(base, _oracle_grads(q, k, v, d_o, scale, 10000.0), Hq // Hkv)
+    for kexp in (-24, -20, 10, 14):      # 6e-8, 1e-6, 1e3, 1.6e4
+        f = 2.0 ** kexp
+        got = [t.float().cpu() for t in mod.corope_gqa_backward(qd, kd, vd, (gd.float() * f).to(torch.bfloat16), scale, 10000.0,
+                                                                  out=out)]
+        torch.cuda.synchronize()
+        for name, a, b in zip(("dQ", "dK", "dV"), got, base):
+            assert torch.isfinite(a).all(), (name, kexp)
+            assert torch.equal(a, b * f), f"{name} at dO x 2^{kexp}: max rel diff {((a - b * f).abs() / (b.abs() * f + 1e-30)).max():.3e}"
