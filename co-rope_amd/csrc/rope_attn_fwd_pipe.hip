@@ -110,6 +110,9 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
   CopyStage<D, BLOCK_N, NT, Cfg::kVPad> vst;
   kst.load(kg, 0, N);
   vst.load(vg, 0, N);
+  // Lane i: largest rotated-key norm of tile i (the first 64 tiles; requested here so that it lands under the Q rows)
+  const uint32_t* tile_kmax_bits = reinterpret_cast<const uint32_t*>(p.tile_kmax) + (int64_t)kvs * n_k_tiles;
+  uint32_t kvec = tile_kmax_bits[min(lane, n_k_tiles - 1)];
 
   // ---- Q rows of this wave: load, rotate, keep as the B operand (through a wave-private LDS tile: the global loads and
   // the copy of the rotated rows kept for the backward then touch whole row segments) ----------------------------------
@@ -145,7 +148,6 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
       }
     q_bound_wave = __builtin_sqrtf(wave_reduce_max(half_sum(ss))) * scale * 1.01f;
   }
-  const uint32_t* tile_kmax_bits = reinterpret_cast<const uint32_t*>(p.tile_kmax) + (int64_t)kvs * n_k_tiles;
 
   f32x16 oacc[NDB];
 #pragma unroll
@@ -195,10 +197,10 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
   // Reference value (raw-score units) that puts every tile this wave will see within the margin.
   float lift_target;
   {
-    uint32_t kall = 0;
-    for (int t0 = 0; t0 <= t_last; t0 += kWave) {
+    uint32_t kall = lane <= t_last ? kvec : 0u;   // non-negative floats order like their bit patterns
+    for (int t0 = kWave; t0 <= t_last; t0 += kWave) {
       const int tt = t0 + lane;
-      kall = max(kall, tt <= t_last ? tile_kmax_bits[tt] : 0u);   // non-negative floats order like their bit patterns
+      kall = max(kall, tt <= t_last ? tile_kmax_bits[tt] : 0u);
     }
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) kall = max(kall, (uint32_t)__shfl_xor((int)kall, m));
@@ -210,7 +212,6 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
   // reference moves.  Lane i of kvec holds the key-norm maximum of tile kvec_base + i.
   uint32_t thr_bits = 0;
   int kvec_base = 0;
-  uint32_t kvec = tile_kmax_bits[min(lane, n_k_tiles - 1)];
 
   auto stage_next = [&](int t) __attribute__((always_inline)) {
     int ko = koff_next, vo = voff_next;
