@@ -19,6 +19,9 @@ LIB = os.path.join(LIBDIR, "libcorope_amd.so")
 TRACE_LIB = os.path.join(LIBDIR, "libcorope_amd_trace.so")
 MFMA_RATE = os.path.join(LIBDIR, "mfma_rate")
 
+# compiled a second time with -DCOROPE_F16 (fp16 elements, namespace corope_f16)
+F16_SOURCES = ["rope_attn_fwd.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip"]
+
 SOURCES = ["abi.hip", "rope_freqs.hip", "rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_fwd_pipe.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip", "corope_gqa_bwd.hip"]
 
 # -packed-fp32-ops is switched off: packed fp32 VALU forms are not used by these kernels.
@@ -56,9 +59,9 @@ def _link(objs, out, shared=True):
 def build(verbose=False, extra_flags=(), extras=True):
     """Compiles every source.  ``extras``: also the trace variant of the library and the mfma_rate program."""
     os.makedirs(LIBDIR, exist_ok=True)
-    jobs = [(s, list(extra_flags), "") for s in SOURCES]
+    jobs = [(s, list(extra_flags), "") for s in SOURCES] + [(s, list(extra_flags) + ["-DCOROPE_F16"], ".f16") for s in F16_SOURCES]
     if extras:
-        jobs += [(s, list(extra_flags) + ["-DCOROPE_TRACE"], ".trace") for s in SOURCES]
+        jobs += [(s, j[1] + ["-DCOROPE_TRACE"], j[2] + ".trace") for j in list(jobs) for s in [j[0]]]
         jobs += [("mfma_rate.hip", [], "")]
     with ThreadPoolExecutor(max_workers=8) as ex:
         results = list(ex.map(lambda j: _compile(*j), jobs))
@@ -66,7 +69,7 @@ def build(verbose=False, extra_flags=(), extras=True):
         for (_, err), j in zip(results, jobs):
             if err.strip():
                 print(f"--- {j[0]}{j[2]}\n{err}", file=sys.stderr)
-    n = len(SOURCES)
+    n = len(SOURCES) + len(F16_SOURCES)
     _link([o for o, _ in results[:n]], LIB)
     if extras:
         _link([o for o, _ in results[n:2 * n]], TRACE_LIB)

@@ -33,14 +33,15 @@ class _CoRopeGqaAttn(torch.autograd.Function):
             raise ValueError(f"CoRoPE backbone currently limits group_size <= 8 (got {Hq // Hkv}).")
         if not (q.is_cuda and k.is_cuda and v.is_cuda):
             raise ValueError("Co-RoPE attention runs on the GPU only: q, k, v must be on a HIP device")
-        if not (q.dtype == k.dtype == v.dtype == torch.bfloat16):
-            raise ValueError(f"q, k, v must be bfloat16 (got {q.dtype}, {k.dtype}, {v.dtype})")
+        if not (q.dtype == k.dtype == v.dtype and q.dtype in (torch.bfloat16, torch.float16)):
+            raise ValueError(f"q, k, v must all be bfloat16 or all float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
         lib = _lib.load()
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         o = torch.empty_like(q)
         with torch.cuda.device(q.device):
-            rc = lib.corope_gqa_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, Hq, Hkv, N, D,
-                                    float(sm_scale), float(theta), torch.cuda.current_stream(q.device).cuda_stream)
+            fwd = lib.corope_gqa_fwd_f16 if q.dtype == torch.float16 else lib.corope_gqa_fwd
+            rc = fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, Hq, Hkv, N, D,
+                     float(sm_scale), float(theta), torch.cuda.current_stream(q.device).cuda_stream)
         _lib.check(rc, "corope_gqa_fwd")
         # what the reference keeps (:451), minus inv_freq (theta is enough), plus the output: the backward takes a
         # reference value for its row sums from it (accuracy of dQ on sharply peaked rows; not needed mathematically)
@@ -54,6 +55,8 @@ class _CoRopeGqaAttn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         q, k, v, o = ctx.saved_tensors
+        if q.dtype != torch.bfloat16:
+            raise ValueError("the Co-RoPE backward is built for bfloat16 tensors only (the forward also takes float16)")
         dq, dk, dv = corope_gqa_backward(q, k, v, grad_output, ctx.sm_scale, ctx.theta, out=o)
         return dq, dk, dv, None, None, None, None
 

@@ -556,6 +556,51 @@ int corope_rope_attn_bwd_gqa(const void* q, const void* k, int prerotated, const
   return launch_status(what, corope::launch_bwd_dq(p, D, causal != 0, st));
 }
 
+// ---- fp16 tensors (the reference's dtype): the same kernels built for fp16 elements -------------------------------------
+int corope_rope_attn_fwd_f16(const void* q, const void* k, const void* v, const float* freqs_cos, const float* freqs_sin,
+                             int64_t freq_row_stride, void* o, float* lse, int B, int H, int N, int D, float sm_scale,
+                             int causal, void* stream) {
+  const char* what = "rope_attn_fwd_f16";
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
+  if (rc) return rc;
+  rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse});
+  if (rc) return rc;
+  corope::FwdParams p{};
+  p.q = static_cast<const uint16_t*>(q);
+  p.k = static_cast<const uint16_t*>(k);
+  p.v = static_cast<const uint16_t*>(v);
+  p.cos = freqs_cos;
+  p.sin = freqs_sin;
+  p.o = static_cast<uint16_t*>(o);
+  p.lse = lse;
+  p.fstride = freq_row_stride;
+  p.qk_scale = sm_scale * kLog2e;
+  p.N = N;
+  p.BH = B * H;
+  p.H = p.Hkv = H;
+  return launch_status(what, corope_f16::launch_rope_attn_fwd(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+}
+
+int corope_rope_attn_bwd_f16(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                             float* delta, const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* dq,
+                             void* dk, void* dv, int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
+  const char* what = "rope_attn_bwd_f16";
+  int rc = validate_bwd(what, B, H, N, D, freq_row_stride, sm_scale,
+                        {q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv});
+  if (rc) return rc;
+  corope::BwdParams p = make_bwd(q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, dk, dv, B, H, N,
+                                 sm_scale);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  rc = launch_status(what, corope_f16::launch_bwd_preprocess(p, D, st));
+  if (rc) return rc;
+  p.o = nullptr;   // delta comes from the pass above, not from the dQ kernel
+  rc = launch_status(what, corope_f16::launch_bwd_dv(p, D, causal != 0, st));
+  if (rc) return rc;
+  rc = launch_status(what, corope_f16::launch_bwd_dk(p, D, causal != 0, st));
+  if (rc) return rc;
+  return launch_status(what, corope_f16::launch_bwd_dq(p, D, causal != 0, st));
+}
+
 int corope_rope_freqs(float* freqs_cos, float* freqs_sin, int n_pos, int D, int width, int64_t freq_row_stride, int pos0,
                       float theta, void* stream) {
   if (n_pos <= 0 || D <= 0 || D % 2 != 0) return fail(COROPE_E_BADARG, "rope_freqs: n_pos must be positive and D even");
@@ -570,11 +615,15 @@ int corope_rope_freqs(float* freqs_cos, float* freqs_sin, int n_pos, int D, int 
                                                                pos0, theta, static_cast<hipStream_t>(stream)));
 }
 
-int corope_gqa_fwd(const void* q, const void* k, const void* v, void* o, int B, int Hq, int Hkv, int N, int D,
-                   float sm_scale, float theta, void* stream) {
+}  // extern "C" (reopened below)
+
+namespace {
+
+int corope_gqa_fwd_impl(const char* what, bool f16, const void* q, const void* k, const void* v, void* o, int B, int Hq, int Hkv,
+                        int N, int D, float sm_scale, float theta, void* stream) {
   int rc = corope_gqa_check(B, Hq, Hkv, N, D, sm_scale, theta);
   if (rc) return rc;
-  rc = check_ptrs("corope_gqa_fwd", {q, k, v, o});
+  rc = check_ptrs(what, {q, k, v, o});
   if (rc) return rc;
   corope::CoropeParams p{};
   p.q = static_cast<const uint16_t*>(q);
@@ -587,7 +636,22 @@ int corope_gqa_fwd(const void* q, const void* k, const void* v, void* o, int B, 
   p.Hq = Hq;
   p.Hkv = Hkv;
   p.N = N;
-  return launch_status("corope_gqa_fwd", corope::launch_corope_gqa_fwd(p, D, static_cast<hipStream_t>(stream)));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return launch_status(what, f16 ? corope_f16::launch_corope_gqa_fwd(p, D, st) : corope::launch_corope_gqa_fwd(p, D, st));
+}
+
+}  // namespace
+
+extern "C" {
+
+int corope_gqa_fwd(const void* q, const void* k, const void* v, void* o, int B, int Hq, int Hkv, int N, int D,
+                   float sm_scale, float theta, void* stream) {
+  return corope_gqa_fwd_impl("corope_gqa_fwd", false, q, k, v, o, B, Hq, Hkv, N, D, sm_scale, theta, stream);
+}
+
+int corope_gqa_fwd_f16(const void* q, const void* k, const void* v, void* o, int B, int Hq, int Hkv, int N, int D,
+                       float sm_scale, float theta, void* stream) {
+  return corope_gqa_fwd_impl("corope_gqa_fwd_f16", true, q, k, v, o, B, Hq, Hkv, N, D, sm_scale, theta, stream);
 }
 
 int64_t corope_gqa_bwd_workspace_bytes(int B, int Hq, int Hkv, int N, int D) {

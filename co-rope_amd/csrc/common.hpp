@@ -8,7 +8,16 @@
 #include <type_traits>
 #include <utility>
 
-namespace corope {
+// The attention kernels are written once for "the 16-bit element type" of q, k, v, dO and of every matrix-core operand:
+// bf16 in the normal build of a source file, fp16 when the same file is compiled with -DCOROPE_F16, which also moves
+// everything into the namespace corope_f16 so that both builds link into one library.
+#ifdef COROPE_F16
+#define COROPE_NS corope_f16
+#else
+#define COROPE_NS corope
+#endif
+
+namespace COROPE_NS {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -34,14 +43,16 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 }
 
 // ---- MFMA ------------------------------------------------------------------------------------
-// D(32x32) += A(32x16) * B(16x32), bf16 in, fp32 accumulate.
+// D(32x32) += A(32x16) * B(16x32), 16-bit elements in (bf16, or fp16 in the COROPE_F16 build), fp32 accumulate.
 //   A operand: lane l holds row (l % 32), contraction slots 8*(l / 32) .. +7
 //   B operand: lane l holds column (l % 32), contraction slots 8*(l / 32) .. +7
 //   D/C      : lane l holds column (l % 32); register i holds row 8*(i / 4) + 4*(l / 32) + (i % 4)
+#ifndef COROPE_F16
 __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
                                                  0, 0, 0);
 }
+#endif
 
 // The same tile shape with fp16 operands (11 significant bits instead of 8).
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
@@ -53,6 +64,21 @@ typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 __device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, f16x2));
 }
+
+#ifdef COROPE_F16
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) { return mfma32_f16(a, b, c); }
+#endif
+
+// ---- the element type of the attention kernels: two elements per 32-bit word, element 0 in the low half -------------
+#ifdef COROPE_F16
+__device__ __forceinline__ float elt_lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
+__device__ __forceinline__ float elt_hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
+__device__ __forceinline__ uint32_t pack_elts(float lo, float hi) { return pack_f16(lo, hi); }
+#else
+__device__ __forceinline__ float elt_lo(uint32_t w) { return bf16_lo(w); }
+__device__ __forceinline__ float elt_hi(uint32_t w) { return bf16_hi(w); }
+__device__ __forceinline__ uint32_t pack_elts(float lo, float hi) { return pack_bf16(lo, hi); }
+#endif
 
 // Row index (0..31) held by accumulator register i of lane-half h in a 32x32 MFMA result.
 __device__ __forceinline__ constexpr int acc_row(int i, int h) { return 8 * (i / 4) + 4 * h + (i % 4); }
@@ -142,12 +168,12 @@ struct RotStage {
   __device__ __forceinline__ void rotate(int it, u32x4& y1, u32x4& y2) const {
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      float a0 = bf16_lo(x1[it][w]), a1 = bf16_hi(x1[it][w]);
-      float b0 = bf16_lo(x2[it][w]), b1 = bf16_hi(x2[it][w]);
+      float a0 = elt_lo(x1[it][w]), a1 = elt_hi(x1[it][w]);
+      float b0 = elt_lo(x2[it][w]), b1 = elt_hi(x2[it][w]);
       float c0 = c[it][w / 2][(2 * w) % 4], c1 = c[it][w / 2][(2 * w) % 4 + 1];
       float s0 = s[it][w / 2][(2 * w) % 4], s1 = s[it][w / 2][(2 * w) % 4 + 1];
-      y1[w] = pack_bf16(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
-      y2[w] = pack_bf16(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+      y1[w] = pack_elts(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+      y2[w] = pack_elts(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
     }
   }
 
@@ -264,11 +290,11 @@ __device__ __forceinline__ void load_b_rows(u32x4 (&out)[D / 16], const uint16_t
       f32x4 s[2] = {*reinterpret_cast<const f32x4*>(sp + 16 * kc), *reinterpret_cast<const f32x4*>(sp + 16 * kc + 4)};
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
-        float a0 = bf16_lo(x1[w]), a1 = bf16_hi(x1[w]), b0 = bf16_lo(x2[w]), b1 = bf16_hi(x2[w]);
+        float a0 = elt_lo(x1[w]), a1 = elt_hi(x1[w]), b0 = elt_lo(x2[w]), b1 = elt_hi(x2[w]);
         float c0 = c[w / 2][(2 * w) % 4], c1 = c[w / 2][(2 * w) % 4 + 1];
         float s0 = s[w / 2][(2 * w) % 4], s1 = s[w / 2][(2 * w) % 4 + 1];
-        out[kc][w] = pack_bf16(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
-        out[kc + KC / 2][w] = pack_bf16(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+        out[kc][w] = pack_elts(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+        out[kc + KC / 2][w] = pack_elts(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
       }
     }
   }
@@ -357,11 +383,11 @@ struct WaveRows<D, true> {
       u32x4 y1, y2;
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
-        float a0 = bf16_lo(x1[i][w]), a1 = bf16_hi(x1[i][w]), b0 = bf16_lo(x2[i][w]), b1 = bf16_hi(x2[i][w]);
+        float a0 = elt_lo(x1[i][w]), a1 = elt_hi(x1[i][w]), b0 = elt_lo(x2[i][w]), b1 = elt_hi(x2[i][w]);
         float c0 = c[i][w / 2][(2 * w) % 4], c1 = c[i][w / 2][(2 * w) % 4 + 1];
         float s0 = s[i][w / 2][(2 * w) % 4], s1 = s[i][w / 2][(2 * w) % 4 + 1];
-        y1[w] = pack_bf16(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
-        y2[w] = pack_bf16(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+        y1[w] = pack_elts(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+        y2[w] = pack_elts(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
       }
       *reinterpret_cast<u32x4*>(wave_tile + RowTile<D>::off(r, u * 8)) = y1;
       *reinterpret_cast<u32x4*>(wave_tile + RowTile<D>::off(r, D / 2 + u * 8)) = y2;
@@ -430,8 +456,8 @@ __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], 
         }
       }
       uint16_t* d = byte_offset(dst, (uint32_t)row * (D * 2) + u * 16);
-      *reinterpret_cast<u32x4*>(d) = u32x4{pack_bf16(o1[0], o1[1]), pack_bf16(o1[2], o1[3]), pack_bf16(o1[4], o1[5]), pack_bf16(o1[6], o1[7])};
-      *reinterpret_cast<u32x4*>(d + D / 2) = u32x4{pack_bf16(o2[0], o2[1]), pack_bf16(o2[2], o2[3]), pack_bf16(o2[4], o2[5]), pack_bf16(o2[6], o2[7])};
+      *reinterpret_cast<u32x4*>(d) = u32x4{pack_elts(o1[0], o1[1]), pack_elts(o1[2], o1[3]), pack_elts(o1[4], o1[5]), pack_elts(o1[6], o1[7])};
+      *reinterpret_cast<u32x4*>(d + D / 2) = u32x4{pack_elts(o2[0], o2[1]), pack_elts(o2[2], o2[3]), pack_elts(o2[4], o2[5]), pack_elts(o2[6], o2[7])};
     }
   }
   lds_order();
@@ -488,6 +514,7 @@ __device__ __forceinline__ float wave_max(float x) {
 __device__ __forceinline__ float bf16_to_f(uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
 __device__ __forceinline__ uint16_t f_to_bf16(float x) { return (uint16_t)(pack_bf16(x, 0.f) & 0xffffu); }
 __device__ __forceinline__ uint16_t f_to_f16(float x) { return (uint16_t)(pack_f16(x, 0.f) & 0xffffu); }
+__device__ __forceinline__ uint16_t f_to_elt(float x) { return (uint16_t)(pack_elts(x, 0.f) & 0xffffu); }
 
 // f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
 // in the body, so register arrays indexed with it never look dynamically indexed to the optimiser.
@@ -500,4 +527,4 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
 }
 
-}  // namespace corope
+}  // namespace COROPE_NS

@@ -29,7 +29,7 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
-namespace corope {
+namespace COROPE_NS {
 
 struct CoropeFreqs {
   float w[64];  // inverse frequencies divided by 2*pi (revolutions per unit of delta), D/2 entries used
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       const u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + 16 * ks);
       u32x4 h16;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) h16[e] = pack_f16(bf16_lo(raw[e]), bf16_hi(raw[e]));
+      for (int e = 0; e < 4; ++e) h16[e] = pack_f16(elt_lo(raw[e]), elt_hi(raw[e]));
       aop[ks] = vr < G ? h16 : u32x4{0, 0, 0, 0};
     }
     const uint16_t* lrow = p.q + ((int64_t)head0 * N + i) * D;
@@ -189,8 +189,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
       for (int e = 0; e < 4; ++e) {
         const float x = __builtin_amdgcn_fractf(delta * fr.w[d0 + e]);
         const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
-        const float k1 = e % 2 ? bf16_hi(w1[e / 2]) : bf16_lo(w1[e / 2]);
-        const float k2 = e % 2 ? bf16_hi(w2[e / 2]) : bf16_lo(w2[e / 2]);
+        const float k1 = e % 2 ? elt_hi(w1[e / 2]) : elt_lo(w1[e / 2]);
+        const float k2 = e % 2 ? elt_hi(w2[e / 2]) : elt_lo(w2[e / 2]);
         r1v[e] = __builtin_fmaf(cs, k1, sn * k2);
         r2v[e] = __builtin_fmaf(cs, k2, -(sn * k1));
       }
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     for (int h = 0; h < G; ++h) {
       const float e = fast_exp2(s2[h] - m_run[h]);   // 0 for the keys beyond the diagonal
       l_run[h] += e;
-      wts[h * WS + lane] = f_to_bf16(e);
+      wts[h * WS + lane] = f_to_elt(e);
     }
     park_block();                          // V replaces the rotated keys
     if (c > 0) fetch_block(kbase, c - 1, std::false_type{});  // K of the next chunk
@@ -262,8 +262,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
-        const u32x2 w = {pack_bf16(oacc[db][4 * g4] * inv_l, oacc[db][4 * g4 + 1] * inv_l),
-                         pack_bf16(oacc[db][4 * g4 + 2] * inv_l, oacc[db][4 * g4 + 3] * inv_l)};
+        const u32x2 w = {pack_elts(oacc[db][4 * g4] * inv_l, oacc[db][4 * g4 + 1] * inv_l),
+                         pack_elts(oacc[db][4 * g4 + 2] * inv_l, oacc[db][4 * g4 + 3] * inv_l)};
         *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
       }
   }
@@ -302,4 +302,4 @@ hipError_t launch_corope_gqa_fwd(const CoropeParams& p, int D, hipStream_t strea
   return D == 128 ? launch_corope_d<128>(p, fr, stream) : launch_corope_d<64>(p, fr, stream);
 }
 
-}  // namespace corope
+}  // namespace COROPE_NS

@@ -114,6 +114,17 @@ struct CoropeBwdParams {
   int B, Hq, Hkv, N;
 };
 
+}  // namespace corope
+
+#ifdef COROPE_F16
+#define COROPE_NS corope_f16
+#else
+#define COROPE_NS corope
+#endif
+
+namespace COROPE_NS {
+using namespace corope;
+
 // y = rotated x for a (BH, N, D) tensor; tile_max (may be null) receives [BH][ceil(N / 64)] largest row norms.
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
                               float* tile_max, int BH, int N, int D, hipStream_t stream);
@@ -131,4 +142,15 @@ hipError_t launch_corope_gqa_bwd(const CoropeBwdParams& p, int D, float* workspa
 hipError_t launch_rope_freqs(float* cosp, float* sinp, int n_pos, int D, int width, int64_t row_stride, int pos0,
                              float theta, hipStream_t stream);
 
-}  // namespace corope
+}  // namespace COROPE_NS
+
+// The launchers of the fp16 build of the attention kernels (the sources compiled with -DCOROPE_F16): fp16 q, k, v, dO,
+// fp16 matrix-core operands, fp16 outputs; same parameter blocks.
+namespace corope_f16 {
+hipError_t launch_rope_attn_fwd(const corope::FwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_bwd_preprocess(const corope::BwdParams& p, int D, hipStream_t stream);
+hipError_t launch_bwd_dv(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_bwd_dk(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_bwd_dq(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_corope_gqa_fwd(const corope::CoropeParams& p, int D, hipStream_t stream);
+}  // namespace corope_f16

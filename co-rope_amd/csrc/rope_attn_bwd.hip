@@ -16,7 +16,7 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
-namespace corope {
+namespace COROPE_NS {
 
 // ===================================================================================== dK / dV
 // Workgroup = NWAVES waves x 32 keys.  K_r and V rows of the wave stay in registers as B operands.
@@ -206,12 +206,12 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
           ds[e] = pv[e] * (dpacc[4 * g + e] - d4[e]);
         }
         if constexpr (DO_DV) {
-          pb[g / 2][2 * (g % 2)] = pack_bf16(pv[0], pv[1]);
-          pb[g / 2][2 * (g % 2) + 1] = pack_bf16(pv[2], pv[3]);
+          pb[g / 2][2 * (g % 2)] = pack_elts(pv[0], pv[1]);
+          pb[g / 2][2 * (g % 2) + 1] = pack_elts(pv[2], pv[3]);
         }
         if constexpr (DO_DK) {
-          dsb[g / 2][2 * (g % 2)] = pack_bf16(ds[0], ds[1]);
-          dsb[g / 2][2 * (g % 2) + 1] = pack_bf16(ds[2], ds[3]);
+          dsb[g / 2][2 * (g % 2)] = pack_elts(ds[0], ds[1]);
+          dsb[g / 2][2 * (g % 2) + 1] = pack_elts(ds[2], ds[3]);
         }
       }
 #pragma unroll
@@ -324,7 +324,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
       const u32x4 ow = orows.x[i], dw = dorows.x[i];
       float acc = 0.f;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) acc += bf16_lo(ow[w]) * bf16_lo(dw[w]) + bf16_hi(ow[w]) * bf16_hi(dw[w]);
+      for (int w = 0; w < 4; ++w) acc += elt_lo(ow[w]) * elt_lo(dw[w]) + elt_hi(ow[w]) * elt_hi(dw[w]);
 #pragma unroll
       for (int m = CPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m);
       if (ch == 0) wave_delta[r] = acc;
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
             float pv = fast_exp2(sacc[i + e] * scale2 - lse_q);
             ds[e] = pv * (dpacc[i + e] - delta_q);
           }
-          dsb[2 * kb + i / 8][(i % 8) / 2] = pack_bf16(ds[0], ds[1]);
+          dsb[2 * kb + i / 8][(i % 8) / 2] = pack_elts(ds[0], ds[1]);
         }
       }
 #pragma unroll
@@ -497,4 +497,4 @@ hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t str
   return causal ? launch_dq_cfg<64, true, false>(p, stream) : launch_dq_cfg<64, false, false>(p, stream);
 }
 
-}  // namespace corope
+}  // namespace COROPE_NS

@@ -6,7 +6,7 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
-namespace corope {
+namespace COROPE_NS {
 
 template <int D>
 __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const uint16_t* __restrict__ o,
@@ -28,7 +28,7 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const uint16_t* __r
   for (int r = 0; r < kRowsPerThread; ++r) {
     float acc = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) acc += bf16_lo(a[r][w]) * bf16_lo(b[r][w]) + bf16_hi(a[r][w]) * bf16_hi(b[r][w]);
+    for (int w = 0; w < 4; ++w) acc += elt_lo(a[r][w]) * elt_lo(b[r][w]) + elt_hi(a[r][w]) * elt_hi(b[r][w]);
 #pragma unroll
     for (int off = kLanesPerRow / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
     int64_t row = base + (int64_t)r * kRowsPerPass;
@@ -50,4 +50,4 @@ hipError_t launch_bwd_preprocess(const BwdParams& p, int D, hipStream_t stream) 
   return hipGetLastError();
 }
 
-}  // namespace corope
+}  // namespace COROPE_NS

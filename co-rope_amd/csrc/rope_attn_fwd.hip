@@ -19,7 +19,7 @@
 
 #include <type_traits>
 
-namespace corope {
+namespace COROPE_NS {
 
 // Workgroup = 8 waves x 32 query rows = 256 rows, two waves per SIMD.
 //
@@ -57,7 +57,11 @@ struct FwdCfg {
 // that grows past kLsumLimit -- some score is ~2^20 above the reference, or the reference is still -inf on the first
 // tile, which shows up as inf/NaN -- the half is redone on the slow path, which moves the reference to the true maximum
 // and rescales the accumulators like a classic online softmax.
+#ifdef COROPE_F16
+constexpr float kLsumLimit = 16384.f;     // fp16 probabilities: everything the matrix cores see stays below 65504
+#else
 constexpr float kLsumLimit = 1048576.f;
+#endif
 
 // Fast-path piece `step` of `n_steps`: exponentiates 8 / n_steps score pairs of a half.
 __device__ __forceinline__ void softmax_fast_piece(int step, int n_steps, const f32x16& sacc, u32x4 (&pb)[2], float& lsum,
@@ -71,7 +75,7 @@ __device__ __forceinline__ void softmax_fast_piece(int step, int n_steps, const 
     float p1 = fast_exp2(sacc[2 * j + 1] * scale - ms);
     // plain adds: the bf16 dot-product instruction would do this in one op but stalls the MFMA pipe
     lsum += p0 + p1;
-    uint32_t w = pack_bf16(p0, p1);
+    uint32_t w = pack_elts(p0, p1);
     asm volatile("" : "+v"(w));  // keeps the piece between the two MFMAs it is written between
     pb[j / 4][j % 4] = w;
   }
@@ -92,7 +96,7 @@ __device__ __forceinline__ float softmax_slow_half(const f32x16& sacc, u32x4 (&p
     float p0 = fast_exp2(sacc[2 * j] * scale - ms);
     float p1 = fast_exp2(sacc[2 * j + 1] * scale - ms);
     lsum += p0 + p1;
-    pb[j / 4][j % 4] = pack_bf16(p0, p1);
+    pb[j / 4][j % 4] = pack_elts(p0, p1);
   }
   l_run = l_run * alpha + lsum;
   m_ref = m_new;
@@ -302,4 +306,4 @@ hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStrea
   return causal ? launch_fwd_cfg<64, 64, true>(p, stream) : launch_fwd_cfg<64, 64, false>(p, stream);
 }
 
-}  // namespace corope
+}  // namespace COROPE_NS

@@ -33,7 +33,7 @@
 #include <type_traits>
 #include <utility>
 
-namespace corope {
+namespace COROPE_NS {
 
 constexpr int kPipeWaves = 8;
 constexpr int kPipeBlockN = 64;
@@ -65,7 +65,7 @@ __device__ __forceinline__ void softmax_pair(int j, const f32x16& sacc, u32x4 (&
   float p1 = fast_exp2(sacc[2 * j + 1] * scale - ms);
   // plain adds: the bf16 dot-product instruction would do this in one op but stalls the MFMA pipe
   lsum += p0 + p1;
-  uint32_t w = pack_bf16(p0, p1);
+  uint32_t w = pack_elts(p0, p1);
   asm volatile("" : "+v"(w), "+v"(lsum));   // ... and ends here, between the two MFMAs it is written between
   pb[j / 4][j % 4] = w;
 }
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
     for (int kc = 0; kc < M; ++kc)
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
-        float x0 = bf16_lo(qb[kc][w]), x1 = bf16_hi(qb[kc][w]);
+        float x0 = elt_lo(qb[kc][w]), x1 = elt_hi(qb[kc][w]);
         ss += x0 * x0 + x1 * x1;
       }
     q_bound_wave = __builtin_sqrtf(wave_reduce_max(half_sum(ss))) * scale * 1.01f;
@@ -410,4 +410,4 @@ hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causa
   return causal ? launch_pipe_cfg<64, true>(p, stream) : launch_pipe_cfg<64, false>(p, stream);
 }
 
-}  // namespace corope
+}  // namespace COROPE_NS

@@ -13,7 +13,7 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
-namespace corope {
+namespace COROPE_NS {
 
 constexpr int kRotRows = 64;
 constexpr int kRotThreads = 256;
@@ -44,7 +44,7 @@ __global__ __launch_bounds__(kRotThreads) void rope_rotate_kernel(const uint16_t
     float ss = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      float a0 = bf16_lo(y1[w]), a1 = bf16_hi(y1[w]), b0 = bf16_lo(y2[w]), b1 = bf16_hi(y2[w]);
+      float a0 = elt_lo(y1[w]), a1 = elt_hi(y1[w]), b0 = elt_lo(y2[w]), b1 = elt_hi(y2[w]);
       ss += (a0 * a0 + a1 * a1) + (b0 * b0 + b1 * b1);
     }
     // the kChunks lanes of a row are consecutive
@@ -83,4 +83,4 @@ hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float*
   return hipGetLastError();
 }
 
-}  // namespace corope
+}  // namespace COROPE_NS

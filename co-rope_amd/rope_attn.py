@@ -5,7 +5,8 @@ like the reference's ``attention = _attention.apply`` (fused-rope/fused_rope_att
 accepted and ignored (it selects a Triton code path there).  ``fused_rope_attn`` is a keyword-friendly wrapper.
 
 Forward and backward run hand-written gfx950 kernels through the C ABI in ``include/corope_amd.h``; there is no
-other implementation behind this module."""
+other implementation behind this module.  Tensors are bfloat16 (the fast paths) or float16 (the reference's dtype,
+fused_rope_attn.py:236; same kernels built for fp16 elements, single-launch forward)."""
 from __future__ import annotations
 
 import torch
@@ -32,8 +33,10 @@ def _check_inputs(q, k, v, freqs_cos, freqs_sin):
         raise ValueError(f"head dim {d} not built for gfx950 (supported: {_SUPPORTED_D})")
     if not (q.is_cuda and k.is_cuda and v.is_cuda and freqs_cos.is_cuda and freqs_sin.is_cuda):
         raise ValueError("fused RoPE attention runs on the GPU only: all tensors must be on a HIP device")
-    if not (q.dtype == k.dtype == v.dtype == torch.bfloat16):
-        raise ValueError(f"q, k, v must be bfloat16 (got {q.dtype}, {k.dtype}, {v.dtype})")
+    if not (q.dtype == k.dtype == v.dtype and q.dtype in (torch.bfloat16, torch.float16)):
+        raise ValueError(f"q, k, v must all be bfloat16 or all float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
+    if q.dtype == torch.float16 and k.shape[1] != q.shape[1]:
+        raise ValueError("grouped-query attention (fewer key/value heads) is built for bfloat16 only")
     n = q.shape[2]
     for name, f in (("freqs_cos", freqs_cos), ("freqs_sin", freqs_sin)):
         if f.dim() != 2 or f.shape[0] < n or f.shape[1] < d // 2:
@@ -79,7 +82,13 @@ def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, k
     rotated = None
     Hkv = k.shape[1]
     with torch.cuda.device(q.device):
-        if Hkv != H:   # grouped-query attention: one entry point covers the three forms
+        if q.dtype == torch.float16:
+            # the reference's dtype: one launch, a true running maximum wherever a probability would leave fp16's range
+            rc = lib.corope_rope_attn_fwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
+                                              fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, N, D, float(sm_scale),
+                                              int(bool(causal)), _stream_ptr(q))
+            _lib.check(rc, "corope_rope_attn_fwd_f16")
+        elif Hkv != H:   # grouped-query attention: one entry point covers the three forms
             q_rot = torch.empty_like(q) if (two_launch and keep_rotated) else None
             k_rot = torch.empty_like(k) if two_launch else None
             kmax = torch.empty((B, Hkv, (N + 63) // 64), device=q.device, dtype=torch.float32) if two_launch else None
@@ -128,7 +137,7 @@ class _FusedRopeAttn(torch.autograd.Function):
         # when a gradient will be asked for, the forward keeps its rotated q and k for the backward and the originals
         # are not saved (the reference saves q and k, fused_rope_attn.py:718, and re-rotates them in its backward)
         o, M, fc, fs, rotated = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin,
-                                         keep_rotated=any(ctx.needs_input_grad[:3]))
+                                         keep_rotated=any(ctx.needs_input_grad[:3]) and q.dtype == torch.bfloat16)
         ctx.rotated = rotated is not None
         if ctx.rotated:
             ctx.save_for_backward(rotated[0], rotated[1], v, o, M, fc, fs)
@@ -144,13 +153,18 @@ class _FusedRopeAttn(torch.autograd.Function):
         q, k, v, o, M, fc, fs = ctx.saved_tensors
         lib = _lib.load()
         do = do.contiguous()
-        if do.dtype != torch.bfloat16:
-            do = do.to(torch.bfloat16)
+        if do.dtype != q.dtype:
+            do = do.to(q.dtype)
         B, H, N, D = q.shape
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         delta = torch.empty_like(M)
         with torch.cuda.device(q.device):
-            if k.shape[1] != H:         # grouped-query attention
+            if q.dtype == torch.float16:
+                rc = lib.corope_rope_attn_bwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
+                                                  M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0),
+                                                  dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, N, D, ctx.sm_scale,
+                                                  int(ctx.causal), _stream_ptr(q))
+            elif k.shape[1] != H:         # grouped-query attention
                 rc = lib.corope_rope_attn_bwd_gqa(q.data_ptr(), k.data_ptr(), int(ctx.rotated), v.data_ptr(), o.data_ptr(),
                                                   do.data_ptr(), M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(),
                                                   fc.stride(0), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H,
@@ -200,6 +214,8 @@ def rope_rotate(x, freqs_cos, freqs_sin, with_tile_max=False):
     """Half-layout rotation of x (B, H, N, D) bf16 on the device (fp32 arithmetic, one rounding to bf16).
     Returns y, or (y, tile_max) with the largest rotated-row norm of every 64-row tile, (B, H, ceil(N/64)) fp32."""
     _check_inputs(x, x, x, freqs_cos, freqs_sin)
+    if x.dtype != torch.bfloat16:
+        raise ValueError("the rotation pass is built for bfloat16 only")
     lib = _lib.load()
     x = x.contiguous()
     fc, fs = _freq_table(freqs_cos), _freq_table(freqs_sin)

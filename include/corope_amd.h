@@ -212,6 +212,23 @@ int corope_rope_attn_bwd_ws(const void *q, const void *k, const void *v, const v
                             int B, int H, int N, int D, float sm_scale, int causal,
                             void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The operator on fp16 tensors -- the only dtype of the reference's kernels (fused-rope/fused_rope_attn.py:236,
+ * verification.py:14): q, k, v, o, d_o, dq, dk, dv are fp16, the matrix cores take fp16 operands, everything else (tables,
+ * lse, delta, accumulation) is fp32 as above.  Same kernels as the bf16 entry points built for the other element type:
+ * the forward is corope_rope_attn_fwd's single launch with a true running maximum per 32-key half whenever a
+ * probability would leave fp16's range (the two-launch forward carries unnormalised probabilities up to 2^64, which only
+ * bf16 can hold); the backward is preprocess + dV + dK + dQ as in corope_rope_attn_bwd.  `delta` is (B,H,N) fp32 scratch.
+ * Replaces _attention.forward / .backward (fused-rope/fused_rope_attn.py:655-777) for callers that keep the reference's dtype. */
+int corope_rope_attn_fwd_f16(const void *q, const void *k, const void *v,
+                             const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                             void *o, float *lse,
+                             int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+int corope_rope_attn_bwd_f16(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                             const float *lse, float *delta,
+                             const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                             void *dq, void *dk, void *dv,
+                             int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+
 /* Grouped-query form of the operator: q (B,Hq,N,D), k and v (B,Hkv,N,D), Hq a multiple of Hkv; query head h reads
  * key/value head h / (Hq/Hkv); dk and dv (B,Hkv,N,D) are sums over the query heads of their group (the key block's
  * workgroup sweeps all of them, no atomics).  The reference's RoPE operator requires Hq == Hkv
@@ -238,6 +255,12 @@ int corope_rope_attn_bwd_gqa(const void *q, const void *k, int prerotated, const
  * on the host here and passed to the kernel by value.  Limits: B*Hkv*N < 2^31, N*D*2 bytes < 4 GiB. */
 int corope_gqa_fwd(const void *q, const void *k, const void *v, void *o,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void *stream);
+
+/* The same forward on fp16 tensors, the dtype of the reference's kernel and of its comparison script
+ * (corope-exp/flash_attn_co_rope_gqa_triton.py:406-456, compare_corope.py:18): fp16 q, k, v, o; same kernel built for
+ * fp16 elements (leader logits, scores and P V all on fp16 matrix-core operands).  The backward is built for bf16 only. */
+int corope_gqa_fwd_f16(const void *q, const void *k, const void *v, void *o,
+                       int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void *stream);
 
 /* Bytes of device workspace corope_gqa_bwd needs for these sizes (-1 for sizes corope_gqa_check rejects):
  * packed lower-triangular N x N fp32 matrices (about N*N/2 + 32*N floats each): two per key/value head (accumulated

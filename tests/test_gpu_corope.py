@@ -90,3 +90,33 @@ def test_corope_validation_errors(pkg):
         pkg.corope_attention(torch.zeros(1, 18, 64, 64, device=dev, dtype=torch.bfloat16), k, k, True, 1.0, 1e4)
     with pytest.raises(ValueError):
         pkg.corope_attention(q.float(), k.float(), k.float(), True, 1.0, 1e4)
+
+
+@pytest.mark.parametrize("scale", [None, 1.0])
+@pytest.mark.parametrize("B,Hq,Hkv,N,D", [(1, 4, 2, 32, 64), (1, 6, 2, 100, 64), (1, 8, 2, 130, 128), (2, 8, 2, 512, 128)])
+def test_corope_forward_fp16(pkg, B, Hq, Hkv, N, D, scale):
+    """fp16 tensors, the dtype of the reference's kernel and comparison script (compare_corope.py:18, whose shape comes
+    first and which runs at sm_scale = 1): the same kernel built for fp16 elements, against the oracle on the same
+    fp16-rounded inputs.  Bar: max-abs <= 2e-2 at 1/sqrt(D); at sm_scale = 1 (logits with a standard deviation of 8 to 11)
+    max <= 0.15 and mean <= 5e-3 as for the other hot cases.  The backward is built for bf16 only and says so."""
+    print(f"case fp16 B={B} Hq={Hq} Hkv={Hkv} N={N} D={D} scale={scale}", flush=True)
+    q, k, v = (t.to(torch.float16).float() for t in (seeded((B, Hq, N, D), 5), seeded((B, Hkv, N, D), 6), seeded((B, Hkv, N, D), 7)))
+    sc = 1 / math.sqrt(D) if scale is None else scale
+    dev = torch.device("cuda:0")
+    qd = q.to(dev, torch.float16).requires_grad_(True)
+    o = pkg.corope_attention(qd, k.to(dev, torch.float16), v.to(dev, torch.float16), True, sc, 10000.0)
+    torch.cuda.synchronize()
+    assert o.dtype == torch.float16
+    if N <= 130:
+        ref = C.corope_gqa_forward(q, k, v, True, sc, 10000.0, torch.float64).float()
+    else:
+        ref = C.corope_gqa_forward_rows(q, k, v, True, sc, 10000.0, torch.arange(N), torch.float32)
+    err = (o.float().cpu() - ref).abs()
+    print(f"  O max-abs {err.max():.3e} mean-abs {err.mean():.3e}")
+    assert torch.isfinite(o).all()
+    if scale is None:
+        assert err.max() <= TOL
+    else:
+        assert err.max() <= 0.15 and err.mean() <= 5e-3
+    with pytest.raises(ValueError, match="bfloat16"):
+        o.sum().backward()
