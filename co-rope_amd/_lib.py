@@ -21,6 +21,7 @@ _P, _I, _F, _L = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_int64
 SIGNATURES = {
     "corope_amd_version": (_I, []),
     "corope_amd_last_error": (ctypes.c_char_p, []),
+    "corope_amd_set_tile_rows": (_I, [_I]),
     "corope_rope_attn_check": (_I, [_I, _I, _I, _I, _L, _F, _I]),
     "corope_gqa_check": (_I, [_I, _I, _I, _I, _I, _F, _F]),
     "corope_rope_freqs": (_I, [_P, _P, _I, _I, _I, _L, _I, _F, _P]),

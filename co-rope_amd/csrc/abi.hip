@@ -13,6 +13,8 @@ namespace corope { uint64_t* g_trace_buf = nullptr; }
 extern "C" void corope_debug_trace(void* buf) { corope::g_trace_buf = static_cast<uint64_t*>(buf); }
 #endif
 
+namespace corope { std::atomic<int> g_tile_rows{0}; }
+
 namespace {
 
 thread_local char g_err[256] = "";
@@ -74,6 +76,12 @@ extern "C" {
 int corope_amd_version(void) { return 1; }
 
 const char* corope_amd_last_error(void) { return g_err; }
+
+int corope_amd_set_tile_rows(int rows) {
+  if (rows != 0 && rows != 128 && rows != 256) return fail(COROPE_E_BADARG, "set_tile_rows: %d is not 0, 128 or 256", rows);
+  corope::g_tile_rows.store(rows);
+  return COROPE_OK;
+}
 
 int corope_rope_attn_check(int B, int H, int N, int D, int64_t freq_row_stride, float sm_scale, int backward) {
   (void)backward;

@@ -43,6 +43,17 @@ extern uint64_t* g_trace_buf;
 #define COROPE_STAMP_ID(tid, extra) do {} while (0)
 #endif
 
+// Rows per workgroup of the attention kernels: 256 (8 waves) or 128 (4 waves).  By shape: a launch whose 256-row blocks
+// number fewer than two per CU of an MI355X takes the 128-row form, which doubles the workgroups and halves the time
+// the heaviest of them runs; `g_tile_rows` (0 = by shape, 128, 256) overrides the rule for tests and tuning.
+extern std::atomic<int> g_tile_rows;
+inline bool use_small_tiles(int n_rows, int slabs) {
+  const int forced = g_tile_rows.load(std::memory_order_relaxed);
+  if (forced == 128) return true;
+  if (forced == 256) return false;
+  return (int64_t)((n_rows + 255) / 256) * slabs < 2 * 256;
+}
+
 struct FwdParams {
   COROPE_TRACE_FIELD
   const uint16_t* q;

@@ -431,9 +431,9 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
 // ===================================================================================== launchers
 // The fused dK+dV kernel sits at 246 of the 256 registers that two waves per SIMD leave each of them; dV alone is
 // small enough for a 128-row tile on pre-rotated operands.
-template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
-static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
-  constexpr int NWAVES = 8, BLOCK_M = (PREROT && !DO_DK) ? 128 : 64;   // the larger tile pays off (and fits) for dV on pre-rotated operands only
+template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT, int NWAVES>
+static hipError_t launch_dkdv_waves(BwdParams p, hipStream_t stream) {
+  constexpr int BLOCK_M = (PREROT && !DO_DK && NWAVES == 8) ? 128 : 64;   // the larger tile pays off (and fits) for dV on pre-rotated operands only
   using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? 8 : 32, DO_DV && DO_DK>;
   auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK, PREROT>;
   static std::atomic<uint64_t> lds_ok{0};
@@ -446,9 +446,15 @@ static hipError_t launch_dkdv_cfg(BwdParams p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int D, bool CAUSAL, bool PREROT>
-static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
-  constexpr int NWAVES = 8, BLOCK_N = 64;
+template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
+static hipError_t launch_dkdv_cfg(const BwdParams& p, hipStream_t stream) {
+  return use_small_tiles(p.N, p.BH / p.H * p.Hkv) ? launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 4>(p, stream)
+                                                   : launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 8>(p, stream);
+}
+
+template <int D, bool CAUSAL, bool PREROT, int NWAVES>
+static hipError_t launch_dq_waves(BwdParams p, hipStream_t stream) {
+  constexpr int BLOCK_N = 64;
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
   auto kern = rope_attn_bwd_dq_kernel<D, NWAVES, BLOCK_N, CAUSAL, PREROT>;
   static std::atomic<uint64_t> lds_ok{0};
@@ -459,6 +465,12 @@ static hipError_t launch_dq_cfg(BwdParams p, hipStream_t stream) {
 #endif
   hipLaunchKernelGGL(kern, dim3(p.num_blocks * p.BH), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
+}
+
+template <int D, bool CAUSAL, bool PREROT>
+static hipError_t launch_dq_cfg(const BwdParams& p, hipStream_t stream) {
+  return use_small_tiles(p.N, p.BH) ? launch_dq_waves<D, CAUSAL, PREROT, 4>(p, stream)
+                                    : launch_dq_waves<D, CAUSAL, PREROT, 8>(p, stream);
 }
 
 // Dispatch on the run-time switches (head dim, causal, pre-rotated operands present).

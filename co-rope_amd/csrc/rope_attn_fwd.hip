@@ -32,19 +32,18 @@ namespace COROPE_NS {
 //     slot C:  O^T += V^T P^T(h0)   +  online softmax of half 1
 //     slot D:  O^T += V^T P^T(h1)
 // Scheduling barriers separate the slots and pin the operand prefetches ahead of the MFMAs that use them.
-constexpr int kFwdWaves = 8;
 constexpr int kFwdStages = 2;
 
-template <int D, int BLOCK_N>
+template <int D, int BLOCK_N, int NW>
 struct FwdCfg {
-  static constexpr int kThreads = kFwdWaves * kWave;
-  static constexpr int kBlockM = kFwdWaves * 32;
+  static constexpr int kThreads = NW * kWave;
+  static constexpr int kBlockM = NW * 32;
   static constexpr int kVPad = 32;                                       // V is read only through load_a_trans
   static constexpr int kKBytes = RowTile<D>::bytes(BLOCK_N);             // K tile, row-major, read row-wise
   static constexpr int kVBytes = RowTile<D, kVPad>::bytes(BLOCK_N);      // V tile, row-major, read transposed
   static constexpr int kStageBytes = kKBytes + kVBytes;
   static constexpr int kLoopBytes = kFwdStages * kStageBytes;
-  static constexpr int kEpilogueBytes = kFwdWaves * 32 * kAccTileStride<D> * 4;   // fp32 O rows of all waves on their way out
+  static constexpr int kEpilogueBytes = NW * 32 * kAccTileStride<D> * 4;   // fp32 O rows of all waves on their way out
   static constexpr int kLdsBytes = kLoopBytes > kEpilogueBytes ? kLoopBytes : kEpilogueBytes;
 };
 
@@ -106,9 +105,9 @@ __device__ __forceinline__ float softmax_slow_half(const f32x16& sacc, u32x4 (&p
 // This kernel knows nothing about the keys in advance, so every half runs the fast pieces and is verified afterwards
 // (two data-dependent branches per tile); the two-launch forward in rope_attn_fwd_pipe.hip gets the same guarantee
 // from key norms computed beforehand and has no such branch.
-template <int D, int BLOCK_N, bool CAUSAL>
-__global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdParams p) {
-  using Cfg = FwdCfg<D, BLOCK_N>;
+template <int D, int BLOCK_N, bool CAUSAL, int NW>
+__global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_fwd_kernel(FwdParams p) {
+  using Cfg = FwdCfg<D, BLOCK_N, NW>;
   static_assert(BLOCK_N == 64, "the slot schedule is written for two 32-key halves");
   constexpr int NT = Cfg::kThreads;
   constexpr int KC = D / 16;        // contraction chunks of QK^T = MFMAs per S^T half
@@ -289,16 +288,22 @@ __global__ __launch_bounds__(kFwdWaves* kWave) void rope_attn_fwd_kernel(FwdPara
 }
 
 // ---- host-side launch -----------------------------------------------------------------------------------------
-template <int D, int BLOCK_N, bool CAUSAL>
-static hipError_t launch_fwd_cfg(FwdParams p, hipStream_t stream) {
-  using Cfg = FwdCfg<D, BLOCK_N>;
-  auto kern = rope_attn_fwd_kernel<D, BLOCK_N, CAUSAL>;
+template <int D, int BLOCK_N, bool CAUSAL, int NW>
+static hipError_t launch_fwd_waves(FwdParams p, hipStream_t stream) {
+  using Cfg = FwdCfg<D, BLOCK_N, NW>;
+  auto kern = rope_attn_fwd_kernel<D, BLOCK_N, CAUSAL, NW>;
   static std::atomic<uint64_t> lds_ok{0};
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
   p.num_m_blocks = (p.N + Cfg::kBlockM - 1) / Cfg::kBlockM;
   dim3 grid(p.num_m_blocks * p.BH);
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
+}
+
+template <int D, int BLOCK_N, bool CAUSAL>
+static hipError_t launch_fwd_cfg(const FwdParams& p, hipStream_t stream) {
+  return use_small_tiles(p.N, p.BH) ? launch_fwd_waves<D, BLOCK_N, CAUSAL, 4>(p, stream)
+                                    : launch_fwd_waves<D, BLOCK_N, CAUSAL, 8>(p, stream);
 }
 
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream) {

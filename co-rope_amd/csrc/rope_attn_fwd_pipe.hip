@@ -35,7 +35,6 @@
 
 namespace COROPE_NS {
 
-constexpr int kPipeWaves = 8;
 constexpr int kPipeBlockN = 64;
 // p stays below 2^kPipeMargin and the fp32 sums below 2^(kPipeMargin + log2 N + log2 max|v|): far from overflow, and
 // bf16 has fp32's exponent range, so P loses nothing either.  The reference is lifted at most kPipeLift above the largest
@@ -45,16 +44,16 @@ constexpr int kPipeBlockN = 64;
 constexpr float kPipeMargin = 64.f;
 constexpr float kPipeLift = 80.f;
 
-template <int D>
+template <int D, int NW>
 struct FwdPipeCfg {
-  static constexpr int kThreads = kPipeWaves * kWave;
-  static constexpr int kBlockM = kPipeWaves * 32;
+  static constexpr int kThreads = NW * kWave;
+  static constexpr int kBlockM = NW * 32;
   static constexpr int kVPad = 32;                                        // V is read only through load_a_trans
   static constexpr int kKBytes = RowTile<D>::bytes(kPipeBlockN);          // K tile, row-major, read row-wise
   static constexpr int kVBytes = RowTile<D, kVPad>::bytes(kPipeBlockN);   // V tile, row-major, read transposed
   static constexpr int kKStages = 2, kVStages = 3;
   static constexpr int kLoopBytes = kKStages * kKBytes + kVStages * kVBytes;
-  static constexpr int kEpilogueBytes = kPipeWaves * 32 * kAccTileStride<D> * 4;   // fp32 O rows of all waves
+  static constexpr int kEpilogueBytes = NW * 32 * kAccTileStride<D> * 4;   // fp32 O rows of all waves
   static constexpr int kLdsBytes = kLoopBytes > kEpilogueBytes ? kLoopBytes : kEpilogueBytes;
 };
 
@@ -76,9 +75,9 @@ __device__ __forceinline__ float wave_reduce_max(float x) {
   return x;
 }
 
-template <int D, bool CAUSAL>
-__global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(FwdParams p) {
-  using Cfg = FwdPipeCfg<D>;
+template <int D, bool CAUSAL, int NW>
+__global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_fwd_pipe_kernel(FwdParams p) {
+  using Cfg = FwdPipeCfg<D, NW>;
   constexpr int BLOCK_N = kPipeBlockN;
   constexpr int NT = Cfg::kThreads;
   constexpr int M = D / 16;         // MFMAs per slot: contraction chunks of a S^T half = MFMAs of a PV half
@@ -390,10 +389,10 @@ __global__ __launch_bounds__(kPipeWaves* kWave) void rope_attn_fwd_pipe_kernel(F
 }
 
 // ---- host-side launch -----------------------------------------------------------------------------------------
-template <int D, bool CAUSAL>
-static hipError_t launch_pipe_cfg(FwdParams p, hipStream_t stream) {
-  using Cfg = FwdPipeCfg<D>;
-  auto kern = rope_attn_fwd_pipe_kernel<D, CAUSAL>;
+template <int D, bool CAUSAL, int NW>
+static hipError_t launch_pipe_waves(FwdParams p, hipStream_t stream) {
+  using Cfg = FwdPipeCfg<D, NW>;
+  auto kern = rope_attn_fwd_pipe_kernel<D, CAUSAL, NW>;
   static std::atomic<uint64_t> lds_ok{0};
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
   p.num_m_blocks = (p.N + Cfg::kBlockM - 1) / Cfg::kBlockM;
@@ -403,6 +402,11 @@ static hipError_t launch_pipe_cfg(FwdParams p, hipStream_t stream) {
   dim3 grid(p.num_m_blocks * p.BH);
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
+}
+
+template <int D, bool CAUSAL>
+static hipError_t launch_pipe_cfg(const FwdParams& p, hipStream_t stream) {
+  return use_small_tiles(p.N, p.BH) ? launch_pipe_waves<D, CAUSAL, 4>(p, stream) : launch_pipe_waves<D, CAUSAL, 8>(p, stream);
 }
 
 hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream) {

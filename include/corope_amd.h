@@ -40,6 +40,11 @@ int corope_amd_version(void);
 /* Text of the last error raised on the calling thread ("" if none). */
 const char *corope_amd_last_error(void);
 
+/* Rows per workgroup of the RoPE attention kernels: 0 = chosen by shape (256, or 128 when a launch would otherwise have
+ * fewer than two workgroups per CU -- the reference picks its tile sizes per shape too, fused-rope/fused_rope_attn.py:
+ * 163-183), 128 or 256 = forced, for tests and tuning.  Process-wide; results do not depend on it beyond rounding. */
+int corope_amd_set_tile_rows(int rows);
+
 /* Argument check only (no HIP call): what corope_rope_attn_fwd/bwd would return for these sizes. */
 int corope_rope_attn_check(int B, int H, int N, int D, int64_t freq_row_stride, float sm_scale, int backward);
 

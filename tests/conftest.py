@@ -24,6 +24,16 @@ def pkg():
     return importlib.import_module("corope_amd")
 
 
+@pytest.fixture(params=[128, 256])
+def tile_rows(request, pkg):
+    """Runs the test once with 128-row (4-wave) and once with 256-row (8-wave) workgroups of the RoPE attention kernels,
+    whatever the library would pick for the shape."""
+    lib = pkg._lib.load()
+    assert lib.corope_amd_set_tile_rows(request.param) == 0
+    yield request.param
+    assert lib.corope_amd_set_tile_rows(0) == 0
+
+
 @pytest.fixture(scope="session")
 def brute():
     """ctypes handle on oracle/libbrute_force.so (built on demand with gcc)."""

@@ -135,6 +135,13 @@ def test_composite_entry_points_check_every_argument_before_the_first_launch(pkg
     assert rc == -2 and "scratch" in pkg._lib.last_error()
 
 
+def test_tile_rows_knob(pkg):
+    lib = pkg._lib.load()
+    assert lib.corope_amd_set_tile_rows(128) == 0 and lib.corope_amd_set_tile_rows(256) == 0
+    assert lib.corope_amd_set_tile_rows(64) == -1 and "tile_rows" in pkg._lib.last_error()
+    assert lib.corope_amd_set_tile_rows(0) == 0
+
+
 def test_grouped_query_argument_checks(pkg):
     """Head-count and pointer checks of the grouped-query entry points happen before any launch."""
     lib = pkg._lib.load()

@@ -44,8 +44,8 @@ SHAPES = [(4, 8, 1024, 64), (1, 8, 1024, 128), (2, 4, 512, 64), (2, 2, 256, 128)
 @pytest.mark.parametrize("two_launch", [False, True])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,N,D", SHAPES)
-def test_backward_parity(pkg, monkeypatch, B, H, N, D, causal, two_launch):
-    print(f"case B={B} H={H} N={N} D={D} causal={causal} two_launch={two_launch}", flush=True)
+def test_backward_parity(pkg, monkeypatch, tile_rows, B, H, N, D, causal, two_launch):
+    print(f"case B={B} H={H} N={N} D={D} causal={causal} two_launch={two_launch} tile_rows={tile_rows}", flush=True)
     _force_path(monkeypatch, pkg, two_launch)
     q, k, v, g, c, s = _case(B, H, N, D)
     scale = 1 / math.sqrt(D)
@@ -145,7 +145,7 @@ def test_forward_keeps_rotated_operands(pkg):
 @pytest.mark.parametrize("two_launch", [False, True])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,Hq,Hkv,N,D", [(1, 8, 2, 320, 128), (2, 4, 1, 200, 64), (1, 6, 3, 1024, 128), (1, 4, 4, 130, 64)])
-def test_grouped_query_parity(pkg, monkeypatch, B, Hq, Hkv, N, D, causal, two_launch):
+def test_grouped_query_parity(pkg, monkeypatch, tile_rows, B, Hq, Hkv, N, D, causal, two_launch):
     """Grouped-query form (k, v with fewer heads): forward and all three gradients against the oracle run on k, v repeated
     over their groups, with dK, dV summed back over the group (the definition of sharing a key/value head)."""
     print(f"case gqa B={B} Hq={Hq} Hkv={Hkv} N={N} D={D} causal={causal} two_launch={two_launch}", flush=True)
@@ -192,7 +192,7 @@ def test_backward_parity_verification_script_cases(pkg, monkeypatch, B, H, N, D,
 
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,N,D", [(1, 2, 512, 128), (2, 2, 300, 64), (1, 3, 257, 128), (1, 1, 77, 64)])
-def test_separate_dv_dk_on_rotated_operands_match_the_fused_kernel(pkg, B, H, N, D, causal):
+def test_separate_dv_dk_on_rotated_operands_match_the_fused_kernel(pkg, tile_rows, B, H, N, D, causal):
     """corope_rope_attn_bwd_dv_prerotated and _dk_prerotated (dV alone with its 128-row tile, dK alone) against the fused
     corope_rope_attn_bwd_dkdv_prerotated, through the C ABI, bit for bit: same operands, same order of accumulation."""
     lib = pkg._lib.load()

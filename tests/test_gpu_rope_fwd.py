@@ -39,8 +39,8 @@ SHAPES = [(2, 4, 512, 64), (1, 8, 1024, 128), (4, 16, 2048, 64), (4, 8, 1024, 64
 @pytest.mark.parametrize("two_launch", [False, True])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,N,D", SHAPES)
-def test_forward_parity(pkg, B, H, N, D, causal, two_launch):
-    print(f"case B={B} H={H} N={N} D={D} causal={causal} two_launch={two_launch}", flush=True)
+def test_forward_parity(pkg, tile_rows, B, H, N, D, causal, two_launch):
+    print(f"case B={B} H={H} N={N} D={D} causal={causal} two_launch={two_launch} tile_rows={tile_rows}", flush=True)
     q, k, v = _inputs(B, H, N, D)
     c, s = O.precompute_freqs_cis(D, N)
     scale = 1 / math.sqrt(D)
@@ -161,7 +161,7 @@ def test_rotate_pass_with_more_slabs_than_a_grid_axis(pkg):
 
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("case", ["large_norms", "outlier_keys", "growing_scores", "tiny_scores", "huge_norms_hot"])
-def test_two_launch_softmax_modes(pkg, case, causal):
+def test_two_launch_softmax_modes(pkg, tile_rows, case, causal):
     """Inputs that push tiles of the two-launch forward onto each of its softmax modes: the per-tile score bound
     (query norm x largest key norm of the tile) decides, so large norms, a few huge keys, and scores that keep
     growing along the sequence all force the exact mode on some tiles while others stay on the unchecked one."""
