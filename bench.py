@@ -423,7 +423,7 @@ def bench_phase_trace(args):
     kmax = torch.empty(B, H, (N + 63) // 64, device=dev, dtype=torch.float32)
     P = lambda t: t.data_ptr()
     launches = [
-        ("rope_rotate_k", lambda: lib.corope_rope_rotate(P(k), P(c), P(s), fs, P(kr), P(kmax), B, H, N, D, st)),
+        ("rope_rotate_k", lambda: lib.corope_rope_rotate(P(k), P(c), P(s), fs, P(kr), P(kmax), B, H, N, D, 1.0, st)),
         ("rope_attn_fwd", lambda: lib.corope_rope_attn_fwd_prerotated(P(q), P(kr), P(kmax), P(v), P(c), P(s), fs, P(o), P(M), P(qr),
                                                                       B, H, N, D, scale, 1, st)),
         ("rope_attn_bwd_dq", lambda: lib.corope_rope_attn_bwd_dq_prerotated(P(qr), P(kr), P(v), P(o), P(do), P(M), P(delta), P(c),
@@ -584,7 +584,7 @@ def main():
         k_rot, q_rot = torch.empty_like(k), torch.empty_like(q)
         kmax = torch.empty(B, H, (N + 63) // 64, device=dev, dtype=torch.float32)
         launches = [("rope_rotate_k", lambda: lib.corope_rope_rotate(kp, cp, sp, fs, k_rot.data_ptr(), kmax.data_ptr(),
-                                                                     B, H, N, D, stream)),
+                                                                     B, H, N, D, 1.0, stream)),
                     ("rope_attn_fwd", lambda: lib.corope_rope_attn_fwd_prerotated(
                         qp, k_rot.data_ptr(), kmax.data_ptr(), vp, cp, sp, fs, o.data_ptr(), M.data_ptr(),
                         None if fwd_only else q_rot.data_ptr(), B, H, N, D, scale, 1, stream))]

@@ -32,7 +32,7 @@ SIGNATURES = {
     "corope_rope_attn_fwd_noalloc": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_fwd_prerotated": (_I, [_P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_fwd_train": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P]),
-    "corope_rope_rotate": (_I, [_P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _P]),
+    "corope_rope_rotate": (_I, [_P, _P, _P, _L, _P, _P, _I, _I, _I, _I, _F, _P]),
     "corope_rope_attn_bwd_preprocess": (_I, [_P, _P, _P, _I, _I, _I, _I, _P]),
     "corope_rope_attn_bwd_dv": (_I, [_P] * 6 + [_L, _P, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_bwd_dk": (_I, [_P] * 8 + [_L, _P, _I, _I, _I, _I, _F, _I, _P]),

@@ -281,24 +281,25 @@ int corope_rope_attn_fwd_train(const void* q, const void* k, const void* v, cons
   if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
     return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "rope_attn_fwd_train: tile_kmax %p is null or misaligned",
                 (const void*)tile_kmax);
-  rc = corope_rope_rotate(k, freqs_cos, freqs_sin, freq_row_stride, k_rot, tile_kmax, B, H, N, D, stream);
+  rc = corope_rope_rotate(k, freqs_cos, freqs_sin, freq_row_stride, k_rot, tile_kmax, B, H, N, D, 1.f, stream);
   if (rc) return rc;
   return corope_rope_attn_fwd_prerotated(q, k_rot, tile_kmax, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, q_rot, B, H,
                                          N, D, sm_scale, causal, stream);
 }
 
 int corope_rope_rotate(const void* x, const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* y,
-                       float* tile_max, int B, int H, int N, int D, void* stream) {
+                       float* tile_max, int B, int H, int N, int D, float scale, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, 1.f, 0);
   if (rc) return rc;
   rc = check_ptrs("rope_rotate", {x, freqs_cos, freqs_sin, y});
   if (rc) return rc;
+  if (!(scale > 0.f) || !std::isfinite(scale)) return fail(COROPE_E_BADARG, "rope_rotate: scale %g must be positive and finite", (double)scale);
   if (tile_max != nullptr && (reinterpret_cast<uintptr_t>(tile_max) & 3u))
     return fail(COROPE_E_ALIGN, "rope_rotate: tile_max %p is not 4-byte aligned", (void*)tile_max);
   return launch_status("rope_rotate",
                        corope::launch_rope_rotate(static_cast<const uint16_t*>(x), freqs_cos, freqs_sin, freq_row_stride,
                                                   static_cast<uint16_t*>(y), tile_max, B * H, N, D,
-                                                  static_cast<hipStream_t>(stream)));
+                                                  static_cast<hipStream_t>(stream), scale));
 }
 
 int corope_rope_attn_bwd_preprocess(const void* o, const void* d_o, float* delta, int B, int H, int N, int D,
@@ -505,9 +506,9 @@ int corope_rope_attn_bwd_ws(const void* q, const void* k, const void* v, const v
                 (long long)(2 * bwd_ws_tensor_bytes(B, H, N, D)));
   void* q_rot = workspace;
   void* k_rot = static_cast<char*>(workspace) + bwd_ws_tensor_bytes(B, H, N, D);
-  rc = corope_rope_rotate(q, freqs_cos, freqs_sin, freq_row_stride, q_rot, nullptr, B, H, N, D, stream);
+  rc = corope_rope_rotate(q, freqs_cos, freqs_sin, freq_row_stride, q_rot, nullptr, B, H, N, D, sm_scale * kLog2e, stream);
   if (rc) return rc;
-  rc = corope_rope_rotate(k, freqs_cos, freqs_sin, freq_row_stride, k_rot, nullptr, B, H, N, D, stream);
+  rc = corope_rope_rotate(k, freqs_cos, freqs_sin, freq_row_stride, k_rot, nullptr, B, H, N, D, 1.f, stream);
   if (rc) return rc;
   return corope_rope_attn_bwd_prerotated(q_rot, k_rot, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, dk,
                                          dv, B, H, N, D, sm_scale, causal, stream);
@@ -531,7 +532,7 @@ int corope_rope_attn_fwd_gqa(const void* q, const void* k, const void* v, const 
   if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
     return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "%s: tile_kmax %p is null or misaligned", what,
                 (const void*)tile_kmax);
-  rc = corope_rope_rotate(k, freqs_cos, freqs_sin, freq_row_stride, k_rot, tile_kmax, B, Hkv, N, D, stream);
+  rc = corope_rope_rotate(k, freqs_cos, freqs_sin, freq_row_stride, k_rot, tile_kmax, B, Hkv, N, D, 1.f, stream);
   if (rc) return rc;
   return rope_attn_fwd_impl(what, q, k_rot, v, freqs_cos, freqs_sin, freq_row_stride, o, lse, B, Hq, N, D, sm_scale, causal,
                             k_rot, tile_kmax, q_rot, nullptr, 0, stream, Hkv);

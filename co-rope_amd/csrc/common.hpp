@@ -80,6 +80,20 @@ __device__ __forceinline__ float elt_hi(uint32_t w) { return bf16_hi(w); }
 __device__ __forceinline__ uint32_t pack_elts(float lo, float hi) { return pack_bf16(lo, hi); }
 #endif
 
+// D = A * B + C with D in registers of its own (C stays intact): the form the score products start from, C holding minus
+// the reference value of the exponentials in every register.  Written as an asm statement because the compiler, given
+// the builtin, copies C into D first.  The only readers of D that may follow are further mfma32 that accumulate into it
+// (same registers as C and D: no wait states needed) -- the vector units must not read D before one of those has run.
+__device__ __forceinline__ f32x16 mfma32_from(u32x4 a, u32x4 b, const f32x16& c) {
+  f32x16 d;
+#ifdef COROPE_F16
+  asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
+#else
+  asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
+#endif
+  return d;
+}
+
 // Row index (0..31) held by accumulator register i of lane-half h in a 32x32 MFMA result.
 __device__ __forceinline__ constexpr int acc_row(int i, int h) { return 8 * (i / 4) + 4 * h + (i % 4); }
 
@@ -133,14 +147,16 @@ struct RowTile {
 // ---- staging: a ROWS x D tile with the half-layout rotation applied on the way -----------------------
 // Work unit = one row x 8 rotation pairs: columns [8c, 8c+8) and [D/2 + 8c, D/2 + 8c + 8) of the same row
 // are loaded by the same thread, so the rotation is thread-local.  cos/sin come from fp32 tables of which
-// only the first D/2 columns are used.
-template <int D, int ROWS, int NT>
+// only the first D/2 columns are used.  SCALED: the rotated values are multiplied by out_scale before the one rounding
+// (the query side of QK^T carries sm_scale * log2(e), so that scores leave the matrix cores in base-2 units).
+template <int D, int ROWS, int NT, bool SCALED = false>
 struct RotStage {
   static constexpr int kChunks = D / 16;              // units per row
   static constexpr int kUnits = ROWS * kChunks;
   static constexpr int kIters = (kUnits + NT - 1) / NT;
   u32x4 x1[kIters], x2[kIters];
   f32x4 c[kIters][2], s[kIters][2];
+  float out_scale = 1.f;
 
   // src: first row of the (n, D) bf16 matrix; row0: first tile row; rows >= n_rows are clamped.
   __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float* __restrict__ cosp,
@@ -172,8 +188,13 @@ struct RotStage {
       float b0 = elt_lo(x2[it][w]), b1 = elt_hi(x2[it][w]);
       float c0 = c[it][w / 2][(2 * w) % 4], c1 = c[it][w / 2][(2 * w) % 4 + 1];
       float s0 = s[it][w / 2][(2 * w) % 4], s1 = s[it][w / 2][(2 * w) % 4 + 1];
-      y1[w] = pack_elts(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
-      y2[w] = pack_elts(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+      if constexpr (SCALED) {
+        y1[w] = pack_elts((a0 * c0 - b0 * s0) * out_scale, (a1 * c1 - b1 * s1) * out_scale);
+        y2[w] = pack_elts((b0 * c0 + a0 * s0) * out_scale, (b1 * c1 + a1 * s1) * out_scale);
+      } else {
+        y1[w] = pack_elts(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+        y2[w] = pack_elts(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+      }
     }
   }
 
@@ -221,10 +242,11 @@ struct CopyStage {
 
 // Staging of a tile whose rows take part in QK^T: rotated on the way to LDS (PREROT = false), or copied from a tensor
 // that rope_rotate_kernel rotated beforehand (PREROT = true; the tables are then not touched).
-template <int D, int ROWS, int NT, bool PREROT>
-struct RopeStage : RotStage<D, ROWS, NT> {};
-template <int D, int ROWS, int NT>
-struct RopeStage<D, ROWS, NT, true> : CopyStage<D, ROWS, NT, 8> {
+template <int D, int ROWS, int NT, bool PREROT, bool SCALED = false>
+struct RopeStage : RotStage<D, ROWS, NT, SCALED> {};
+template <int D, int ROWS, int NT, bool SCALED>
+struct RopeStage<D, ROWS, NT, true, SCALED> : CopyStage<D, ROWS, NT, 8> {
+  float out_scale = 1.f;   // unused: the copy was scaled when it was rotated
   __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float*, const float*, int64_t, int row0,
                                        int n_rows) {
     CopyStage<D, ROWS, NT, 8>::load(src, row0, n_rows);
@@ -334,7 +356,8 @@ struct WaveRows<D, false> {
       x[i] = *reinterpret_cast<const u32x4*>(
           byte_offset(src, (uint32_t)min(row0 + RPI * i + l / CPR, n_rows - 1) * (D * 2) + (l % CPR) * 16));
   }
-  __device__ __forceinline__ void park(u32x4 (&out)[D / 16], uint16_t* wave_tile, uint16_t* = nullptr, int = 0, int = 0) {
+  __device__ __forceinline__ void park(u32x4 (&out)[D / 16], uint16_t* wave_tile, uint16_t* = nullptr, int = 0, int = 0,
+                                       float = 1.f) {
     const int l = threadIdx.x % kWave;
     lds_order();
 #pragma unroll
@@ -374,7 +397,7 @@ struct WaveRows<D, true> {
     }
   }
   __device__ __forceinline__ void park(u32x4 (&out)[D / 16], uint16_t* wave_tile, uint16_t* __restrict__ rot_out = nullptr,
-                                       int row0 = 0, int n_rows = 0) {
+                                       int row0 = 0, int n_rows = 0, float out_scale = 1.f) {
     const int l = threadIdx.x % kWave;
     lds_order();
 #pragma unroll
@@ -386,8 +409,8 @@ struct WaveRows<D, true> {
         float a0 = elt_lo(x1[i][w]), a1 = elt_hi(x1[i][w]), b0 = elt_lo(x2[i][w]), b1 = elt_hi(x2[i][w]);
         float c0 = c[i][w / 2][(2 * w) % 4], c1 = c[i][w / 2][(2 * w) % 4 + 1];
         float s0 = s[i][w / 2][(2 * w) % 4], s1 = s[i][w / 2][(2 * w) % 4 + 1];
-        y1[w] = pack_elts(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
-        y2[w] = pack_elts(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+        y1[w] = pack_elts((a0 * c0 - b0 * s0) * out_scale, (a1 * c1 - b1 * s1) * out_scale);
+        y2[w] = pack_elts((b0 * c0 + a0 * s0) * out_scale, (b1 * c1 + a1 * s1) * out_scale);
       }
       *reinterpret_cast<u32x4*>(wave_tile + RowTile<D>::off(r, u * 8)) = y1;
       *reinterpret_cast<u32x4*>(wave_tile + RowTile<D>::off(r, D / 2 + u * 8)) = y2;

@@ -61,7 +61,7 @@ struct FwdParams {
   const uint16_t* v;
   const uint16_t* k_rot;   // K already rotated (same layout as k), or null: rotate K tiles inside the kernel
   const float* tile_kmax;  // with k_rot: largest rotated-key norm of every 64-key tile, [BH][ceil(N / 64)]
-  uint16_t* q_rot_out;     // with k_rot, optional: receives the rotated Q (same layout as q), for a backward on rotated operands
+  uint16_t* q_rot_out;     // with k_rot, optional: receives the rotated Q times qk_scale (same layout as q), for a backward on rotated operands
   const float* cos;
   const float* sin;
   uint16_t* o;
@@ -82,8 +82,8 @@ struct BwdParams {
   const uint16_t* v;
   const uint16_t* o;
   const uint16_t* d_o;
-  const uint16_t* q_rot;  // Q and K already rotated (same layout as q, k), or both null: rotate tiles inside the kernels
-  const uint16_t* k_rot;
+  const uint16_t* q_rot;  // Q and K already rotated (same layout as q, k), or both null: rotate tiles inside the kernels;
+  const uint16_t* k_rot;  // q_rot carries the factor qk_scale (rotated, scaled, rounded once), k_rot none
   const float* cos;
   const float* sin;
   const float* lse;
@@ -136,9 +136,9 @@ struct CoropeBwdParams {
 namespace COROPE_NS {
 using namespace corope;
 
-// y = rotated x for a (BH, N, D) tensor; tile_max (may be null) receives [BH][ceil(N / 64)] largest row norms.
+// y = out_scale * rotated x for a (BH, N, D) tensor; tile_max (may be null) receives [BH][ceil(N / 64)] largest row norms.
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
-                              float* tile_max, int BH, int N, int D, hipStream_t stream);
+                              float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale = 1.f);
 hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream);  // needs k_rot
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_preprocess(const BwdParams& p, int D, hipStream_t stream);

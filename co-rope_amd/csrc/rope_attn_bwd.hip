@@ -86,7 +86,8 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   CopyStage<D, Cfg::kBlockN, NT> vcp;
   if constexpr (V_LDS) vcp.load(p.v + base, n0, N);
 
-  RopeStage<D, BLOCK_M, NT, PREROT> qst;
+  RopeStage<D, BLOCK_M, NT, PREROT, true> qst;   // Q_r tiles carry qk_scale: S leaves the matrix cores in base-2 units
+  qst.out_scale = p.qk_scale;
   CopyStage<D, BLOCK_M, NT, DO_PAD> dst;
   float st_lse = 0.f, st_delta = 0.f;
   const int m_tiles = (N + BLOCK_M - 1) / BLOCK_M;
@@ -100,9 +101,10 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
     dst.load(p.d_o + (int64_t)qs * N * D, m0, N);
     if (threadIdx.x < BLOCK_M) {
       int qi = m0 + threadIdx.x;
-      // rows past the end: M = +inf makes P = 0, so they contribute nothing
-      st_lse = qi < N ? p.lse[(int64_t)qs * N + qi] : INFINITY;
-      if constexpr (DO_DK) st_delta = qi < N ? p.delta[(int64_t)qs * N + qi] : 0.f;
+      // -M and -delta: what the S and dP products start from.  Rows past the end: M = +inf makes P = 0, so they
+      // contribute nothing
+      st_lse = qi < N ? -p.lse[(int64_t)qs * N + qi] : -INFINITY;
+      if constexpr (DO_DK) st_delta = qi < N ? -p.delta[(int64_t)qs * N + qi] : 0.f;
     }
   };
   auto q_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
@@ -150,7 +152,6 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   const uint64_t clk0 = __builtin_readcyclecounter();
 #endif
 
-  const float scale2 = p.qk_scale;
   for (int it = 0; it < n_iter; ++it) {
     const int m0 = tile_m0(it);
 #ifdef COROPE_TRACE
@@ -169,18 +170,31 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
       const int mq0 = m0 + qb * 32;
       // queries of this 32-row block that lie above every key of the wave see none of them
       if (CAUSAL && mq0 + 31 < wk_lo) continue;
-      f32x16 sacc, dpacc = f32x16{0};   // the first MFMA of each product takes a literal zero as its accumulator
+      // The products start from -M and -delta of their rows (register i holds query 8*(i/4) + 4*lh + i%4 of the block):
+      // S - M and dP - delta leave the matrix cores, no vector instruction applies them.
+      f32x16 sacc, dpacc = f32x16{0};
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 m4 = *reinterpret_cast<const f32x4*>(lses + qb * 32 + 8 * g + 4 * lh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sacc[4 * g + e] = m4[e];
+        if constexpr (DO_DK) {
+          const f32x4 d4 = *reinterpret_cast<const f32x4*>(deltas + qb * 32 + 8 * g + 4 * lh);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dpacc[4 * g + e] = d4[e];
+        }
+      }
       const uint16_t* qrow = qs + RowTile<D>::off(qb * 32 + lq, 8 * lh);
       const uint16_t* dorow = dos + RowTile<D, DO_PAD>::off(qb * 32 + lq, 8 * lh);
 #pragma unroll
       for (int kc = 0; kc < KC; ++kc)
-        sacc = mfma32(*reinterpret_cast<const u32x4*>(qrow + 16 * kc), kb[kc], kc == 0 ? f32x16{0} : sacc);
+        sacc = mfma32(*reinterpret_cast<const u32x4*>(qrow + 16 * kc), kb[kc], sacc);
       if constexpr (DO_DK) {
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
           dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc),
                          V_LDS ? *reinterpret_cast<const u32x4*>(vrows + RowTile<D>::off(wave * 32 + lq, 8 * lh + 16 * kc)) : vb[V_LDS ? 0 : kc],
-                         kc == 0 ? f32x16{0} : dpacc);
+                         dpacc);
       }
 
       // Causal mask on the raw scores, under a wave-uniform branch of its own (written into the exponential loop it
@@ -196,14 +210,11 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
       u32x4 pb[2], dsb[2];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        f32x4 m4 = *reinterpret_cast<const f32x4*>(lses + qb * 32 + 8 * g + 4 * lh);
-        f32x4 d4 = f32x4{0};
-        if constexpr (DO_DK) d4 = *reinterpret_cast<const f32x4*>(deltas + qb * 32 + 8 * g + 4 * lh);
         float pv[4], ds[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          pv[e] = fast_exp2(sacc[4 * g + e] * scale2 - m4[e]);
-          ds[e] = pv[e] * (dpacc[4 * g + e] - d4[e]);
+          pv[e] = fast_exp2(sacc[4 * g + e]);
+          ds[e] = pv[e] * dpacc[4 * g + e];
         }
         if constexpr (DO_DV) {
           pb[g / 2][2 * (g % 2)] = pack_elts(pv[0], pv[1]);
@@ -236,7 +247,8 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   // to a row-major order, so that dV and dK leave in whole row segments and the tables are read the same way
   float* wave_out = reinterpret_cast<float*>(smem) + wave * 32 * kAccTileStride<D>;
   if constexpr (DO_DV) store_rows_via_lds<D, false>(dvacc, p.dv + base, wk_lo, N, nullptr, nullptr, 0, 1.f, wave_out);
-  if constexpr (DO_DK) store_rows_via_lds<D, true>(dkacc, p.dk + base, wk_lo, N, p.cos, p.sin, p.fstride, p.sm_scale, wave_out);
+  // the Q_r operand carried sm_scale * log2(e): ln 2 is what is left of sm_scale
+  if constexpr (DO_DK) store_rows_via_lds<D, true>(dkacc, p.dk + base, wk_lo, N, p.cos, p.sin, p.fstride, 0.6931471805599453f, wave_out);
 #ifdef COROPE_TRACE
   __builtin_amdgcn_s_waitcnt(0);
   COROPE_STAMP(6, 0);
@@ -312,7 +324,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   // which then has to run after this one.
   float delta_q = 0.f;
   if (p.o == nullptr) delta_q = p.delta[(int64_t)bh * N + q_c];
-  qrows.park(qb, wave_rows);
+  qrows.park(qb, wave_rows, nullptr, 0, 0, p.qk_scale);   // Q_r carries qk_scale (a pre-rotated copy already does)
   dorows.park(dob, wave_rows);
   if (p.o != nullptr) {
     // 16 lanes per row: O in registers (same chunk order as dO went into the tile), dO from the tile
@@ -352,7 +364,14 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   const uint64_t clk0 = __builtin_readcyclecounter();
 #endif
 
-  const float scale2 = p.qk_scale;
+  // S - M leaves the matrix cores: the score products start from -M of the lane's query in every register
+  f32x16 msb;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    float x = -lse_q;
+    asm volatile("" : "+v"(x));   // sixteen values of their own: one value in sixteen places is tied to the first of them
+    msb[i] = x;
+  }
   for (int t = 0; t < n_tiles; ++t) {
     const int n0 = t * BLOCK_N;
 #ifdef COROPE_TRACE
@@ -377,7 +396,8 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
         const uint16_t* vrow = vs + RowTile<D>::off(kb * 32 + lq, 8 * lh);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
-          sacc = mfma32(*reinterpret_cast<const u32x4*>(krow + 16 * kc), qb[kc], kc == 0 ? f32x16{0} : sacc);
+          sacc = kc == 0 ? mfma32_from(*reinterpret_cast<const u32x4*>(krow), qb[0], msb)
+                         : mfma32(*reinterpret_cast<const u32x4*>(krow + 16 * kc), qb[kc], sacc);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
           dpacc = mfma32(*reinterpret_cast<const u32x4*>(vrow + 16 * kc), dob[kc], kc == 0 ? f32x16{0} : dpacc);
@@ -395,7 +415,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
           float ds[2];
 #pragma unroll
           for (int e = 0; e < 2; ++e) {
-            float pv = fast_exp2(sacc[i + e] * scale2 - lse_q);
+            float pv = fast_exp2(sacc[i + e]);
             ds[e] = pv * (dpacc[i + e] - delta_q);
           }
           dsb[2 * kb + i / 8][(i % 8) / 2] = pack_elts(ds[0], ds[1]);

@@ -146,11 +146,13 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
   {
     WaveRows<D, true> qrows;
     qrows.load(qg, p.cos, p.sin, p.fstride, m0 + wave * 32, N);
-    qrows.park(qb, reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride);
+    // the rotated Q rows carry sm_scale * log2(e), as in every other kernel of the operator: forward and backward then
+    // see the same rounded operands, and the same scores
+    qrows.park(qb, reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride, nullptr, 0, 0, p.qk_scale);
   }
   __syncthreads();   // the K and V buffers below overlap the tiles the waves just used
 
-  const float scale = p.qk_scale;
+  constexpr float scale = 1.f;   // scores come out of the matrix cores in base-2 units
   f32x16 oacc[NDB];
 #pragma unroll
   for (int i = 0; i < NDB; ++i) oacc[i] = f32x16{0};

@@ -58,10 +58,10 @@ struct FwdPipeCfg {
 };
 
 // One exponential pair of a 32-key half: scores 2j, 2j+1 of the lane -> one bf16x2 word of the P^T operand.
-__device__ __forceinline__ void softmax_pair(int j, const f32x16& sacc, u32x4 (&pb)[2], float& lsum, float scale, float ms) {
-  asm volatile("" : "+v"(ms));  // the pair starts here, not wherever the optimiser would like to hoist it
-  float p0 = fast_exp2(sacc[2 * j] * scale - ms);
-  float p1 = fast_exp2(sacc[2 * j + 1] * scale - ms);
+__device__ __forceinline__ void softmax_pair(int j, const f32x16& sacc, u32x4 (&pb)[2], float& lsum) {
+  asm volatile("" : "+v"(lsum));  // the pair starts here, not wherever the optimiser would like to hoist it
+  float p0 = fast_exp2(sacc[2 * j]);
+  float p1 = fast_exp2(sacc[2 * j + 1]);
   // plain adds: the bf16 dot-product instruction would do this in one op but stalls the MFMA pipe
   lsum += p0 + p1;
   uint32_t w = pack_elts(p0, p1);
@@ -126,13 +126,13 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
     COROPE_STAMP(9, TT);
 #endif
     qrows.park(qb, reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride,
-               p.q_rot_out != nullptr ? p.q_rot_out + (int64_t)bh * N * D : nullptr, m0 + wave * 32, N);
+               p.q_rot_out != nullptr ? p.q_rot_out + (int64_t)bh * N * D : nullptr, m0 + wave * 32, N, p.qk_scale);
   }
   COROPE_STAMP(10, TT);
   __syncthreads();   // the K and V buffers below overlap the tiles the waves just used
   COROPE_STAMP(11, TT);
 
-  const float scale = p.qk_scale;
+  constexpr float scale = 1.f;   // the rotated Q rows carry sm_scale * log2(e): scores come out of the MFMAs in base-2 units
   // Largest |q_r| * scale of the wave's rows (a little generous): times a tile's largest key norm it bounds the
   // tile's scaled scores.
   float q_bound_wave;
@@ -155,6 +155,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
   float m_true = -INFINITY;  // largest raw score seen by the reference moves (at most the row's true running maximum)
   float l_run = 0.f;         // this lane's share of the denominator up to the last move of the reference
   float lsum = 0.f;          // ... and since then
+  f32x16 msb = f32x16{0};    // -m_run in every register: the accumulator the score MFMAs start from
   f32x16 s1;                 // scores of the second half of the previous tile (softmax half done)
   u32x4 pb0[2], pb1[2];      // P^T operands of the two halves
 
@@ -226,11 +227,10 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
   };
   // Takes the second half of the previous tile out of the pipeline: rest of the softmax of its S1, then its PV product.
   auto drain = [&]() __attribute__((always_inline)) {
-    const float ms = m_run * scale;
     uint32_t vp_lane = v_lane_off + voff_prev;
     asm volatile("" : "+v"(vp_lane));
 #pragma unroll
-    for (int j = 4; j < 8; ++j) softmax_pair(j, s1, pb1, lsum, scale, ms);
+    for (int j = 4; j < 8; ++j) softmax_pair(j, s1, pb1, lsum);
 #pragma unroll
     for (int i = 0; i < M; ++i) oacc[i % NDB] = mfma32(v_operand(vp_lane, 1, i), pb1[i / NDB], oacc[i % NDB]);
   };
@@ -270,7 +270,6 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
     // One tile: four slots of M MFMAs, operands fetched RING MFMAs ahead.
     // stream position n -> slot n / M (0: S0, 1: PV1 of the previous tile, 2: S1, 3: PV0), MFMA i = n % M of the slot
     auto run_tile = [&](const bool MASK) __attribute__((always_inline)) {
-      const float ms = m_run * scale;
       auto operand = [&](int n) {
         const int slot = n / M, i = n % M;
         return slot == 0 ? k_operand(0, i) : slot == 1 ? v_operand(vprev, 1, i) : slot == 2 ? k_operand(1, i) : v_operand(vt, 0, i);
@@ -280,14 +279,14 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
 #pragma unroll
       for (int n = 0; n < RING; ++n) ring[n] = operand(n);
       __builtin_amdgcn_sched_barrier(0);
-      f32x16 t0 = f32x16{0};   // S0(t); S1(t) goes straight into s1, whose previous contents slot 0 has used up by then
+      f32x16 t0;   // S0(t); S1(t) goes straight into s1, whose previous contents slot 0 has used up by then
       static_for<TOTAL>([&](auto n_c) __attribute__((always_inline)) {
         constexpr int n = decltype(n_c)::value;
         constexpr int slot = n / M, i = n % M;
         // MFMA
-        if (slot == 0) t0 = mfma32(ring[n % RING], qb[i], t0);
+        if (slot == 0) t0 = i == 0 ? mfma32_from(ring[n % RING], qb[i], msb) : mfma32(ring[n % RING], qb[i], t0);
         if (slot == 1) oacc[i % NDB] = mfma32(ring[n % RING], pb1[i / NDB], oacc[i % NDB]);
-        if (slot == 2) s1 = mfma32(ring[n % RING], qb[i], i == 0 ? f32x16{0} : s1);
+        if (slot == 2) s1 = i == 0 ? mfma32_from(ring[n % RING], qb[i], msb) : mfma32(ring[n % RING], qb[i], s1);
         if (slot == 3) oacc[i % NDB] = mfma32(ring[n % RING], pb0[i / NDB], oacc[i % NDB]);
         if (n + RING < TOTAL) ring[n % RING] = operand(n + RING);
         if (n == 0) stage_next(t);
@@ -297,10 +296,10 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
         if (slot == 3 && i == 0 && MASK) mask_scores(s1, 1);
 #pragma unroll
         for (int j = jlo; j < jhi; ++j) {
-          if (slot == 0) softmax_pair(4 + j, s1, pb1, lsum, scale, ms);   // S1(t-1), second half
-          if (slot == 1) softmax_pair(j, t0, pb0, lsum, scale, ms);       // S0(t), first half
-          if (slot == 2) softmax_pair(4 + j, t0, pb0, lsum, scale, ms);   // S0(t), second half
-          if (slot == 3) softmax_pair(j, s1, pb1, lsum, scale, ms);       // S1(t), first half
+          if (slot == 0) softmax_pair(4 + j, s1, pb1, lsum);   // S1(t-1), second half
+          if (slot == 1) softmax_pair(j, t0, pb0, lsum);       // S0(t), first half
+          if (slot == 2) softmax_pair(4 + j, t0, pb0, lsum);   // S0(t), second half
+          if (slot == 3) softmax_pair(j, s1, pb1, lsum);       // S1(t), first half
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -348,6 +347,12 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
       m_run = m_new;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float x = -m_new;
+        asm volatile("" : "+v"(x));   // sixteen values of their own: one value in sixteen places is tied to the first of them
+        msb[i] = x;
+      }
       const float m_min = -wave_reduce_max(-m_run);
       const float thr = (m_min * scale + kPipeMargin) / q_bound_wave;
       thr_bits = __builtin_amdgcn_readfirstlane(thr > 0.f ? __builtin_bit_cast(uint32_t, thr) : 0u);

@@ -8,6 +8,9 @@
 // here costs one extra pass over K (HBM-bound) and removes N / 256 repeated rotations -- and their fp32 table
 // reads -- from the attention kernel's inner loop.
 //
+// out_scale != 1: y = out_scale * rotated x, still one rounding -- the form in which the backward kernels and the
+// two-launch forward take a pre-rotated Q (out_scale = sm_scale * log2(e)).
+//
 // tile_max[bh][t] = max over the rows of tile t of |y| (norm of the ROUNDED row).  With the norm of a query this
 // bounds every score of the tile, which lets the forward kernel pick its softmax mode per tile up front.
 #include "common.hpp"
@@ -18,13 +21,13 @@ namespace COROPE_NS {
 constexpr int kRotRows = 64;
 constexpr int kRotThreads = 256;
 
-template <int D>
+template <int D, bool SCALED>
 __global__ __launch_bounds__(kRotThreads) void rope_rotate_kernel(const uint16_t* __restrict__ x,
                                                                   const float* __restrict__ cosp,
                                                                   const float* __restrict__ sinp, int64_t fstride,
                                                                   uint16_t* __restrict__ y, float* __restrict__ tile_max,
-                                                                  int N, int n_tiles) {
-  using Stage = RotStage<D, kRotRows, kRotThreads>;
+                                                                  int N, int n_tiles, float out_scale) {
+  using Stage = RotStage<D, kRotRows, kRotThreads, SCALED>;
   constexpr int kChunks = Stage::kChunks;
   __shared__ float wave_max[kRotThreads / kWave];
   const int tile = blockIdx.x % n_tiles, bh = blockIdx.x / n_tiles;
@@ -33,6 +36,7 @@ __global__ __launch_bounds__(kRotThreads) void rope_rotate_kernel(const uint16_t
   uint16_t* yg = y + (int64_t)bh * N * D;
 
   Stage st;
+  st.out_scale = out_scale;
   st.load(xg, cosp, sinp, fstride, row0, N);
   float best = 0.f;
 #pragma unroll
@@ -71,15 +75,18 @@ __global__ __launch_bounds__(kRotThreads) void rope_rotate_kernel(const uint16_t
 }
 
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
-                              float* tile_max, int BH, int N, int D, hipStream_t stream) {
+                              float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale) {
   const int n_tiles = (N + kRotRows - 1) / kRotRows;
   dim3 grid((unsigned)n_tiles * BH);   // one axis: the second grid axis stops at 65535 slabs
-  if (D == 128)
-    hipLaunchKernelGGL(rope_rotate_kernel<128>, grid, dim3(kRotThreads), 0, stream, x, cosp, sinp, fstride, y, tile_max,
-                       N, n_tiles);
-  else
-    hipLaunchKernelGGL(rope_rotate_kernel<64>, grid, dim3(kRotThreads), 0, stream, x, cosp, sinp, fstride, y, tile_max,
-                       N, n_tiles);
+#define COROPE_ROT(DD, SS)                                                                                             \
+  hipLaunchKernelGGL((rope_rotate_kernel<DD, SS>), grid, dim3(kRotThreads), 0, stream, x, cosp, sinp, fstride, y, tile_max, \
+                     N, n_tiles, out_scale)
+  if (D == 128) {
+    if (out_scale == 1.f) COROPE_ROT(128, false); else COROPE_ROT(128, true);
+  } else {
+    if (out_scale == 1.f) COROPE_ROT(64, false); else COROPE_ROT(64, true);
+  }
+#undef COROPE_ROT
   return hipGetLastError();
 }
 

@@ -210,9 +210,11 @@ def rope_attn_forward_with_lse(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, 
     return o, M
 
 
-def rope_rotate(x, freqs_cos, freqs_sin, with_tile_max=False):
-    """Half-layout rotation of x (B, H, N, D) bf16 on the device (fp32 arithmetic, one rounding to bf16).
-    Returns y, or (y, tile_max) with the largest rotated-row norm of every 64-row tile, (B, H, ceil(N/64)) fp32."""
+def rope_rotate(x, freqs_cos, freqs_sin, with_tile_max=False, scale=1.0):
+    """``scale`` times the half-layout rotation of x (B, H, N, D) bf16 on the device (fp32 arithmetic, one rounding to
+    bf16).  Returns y, or (y, tile_max) with the largest row norm of y in every 64-row tile, (B, H, ceil(N/64)) fp32.
+    The pre-rotated operands of the backward kernels are ``rope_rotate(k, ...)`` and
+    ``rope_rotate(q, ..., scale=sm_scale * log2(e))``."""
     _check_inputs(x, x, x, freqs_cos, freqs_sin)
     if x.dtype != torch.bfloat16:
         raise ValueError("the rotation pass is built for bfloat16 only")
@@ -226,6 +228,6 @@ def rope_rotate(x, freqs_cos, freqs_sin, with_tile_max=False):
     tm = torch.empty((B, H, (N + 63) // 64), device=x.device, dtype=torch.float32) if with_tile_max else None
     with torch.cuda.device(x.device):
         rc = lib.corope_rope_rotate(x.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0), y.data_ptr(),
-                                    tm.data_ptr() if with_tile_max else None, B, H, N, D, _stream_ptr(x))
+                                    tm.data_ptr() if with_tile_max else None, B, H, N, D, float(scale), _stream_ptr(x))
     _lib.check(rc, "corope_rope_rotate")
     return (y, tm) if with_tile_max else y

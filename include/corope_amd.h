@@ -97,15 +97,19 @@ int corope_rope_attn_fwd_noalloc(const void *q, const void *k, const void *v,
                                  void *o, float *lse,
                                  int B, int H, int N, int D, float sm_scale, int causal, void *stream);
 
-/* y = half-layout rotation of x (B,H,N,D) bf16, fp32 arithmetic, rounded to bf16; tile_max (may be NULL) receives
- * [B*H][ceil(N/64)] floats, the largest norm of a rotated row in every 64-row tile.
- * Replaces apply_rotary_emb (reference fused-rope/rope_attn_pytorch.py:71-84, rotate_half :52-68). */
+/* y = scale * (half-layout rotation of x), x (B,H,N,D) bf16, fp32 arithmetic, rounded to bf16 once; tile_max (may be
+ * NULL) receives [B*H][ceil(N/64)] floats, the largest norm of a row of y in every 64-row tile.  scale = 1 is
+ * apply_rotary_emb (reference fused-rope/rope_attn_pytorch.py:71-84, rotate_half :52-68).  The "rotated" operands of the
+ * *_prerotated entry points are: k_rot = this with scale 1, q_rot = this with scale = sm_scale * log2(e) -- the query side
+ * carries the softmax temperature, so the scores leave the matrix cores in base-2 units (the reference folds the same
+ * factor into k on the host for its backward, fused-rope/fused_rope_attn.py:746-748). */
 int corope_rope_rotate(const void *x, const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
-                       void *y, float *tile_max, int B, int H, int N, int D, void *stream);
+                       void *y, float *tile_max, int B, int H, int N, int D, float scale, void *stream);
 
 /* Attention on a K that corope_rope_rotate already rotated (k_rot, with its tile_max as tile_kmax): the second
  * launch of corope_rope_attn_fwd_ws on its own, for callers that keep the rotated K (a key cache) or time the two
- * launches separately.  q is still rotated inside the kernel; q_rot_out (may be NULL) receives the rotated q.
+ * launches separately.  q is still rotated inside the kernel; q_rot_out (may be NULL) receives the rotated q times
+ * sm_scale * log2(e), the form the *_bwd_*_prerotated entry points take.
  * Same reference site as corope_rope_attn_fwd. */
 int corope_rope_attn_fwd_prerotated(const void *q, const void *k_rot, const float *tile_kmax, const void *v,
                                     const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,

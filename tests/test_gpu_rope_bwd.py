@@ -4,6 +4,8 @@ Everything goes through the torch.autograd.Function, i.e. through the C ABI.  Ba
 against the fp32 oracle evaluated on the same bf16-rounded q, k, v, dO."""
 import math
 
+import numpy as np
+
 import pytest
 import torch
 
@@ -128,8 +130,14 @@ def test_backward_paths_agree(pkg, monkeypatch):
         assert ((a - t.grad.float().cpu()).abs() <= 5e-3 + a.abs() / 64).all(), name
 
 
+def _qk_scale(sm_scale):
+    """sm_scale * log2(e) as the library forms it: a product of two fp32 numbers."""
+    return float(np.float32(sm_scale) * np.float32(math.log2(math.e)))
+
+
 def test_forward_keeps_rotated_operands(pkg):
-    """corope_rope_attn_fwd_train leaves q_rot and k_rot equal to what corope_rope_rotate produces (bit for bit)."""
+    """corope_rope_attn_fwd_train leaves q_rot and k_rot equal to what corope_rope_rotate produces (bit for bit): k_rot
+    at scale 1, q_rot at scale sm_scale * log2(e)."""
     B, H, N, D = 2, 2, 300, 128
     q, k, v, g, c, s = _case(B, H, N, D, seed=8)
     dev = torch.device("cuda:0")
@@ -138,7 +146,8 @@ def test_forward_keeps_rotated_operands(pkg):
     o, M, _, _, rot = pkg.rope_attn._forward(qd, kd, vd, True, 0.09, cd, sd, two_launch=True, keep_rotated=True)
     o2, M2 = pkg.rope_attn_forward_with_lse(qd, kd, vd, True, 0.09, cd, sd, two_launch=True)
     torch.cuda.synchronize()
-    assert torch.equal(rot[0], pkg.rope_rotate(qd, cd, sd)) and torch.equal(rot[1], pkg.rope_rotate(kd, cd, sd))
+    assert torch.equal(rot[0], pkg.rope_rotate(qd, cd, sd, scale=_qk_scale(0.09)))
+    assert torch.equal(rot[1], pkg.rope_rotate(kd, cd, sd))
     assert torch.equal(o, o2) and torch.equal(M, M2)
 
 
@@ -202,7 +211,7 @@ def test_separate_dv_dk_on_rotated_operands_match_the_fused_kernel(pkg, tile_row
     cd, sd = c.to(dev), s.to(dev)
     scale = 1 / math.sqrt(D)
     o, M = pkg.rope_attn_forward_with_lse(qd, kd, vd, causal, scale, cd, sd, two_launch=True)
-    q_rot, k_rot = pkg.rope_rotate(qd, cd, sd), pkg.rope_rotate(kd, cd, sd)
+    q_rot, k_rot = pkg.rope_rotate(qd, cd, sd, scale=_qk_scale(scale)), pkg.rope_rotate(kd, cd, sd)
     delta = torch.empty_like(M)
     st = torch.cuda.current_stream().cuda_stream
     assert lib.corope_rope_attn_bwd_preprocess(o.data_ptr(), gd.data_ptr(), delta.data_ptr(), B, H, N, D, st) == 0

@@ -2,7 +2,10 @@
 
 fused-rope/verification.py runs its six cases in fp16 at sm_scale = 0.5 and passes with O max-abs < 1e-2
 (verification.py:67) and max < 0.15, mean < 5e-3 per gradient (verification.py:116) against the PyTorch path in fp16;
-here the same cases run against the fp32 oracle on the same fp16-rounded inputs with those numbers as the bar."""
+here the same cases run against the fp32 oracle on the same fp16-rounded inputs.  The gradients keep the script's
+numbers as the bar.  For O the bar is the operator's own 2e-2: the script's 1e-2 separates two fp16 implementations that
+round the rotated q and k at the same points, so those roundings cancel in its comparison, while against an fp32 oracle
+they show in full (at sm_scale = 0.5 the largest of a million outputs lands between 0.8e-2 and 1.2e-2, seed by seed)."""
 import math
 
 import pytest
@@ -43,7 +46,7 @@ def test_fp16_verification_script_cases(pkg, B, H, N, D, causal):
         print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
         assert torch.isfinite(a).all(), name
         if name == "O":
-            assert err.max() < 1e-2                                  # verification.py:67
+            assert err.max() < 2e-2 and err.mean() < 1e-3             # verification.py:67 has 1e-2 between two fp16 paths
         else:
             assert err.max() < 0.15 and err.mean() < 5e-3, name      # verification.py:116
 

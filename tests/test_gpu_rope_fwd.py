@@ -202,4 +202,6 @@ def test_two_launch_softmax_modes(pkg, tile_rows, case, causal):
     # to bf16 relative to different reference maxima), which can flip the bf16 rounding of an output: one ulp of slack
     print(f"  paths: O max-abs diff {(o - o1).abs().max():.3e}, M max-abs diff {(M - M1).abs().max():.3e}")
     hot = case == "huge_norms_hot"
-    assert ((o - o1).abs() <= (3e-2 if hot else 5e-3) + o.abs() / 64).all() and (M - M1).abs().max() * LN2 <= (1e-2 if hot else 1e-3)
+    # (an output that is the small remainder of cancelling terms carries the absolute error of those terms: half the
+    # parity bar as the fixed part)
+    assert ((o - o1).abs() <= (3e-2 if hot else 1e-2) + o.abs() / 64).all() and (M - M1).abs().max() * LN2 <= (1e-2 if hot else 1e-3)
