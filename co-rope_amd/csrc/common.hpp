@@ -378,9 +378,11 @@ struct WaveRows<D, true> {
   static constexpr int IT = 32 / RPI;
   u32x4 x1[IT], x2[IT];
   f32x4 c[IT][2], s[IT][2];
+  // l: the lane (callers inside a loop over work items pass a value the optimiser cannot see through, so that the
+  // per-lane address parts are recomputed per item instead of being kept in registers across the whole loop)
   __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float* __restrict__ cosp,
-                                       const float* __restrict__ sinp, int64_t fstride, int row0, int n_rows) {
-    const int l = threadIdx.x % kWave;
+                                       const float* __restrict__ sinp, int64_t fstride, int row0, int n_rows,
+                                       int l = threadIdx.x % kWave) {
 #pragma unroll
     for (int i = 0; i < IT; ++i) {
       const int row = min(row0 + RPI * i + l / UPR, n_rows - 1), u = l % UPR;
@@ -427,6 +429,81 @@ struct WaveRows<D, true> {
     lds_order();
   }
 };
+
+// ---- a wave's private 32 x D tile of 16-bit elements without row padding ---------------------------------------------
+// 16-byte chunk c of row r is kept at chunk c ^ swz(r) of the row: sixteen consecutive rows read at one chunk index (the
+// B-operand read, lane = row) then touch sixteen different bank groups, and so do the chunks of one row.  8 KB at D = 128.
+template <int D>
+struct WaveTile {
+  static constexpr int CPR = D / 8;                      // 16-byte chunks per row
+  static constexpr int RP = 16 / CPR > 0 ? 16 / CPR : 1;  // rows per 256 bytes
+  static constexpr int kBytes = 32 * D * 2;
+  __device__ static __forceinline__ int swz(int r) { return (r / RP) & (CPR - 1); }
+  __device__ static __forceinline__ int off(int r, int c) { return r * (D * 2) + ((c ^ swz(r)) << 4); }   // bytes
+};
+
+// WaveRows<D, true>::load's rows, rotated, scaled and rounded, through a WaveTile: rot_out (may be null) receives the rows
+// that lie inside the matrix, `out` the B operand chunks.
+template <int D>
+__device__ __forceinline__ void park_rotated_rows(const WaveRows<D, true>& w, u32x4 (&out)[D / 16], uint8_t* tile,
+                                                  uint16_t* __restrict__ rot_out, int row0, int n_rows, float out_scale,
+                                                  int l = threadIdx.x % kWave) {
+  using WR = WaveRows<D, true>;
+  using T = WaveTile<D>;
+  lds_order();
+#pragma unroll
+  for (int i = 0; i < WR::IT; ++i) {
+    const int r = WR::RPI * i + l / WR::UPR, u = l % WR::UPR;
+    u32x4 y1, y2;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float a0 = elt_lo(w.x1[i][k]), a1 = elt_hi(w.x1[i][k]), b0 = elt_lo(w.x2[i][k]), b1 = elt_hi(w.x2[i][k]);
+      float c0 = w.c[i][k / 2][(2 * k) % 4], c1 = w.c[i][k / 2][(2 * k) % 4 + 1];
+      float s0 = w.s[i][k / 2][(2 * k) % 4], s1 = w.s[i][k / 2][(2 * k) % 4 + 1];
+      y1[k] = pack_elts((a0 * c0 - b0 * s0) * out_scale, (a1 * c1 - b1 * s1) * out_scale);
+      y2[k] = pack_elts((b0 * c0 + a0 * s0) * out_scale, (b1 * c1 + a1 * s1) * out_scale);
+    }
+    *reinterpret_cast<u32x4*>(tile + T::off(r, u)) = y1;
+    *reinterpret_cast<u32x4*>(tile + T::off(r, u + T::CPR / 2)) = y2;
+    if (rot_out != nullptr && row0 + r < n_rows) {
+      uint16_t* dst = byte_offset(rot_out, (uint32_t)(row0 + r) * (D * 2) + u * 16);
+      *reinterpret_cast<u32x4*>(dst) = y1;
+      *reinterpret_cast<u32x4*>(dst + D / 2) = y2;
+    }
+  }
+  lds_order();
+#pragma unroll
+  for (int kc = 0; kc < D / 16; ++kc) out[kc] = *reinterpret_cast<const u32x4*>(tile + T::off(l % 32, 2 * kc + l / 32));
+  lds_order();
+}
+
+// Rows row0 .. row0 + 31 of a (n_rows, D) matrix of 16-bit elements from transposed fp32 accumulators (layout as for
+// store_rows_via_lds below), every value multiplied by `scale` (per lane = per row), one rounding, through a WaveTile:
+// 16-byte stores that cover whole rows.
+template <int D>
+__device__ __forceinline__ void store_rows_via_wave_tile(const f32x16 (&acc)[D / 32], uint16_t* __restrict__ dst, int row0,
+                                                         int n_rows, float scale, uint8_t* tile,
+                                                         int l = threadIdx.x % kWave) {
+  using T = WaveTile<D>;
+  const int lq = l % 32, lh = l / 32;
+  lds_order();
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      *reinterpret_cast<u32x2*>(tile + T::off(lq, db * 4 + g) + 8 * lh) =
+          u32x2{pack_elts(acc[db][4 * g] * scale, acc[db][4 * g + 1] * scale),
+                pack_elts(acc[db][4 * g + 2] * scale, acc[db][4 * g + 3] * scale)};
+  lds_order();
+  constexpr int RPI = kWave / T::CPR;
+#pragma unroll
+  for (int i = 0; i < 32 / RPI; ++i) {
+    const int r = RPI * i + l / T::CPR, c = l % T::CPR, row = row0 + r;
+    const u32x4 x = *reinterpret_cast<const u32x4*>(tile + T::off(r, c));
+    if (row < n_rows) *reinterpret_cast<u32x4*>(byte_offset(dst, (uint32_t)row * (D * 2) + c * 16)) = x;
+  }
+  lds_order();
+}
 
 // Rows row0 .. row0 + 31 of a (n_rows, D) bf16 matrix from transposed fp32 accumulators (lane = row l % 32, acc[db][i] =
 // column db*32 + 8*(i/4) + 4*(l/32) + i%4): every value is multiplied by `scale` (which may

@@ -22,6 +22,19 @@ inline hipError_t allow_dynamic_lds(const void* kernel, int bytes, std::atomic<u
 }
 
 
+// Compute units of the current device (cached per device; 256 on an MI355X): the size of a persistent launch, one
+// workgroup per compute unit.
+inline int device_cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  int n = cached[dev & 63].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+  cached[dev & 63].store(n, std::memory_order_relaxed);
+  return n;
+}
+
 #ifdef COROPE_TRACE
 // Experiment builds only: per-workgroup time stamps (100 MHz counter) for splitting a launch into its phases.
 extern uint64_t* g_trace_buf;
