@@ -349,8 +349,7 @@ struct WaveRows<D, false> {
   static constexpr int IT = 32 / RPI;
   u32x4 x[IT];
   __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float*, const float*, int64_t, int row0,
-                                       int n_rows) {
-    const int l = threadIdx.x % kWave;
+                                       int n_rows, int l = threadIdx.x % kWave) {
 #pragma unroll
     for (int i = 0; i < IT; ++i)
       x[i] = *reinterpret_cast<const u32x4*>(
@@ -477,6 +476,46 @@ __device__ __forceinline__ void park_rotated_rows(const WaveRows<D, true>& w, u3
   lds_order();
 }
 
+// WaveRows<D, false>::load's rows through a WaveTile, as B operand chunks.
+template <int D>
+__device__ __forceinline__ void park_plain_rows(const WaveRows<D, false>& w, u32x4 (&out)[D / 16], uint8_t* tile,
+                                                int l = threadIdx.x % kWave) {
+  using WR = WaveRows<D, false>;
+  using T = WaveTile<D>;
+  lds_order();
+#pragma unroll
+  for (int i = 0; i < WR::IT; ++i) *reinterpret_cast<u32x4*>(tile + T::off(WR::RPI * i + l / WR::CPR, l % WR::CPR)) = w.x[i];
+  lds_order();
+#pragma unroll
+  for (int kc = 0; kc < D / 16; ++kc) out[kc] = *reinterpret_cast<const u32x4*>(tile + T::off(l % 32, 2 * kc + l / 32));
+  lds_order();
+}
+template <int D>
+__device__ __forceinline__ void park_rows(const WaveRows<D, false>& w, u32x4 (&out)[D / 16], uint8_t* tile, float, int l) {
+  park_plain_rows<D>(w, out, tile, l);
+}
+template <int D>
+__device__ __forceinline__ void park_rows(const WaveRows<D, true>& w, u32x4 (&out)[D / 16], uint8_t* tile, float out_scale,
+                                          int l) {
+  park_rotated_rows<D>(w, out, tile, nullptr, 0, 0, out_scale, l);
+}
+
+// Persistent launches: one workgroup per compute unit (or per item, if those are fewer), every workgroup walking a list
+// of items that is fixed by arithmetic.  Items are numbered heaviest first and dealt to the workgroups in rounds,
+// forwards in even rounds and backwards in odd ones, so that the workgroups end up with equal work when the rounds are
+// full and the weights fall linearly (causal attention).  Workgroup ids are dealt round-robin to the 8 XCDs and both
+// directions keep id % 8: with the slab index running fastest in the item number (and slabs a multiple of 8), all items
+// of a slab stay on one XCD and share its L2.
+struct ItemList {
+  int G, fwd, back;
+  __device__ __forceinline__ ItemList() {
+    G = gridDim.x;
+    fwd = blockIdx.x;
+    back = (G % 8 == 0) ? (G - 8 - (fwd & ~7)) + (fwd & 7) : G - 1 - fwd;
+  }
+  __device__ __forceinline__ int at(int round) const { return round * G + ((round & 1) ? back : fwd); }
+};
+
 // Rows row0 .. row0 + 31 of a (n_rows, D) matrix of 16-bit elements from transposed fp32 accumulators (layout as for
 // store_rows_via_lds below), every value multiplied by `scale` (per lane = per row), one rounding, through a WaveTile:
 // 16-byte stores that cover whole rows.
@@ -494,6 +533,59 @@ __device__ __forceinline__ void store_rows_via_wave_tile(const f32x16 (&acc)[D /
       *reinterpret_cast<u32x2*>(tile + T::off(lq, db * 4 + g) + 8 * lh) =
           u32x2{pack_elts(acc[db][4 * g] * scale, acc[db][4 * g + 1] * scale),
                 pack_elts(acc[db][4 * g + 2] * scale, acc[db][4 * g + 3] * scale)};
+  lds_order();
+  constexpr int RPI = kWave / T::CPR;
+#pragma unroll
+  for (int i = 0; i < 32 / RPI; ++i) {
+    const int r = RPI * i + l / T::CPR, c = l % T::CPR, row = row0 + r;
+    const u32x4 x = *reinterpret_cast<const u32x4*>(tile + T::off(r, c));
+    if (row < n_rows) *reinterpret_cast<u32x4*>(byte_offset(dst, (uint32_t)row * (D * 2) + c * 16)) = x;
+  }
+  lds_order();
+}
+
+// The same for accumulators of rotated rows (dQ_r, dK_r): the half-layout rotation is undone in fp32 before the one
+// rounding, d1 = d1r c + d2r s, d2 = d2r c - d1r s.  A lane holds both partners of a pair (columns j and j + D/2 of its
+// row), so this needs no exchange; its 2 x D/4 table values are read in 16-byte pieces, in a step of their own so that a
+// kernel can request them ahead of other loads (loads return in the order they were issued).
+template <int D>
+struct UnrotateTables {
+  static constexpr int NP = (D / 64) * 4;   // 16-byte pieces per table
+  f32x4 c[NP], s[NP];
+  __device__ __forceinline__ void load(const float* __restrict__ cosp, const float* __restrict__ sinp, int64_t fstride,
+                                       int row0, int n_rows, int l = threadIdx.x % kWave) {
+    const uint32_t frow = (uint32_t)min(row0 + l % 32, n_rows - 1) * (uint32_t)fstride;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const uint32_t foff = (frow + (i / 4) * 32 + 8 * (i % 4) + 4 * (l / 32)) * 4;
+      c[i] = *reinterpret_cast<const f32x4*>(byte_offset(cosp, foff));
+      s[i] = *reinterpret_cast<const f32x4*>(byte_offset(sinp, foff));
+    }
+  }
+};
+template <int D>
+__device__ __forceinline__ void store_unrotated_rows_via_wave_tile(const f32x16 (&acc)[D / 32], const UnrotateTables<D>& tb,
+                                                                   uint16_t* __restrict__ dst, int row0, int n_rows,
+                                                                   float scale, uint8_t* tile, int l = threadIdx.x % kWave) {
+  using T = WaveTile<D>;
+  constexpr int NH = D / 64;   // 32-column blocks per half
+  const int lq = l % 32, lh = l / 32;
+  lds_order();
+#pragma unroll
+  for (int db = 0; db < NH; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 c = tb.c[db * 4 + g], s = tb.s[db * 4 + g];
+      float o1[4], o2[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float r1 = acc[db][4 * g + e] * scale, r2 = acc[db + NH][4 * g + e] * scale;
+        o1[e] = r1 * c[e] + r2 * s[e];
+        o2[e] = r2 * c[e] - r1 * s[e];
+      }
+      *reinterpret_cast<u32x2*>(tile + T::off(lq, db * 4 + g) + 8 * lh) = u32x2{pack_elts(o1[0], o1[1]), pack_elts(o1[2], o1[3])};
+      *reinterpret_cast<u32x2*>(tile + T::off(lq, (db + NH) * 4 + g) + 8 * lh) = u32x2{pack_elts(o2[0], o2[1]), pack_elts(o2[2], o2[3])};
+    }
   lds_order();
   constexpr int RPI = kWave / T::CPR;
 #pragma unroll
@@ -596,6 +688,14 @@ __device__ __forceinline__ float wave_prefix_sum(float x) {   // inclusive: lane
   x += dpp_move<0x118, 0xf>(0.f, x);
   x += dpp_move<0x142, 0xa>(0.f, x);
   x += dpp_move<0x143, 0xc>(0.f, x);
+  return x;
+}
+// Sum over each row of 16 lanes, in every lane of the row (rotations within the row: no LDS round trips).
+__device__ __forceinline__ float row16_sum(float x) {
+  x += dpp_move<0x128, 0xf>(0.f, x);   // row_ror:8
+  x += dpp_move<0x124, 0xf>(0.f, x);   // row_ror:4
+  x += dpp_move<0x122, 0xf>(0.f, x);   // row_ror:2
+  x += dpp_move<0x121, 0xf>(0.f, x);   // row_ror:1
   return x;
 }
 __device__ __forceinline__ float wave_last(float x) {          // lane 63's value, wave-uniform

@@ -50,10 +50,24 @@ extern uint64_t* g_trace_buf;
       p.trace[(int64_t)blockIdx.x * 16 + 15] = (uint64_t)(extra);                                              \
     }                                                                                                        \
   } while (0)
+// the same for persistent kernels: stamps are filed under the item (variables `item` and `TT` of the kernel)
+#define COROPE_ISTAMP(slot)                                                                                   \
+  do {                                                                                                        \
+    if (p.trace != nullptr && threadIdx.x == TT) p.trace[(int64_t)item * 16 + (slot)] = __builtin_amdgcn_s_memrealtime(); \
+  } while (0)
+#define COROPE_ISTAMP_ID(extra)                                                                               \
+  do {                                                                                                        \
+    if (p.trace != nullptr && threadIdx.x == TT) {                                                            \
+      p.trace[(int64_t)item * 16 + 14] = (uint64_t)__builtin_amdgcn_s_getreg(63492) | ((uint64_t)__builtin_amdgcn_s_getreg(63508) << 32); \
+      p.trace[(int64_t)item * 16 + 15] = (uint64_t)(extra);                                                    \
+    }                                                                                                         \
+  } while (0)
 #else
 #define COROPE_TRACE_FIELD
 #define COROPE_STAMP(slot, tid) do {} while (0)
 #define COROPE_STAMP_ID(tid, extra) do {} while (0)
+#define COROPE_ISTAMP(slot) do {} while (0)
+#define COROPE_ISTAMP_ID(extra) do {} while (0)
 #endif
 
 // Rows per workgroup of the attention kernels: 256 (8 waves) or 128 (4 waves).  By shape: a launch whose 256-row blocks

@@ -268,14 +268,17 @@ struct DqCfg {
   static constexpr int kBlockM = NWAVES * 32;
   static constexpr int kTileBytes = RowTile<D>::bytes(BLOCK_N);
   static constexpr int kStageBytes = 2 * kTileBytes;
-  static constexpr int kLoopBytes = 2 * kStageBytes;
-  static constexpr int kEpilogueBytes = NWAVES * 32 * kAccTileStride<D> * 4;   // fp32 dQ rows of all waves on their way out
-  // prologue: each wave's 32 operand rows (bf16) and their 32 delta values
-  static constexpr int kPrologueBytes = NWAVES * (RowTile<D>::bytes(32) + 32 * 4);
-  static constexpr int kLdsBytes = kLoopBytes > kEpilogueBytes ? (kLoopBytes > kPrologueBytes ? kLoopBytes : kPrologueBytes)
-                                                               : (kEpilogueBytes > kPrologueBytes ? kEpilogueBytes : kPrologueBytes);
+  static constexpr int kRingBytes = 2 * kStageBytes;
+  // behind the ring, per wave: a private tile for its operand rows on their way in and its dQ rows on their way out, and
+  // the 32 delta values of its rows
+  static constexpr int kWaveBytes = WaveTile<D>::kBytes + 32 * 4;
+  static constexpr int kLdsBytes = kRingBytes + NWAVES * kWaveBytes;
+  static_assert(kLdsBytes <= 160 * 1024, "LDS of a compute unit");
 };
 
+// Persistent, like the forward on a pre-rotated K: one workgroup per compute unit walks a balanced list of (head, query
+// block) items, the stream of K/V tiles runs on from item to item, and nothing at the change of items needs a workgroup
+// barrier (a wave's operand rows and its dQ rows go through an LDS tile of its own).
 template <int D, int NWAVES, int BLOCK_N, bool CAUSAL, bool PREROT>
 __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_bwd_dq_kernel(BwdParams p) {
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
@@ -284,114 +287,175 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   constexpr int LS = RowTile<D>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
-  [[maybe_unused]] constexpr int TT = NT - kWave;   // stamping thread: first lane of the last wave (it sees every tile)
-  COROPE_STAMP(0, TT);
-  const int bh = blockIdx.x % p.BH;
-  const int mb = p.num_blocks - 1 - blockIdx.x / p.BH;  // heaviest (last) query blocks first
-  const int m0 = mb * Cfg::kBlockM;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int lq = lane % 32, lh = lane / 32;
+  // 32-row block of the item this wave owns; waves w and w + 4 share a SIMD, blocks (0,7), (1,6), (2,5), (3,4) give
+  // every SIMD the same number of diagonal tiles
+  const int rb = NWAVES == 8 ? (wave < 4 ? wave : 11 - wave) : wave;
+  [[maybe_unused]] constexpr int TT = NWAVES == 8 ? 4 * kWave : (NWAVES - 1) * kWave;   // stamping thread: first lane of the wave with the last rows
   const int N = p.N;
-  const int64_t base = (int64_t)bh * N * D;
-  const int64_t kv_base = (int64_t)kv_slab(bh, p.H, p.Hkv) * N * D;   // key/value slab of this query head
-  const uint16_t* kg = (PREROT ? p.k_rot : p.k) + kv_base;
-  const uint16_t* vg = p.v + kv_base;
+  uint8_t* const wave_tile = smem + Cfg::kRingBytes + wave * Cfg::kWaveBytes;
+  float* const wave_delta = reinterpret_cast<float*>(wave_tile + WaveTile<D>::kBytes);
 
-  const int q_row = m0 + wave * 32 + lq;
-  const int q_c = min(q_row, N - 1);
-  const int wq_lo = m0 + wave * 32, wq_hi = wq_lo + 31;
-  const int key_limit = CAUSAL ? q_row : N - 1;   // last key this lane's query attends to
+  const ItemList items;
+  const int total = p.num_blocks * p.BH;   // item i (heaviest first): query block num_blocks - 1 - i / BH of head i % BH
+  const int n_k_tiles = (N + BLOCK_N - 1) / BLOCK_N;
+  auto tiles_of = [&](int mb) {
+    return CAUSAL ? min((mb * Cfg::kBlockM + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, n_k_tiles) : n_k_tiles;
+  };
 
-  const int n_tiles = CAUSAL ? min((m0 + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, (N + BLOCK_N - 1) / BLOCK_N)
-                             : (N + BLOCK_N - 1) / BLOCK_N;
+  // ---- the stream of K/V tiles: a cursor one tile ahead of the tile being consumed -------------------------------------
   RopeStage<D, BLOCK_N, NT, PREROT> kst;
   CopyStage<D, BLOCK_N, NT> vst;
-  kst.load(kg, p.cos, p.sin, p.fstride, 0, N);
-  vst.load(vg, 0, N);
-
-  // Q_r and dO rows of the wave as B operands, through a wave-private LDS tile (whole row segments per global load).
-  // Every load of the prologue is issued before the first of them is waited for.
-  u32x4 qb[KC], dob[KC];
-  uint16_t* wave_rows = reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride;
-  WaveRows<D, !PREROT> qrows;
-  WaveRows<D, false> dorows, orows;
-  qrows.load((PREROT ? p.q_rot : p.q) + base, p.cos, p.sin, p.fstride, wq_lo, N);
-  dorows.load(p.d_o + base, nullptr, nullptr, 0, wq_lo, N);
-  if (p.o != nullptr) orows.load(p.o + base, nullptr, nullptr, 0, wq_lo, N);
-  const float lse_q = p.lse[(int64_t)bh * N + q_c];
-  // delta_i = sum_d o_id * do_id (reference _attn_bwd_preprocess, :324-337): read from the preprocess pass, or -- when the
-  // caller hands over O instead -- computed here for the rows this workgroup owns and written out for the dK kernel,
-  // which then has to run after this one.
-  float delta_q = 0.f;
-  if (p.o == nullptr) delta_q = p.delta[(int64_t)bh * N + q_c];
-  qrows.park(qb, wave_rows, nullptr, 0, 0, p.qk_scale);   // Q_r carries qk_scale (a pre-rotated copy already does)
-  dorows.park(dob, wave_rows);
-  if (p.o != nullptr) {
-    // 16 lanes per row: O in registers (same chunk order as dO went into the tile), dO from the tile
-    constexpr int CPR = D / 8, RPI = kWave / CPR;
-    float* wave_delta = reinterpret_cast<float*>(smem + NWAVES * RowTile<D>::bytes(32)) + wave * 32;
-#pragma unroll
-    for (int i = 0; i < 32 / RPI; ++i) {
-      const int r = RPI * i + lane / CPR, ch = lane % CPR;
-      const u32x4 ow = orows.x[i], dw = dorows.x[i];
-      float acc = 0.f;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) acc += elt_lo(ow[w]) * elt_lo(dw[w]) + elt_hi(ow[w]) * elt_hi(dw[w]);
-#pragma unroll
-      for (int m = CPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m);
-      if (ch == 0) wave_delta[r] = acc;
-    }
-    lds_order();
-    delta_q = wave_delta[lq];
-    lds_order();
-    if (lh == 0 && q_row < N) p.delta[(int64_t)bh * N + q_row] = delta_q;
-  }
-
+  int l_round = 0, l_tile = 0, l_tiles;
+  const uint16_t *l_kg, *l_vg;
+  auto load_item = [&](int r) {    // false: no such item
+    const int i = items.at(r);
+    if (i >= total) return false;
+    const int64_t kv_base = (int64_t)kv_slab(i % p.BH, p.H, p.Hkv) * N * D;
+    l_kg = (PREROT ? p.k_rot : p.k) + kv_base;
+    l_vg = p.v + kv_base;
+    l_tiles = tiles_of(p.num_blocks - 1 - i / p.BH);
+    return true;
+  };
+  auto load_next_tile = [&]() __attribute__((always_inline)) {   // moves the cursor on and requests that tile
+    if (l_tile + 1 < l_tiles) {
+      ++l_tile;
+    } else if (load_item(l_round + 1)) {
+      ++l_round;
+      l_tile = 0;
+    }   // else: past the last tile of the last item; the same tile is requested again and never used
+    kst.load(l_kg, p.cos, p.sin, p.fstride, l_tile * BLOCK_N, N);
+    vst.load(l_vg, l_tile * BLOCK_N, N);
+  };
   auto k_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
   auto v_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes + Cfg::kTileBytes); };
+  int cur = 0;   // ring stage of the tile being consumed
 
-  f32x16 dqacc[NDB];
+  // ---- operand rows of an item: Q_r (rotated and scaled here unless a pre-rotated copy is given), dO, O for delta ------
+  // (the lane index goes in as a value the optimiser cannot see through: the per-lane address parts of these steps are
+  // then recomputed per item instead of being kept in registers, or in scratch memory, across the whole loop)
+  auto opaque_lane = [&]() __attribute__((always_inline)) {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    return l;
+  };
+  WaveRows<D, !PREROT> qrows;
+  WaveRows<D, false> dorows, orows;
+  float lse_q, delta_in;
+  u32x4 qb[KC], dob[KC];
+  float delta_q;
+  auto request_rows = [&](int i) __attribute__((always_inline)) {
+    const int bh = i % p.BH, row0 = (p.num_blocks - 1 - i / p.BH) * Cfg::kBlockM + rb * 32;
+    const int64_t base = (int64_t)bh * N * D;
+    const int l = opaque_lane();
+    qrows.load((PREROT ? p.q_rot : p.q) + base, p.cos, p.sin, p.fstride, row0, N, l);
+    dorows.load(p.d_o + base, nullptr, nullptr, 0, row0, N, l);
+    // (without O the dO rows are requested twice: the request is then unconditional and the registers it fills are free
+    // during the tile loop on every path)
+    orows.load((p.o != nullptr ? p.o : p.d_o) + base, nullptr, nullptr, 0, row0, N, l);
+    const int q_c = min(row0 + l % 32, N - 1);
+    lse_q = p.lse[(int64_t)bh * N + q_c];
+    // delta_i = sum_d o_id * do_id (reference _attn_bwd_preprocess, :324-337): read from the preprocess pass, or -- when the
+    // caller hands over O instead -- computed here for the rows this workgroup owns and written out for the dK kernel,
+    // which then has to run after this one.
+    delta_in = 0.f;
+    if (p.o == nullptr) delta_in = p.delta[(int64_t)bh * N + q_c];
+  };
+  auto take_rows = [&](int i) __attribute__((always_inline)) {
+    const int bh = i % p.BH, row0 = (p.num_blocks - 1 - i / p.BH) * Cfg::kBlockM + rb * 32;
+    const int l = opaque_lane();
+    park_rows<D>(qrows, qb, wave_tile, p.qk_scale, l);   // Q_r carries qk_scale (a pre-rotated copy already does)
+    park_plain_rows<D>(dorows, dob, wave_tile, l);
+    delta_q = delta_in;
+    if (p.o != nullptr) {
+      // 16 lanes per row: O and dO in registers, same chunk order
+      constexpr int CPR = D / 8, RPI = kWave / CPR;
 #pragma unroll
-  for (int i = 0; i < NDB; ++i) dqacc[i] = f32x16{0};
+      for (int i2 = 0; i2 < 32 / RPI; ++i2) {
+        const int r = RPI * i2 + l / CPR, ch = l % CPR;
+        const u32x4 ow = orows.x[i2], dw = dorows.x[i2];
+        float acc = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) acc += elt_lo(ow[w]) * elt_lo(dw[w]) + elt_hi(ow[w]) * elt_hi(dw[w]);
+        if constexpr (CPR == 16) {
+          acc = row16_sum(acc);
+        } else {
+#pragma unroll
+          for (int m = CPR / 2; m >= 1; m >>= 1) acc += __shfl_xor(acc, m);
+        }
+        if (ch == 0) wave_delta[r] = acc;
+      }
+      lds_order();
+      delta_q = wave_delta[l % 32];
+      lds_order();
+      if (l / 32 == 0 && row0 + l % 32 < N) p.delta[(int64_t)bh * N + row0 + l % 32] = delta_q;
+    }
+  };
 
-  __syncthreads();   // the tile stages overlap the tiles the waves parked their rows in
+  // ---- first item: nothing to hide its prologue behind ----------------------------------------------------------------
+  int item = items.at(0);
+  COROPE_ISTAMP(0);
+  load_item(0);
+  kst.load(l_kg, p.cos, p.sin, p.fstride, 0, N);
+  vst.load(l_vg, 0, N);
+  request_rows(item);
+  take_rows(item);
   kst.store_rows(k_tile(0));
   vst.store_rows(v_tile(0));
   __syncthreads();
-  COROPE_STAMP(1, TT);
-  COROPE_STAMP_ID(TT, n_tiles);
+
+  for (int round = 0;; ++round) {
+    const int bh = item % p.BH, mb = p.num_blocks - 1 - item / p.BH;
+    const int m0 = mb * Cfg::kBlockM;
+    const int n_tiles = tiles_of(mb);
+    const int q_row = m0 + rb * 32 + lq;
+    const int wq_lo = m0 + rb * 32, wq_hi = wq_lo + 31;
+    const int key_limit = CAUSAL ? q_row : N - 1;   // last key this lane's query attends to
+    // last tile this wave's rows can see
+    const int t_last = __builtin_amdgcn_readfirstlane(CAUSAL ? min(n_tiles - 1, wq_hi / BLOCK_N) : n_tiles - 1);
+    COROPE_ISTAMP(1);
+    COROPE_ISTAMP_ID(n_tiles);
 #ifdef COROPE_TRACE
-  const uint64_t clk0 = __builtin_readcyclecounter();
+    const uint64_t clk0 = __builtin_readcyclecounter();
 #endif
 
-  // S - M leaves the matrix cores: the score products start from -M of the lane's query in every register
-  f32x16 msb;
+    f32x16 dqacc[NDB];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    float x = -lse_q;
-    asm volatile("" : "+v"(x));   // sixteen values of their own: one value in sixteen places is tied to the first of them
-    msb[i] = x;
-  }
-  for (int t = 0; t < n_tiles; ++t) {
-    const int n0 = t * BLOCK_N;
-#ifdef COROPE_TRACE
-    if (t == 1) COROPE_STAMP(3, TT);
-    if (n0 == m0) COROPE_STAMP(4, TT);
-#endif
-    const int cur = t & 1;
-    if (t + 1 < n_tiles) {
-      kst.load(kg, p.cos, p.sin, p.fstride, n0 + BLOCK_N, N);
-      vst.load(vg, n0 + BLOCK_N, N);
+    for (int i = 0; i < NDB; ++i) dqacc[i] = f32x16{0};
+    // S - M leaves the matrix cores: the score products start from -M of the lane's query in every register
+    f32x16 msb;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float x = -lse_q;
+      asm volatile("" : "+v"(x));   // sixteen values of their own: one value in sixteen places is tied to the first of them
+      msb[i] = x;
     }
-    const bool active = !CAUSAL || n0 <= wq_hi;
-    if (active) {
+    // the wave's operands have landed on every path into the loop (left to their first use, the wait would sit inside
+    // the loop and there also wait for the next tile's loads)
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) asm volatile("" ::"v"(qb[kc]), "v"(dob[kc]));
+    asm volatile("" ::"v"(delta_q));
+
+    auto stage_next = [&]() __attribute__((always_inline)) {
+      kst.store_rows(k_tile(cur ^ 1));
+      vst.store_rows(v_tile(cur ^ 1));
+    };
+
+    for (int t = 0; t <= t_last; ++t) {
+      const int n0 = t * BLOCK_N;
+#ifdef COROPE_TRACE
+      if (t == 1) COROPE_ISTAMP(3);
+      if (n0 == m0) COROPE_ISTAMP(4);
+#endif
+      load_next_tile();
       const uint16_t* ks = k_tile(cur);
       const uint16_t* vs = v_tile(cur);
       const bool need_mask = (CAUSAL && n0 + BLOCK_N - 1 > wq_lo) || (!CAUSAL && n0 + BLOCK_N > N);
       u32x4 dsb[BLOCK_N / 16];
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb) {
-        f32x16 sacc, dpacc;   // the first MFMA of each product takes a literal zero as its accumulator
+        f32x16 sacc, dpacc;   // dP starts from a literal zero, S from -M
         const uint16_t* krow = ks + RowTile<D>::off(kb * 32 + lq, 8 * lh);
         const uint16_t* vrow = vs + RowTile<D>::off(kb * 32 + lq, 8 * lh);
 #pragma unroll
@@ -426,26 +490,42 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
           dqacc[db] = mfma32(load_a_trans(ks, LS, 16 * c, db * 32), dsb[c], dqacc[db]);
+      stage_next();
+      cur ^= 1;
+      __syncthreads();
     }
-    if (t + 1 < n_tiles) {
-      kst.store_rows(k_tile(cur ^ 1));
-      vst.store_rows(v_tile(cur ^ 1));
+    COROPE_ISTAMP(5);
+#ifdef COROPE_TRACE
+    if (p.trace != nullptr && threadIdx.x == TT) p.trace[(int64_t)item * 16 + 7] = __builtin_readcyclecounter() - clk0;
+#endif
+    // The next item's rows are requested as soon as the registers of this item's rows are free.  (After the last item its
+    // own rows are requested once more and never used: the request is then unconditional, and the registers it fills are
+    // free during the tile loop on every path.)
+    // Ahead of them go the table values that the item's dQ rows need on their way out: loads return in the order they
+    // were issued, and those must not wait for the next item's rows.
+    // (Only on pre-rotated operands: rows that are rotated here travel with their own table values, and both sets do not
+    // fit the registers.)
+    UnrotateTables<D> tb;
+    if constexpr (PREROT) tb.load(p.cos, p.sin, p.fstride, wq_lo, N, opaque_lane());
+    const int next_item = items.at(round + 1);
+    const bool has_next = next_item < total;
+    request_rows(has_next ? next_item : item);
+    // of the tiles entirely above this wave's diagonal it only stages its share
+    for (int t = t_last + 1; t < n_tiles; ++t) {
+      load_next_tile();
+      stage_next();
+      cur ^= 1;
+      __syncthreads();
     }
-    __syncthreads();
+    // dQ_r -> dQ: scaled, un-rotated in fp32, rounded once, whole rows per store
+    if constexpr (!PREROT) tb.load(p.cos, p.sin, p.fstride, wq_lo, N, opaque_lane());
+    store_unrotated_rows_via_wave_tile<D>(dqacc, tb, p.dq + (int64_t)bh * N * D, wq_lo, N, p.sm_scale, wave_tile, opaque_lane());
+    COROPE_ISTAMP(6);
+    if (!has_next) break;
+    item = next_item;
+    COROPE_ISTAMP(0);
+    take_rows(item);
   }
-
-  COROPE_STAMP(5, TT);
-#ifdef COROPE_TRACE
-  if (p.trace != nullptr && threadIdx.x == TT) p.trace[(int64_t)blockIdx.x * 16 + 7] = __builtin_readcyclecounter() - clk0;
-#endif
-  // every wave is past its last read of the tiles (the loop ends with a barrier): their LDS now carries dQ_r to a
-  // row-major order, so that the tables are read and dQ is written in whole row segments
-  store_rows_via_lds<D, true>(dqacc, p.dq + base, wq_lo, N, p.cos, p.sin, p.fstride, p.sm_scale,
-                              reinterpret_cast<float*>(smem) + wave * 32 * kAccTileStride<D>);
-#ifdef COROPE_TRACE
-  __builtin_amdgcn_s_waitcnt(0);
-  COROPE_STAMP(6, TT);
-#endif
 }
 
 // ===================================================================================== launchers
@@ -483,7 +563,10 @@ static hipError_t launch_dq_waves(BwdParams p, hipStream_t stream) {
 #ifdef COROPE_TRACE
   p.trace = g_trace_buf;
 #endif
-  hipLaunchKernelGGL(kern, dim3(p.num_blocks * p.BH), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
+  // one workgroup per compute unit, or per item if those are fewer
+  const int64_t n_items = (int64_t)p.num_blocks * p.BH;
+  const int cus = device_cu_count();
+  hipLaunchKernelGGL(kern, dim3((unsigned)(n_items < cus ? n_items : cus)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
 }
 

@@ -74,15 +74,6 @@ __device__ __forceinline__ void softmax_pair(int j, const f32x16& sacc, u32x4 (&
 
 __device__ __forceinline__ float wave_reduce_max(float x) { return wave_max(x); }   // data-parallel-primitive moves, no LDS round trips
 
-#ifdef COROPE_TRACE
-#define COROPE_ISTAMP(slot)                                                                                   \
-  do {                                                                                                        \
-    if (p.trace != nullptr && threadIdx.x == TT) p.trace[(int64_t)item * 16 + (slot)] = __builtin_amdgcn_s_memrealtime(); \
-  } while (0)
-#else
-#define COROPE_ISTAMP(slot) do {} while (0)
-#endif
-
 // Persistent: the launch has one workgroup per compute unit (or per item, if those are fewer) and every workgroup walks
 // its own list of items, an item being 32*NW query rows of one (batch, head).  The lists are fixed by arithmetic: items
 // are ordered heaviest first (causal: last query block first; within a block over the heads), dealt to the workgroups in
@@ -116,10 +107,9 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
   uint8_t* const wave_tile = smem + Cfg::kRingBytes + wave * WaveTile<D>::kBytes;
 
   // ---- the workgroup's list of items --------------------------------------------------------------------------------
-  const int G = gridDim.x, g = blockIdx.x;
+  const ItemList items;
   const int total = p.num_m_blocks * p.BH;
-  const int g_back = (G % 8 == 0) ? (G - 8 - (g & ~7)) + (g & 7) : G - 1 - g;
-  auto item_at = [&](int r) { return r * G + ((r & 1) ? g_back : g); };   // position in the heaviest-first order; >= total: none
+  auto item_at = [&](int r) { return items.at(r); };   // position in the heaviest-first order; >= total: none
   const int n_k_tiles = (N + BLOCK_N - 1) / BLOCK_N;
   auto tiles_of = [&](int mb) {
     return CAUSAL ? min((mb * Cfg::kBlockM + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, n_k_tiles) : n_k_tiles;
@@ -295,10 +285,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
     asm volatile("" ::"v"(kvec));
     COROPE_ISTAMP(2);
 #ifdef COROPE_TRACE
-    if (p.trace != nullptr && threadIdx.x == TT) {
-      p.trace[(int64_t)item * 16 + 14] = (uint64_t)__builtin_amdgcn_s_getreg(63492) | ((uint64_t)__builtin_amdgcn_s_getreg(63508) << 32);
-      p.trace[(int64_t)item * 16 + 15] = (uint64_t)n_tiles;
-    }
+    COROPE_ISTAMP_ID(n_tiles);
     const uint64_t clk0 = __builtin_readcyclecounter();
     uint64_t exact_passes = 0;   // tiles of this wave that were examined a second time to move the reference
 #endif
