@@ -452,6 +452,8 @@ def bench_phase_trace(args):
     print(f"Workload: {cfg['name']}, data {args.data}; times in microseconds per workgroup (256 rows) unless said otherwise.\n")
     for name, buf in bufs.items():
         a = buf.cpu().numpy().reshape(-1, 16)
+        if args.trace_dump:
+            np.save(os.path.join(args.trace_dump, f"trace_{name}_{args.data}.npy"), a)
         a = a[a[:, 0] != 0]
         t = a[:, :14].astype(np.float64) * 0.01
         t = np.where(a[:, :14] != 0, t - t[:, 0].min(), np.nan)
@@ -517,6 +519,8 @@ def main():
                     help="synthetic inputs: N(0,1), or attention-sink-like keys (see make_inputs)")
     ap.add_argument("--phase-trace", action="store_true",
                     help="split the attention kernels of the chosen RoPE config into phases (trace build of the library)")
+    ap.add_argument("--trace-dump", default=None, metavar="DIR",
+                    help="with --phase-trace: also save the raw stamps of every kernel (one row of 16 per item) as .npy files there")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()

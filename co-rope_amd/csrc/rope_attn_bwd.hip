@@ -28,9 +28,14 @@ namespace COROPE_NS {
 //   dK_r^T += Q_r^T dS        (A = Q_r tile read transposed, B = dS)
 // DO_PAD: row padding of the dO tile.  The dV-only kernel reads dO through the transposing load alone and takes the
 // padding that is conflict-free for it (32); the dK kernel reads dO row-wise (8).
-// V_LDS: the workgroup's V rows live in LDS (behind the two tile stages) instead of registers -- the fused dK+dV kernel,
-// whose two sets of accumulators leave no room for them.
-template <int D, int NWAVES, int BLOCK_M, int DO_PAD, bool V_LDS>
+// V_LDS: the waves' V rows live in LDS instead of registers -- the fused dK+dV kernel, whose two sets of accumulators
+// leave no room for them.
+//
+// Persistent, like the other attention kernels: one workgroup per compute unit walks a balanced list of (key/value slab,
+// key block) items and the stream of query tiles runs on from item to item.  Behind the two tile stages every wave has an
+// LDS slot of its own (32 padded rows): its V rows during an item (V_LDS), and at the change of items the tile through
+// which its dV and dK rows leave and its next K_r rows come in -- nothing there needs a workgroup barrier.
+template <int D, int NWAVES, int BLOCK_M, int DO_PAD>
 struct DkdvCfg {
   static constexpr int kThreads = NWAVES * kWave;
   static constexpr int kBlockN = NWAVES * 32;
@@ -38,12 +43,11 @@ struct DkdvCfg {
   static constexpr int kDoTileBytes = RowTile<D, DO_PAD>::bytes(BLOCK_M);
   static constexpr int kStatBytes = BLOCK_M * 4;
   static constexpr int kStageBytes = kTileBytes + kDoTileBytes + 2 * kStatBytes;
-  static constexpr int kVRowsBytes = V_LDS ? RowTile<D>::bytes(kBlockN) : 0;
-  static constexpr int kLoopBytes = 2 * kStageBytes + kVRowsBytes;
-  static constexpr int kEpilogueBytes = NWAVES * 32 * kAccTileStride<D> * 4;   // fp32 rows of all waves on their way out
-  static constexpr int kLdsBytes = kLoopBytes > kEpilogueBytes ? kLoopBytes : kEpilogueBytes;
-  // the prologue parks each wave's 32 operand rows in the two tile stages, next to (not on) the V rows
-  static_assert(NWAVES * RowTile<D>::bytes(32) <= 2 * kStageBytes, "prologue tiles do not fit the tile stages");
+  static constexpr int kRingBytes = 2 * kStageBytes;
+  static constexpr int kWaveBytes = RowTile<D>::bytes(32);
+  static_assert(kWaveBytes >= WaveTile<D>::kBytes, "a wave's slot holds its unpadded tile too");
+  static constexpr int kLdsBytes = kRingBytes + NWAVES * kWaveBytes;
+  static_assert(kLdsBytes <= 160 * 1024, "LDS of a compute unit");
 };
 
 // PREROT: Q and K come from copies that rope_rotate_kernel rotated beforehand (no table reads in the loop).
@@ -51,52 +55,58 @@ template <int D, int NWAVES, int BLOCK_M, bool CAUSAL, bool DO_DV, bool DO_DK, b
 __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
   constexpr int DO_PAD = DO_DK ? 8 : 32;
   constexpr bool V_LDS = DO_DV && DO_DK;
-  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_PAD, V_LDS>;
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_PAD>;
   constexpr int NT = Cfg::kThreads;
   constexpr int KC = D / 16, NDB = D / 32, NQB = BLOCK_M / 32;
   constexpr int LS = RowTile<D>::kStride, LSDO = RowTile<D, DO_PAD>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
-  // The workgroup owns a key block of one key/value slab and sweeps the query tiles of every query head of its group
-  // (one head without grouped-query attention), accumulating dK and dV over all of them.
-  COROPE_STAMP(0, 0);
-  const int BHkv = p.BH / p.H * p.Hkv, GQ = p.H / p.Hkv;
-  const int bkv = blockIdx.x % BHkv;
-  const int nb = blockIdx.x / BHkv;  // key block; for causal the low blocks are the heavy ones and start first
-  const int n0 = nb * Cfg::kBlockN;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int lq = lane % 32, lh = lane / 32;
+  // 32-key block of the item this wave owns; waves w and w + 4 share a SIMD, blocks (0,7), (1,6), (2,5), (3,4) give
+  // every SIMD the same number of diagonal tiles
+  const int rb = NWAVES == 8 ? (wave < 4 ? wave : 11 - wave) : wave;
+  [[maybe_unused]] constexpr int TT = 0;   // stamping thread: first lane of the wave with the first keys (it sees every tile)
   const int N = p.N;
-  const int64_t base = (int64_t)bkv * N * D;                           // k, v, dk, dv
-  const int q_slab0 = (bkv / p.Hkv) * p.H + (bkv % p.Hkv) * GQ;        // first query head of the group
+  uint8_t* const wave_slot = smem + Cfg::kRingBytes + wave * Cfg::kWaveBytes;
+  uint16_t* const vrows = reinterpret_cast<uint16_t*>(wave_slot);   // V_LDS: the wave's V rows, row-major, padded
+
+  // An item: a key block of one key/value slab; its workgroup sweeps the query tiles of every query head of the group
+  // (one head without grouped-query attention), accumulating dK and dV over all of them.  Heaviest first: causal key
+  // blocks see fewer query tiles the later they lie.
+  const ItemList items;
+  const int BHkv = p.BH / p.H * p.Hkv, GQ = p.H / p.Hkv;
+  const int total = p.num_blocks * BHkv;   // item i: key block i / BHkv of slab i % BHkv
+  const int m_tiles = (N + BLOCK_M - 1) / BLOCK_M;
   const uint16_t* q_all = PREROT ? p.q_rot : p.q;
 
-  const int key = n0 + wave * 32 + lq;
-  const int wk_lo = n0 + wave * 32, wk_hi = wk_lo + 31;
-
-  // The wave's K_r (and V) rows as B operands, through a wave-private LDS tile (whole row segments per global load).
-  // Every load of the prologue is issued before the first of them is waited for.
-  u32x4 kb[KC], vb[(DO_DK && !V_LDS) ? KC : 1];
-  uint16_t* wave_rows = reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride;
-  uint16_t* vrows = reinterpret_cast<uint16_t*>(smem + 2 * Cfg::kStageBytes);   // V_LDS: the block's V rows, row-major
-  WaveRows<D, !PREROT> krows;
-  krows.load((PREROT ? p.k_rot : p.k) + base, p.cos, p.sin, p.fstride, wk_lo, N);
-  WaveRows<D, false> vrows_regs;
-  if constexpr (DO_DK && !V_LDS) vrows_regs.load(p.v + base, nullptr, nullptr, 0, wk_lo, N);
-  CopyStage<D, Cfg::kBlockN, NT> vcp;
-  if constexpr (V_LDS) vcp.load(p.v + base, n0, N);
-
+  // ---- the stream of query tiles: a cursor one tile ahead of the tile being consumed -----------------------------------
   RopeStage<D, BLOCK_M, NT, PREROT, true> qst;   // Q_r tiles carry qk_scale: S leaves the matrix cores in base-2 units
   qst.out_scale = p.qk_scale;
   CopyStage<D, BLOCK_M, NT, DO_PAD> dst;
   float st_lse = 0.f, st_delta = 0.f;
-  const int m_tiles = (N + BLOCK_M - 1) / BLOCK_M;
-  const int mt0 = CAUSAL ? n0 / BLOCK_M : 0;
-  const int tiles_per_head = max(m_tiles - mt0, 0), n_iter = GQ * tiles_per_head;
-  // iteration it -> query head q_slab0 + it / tiles_per_head, query tile mt0 + it % tiles_per_head
-  auto tile_m0 = [&](int it) { return (mt0 + it % tiles_per_head) * BLOCK_M; };
-  auto load_tile = [&](int it) {
-    const int qs = q_slab0 + it / tiles_per_head, m0 = tile_m0(it);
+  int l_round = 0, l_it = 0, l_iters, l_slab0, l_mt0, l_tph;
+  auto load_item = [&](int r) {    // false: no such item
+    const int i = items.at(r);
+    if (i >= total) return false;
+    const int bkv = i % BHkv, n0 = (i / BHkv) * Cfg::kBlockN;
+    l_slab0 = (bkv / p.Hkv) * p.H + (bkv % p.Hkv) * GQ;   // first query head of the group
+    l_mt0 = CAUSAL ? n0 / BLOCK_M : 0;
+    l_tph = max(m_tiles - l_mt0, 0);
+    l_iters = GQ * l_tph;
+    return true;
+  };
+  // iteration it of an item -> query head slab0 + it / tph, query tile mt0 + it % tph
+  auto load_next_tile = [&](bool advance) __attribute__((always_inline)) {
+    if (advance) {
+      if (l_it + 1 < l_iters) {
+        ++l_it;
+      } else if (load_item(l_round + 1)) {
+        ++l_round;
+        l_it = 0;
+      }   // else: past the last tile of the last item; the same tile is requested again and never used
+    }
+    const int qs = l_slab0 + l_it / l_tph, m0 = (l_mt0 + l_it % l_tph) * BLOCK_M;
     qst.load(q_all + (int64_t)qs * N * D, p.cos, p.sin, p.fstride, m0, N);
     dst.load(p.d_o + (int64_t)qs * N * D, m0, N);
     if (threadIdx.x < BLOCK_M) {
@@ -115,7 +125,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   auto delta_tile = [&](int buf) {
     return reinterpret_cast<float*>(smem + buf * Cfg::kStageBytes + Cfg::kTileBytes + Cfg::kDoTileBytes + Cfg::kStatBytes);
   };
-  auto store_tile = [&](int buf) {
+  auto store_tile = [&](int buf) __attribute__((always_inline)) {
     qst.store_rows(q_tile(buf));
     dst.store_rows(do_tile(buf));
     if (threadIdx.x < BLOCK_M) {
@@ -123,136 +133,192 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
       if constexpr (DO_DK) delta_tile(buf)[threadIdx.x] = st_delta;
     }
   };
+  int cur = 0;   // ring stage of the tile being consumed
 
-  f32x16 dvacc[DO_DV ? NDB : 1], dkacc[DO_DK ? NDB : 1];
+  // ---- the wave's K_r (and V) rows of an item ----------------------------------------------------------------------
+  // (the lane index goes in as a value the optimiser cannot see through: the per-lane address parts of these steps are
+  // then recomputed per item instead of being kept in registers, or in scratch memory, across the whole loop)
+  auto opaque_lane = [&]() __attribute__((always_inline)) {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    return l;
+  };
+  WaveRows<D, !PREROT> krows;
+  WaveRows<D, false> vrows_regs;
+  u32x4 kb[KC], vb[(DO_DK && !V_LDS) ? KC : 1];
+  auto request_rows = [&](int i) __attribute__((always_inline)) {
+    const int64_t base = (int64_t)(i % BHkv) * N * D;
+    const int row0 = (i / BHkv) * Cfg::kBlockN + rb * 32, l = opaque_lane();
+    krows.load((PREROT ? p.k_rot : p.k) + base, p.cos, p.sin, p.fstride, row0, N, l);
+    if constexpr (DO_DK) vrows_regs.load(p.v + base, nullptr, nullptr, 0, row0, N, l);
+  };
+  auto take_rows = [&]() __attribute__((always_inline)) {
+    const int l = opaque_lane();
+    park_rows<D>(krows, kb, wave_slot, 1.f, l);
+    if constexpr (DO_DK && !V_LDS) park_plain_rows<D>(vrows_regs, vb, wave_slot, l);
+    if constexpr (V_LDS) {
+      using WR = WaveRows<D, false>;
+      lds_order();
 #pragma unroll
-  for (int i = 0; i < NDB; ++i) {
-    if constexpr (DO_DV) dvacc[i] = f32x16{0};
-    if constexpr (DO_DK) dkacc[i] = f32x16{0};
-  }
+      for (int i = 0; i < WR::IT; ++i)
+        *reinterpret_cast<u32x4*>(vrows + RowTile<D>::off(WR::RPI * i + l / WR::CPR, (l % WR::CPR) * 8)) = vrows_regs.x[i];
+      lds_order();
+    }
+  };
 
-  if (n_iter > 0) load_tile(0);
-  krows.park(kb, wave_rows);
-  if constexpr (DO_DK && !V_LDS) vrows_regs.park(vb, wave_rows);
-  if constexpr (V_LDS) vcp.store_rows(vrows);    // visible after the barrier that ends the prologue
-  __syncthreads();   // the tile stages overlap the tiles the waves parked their rows in
-  if (n_iter > 0) store_tile(0);
-  // The wave's K_r (and V) rows must have landed on EVERY path into the loop: left to the first product that reads them,
-  // the wait for them is placed inside the loop, where each time round it also waits for the next tile's loads issued
-  // a few instructions earlier, and the prefetch hides less.
-#pragma unroll
-  for (int kc = 0; kc < KC; ++kc) {
-    asm volatile("" ::"v"(kb[kc]));
-    if constexpr (DO_DK && !V_LDS) asm volatile("" ::"v"(vb[kc]));
-  }
+  // ---- first item: nothing to hide its prologue behind ----------------------------------------------------------------
+  int item = items.at(0);
+  COROPE_ISTAMP(0);
+  load_item(0);
+  load_next_tile(false);
+  request_rows(item);
+  take_rows();
+  store_tile(0);
   __syncthreads();
-  COROPE_STAMP(1, 0);
-  COROPE_STAMP_ID(0, n_iter);
+
+  for (int round = 0;; ++round) {
+    const int bkv = item % BHkv, n0 = (item / BHkv) * Cfg::kBlockN;
+    const int64_t base = (int64_t)bkv * N * D;                           // k, v, dk, dv
+    const int mt0 = CAUSAL ? n0 / BLOCK_M : 0;
+    const int tiles_per_head = max(m_tiles - mt0, 0), n_iter = GQ * tiles_per_head;
+    const int wk_lo = n0 + rb * 32, wk_hi = wk_lo + 31;
+    const int key = wk_lo + lq;
+    COROPE_ISTAMP(1);
+    COROPE_ISTAMP_ID(n_iter);
 #ifdef COROPE_TRACE
-  const uint64_t clk0 = __builtin_readcyclecounter();
+    const uint64_t clk0 = __builtin_readcyclecounter();
 #endif
 
-  for (int it = 0; it < n_iter; ++it) {
-    const int m0 = tile_m0(it);
-#ifdef COROPE_TRACE
-    if (it == 1) COROPE_STAMP(3, 0);
-    if (it == Cfg::kBlockN / BLOCK_M) COROPE_STAMP(4, 0);   // first tile past the diagonal block
-#endif
-    const int cur = it & 1;
-    if (it + 1 < n_iter) load_tile(it + 1);
+    f32x16 dvacc[DO_DV ? NDB : 1], dkacc[DO_DK ? NDB : 1];
+#pragma unroll
+    for (int i = 0; i < NDB; ++i) {
+      if constexpr (DO_DV) dvacc[i] = f32x16{0};
+      if constexpr (DO_DK) dkacc[i] = f32x16{0};
+    }
+    // The wave's K_r (and V) rows must have landed on EVERY path into the loop: left to the first product that reads
+    // them, the wait for them is placed inside the loop, where each time round it also waits for the next tile's loads
+    // issued a few instructions earlier, and the prefetch hides less.
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) {
+      asm volatile("" ::"v"(kb[kc]));
+      if constexpr (DO_DK && !V_LDS) asm volatile("" ::"v"(vb[kc]));
+    }
 
-    const uint16_t* qs = q_tile(cur);
-    const uint16_t* dos = do_tile(cur);
-    const float* lses = lse_tile(cur);
-    const float* deltas = delta_tile(cur);
+    for (int it = 0; it < n_iter; ++it) {
+      const int m0 = (mt0 + it % tiles_per_head) * BLOCK_M;
+#ifdef COROPE_TRACE
+      if (it == 1) COROPE_ISTAMP(3);
+      if (it == Cfg::kBlockN / BLOCK_M) COROPE_ISTAMP(4);   // first tile past the diagonal block
+#endif
+      load_next_tile(true);
+
+      const uint16_t* qs = q_tile(cur);
+      const uint16_t* dos = do_tile(cur);
+      const float* lses = lse_tile(cur);
+      const float* deltas = delta_tile(cur);
 #pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) {
-      const int mq0 = m0 + qb * 32;
-      // queries of this 32-row block that lie above every key of the wave see none of them
-      if (CAUSAL && mq0 + 31 < wk_lo) continue;
-      // The products start from -M and -delta of their rows (register i holds query 8*(i/4) + 4*lh + i%4 of the block):
-      // S - M and dP - delta leave the matrix cores, no vector instruction applies them.
-      f32x16 sacc, dpacc = f32x16{0};
+      for (int qb = 0; qb < NQB; ++qb) {
+        const int mq0 = m0 + qb * 32;
+        // queries of this 32-row block that lie above every key of the wave see none of them
+        if (CAUSAL && mq0 + 31 < wk_lo) continue;
+        // The products start from -M and -delta of their rows (register i holds query 8*(i/4) + 4*lh + i%4 of the block):
+        // S - M and dP - delta leave the matrix cores, no vector instruction applies them.
+        f32x16 sacc, dpacc = f32x16{0};
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x4 m4 = *reinterpret_cast<const f32x4*>(lses + qb * 32 + 8 * g + 4 * lh);
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 m4 = *reinterpret_cast<const f32x4*>(lses + qb * 32 + 8 * g + 4 * lh);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) sacc[4 * g + e] = m4[e];
-        if constexpr (DO_DK) {
-          const f32x4 d4 = *reinterpret_cast<const f32x4*>(deltas + qb * 32 + 8 * g + 4 * lh);
+          for (int e = 0; e < 4; ++e) sacc[4 * g + e] = m4[e];
+          if constexpr (DO_DK) {
+            const f32x4 d4 = *reinterpret_cast<const f32x4*>(deltas + qb * 32 + 8 * g + 4 * lh);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) dpacc[4 * g + e] = d4[e];
+            for (int e = 0; e < 4; ++e) dpacc[4 * g + e] = d4[e];
+          }
         }
-      }
-      const uint16_t* qrow = qs + RowTile<D>::off(qb * 32 + lq, 8 * lh);
-      const uint16_t* dorow = dos + RowTile<D, DO_PAD>::off(qb * 32 + lq, 8 * lh);
-#pragma unroll
-      for (int kc = 0; kc < KC; ++kc)
-        sacc = mfma32(*reinterpret_cast<const u32x4*>(qrow + 16 * kc), kb[kc], sacc);
-      if constexpr (DO_DK) {
+        const uint16_t* qrow = qs + RowTile<D>::off(qb * 32 + lq, 8 * lh);
+        const uint16_t* dorow = dos + RowTile<D, DO_PAD>::off(qb * 32 + lq, 8 * lh);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
-          dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc),
-                         V_LDS ? *reinterpret_cast<const u32x4*>(vrows + RowTile<D>::off(wave * 32 + lq, 8 * lh + 16 * kc)) : vb[V_LDS ? 0 : kc],
-                         dpacc);
-      }
-
-      // Causal mask on the raw scores, under a wave-uniform branch of its own (written into the exponential loop it
-      // is turned into compare + select on every tile).  Register i holds query mq0 + 8*(i/4) + 4*lh + i%4; the
-      // lane-dependent part of the threshold goes into one opaque value so that the 16 thresholds stay immediates.
-      if (CAUSAL && mq0 < wk_hi) {
-        int rel = key - mq0 - 4 * lh;
-        asm volatile("" : "+v"(rel));
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-          if (8 * (i / 4) + i % 4 < rel) sacc[i] = -INFINITY;
-      }
-      u32x4 pb[2], dsb[2];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        float pv[4], ds[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          pv[e] = fast_exp2(sacc[4 * g + e]);
-          ds[e] = pv[e] * dpacc[4 * g + e];
-        }
-        if constexpr (DO_DV) {
-          pb[g / 2][2 * (g % 2)] = pack_elts(pv[0], pv[1]);
-          pb[g / 2][2 * (g % 2) + 1] = pack_elts(pv[2], pv[3]);
-        }
+          sacc = mfma32(*reinterpret_cast<const u32x4*>(qrow + 16 * kc), kb[kc], sacc);
         if constexpr (DO_DK) {
-          dsb[g / 2][2 * (g % 2)] = pack_elts(ds[0], ds[1]);
-          dsb[g / 2][2 * (g % 2) + 1] = pack_elts(ds[2], ds[3]);
-        }
-      }
 #pragma unroll
-      for (int cc = 0; cc < 2; ++cc) {
-        const int kbase = qb * 32 + 16 * cc;
-#pragma unroll
-        for (int db = 0; db < NDB; ++db) {
-          if constexpr (DO_DV) dvacc[db] = mfma32(load_a_trans(dos, LSDO, kbase, db * 32), pb[cc], dvacc[db]);
-          if constexpr (DO_DK) dkacc[db] = mfma32(load_a_trans(qs, LS, kbase, db * 32), dsb[cc], dkacc[db]);
+          for (int kc = 0; kc < KC; ++kc)
+            dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc),
+                           V_LDS ? *reinterpret_cast<const u32x4*>(vrows + RowTile<D>::off(lq, 8 * lh + 16 * kc)) : vb[V_LDS ? 0 : kc],
+                           dpacc);
         }
-      }
-    }
-    if (it + 1 < n_iter) store_tile(cur ^ 1);
-    __syncthreads();
-  }
 
-  COROPE_STAMP(5, 0);
+        // Causal mask on the raw scores, under a wave-uniform branch of its own (written into the exponential loop it
+        // is turned into compare + select on every tile).  Register i holds query mq0 + 8*(i/4) + 4*lh + i%4; the
+        // lane-dependent part of the threshold goes into one opaque value so that the 16 thresholds stay immediates.
+        if (CAUSAL && mq0 < wk_hi) {
+          int rel = key - mq0 - 4 * lh;
+          asm volatile("" : "+v"(rel));
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            if (8 * (i / 4) + i % 4 < rel) sacc[i] = -INFINITY;
+        }
+        u32x4 pb[2], dsb[2];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          float pv[4], ds[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            pv[e] = fast_exp2(sacc[4 * g + e]);
+            ds[e] = pv[e] * dpacc[4 * g + e];
+          }
+          if constexpr (DO_DV) {
+            pb[g / 2][2 * (g % 2)] = pack_elts(pv[0], pv[1]);
+            pb[g / 2][2 * (g % 2) + 1] = pack_elts(pv[2], pv[3]);
+          }
+          if constexpr (DO_DK) {
+            dsb[g / 2][2 * (g % 2)] = pack_elts(ds[0], ds[1]);
+            dsb[g / 2][2 * (g % 2) + 1] = pack_elts(ds[2], ds[3]);
+          }
+        }
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+          const int kbase = qb * 32 + 16 * cc;
+#pragma unroll
+          for (int db = 0; db < NDB; ++db) {
+            if constexpr (DO_DV) dvacc[db] = mfma32(load_a_trans(dos, LSDO, kbase, db * 32), pb[cc], dvacc[db]);
+            if constexpr (DO_DK) dkacc[db] = mfma32(load_a_trans(qs, LS, kbase, db * 32), dsb[cc], dkacc[db]);
+          }
+        }
+        // without the causal branches the two blocks of a tile are one stretch of code: kept apart, or the scheduler
+        // interleaves them and needs both blocks' score registers at once
+        if constexpr (!CAUSAL) __builtin_amdgcn_sched_barrier(0);
+      }
+      store_tile(cur ^ 1);
+      cur ^= 1;
+      __syncthreads();
+    }
+
+    COROPE_ISTAMP(5);
 #ifdef COROPE_TRACE
-  if (p.trace != nullptr && threadIdx.x == 0) p.trace[(int64_t)blockIdx.x * 16 + 7] = __builtin_readcyclecounter() - clk0;
+    if (p.trace != nullptr && threadIdx.x == TT) p.trace[(int64_t)item * 16 + 7] = __builtin_readcyclecounter() - clk0;
 #endif
-  // every wave is past its last read of the tiles (the loop ends with a barrier): their LDS now carries the accumulators
-  // to a row-major order, so that dV and dK leave in whole row segments and the tables are read the same way
-  float* wave_out = reinterpret_cast<float*>(smem) + wave * 32 * kAccTileStride<D>;
-  if constexpr (DO_DV) store_rows_via_lds<D, false>(dvacc, p.dv + base, wk_lo, N, nullptr, nullptr, 0, 1.f, wave_out);
-  // the Q_r operand carried sm_scale * log2(e): ln 2 is what is left of sm_scale
-  if constexpr (DO_DK) store_rows_via_lds<D, true>(dkacc, p.dk + base, wk_lo, N, p.cos, p.sin, p.fstride, 0.6931471805599453f, wave_out);
-#ifdef COROPE_TRACE
-  __builtin_amdgcn_s_waitcnt(0);
-  COROPE_STAMP(6, 0);
-#endif
+    // ---- change of items, all within the wave's own LDS slot.  The table values dK needs on its way out are requested
+    // first and land while dV leaves (which waits for nothing); behind them (loads return in the order they were issued)
+    // the next item's rows, which land while dK leaves.  After the last item its own rows are requested once more and
+    // never used: the request is then unconditional, and the registers it fills are free during the tile loop on every path.
+    UnrotateTables<D> tb;
+    if constexpr (DO_DK && PREROT) tb.load(p.cos, p.sin, p.fstride, wk_lo, N, opaque_lane());
+    if constexpr (DO_DV) store_rows_via_wave_tile<D>(dvacc, p.dv + base, wk_lo, N, 1.f, wave_slot, opaque_lane());
+    const int next_item = items.at(round + 1);
+    const bool has_next = next_item < total;
+    request_rows(has_next ? next_item : item);
+    if constexpr (DO_DK) {
+      if constexpr (!PREROT) tb.load(p.cos, p.sin, p.fstride, wk_lo, N, opaque_lane());
+      // the Q_r operand carried sm_scale * log2(e): ln 2 is what is left of sm_scale
+      store_unrotated_rows_via_wave_tile<D>(dkacc, tb, p.dk + base, wk_lo, N, 0.6931471805599453f, wave_slot, opaque_lane());
+    }
+    COROPE_ISTAMP(6);
+    if (!has_next) break;
+    item = next_item;
+    COROPE_ISTAMP(0);
+    take_rows();
+  }
 }
 
 // ===================================================================================== dQ
@@ -529,12 +595,10 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
 }
 
 // ===================================================================================== launchers
-// The fused dK+dV kernel sits at 246 of the 256 registers that two waves per SIMD leave each of them; dV alone is
-// small enough for a 128-row tile on pre-rotated operands.
 template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT, int NWAVES>
 static hipError_t launch_dkdv_waves(BwdParams p, hipStream_t stream) {
-  constexpr int BLOCK_M = (PREROT && !DO_DK && NWAVES == 8) ? 128 : 64;   // the larger tile pays off (and fits) for dV on pre-rotated operands only
-  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? 8 : 32, DO_DV && DO_DK>;
+  constexpr int BLOCK_M = 64;
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? 8 : 32>;
   auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK, PREROT>;
   static std::atomic<uint64_t> lds_ok{0};
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
@@ -542,7 +606,10 @@ static hipError_t launch_dkdv_waves(BwdParams p, hipStream_t stream) {
 #ifdef COROPE_TRACE
   p.trace = g_trace_buf;
 #endif
-  hipLaunchKernelGGL(kern, dim3(p.num_blocks * (p.BH / p.H * p.Hkv)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
+  // one workgroup per compute unit, or per item if those are fewer
+  const int64_t n_items = (int64_t)p.num_blocks * (p.BH / p.H * p.Hkv);
+  const int cus = device_cu_count();
+  hipLaunchKernelGGL(kern, dim3((unsigned)(n_items < cus ? n_items : cus)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
 }
 
