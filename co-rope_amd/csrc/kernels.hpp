@@ -22,19 +22,6 @@ inline hipError_t allow_dynamic_lds(const void* kernel, int bytes, std::atomic<u
 }
 
 
-// Compute units of the current device (cached per device; 256 on an MI355X): the size of a persistent launch, one
-// workgroup per compute unit.
-inline int device_cu_count() {
-  static std::atomic<int> cached[64];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return 256;
-  int n = cached[dev & 63].load(std::memory_order_relaxed);
-  if (n > 0) return n;
-  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-  cached[dev & 63].store(n, std::memory_order_relaxed);
-  return n;
-}
-
 #ifdef COROPE_TRACE
 // Experiment builds only: per-workgroup time stamps (100 MHz counter) for splitting a launch into its phases.
 extern uint64_t* g_trace_buf;
@@ -70,15 +57,36 @@ extern uint64_t* g_trace_buf;
 #define COROPE_ISTAMP_ID(extra) do {} while (0)
 #endif
 
-// Rows per workgroup of the attention kernels: 256 (8 waves) or 128 (4 waves).  By shape: a launch whose 256-row blocks
-// number fewer than two per CU of an MI355X takes the 128-row form, which doubles the workgroups and halves the time
-// the heaviest of them runs; `g_tile_rows` (0 = by shape, 128, 256) overrides the rule for tests and tuning.
+// Compute units of the current device (cached per device; 256 on an MI355X): the size of a persistent launch, one
+// workgroup per compute unit.
+inline int device_cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  int n = cached[dev & 63].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+  cached[dev & 63].store(n, std::memory_order_relaxed);
+  return n;
+}
+
+// Rows per workgroup of the attention kernels: 256 (8 waves) or 128 (4 waves).  By shape: a launch whose 256-row items
+// number fewer than the compute units takes the 128-row form, which doubles the items and halves the time the heaviest
+// of them runs; `g_tile_rows` (0 = by shape, 128, 256) overrides the rule for tests and tuning.
 extern std::atomic<int> g_tile_rows;
 inline bool use_small_tiles(int n_rows, int slabs) {
   const int forced = g_tile_rows.load(std::memory_order_relaxed);
   if (forced == 128) return true;
   if (forced == 256) return false;
-  return (int64_t)((n_rows + 255) / 256) * slabs < 2 * 256;
+  return (int64_t)((n_rows + 255) / 256) * slabs < device_cu_count();
+}
+
+// Workgroups of a persistent launch: one per compute unit -- two where two fit (4-wave workgroups whose LDS leaves room
+// for a second one: the attention kernels are compiled for two waves per SIMD) -- or one per item if those are fewer.
+inline unsigned persistent_grid(int64_t n_items, int waves, int lds_bytes) {
+  const int per_cu = (waves <= 4 && 2 * lds_bytes <= 160 * 1024) ? 2 : 1;
+  const int64_t slots = (int64_t)device_cu_count() * per_cu;
+  return (unsigned)(n_items < slots ? n_items : slots);
 }
 
 struct FwdParams {

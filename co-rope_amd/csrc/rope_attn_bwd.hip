@@ -606,10 +606,8 @@ static hipError_t launch_dkdv_waves(BwdParams p, hipStream_t stream) {
 #ifdef COROPE_TRACE
   p.trace = g_trace_buf;
 #endif
-  // one workgroup per compute unit, or per item if those are fewer
-  const int64_t n_items = (int64_t)p.num_blocks * (p.BH / p.H * p.Hkv);
-  const int cus = device_cu_count();
-  hipLaunchKernelGGL(kern, dim3((unsigned)(n_items < cus ? n_items : cus)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
+  const unsigned grid = persistent_grid((int64_t)p.num_blocks * (p.BH / p.H * p.Hkv), NWAVES, Cfg::kLdsBytes);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
 }
 
@@ -630,10 +628,8 @@ static hipError_t launch_dq_waves(BwdParams p, hipStream_t stream) {
 #ifdef COROPE_TRACE
   p.trace = g_trace_buf;
 #endif
-  // one workgroup per compute unit, or per item if those are fewer
-  const int64_t n_items = (int64_t)p.num_blocks * p.BH;
-  const int cus = device_cu_count();
-  hipLaunchKernelGGL(kern, dim3((unsigned)(n_items < cus ? n_items : cus)), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
+  const unsigned grid = persistent_grid((int64_t)p.num_blocks * p.BH, NWAVES, Cfg::kLdsBytes);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
 }
 

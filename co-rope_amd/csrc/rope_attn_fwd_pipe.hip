@@ -460,10 +460,7 @@ static hipError_t launch_pipe_waves(FwdParams p, hipStream_t stream) {
 #ifdef COROPE_TRACE
   p.trace = g_trace_buf;
 #endif
-  // one workgroup per compute unit (its LDS and registers leave room for no second one), or per item if those are fewer
-  const int64_t items = (int64_t)p.num_m_blocks * p.BH;
-  const int cus = device_cu_count();
-  dim3 grid((unsigned)(items < cus ? items : cus));
+  dim3 grid(persistent_grid((int64_t)p.num_m_blocks * p.BH, NW, Cfg::kLdsBytes));
   hipLaunchKernelGGL(kern, grid, dim3(Cfg::kThreads), Cfg::kLdsBytes, stream, p);
   return hipGetLastError();
 }

@@ -16,8 +16,31 @@ from . import _lib
 _SUPPORTED_D = (64, 128)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(t):
+    """The current HIP stream of t's device as an integer handle (the short way when this torch has it: at the small
+    shapes the operator is bound by the host, and torch.cuda.current_stream() builds a Python object per call)."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on_device(t):
+    """Context in which t's device is the current one; nothing to enter when it already is."""
+    return _NO_GUARD if torch.cuda.current_device() == t.device.index else torch.cuda.device(t.device)
 
 
 def _check_inputs(q, k, v, freqs_cos, freqs_sin):
@@ -81,7 +104,7 @@ def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, k
         two_launch = use_rotated_path(N, D, training=keep_rotated)
     rotated = None
     Hkv = k.shape[1]
-    with torch.cuda.device(q.device):
+    with _on_device(q):
         if q.dtype == torch.float16:
             # the reference's dtype: one launch, a true running maximum wherever a probability would leave fp16's range
             rc = lib.corope_rope_attn_fwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
@@ -158,7 +181,7 @@ class _FusedRopeAttn(torch.autograd.Function):
         B, H, N, D = q.shape
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         delta = torch.empty_like(M)
-        with torch.cuda.device(q.device):
+        with _on_device(q):
             if q.dtype == torch.float16:
                 rc = lib.corope_rope_attn_bwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
                                                   M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0),
@@ -226,7 +249,7 @@ def rope_rotate(x, freqs_cos, freqs_sin, with_tile_max=False, scale=1.0):
     B, H, N, D = x.shape
     y = torch.empty_like(x)
     tm = torch.empty((B, H, (N + 63) // 64), device=x.device, dtype=torch.float32) if with_tile_max else None
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         rc = lib.corope_rope_rotate(x.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0), y.data_ptr(),
                                     tm.data_ptr() if with_tile_max else None, B, H, N, D, float(scale), _stream_ptr(x))
     _lib.check(rc, "corope_rope_rotate")
