@@ -592,7 +592,8 @@ int corope_rope_attn_fwd_f16(const void* q, const void* k, const void* v, const 
 
 int corope_rope_attn_bwd_f16(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                              float* delta, const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* dq,
-                             void* dk, void* dv, int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
+                             void* dk, void* dv, int B, int H, int N, int D, float sm_scale, int causal, void* workspace,
+                             int64_t workspace_bytes, void* stream) {
   const char* what = "rope_attn_bwd_f16";
   int rc = validate_bwd(what, B, H, N, D, freq_row_stride, sm_scale,
                         {q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv});
@@ -600,6 +601,27 @@ int corope_rope_attn_bwd_f16(const void* q, const void* k, const void* v, const 
   corope::BwdParams p = make_bwd(q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, dk, dv, B, H, N,
                                  sm_scale);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (workspace != nullptr) {
+    // as corope_rope_attn_bwd_ws: q (scaled) and k are rotated once, the dQ kernel computes delta on its way, dK and dV
+    // come from one kernel
+    if (!aligned16(workspace)) return fail(COROPE_E_ALIGN, "%s: pointer %p is not 16-byte aligned", what, workspace);
+    const int64_t each = bwd_ws_tensor_bytes(B, H, N, D);
+    if (workspace_bytes < 2 * each)
+      return fail(COROPE_E_BADARG, "%s: workspace of %lld bytes, %lld needed", what, (long long)workspace_bytes,
+                  (long long)(2 * each));
+    uint16_t* q_rot = static_cast<uint16_t*>(workspace);
+    uint16_t* k_rot = reinterpret_cast<uint16_t*>(static_cast<char*>(workspace) + each);
+    rc = launch_status(what, corope_f16::launch_rope_rotate(p.q, p.cos, p.sin, p.fstride, q_rot, nullptr, p.BH, N, D, st,
+                                                            p.qk_scale));
+    if (rc) return rc;
+    rc = launch_status(what, corope_f16::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, k_rot, nullptr, p.BH, N, D, st, 1.f));
+    if (rc) return rc;
+    p.q = p.q_rot = q_rot;
+    p.k = p.k_rot = k_rot;
+    rc = launch_status(what, corope_f16::launch_bwd_dq(p, D, causal != 0, st));
+    if (rc) return rc;
+    return launch_status(what, corope_f16::launch_bwd_dkdv_fused(p, D, causal != 0, st));
+  }
   rc = launch_status(what, corope_f16::launch_bwd_preprocess(p, D, st));
   if (rc) return rc;
   p.o = nullptr;   // delta comes from the pass above, not from the dQ kernel

@@ -198,5 +198,8 @@ hipError_t launch_bwd_preprocess(const corope::BwdParams& p, int D, hipStream_t 
 hipError_t launch_bwd_dv(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_dk(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_dq(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_bwd_dkdv_fused(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
+                              float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale);
 hipError_t launch_corope_gqa_fwd(const corope::CoropeParams& p, int D, hipStream_t stream);
 }  // namespace corope_f16

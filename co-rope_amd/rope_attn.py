@@ -183,10 +183,15 @@ class _FusedRopeAttn(torch.autograd.Function):
         delta = torch.empty_like(M)
         with _on_device(q):
             if q.dtype == torch.float16:
+                ws, nbytes = None, 0
+                if use_rotated_path(N, D, training=True):   # rotate q and k once, then the kernels on the rotated copies
+                    nbytes = lib.corope_rope_attn_bwd_workspace_bytes(B, H, N, D)
+                    ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
                 rc = lib.corope_rope_attn_bwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
                                                   M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0),
                                                   dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, N, D, ctx.sm_scale,
-                                                  int(ctx.causal), _stream_ptr(q))
+                                                  int(ctx.causal), ws.data_ptr() if ws is not None else None, nbytes,
+                                                  _stream_ptr(q))
             elif k.shape[1] != H:         # grouped-query attention
                 rc = lib.corope_rope_attn_bwd_gqa(q.data_ptr(), k.data_ptr(), int(ctx.rotated), v.data_ptr(), o.data_ptr(),
                                                   do.data_ptr(), M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(),

@@ -226,7 +226,9 @@ int corope_rope_attn_bwd_ws(const void *q, const void *k, const void *v, const v
  * lse, delta, accumulation) is fp32 as above.  Same kernels as the bf16 entry points built for the other element type:
  * the forward is corope_rope_attn_fwd's single launch with a true running maximum per 32-key half whenever a
  * probability would leave fp16's range (the two-launch forward carries unnormalised probabilities up to 2^64, which only
- * bf16 can hold); the backward is preprocess + dV + dK + dQ as in corope_rope_attn_bwd.  `delta` is (B,H,N) fp32 scratch.
+ * bf16 can hold); the backward is preprocess + dV + dK + dQ as in corope_rope_attn_bwd, or -- given a workspace of
+ * corope_rope_attn_bwd_workspace_bytes (may be NULL) -- the rotation of q and k into it followed by the dQ and the fused
+ * dK+dV kernel as in corope_rope_attn_bwd_ws, which is the faster form from N * D = 65536 on.  `delta` is (B,H,N) fp32 scratch.
  * Replaces _attention.forward / .backward (fused-rope/fused_rope_attn.py:655-777) for callers that keep the reference's dtype. */
 int corope_rope_attn_fwd_f16(const void *q, const void *k, const void *v,
                              const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
@@ -236,7 +238,8 @@ int corope_rope_attn_bwd_f16(const void *q, const void *k, const void *v, const 
                              const float *lse, float *delta,
                              const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
                              void *dq, void *dk, void *dv,
-                             int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+                             int B, int H, int N, int D, float sm_scale, int causal,
+                             void *workspace, int64_t workspace_bytes, void *stream);
 
 /* Grouped-query form of the operator: q (B,Hq,N,D), k and v (B,Hkv,N,D), Hq a multiple of Hkv; query head h reads
  * key/value head h / (Hq/Hkv); dk and dv (B,Hkv,N,D) are sums over the query heads of their group (the key block's
