@@ -149,7 +149,7 @@ struct RowTile {
 // are loaded by the same thread, so the rotation is thread-local.  cos/sin come from fp32 tables of which
 // only the first D/2 columns are used.  SCALED: the rotated values are multiplied by out_scale before the one rounding
 // (the query side of QK^T carries sm_scale * log2(e), so that scores leave the matrix cores in base-2 units).
-template <int D, int ROWS, int NT, bool SCALED = false>
+template <int D, int ROWS, int NT, bool SCALED = false, int PAD = 8>
 struct RotStage {
   static constexpr int kChunks = D / 16;              // units per row
   static constexpr int kUnits = ROWS * kChunks;
@@ -207,8 +207,8 @@ struct RotStage {
       int r = u / kChunks, ch = u % kChunks;
       u32x4 y1, y2;
       rotate(it, y1, y2);
-      *reinterpret_cast<u32x4*>(lds + RowTile<D>::off(r, ch * 8)) = y1;
-      *reinterpret_cast<u32x4*>(lds + RowTile<D>::off(r, D / 2 + ch * 8)) = y2;
+      *reinterpret_cast<u32x4*>(lds + RowTile<D, PAD>::off(r, ch * 8)) = y1;
+      *reinterpret_cast<u32x4*>(lds + RowTile<D, PAD>::off(r, D / 2 + ch * 8)) = y2;
     }
   }
 };
@@ -242,14 +242,14 @@ struct CopyStage {
 
 // Staging of a tile whose rows take part in QK^T: rotated on the way to LDS (PREROT = false), or copied from a tensor
 // that rope_rotate_kernel rotated beforehand (PREROT = true; the tables are then not touched).
-template <int D, int ROWS, int NT, bool PREROT, bool SCALED = false>
-struct RopeStage : RotStage<D, ROWS, NT, SCALED> {};
-template <int D, int ROWS, int NT, bool SCALED>
-struct RopeStage<D, ROWS, NT, true, SCALED> : CopyStage<D, ROWS, NT, 8> {
+template <int D, int ROWS, int NT, bool PREROT, bool SCALED = false, int PAD = 8>
+struct RopeStage : RotStage<D, ROWS, NT, SCALED, PAD> {};
+template <int D, int ROWS, int NT, bool SCALED, int PAD>
+struct RopeStage<D, ROWS, NT, true, SCALED, PAD> : CopyStage<D, ROWS, NT, PAD> {
   float out_scale = 1.f;   // unused: the copy was scaled when it was rotated
   __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float*, const float*, int64_t, int row0,
                                        int n_rows) {
-    CopyStage<D, ROWS, NT, 8>::load(src, row0, n_rows);
+    CopyStage<D, ROWS, NT, PAD>::load(src, row0, n_rows);
   }
 };
 

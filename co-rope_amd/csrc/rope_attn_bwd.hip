@@ -18,6 +18,13 @@
 
 namespace COROPE_NS {
 
+// Row padding (elements) of LDS tiles that are read both row-wise (16 bytes per lane, lane = row) and through the
+// transposing read (8 bytes per lane, 4 rows x 32 bytes per 16 lanes).  16 bytes of padding keep the row-wise reads free
+// of bank conflicts and leave the transposing ones four-way conflicted, 64 bytes do the opposite; 48 bytes (a row stride
+// of 12 dwords past a multiple of 64) was the best of 16 / 32 / 48 / 64 / 80 measured on the fused dK+dV kernel at
+// B2 H32 N4096 D128: 0.551 / 0.524 / 0.512 / 0.561 / 0.523 ms.
+constexpr int kBothWaysPad = 24;
+
 // ===================================================================================== dK / dV
 // Workgroup = NWAVES waves x 32 keys.  K_r and V rows of the wave stay in registers as B operands.
 // Per query tile (BLOCK_M rows, staged: rotated Q and dO, plus M and delta):
@@ -35,11 +42,11 @@ namespace COROPE_NS {
 // key block) items and the stream of query tiles runs on from item to item.  Behind the two tile stages every wave has an
 // LDS slot of its own (32 padded rows): its V rows during an item (V_LDS), and at the change of items the tile through
 // which its dV and dK rows leave and its next K_r rows come in -- nothing there needs a workgroup barrier.
-template <int D, int NWAVES, int BLOCK_M, int DO_PAD>
+template <int D, int NWAVES, int BLOCK_M, int DO_PAD, int Q_PAD>
 struct DkdvCfg {
   static constexpr int kThreads = NWAVES * kWave;
   static constexpr int kBlockN = NWAVES * 32;
-  static constexpr int kTileBytes = RowTile<D>::bytes(BLOCK_M);
+  static constexpr int kTileBytes = RowTile<D, Q_PAD>::bytes(BLOCK_M);
   static constexpr int kDoTileBytes = RowTile<D, DO_PAD>::bytes(BLOCK_M);
   static constexpr int kStatBytes = BLOCK_M * 4;
   static constexpr int kStageBytes = kTileBytes + kDoTileBytes + 2 * kStatBytes;
@@ -53,12 +60,13 @@ struct DkdvCfg {
 // PREROT: Q and K come from copies that rope_rotate_kernel rotated beforehand (no table reads in the loop).
 template <int D, int NWAVES, int BLOCK_M, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
 __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
-  constexpr int DO_PAD = DO_DK ? 8 : 32;
+  constexpr int DO_PAD = DO_DK ? (DO_DV ? kBothWaysPad : 8) : 32;
+  constexpr int Q_PAD = DO_DK ? kBothWaysPad : 8;
   constexpr bool V_LDS = DO_DV && DO_DK;
-  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_PAD>;
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_PAD, Q_PAD>;
   constexpr int NT = Cfg::kThreads;
   constexpr int KC = D / 16, NDB = D / 32, NQB = BLOCK_M / 32;
-  constexpr int LS = RowTile<D>::kStride, LSDO = RowTile<D, DO_PAD>::kStride;
+  constexpr int LS = RowTile<D, Q_PAD>::kStride, LSDO = RowTile<D, DO_PAD>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -81,7 +89,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   const uint16_t* q_all = PREROT ? p.q_rot : p.q;
 
   // ---- the stream of query tiles: a cursor one tile ahead of the tile being consumed -----------------------------------
-  RopeStage<D, BLOCK_M, NT, PREROT, true> qst;   // Q_r tiles carry qk_scale: S leaves the matrix cores in base-2 units
+  RopeStage<D, BLOCK_M, NT, PREROT, true, Q_PAD> qst;   // Q_r tiles carry qk_scale: S leaves the matrix cores in base-2 units
   qst.out_scale = p.qk_scale;
   CopyStage<D, BLOCK_M, NT, DO_PAD> dst;
   float st_lse = 0.f, st_delta = 0.f;
@@ -235,7 +243,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
             for (int e = 0; e < 4; ++e) dpacc[4 * g + e] = d4[e];
           }
         }
-        const uint16_t* qrow = qs + RowTile<D>::off(qb * 32 + lq, 8 * lh);
+        const uint16_t* qrow = qs + RowTile<D, Q_PAD>::off(qb * 32 + lq, 8 * lh);
         const uint16_t* dorow = dos + RowTile<D, DO_PAD>::off(qb * 32 + lq, 8 * lh);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
@@ -332,8 +340,9 @@ template <int D, int NWAVES, int BLOCK_N>
 struct DqCfg {
   static constexpr int kThreads = NWAVES * kWave;
   static constexpr int kBlockM = NWAVES * 32;
-  static constexpr int kTileBytes = RowTile<D>::bytes(BLOCK_N);
-  static constexpr int kStageBytes = 2 * kTileBytes;
+  static constexpr int kKTileBytes = RowTile<D, kBothWaysPad>::bytes(BLOCK_N);   // K_r: read row-wise and transposed
+  static constexpr int kVTileBytes = RowTile<D>::bytes(BLOCK_N);                 // V: read row-wise
+  static constexpr int kStageBytes = kKTileBytes + kVTileBytes;
   static constexpr int kRingBytes = 2 * kStageBytes;
   // behind the ring, per wave: a private tile for its operand rows on their way in and its dQ rows on their way out, and
   // the 32 delta values of its rows
@@ -350,7 +359,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
   constexpr int NT = Cfg::kThreads;
   constexpr int KC = D / 16, NDB = D / 32, NKB = BLOCK_N / 32;
-  constexpr int LS = RowTile<D>::kStride;
+  constexpr int LS = RowTile<D, kBothWaysPad>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -371,7 +380,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   };
 
   // ---- the stream of K/V tiles: a cursor one tile ahead of the tile being consumed -------------------------------------
-  RopeStage<D, BLOCK_N, NT, PREROT> kst;
+  RopeStage<D, BLOCK_N, NT, PREROT, false, kBothWaysPad> kst;
   CopyStage<D, BLOCK_N, NT> vst;
   int l_round = 0, l_tile = 0, l_tiles;
   const uint16_t *l_kg, *l_vg;
@@ -395,7 +404,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
     vst.load(l_vg, l_tile * BLOCK_N, N);
   };
   auto k_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes); };
-  auto v_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes + Cfg::kTileBytes); };
+  auto v_tile = [&](int buf) { return reinterpret_cast<uint16_t*>(smem + buf * Cfg::kStageBytes + Cfg::kKTileBytes); };
   int cur = 0;   // ring stage of the tile being consumed
 
   // ---- operand rows of an item: Q_r (rotated and scaled here unless a pre-rotated copy is given), dO, O for delta ------
@@ -522,7 +531,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb) {
         f32x16 sacc, dpacc;   // dP starts from a literal zero, S from -M
-        const uint16_t* krow = ks + RowTile<D>::off(kb * 32 + lq, 8 * lh);
+        const uint16_t* krow = ks + RowTile<D, kBothWaysPad>::off(kb * 32 + lq, 8 * lh);
         const uint16_t* vrow = vs + RowTile<D>::off(kb * 32 + lq, 8 * lh);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
@@ -598,7 +607,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
 template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT, int NWAVES>
 static hipError_t launch_dkdv_waves(BwdParams p, hipStream_t stream) {
   constexpr int BLOCK_M = 64;
-  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? 8 : 32>;
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? (DO_DV ? kBothWaysPad : 8) : 32, DO_DK ? kBothWaysPad : 8>;
   auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK, PREROT>;
   static std::atomic<uint64_t> lds_ok{0};
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
