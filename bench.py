@@ -36,9 +36,9 @@ PEAK_HBM_GBS = 8000.0
 # benchmark (summary and commands: profiles/rope_attn_c3_hbm_traffic.md); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE
 # by 1.0, the factors a plain 1 GiB device copy gives for the same counters.
 HBM_TRAFFIC_BYTES = {
-    ("c3", "rope_attn_fwd"): int((252746 * 2.0 + 132101) * 1024),
-    ("c3", "rope_attn_bwd_dq"): int((330591 * 2.0 + 66565) * 1024),
-    ("c3", "rope_attn_bwd_dkdv"): int((285381 * 2.0 + 137995) * 1024),
+    ("c3", "rope_attn_fwd"): int((307460 * 2.0 + 132096) * 1024),
+    ("c3", "rope_attn_bwd_dq"): int((402667 * 2.0 + 91136) * 1024),
+    ("c3", "rope_attn_bwd_dkdv"): int((315363 * 2.0 + 131072) * 1024),
 }
 
 CONFIGS = {
@@ -396,9 +396,10 @@ def forward_ms(pkg, q, k, v, cos, sin, scale, torch, reps=100):
 
 
 def bench_phase_trace(args):
-    """Where the time of the forward, dQ and dK+dV kernels goes at the chosen shape: every workgroup of the trace build
-    stamps the constant 100 MHz counter at its phase boundaries (one lane of the wave that sees every tile) and the
-    core-clock counter around its tile loop.  Prints a markdown table (one traced step in the middle of a run of steps)."""
+    """Where the time of the forward, dQ and dK+dV kernels goes at the chosen shape: the kernels of the trace build stamp
+    the constant 100 MHz counter at the phase boundaries of every item they work on (one lane of the wave that sees every
+    tile) and the core-clock counter around its tile loop.  Prints a markdown table (one traced step in the middle of a run
+    of steps)."""
     import ctypes
     import numpy as np
     import torch
@@ -449,7 +450,7 @@ def bench_phase_trace(args):
         x = np.asarray(x, dtype=float)
         return f"| {label} | {x.mean():.2f} | {np.percentile(x, 10):.2f} | {np.percentile(x, 50):.2f} | {np.percentile(x, 90):.2f} | {x.max():.2f} |"
 
-    print(f"Workload: {cfg['name']}, data {args.data}; times in microseconds per workgroup (256 rows) unless said otherwise.\n")
+    print(f"Workload: {cfg['name']}, data {args.data}; times in microseconds per item (256 rows) unless said otherwise.\n")
     for name, buf in bufs.items():
         a = buf.cpu().numpy().reshape(-1, 16)
         if args.trace_dump:
@@ -469,12 +470,12 @@ def bench_phase_trace(args):
             busy.append(sum(t[i, 6] - t[i, 0] for i in idx))
         span = np.nanmax(t[:, 6])
         ghz = a[:, 7] / ((a[:, 5] - (a[:, 1] if name != "rope_attn_fwd" else a[:, 2])) * 10.0)
-        print(f"### {name}: {len(a)} workgroups on {len(set(cu_key))} CUs, {len(a) / len(set(cu_key)):.1f} per CU, "
+        print(f"### {name}: {len(a)} items on {len(set(cu_key))} CUs, {len(a) / len(set(cu_key)):.1f} per CU, "
               f"launch span {span:.1f} us, mean busy time per CU {np.mean(busy):.1f} us\n")
         print("| phase | mean | p10 | p50 | p90 | max |\n|---|---|---|---|---|---|")
-        print(row("whole workgroup", t[:, 6] - t[:, 0]))
-        print(row("gap to the next workgroup on the same CU", gaps))
-        print(row("prologue (entry -> first tile staged)", t[:, 1] - t[:, 0]))
+        print(row("whole item", t[:, 6] - t[:, 0]))
+        print(row("gap to the next item on the same CU", gaps))
+        print(row("prologue (previous item's stores issued -> operand rows in registers)", t[:, 1] - t[:, 0]))
         big = ntile > 5
         if dkdv:      # the key block's diagonal query tiles come first
             print(row("first tile", t[:, 3] - t[:, 1]))
@@ -482,10 +483,6 @@ def bench_phase_trace(args):
             print(row("steady state, per tile (64 queries x 256 keys)", (t[big, 5] - t[big, 4]) / (ntile[big] - 4)))
         else:
             if name == "rope_attn_fwd":
-                print(row("  of which: loads issued", t[:, 8] - t[:, 0]))
-                print(row("  of which: loads landed", t[:, 9] - t[:, 8]))
-                print(row("  of which: rotate Q, through LDS, rotated copy stored", t[:, 10] - t[:, 9]))
-                print(row("  of which: K/V tile 0 to LDS, tile 1 requested, barriers", t[:, 1] - t[:, 10]))
                 print(row("key-norm bounds of the wave's tiles", t[:, 2] - t[:, 1]))
                 print(row("first tile (with its exact pass)", t[:, 3] - t[:, 2]))
                 print(row("tiles examined twice, fraction of the wave's tiles", a[:, 13] / ntile))
@@ -493,11 +490,11 @@ def bench_phase_trace(args):
                 print(row("first tile", t[:, 3] - t[:, 1]))
             print(row("steady state, per tile (256 queries x 64 keys)", (t[big, 4] - t[big, 3]) / (ntile[big] - 5)))
             print(row("diagonal block, per tile (4 tiles, waves drop out)", (t[:, 5] - t[:, 4]) / 4))
-        print(row("epilogue (last tile -> stores done)", t[:, 6] - t[:, 5]))
+        print(row("epilogue (last tile -> stores issued, next rows requested)", t[:, 6] - t[:, 5]))
         print(row("shader clock in the tile loop [GHz]", ghz))
         per_cu = len(a) / len(set(cu_key))
         edge = np.nanmean(t[:, 1] - t[:, 0]) + np.nanmean(t[:, 6] - t[:, 5]) + np.mean(gaps)
-        print(f"\nPer CU: {per_cu:.0f} workgroups x {edge:.1f} us of prologue + epilogue + gap = {per_cu * edge:.0f} us "
+        print(f"\nPer CU: {per_cu:.0f} items x {edge:.1f} us of prologue + epilogue + gap = {per_cu * edge:.0f} us "
               f"of {np.mean(busy):.0f} us ({100 * per_cu * edge / np.mean(busy):.0f} %).\n")
 
 
