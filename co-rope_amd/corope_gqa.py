@@ -11,6 +11,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
+from .rope_attn import _PADDED_D, gather_halves, spread_halves
 
 
 class _CoRopeGqaAttn(torch.autograd.Function):
@@ -115,7 +116,18 @@ def corope_gqa_backward(q, k, v, grad_output, sm_scale, theta, workspace=None, o
     return dq, dk, dv
 
 
-attention = _CoRopeGqaAttn.apply
+def attention(q, k, v, causal, sm_scale, theta, warp_specialize=False):
+    """The reference's ``attention = _attention.apply`` (corope-exp/flash_attn_co_rope_gqa_triton.py:580): positional
+    arguments in its order.  Head dims 64 and 128 go to the kernels as they are.  16 and 32 -- the reference's own
+    self-check runs at 32 (corope_attn_gqa_pytorch.py:309-321) -- run at D = 64 with each half of a row padded with zeros:
+    the rotation pairs and every dot product keep their values, and the inverse frequencies theta^(-2d/D) of the pairs
+    that carry data are those of theta^(64/D) at D = 64."""
+    d = q.shape[-1] if q.ndim == 4 else 0
+    if d in _PADDED_D and k.ndim == 4 and v.ndim == 4 and k.shape[-1] == d and v.shape[-1] == d:
+        o = _CoRopeGqaAttn.apply(spread_halves(q, 64), spread_halves(k, 64), spread_halves(v, 64), causal, sm_scale,
+                                 float(theta) ** (64 // d), warp_specialize)
+        return gather_halves(o, d)
+    return _CoRopeGqaAttn.apply(q, k, v, causal, sm_scale, theta, warp_specialize)
 
 
 def corope_attn_gqa(q, k, v, sm_scale=None, theta=10000.0, causal=True):

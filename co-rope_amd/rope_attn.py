@@ -14,6 +14,22 @@ import torch
 from . import _lib
 
 _SUPPORTED_D = (64, 128)
+# Head dims of the reference (fused_rope_attn.py:661) below the kernels' own: run at D = 64 with each half of a row padded
+# with zeros (the rotation pairs column j with column j + D/2, so the halves must stay the starts of the new halves).
+_PADDED_D = (16, 32)
+
+
+def spread_halves(x, d_to):
+    """(..., D) -> (..., d_to): [x[:D/2], 0, x[D/2:], 0]; zero columns add nothing to any dot product."""
+    d = x.shape[-1]
+    h, z = d // 2, x.new_zeros(x.shape[:-1] + ((d_to - d) // 2,))
+    return torch.cat([x[..., :h], z, x[..., h:], z], dim=-1)
+
+
+def gather_halves(y, d):
+    """Inverse of spread_halves on the columns that carry data."""
+    h, hp = d // 2, y.shape[-1] // 2
+    return torch.cat([y[..., :h], y[..., hp:hp + h]], dim=-1)
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -53,7 +69,7 @@ def _check_inputs(q, k, v, freqs_cos, freqs_sin):
     assert q.shape[0] == k.shape[0] and q.shape[2:] == k.shape[2:], "q and k must agree in batch, sequence and head dim"
     assert q.shape[1] % k.shape[1] == 0, "the number of query heads must be a multiple of the number of key/value heads"
     if d not in _SUPPORTED_D:
-        raise ValueError(f"head dim {d} not built for gfx950 (supported: {_SUPPORTED_D})")
+        raise ValueError(f"head dim {d} not built for gfx950 (kernels: {_SUPPORTED_D}; padded to 64: {_PADDED_D})")
     if not (q.is_cuda and k.is_cuda and v.is_cuda and freqs_cos.is_cuda and freqs_sin.is_cuda):
         raise ValueError("fused RoPE attention runs on the GPU only: all tensors must be on a HIP device")
     if not (q.dtype == k.dtype == v.dtype and q.dtype in (torch.bfloat16, torch.float16)):
@@ -219,7 +235,19 @@ class _FusedRopeAttn(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None, None
 
 
-attention = _FusedRopeAttn.apply
+def attention(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, warp_specialize=True):
+    """The reference's ``attention = _attention.apply`` (fused-rope/fused_rope_attn.py:780): positional arguments in its
+    order.  Head dims 64 and 128 go to the kernels as they are; 16 and 32 are padded to 64 around the same kernels (zero
+    columns, tables padded with the identity rotation), which changes no value of the result."""
+    d = q.shape[-1]
+    if d in _PADDED_D and q.dim() == 4 and k.shape[-1] == d and v.shape[-1] == d:
+        h, pad = d // 2, (64 - d) // 2
+        fc = torch.cat([freqs_cos[:, :h].float(), freqs_cos.new_ones((freqs_cos.shape[0], pad), dtype=torch.float32)], dim=1)
+        fs = torch.cat([freqs_sin[:, :h].float(), freqs_sin.new_zeros((freqs_sin.shape[0], pad), dtype=torch.float32)], dim=1)
+        o = _FusedRopeAttn.apply(spread_halves(q, 64), spread_halves(k, 64), spread_halves(v, 64), causal, sm_scale, fc, fs,
+                                 warp_specialize)
+        return gather_halves(o, d)
+    return _FusedRopeAttn.apply(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, warp_specialize)
 
 
 def fused_rope_attn(q, k, v, freqs_cos, freqs_sin, causal=True, sm_scale=None):

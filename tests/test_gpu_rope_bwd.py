@@ -260,3 +260,20 @@ def test_item_lists_with_partial_rounds(pkg, tile_rows, B, Hq, Hkv, N, D, causal
         print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
         assert a.shape == b.shape and torch.isfinite(a).all(), name
         assert within_bar(a, b, TOL * (math.sqrt(G) if name in ("dK", "dV") else 1.0))[0], name
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,N,D", [(2, 3, 300, 32), (1, 2, 1100, 32), (1, 4, 130, 16)])
+def test_head_dims_below_the_kernels_own(pkg, B, H, N, D, causal):
+    """The reference admits head dims 16 and 32 (fused-rope/fused_rope_attn.py:661); here they run padded to the kernels'
+    D = 64 (zero columns, identity rotation on the padding), forward and backward, against the oracle at the true D."""
+    print(f"case small-D B={B} H={H} N={N} D={D} causal={causal}", flush=True)
+    q, k, v, g, c, s = _case(B, H, N, D, seed=17)
+    scale = 1 / math.sqrt(D)
+    o, dq, dk, dv = _gpu_fwd_bwd(pkg, q, k, v, g, causal, scale, c, s)
+    ro, _, rdq, rdk, rdv, _ = O.rope_attn_fwd_bwd_blocked(q, k, v, g, causal, scale, c, s)
+    for name, a, b in (("O", o, ro), ("dQ", dq, rdq), ("dK", dk, rdk), ("dV", dv, rdv)):
+        err = (a - b).abs()
+        print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
+        assert a.shape == b.shape and torch.isfinite(a).all(), name
+        assert within_bar(a, b, TOL)[0], name
