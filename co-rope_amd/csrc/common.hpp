@@ -136,12 +136,20 @@ __device__ __forceinline__ int kv_slab(int bh, int H, int Hkv) {
 //                        bank groups -- the layout for tiles read row-wise as MFMA operands;
 //   PAD = 32 (64 bytes): the row stride is 16 dwords past a multiple of 64, so the 4 rows x 32 bytes a 16-lane
 //                        block touches in a transposing read (and the 8 rows of a whole wave) spread over all
-//                        banks -- the layout for tiles read only through load_a_trans.
+//                        banks -- the layout for tiles read only through load_a_trans;
+//   PAD = kStaggerPad:   for tiles read both ways: 64 bytes of padding as with PAD = 32, and every fourth row another 16
+//                        bytes.  Row r then starts 4 * r + r / 4 sixteen-byte groups past a multiple of 16 groups: 16
+//                        consecutive rows sit in 16 different groups (row-wise reads), and the 4 rows x 64 bytes that
+//                        two 16-lane blocks of a transposing read touch still cover every bank once.  The extra 16 bytes
+//                        per 4 rows are the same for rows 4 apart in lane terms (lane part + compile-time constant).
+constexpr int kStaggerPad = 9;
 template <int D, int PAD = 8>
 struct RowTile {
-  static constexpr int kStride = D + PAD;  // elements
-  static constexpr int bytes(int rows) { return rows * kStride * 2; }
-  __device__ static __forceinline__ int off(int row, int col) { return row * kStride + col; }
+  static constexpr bool kStaggered = PAD == kStaggerPad;
+  static constexpr int kStride = D + (kStaggered ? 32 : PAD);  // elements
+  static constexpr int bytes(int rows) { return (rows * kStride + (kStaggered ? 8 * ((rows + 3) / 4) : 0)) * 2; }
+  __device__ static __forceinline__ int stagger(int row) { return kStaggered ? 8 * (row >> 2) : 0; }
+  __device__ static __forceinline__ int off(int row, int col) { return row * kStride + stagger(row) + col; }
 };
 
 // ---- staging: a ROWS x D tile with the half-layout rotation applied on the way -----------------------
@@ -269,6 +277,20 @@ __device__ __forceinline__ u32x4 load_a_trans(const uint16_t* tile, int stride, 
   const uint16_t* p = tile + (kbase + 4 * h + s / 4) * stride + m0 + 16 * (blk % 2) + 4 * (s % 4);
   s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
   s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 8 * stride));
+  u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
+  return u32x4{a[0], a[1], b[0], b[1]};
+}
+
+// The same read from a tile of layout T (a RowTile); kbase: a multiple of 4.
+template <typename T>
+__device__ __forceinline__ u32x4 load_a_trans_of(const uint16_t* tile, int kbase, int m0) {
+  typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+  const int l = threadIdx.x % kWave;
+  const int blk = l / 16, s = l % 16, h = blk / 2;
+  // rows kbase + 4h + s/4 and, 8 further, the second half
+  const uint16_t* p = tile + T::off(kbase, 0) + T::off(4 * h + s / 4, m0 + 16 * (blk % 2) + 4 * (s % 4));
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + T::off(8, 0)));
   u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
   return u32x4{a[0], a[1], b[0], b[1]};
 }

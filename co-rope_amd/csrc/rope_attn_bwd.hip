@@ -18,12 +18,14 @@
 
 namespace COROPE_NS {
 
-// Row padding (elements) of LDS tiles that are read both row-wise (16 bytes per lane, lane = row) and through the
-// transposing read (8 bytes per lane, 4 rows x 32 bytes per 16 lanes).  16 bytes of padding keep the row-wise reads free
-// of bank conflicts and leave the transposing ones four-way conflicted, 64 bytes do the opposite; 48 bytes (a row stride
-// of 12 dwords past a multiple of 64) was the best of 16 / 32 / 48 / 64 / 80 measured on the fused dK+dV kernel at
-// B2 H32 N4096 D128: 0.551 / 0.524 / 0.512 / 0.561 / 0.523 ms.
+// Layout of LDS tiles that are read both row-wise (16 bytes per lane, lane = row) and through the transposing read
+// (8 bytes per lane, 4 rows x 32 bytes per 16 lanes).  With plain row padding, 16 bytes keep the row-wise reads free of
+// bank conflicts and leave the transposing ones four-way conflicted, 64 bytes do the opposite; measured on the fused
+// dK+dV kernel at B2 H32 N4096 D128, paddings of 16 / 32 / 48 / 64 / 80 bytes gave 0.551 / 0.524 / 0.512 / 0.561 /
+// 0.523 ms.  The staggered layout (free of conflicts both ways, 68 bytes a row) gains another 1.4 % there, side by side
+// on one device; in the dQ kernel it loses 2.8 % to the 48-byte padding (more registers spilled for its addresses).
 constexpr int kBothWaysPad = 24;
+constexpr int kDkdvBothWaysPad = kStaggerPad;
 
 // ===================================================================================== dK / dV
 // Workgroup = NWAVES waves x 32 keys.  K_r and V rows of the wave stay in registers as B operands.
@@ -60,13 +62,12 @@ struct DkdvCfg {
 // PREROT: Q and K come from copies that rope_rotate_kernel rotated beforehand (no table reads in the loop).
 template <int D, int NWAVES, int BLOCK_M, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
 __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
-  constexpr int DO_PAD = DO_DK ? (DO_DV ? kBothWaysPad : 8) : 32;
-  constexpr int Q_PAD = DO_DK ? kBothWaysPad : 8;
+  constexpr int DO_PAD = DO_DK ? (DO_DV ? kDkdvBothWaysPad : 8) : 32;
+  constexpr int Q_PAD = DO_DK ? kDkdvBothWaysPad : 8;
   constexpr bool V_LDS = DO_DV && DO_DK;
   using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_PAD, Q_PAD>;
   constexpr int NT = Cfg::kThreads;
   constexpr int KC = D / 16, NDB = D / 32, NQB = BLOCK_M / 32;
-  constexpr int LS = RowTile<D, Q_PAD>::kStride, LSDO = RowTile<D, DO_PAD>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -289,8 +290,8 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
           const int kbase = qb * 32 + 16 * cc;
 #pragma unroll
           for (int db = 0; db < NDB; ++db) {
-            if constexpr (DO_DV) dvacc[db] = mfma32(load_a_trans(dos, LSDO, kbase, db * 32), pb[cc], dvacc[db]);
-            if constexpr (DO_DK) dkacc[db] = mfma32(load_a_trans(qs, LS, kbase, db * 32), dsb[cc], dkacc[db]);
+            if constexpr (DO_DV) dvacc[db] = mfma32(load_a_trans_of<RowTile<D, DO_PAD>>(dos, kbase, db * 32), pb[cc], dvacc[db]);
+            if constexpr (DO_DK) dkacc[db] = mfma32(load_a_trans_of<RowTile<D, Q_PAD>>(qs, kbase, db * 32), dsb[cc], dkacc[db]);
           }
         }
         // without the causal branches the two blocks of a tile are one stretch of code: kept apart, or the scheduler
@@ -359,7 +360,6 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
   constexpr int NT = Cfg::kThreads;
   constexpr int KC = D / 16, NDB = D / 32, NKB = BLOCK_N / 32;
-  constexpr int LS = RowTile<D, kBothWaysPad>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -564,7 +564,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
       for (int c = 0; c < BLOCK_N / 16; ++c)
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
-          dqacc[db] = mfma32(load_a_trans(ks, LS, 16 * c, db * 32), dsb[c], dqacc[db]);
+          dqacc[db] = mfma32(load_a_trans_of<RowTile<D, kBothWaysPad>>(ks, 16 * c, db * 32), dsb[c], dqacc[db]);
       stage_next();
       cur ^= 1;
       __syncthreads();
@@ -607,7 +607,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
 template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT, int NWAVES>
 static hipError_t launch_dkdv_waves(BwdParams p, hipStream_t stream) {
   constexpr int BLOCK_M = 64;
-  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? (DO_DV ? kBothWaysPad : 8) : 32, DO_DK ? kBothWaysPad : 8>;
+  using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? (DO_DV ? kDkdvBothWaysPad : 8) : 32, DO_DK ? kDkdvBothWaysPad : 8>;
   auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK, PREROT>;
   static std::atomic<uint64_t> lds_ok{0};
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
