@@ -39,6 +39,16 @@ int check_ptrs(const char* what, std::initializer_list<const void*> ptrs) {
   return COROPE_OK;
 }
 
+// Head dim 256 is built for the kernels that take q and k as they are (single-launch forward; dV, dK and dQ that rotate
+// while they stage): entry points that work on rotated copies say so instead of launching.
+int rotated_copies_built(const char* what, int D) {
+  if (D > 128)
+    return fail(COROPE_E_UNSUPPORTED,
+                "%s: head dim %d runs on the original operands only (corope_rope_attn_fwd, corope_rope_attn_bwd and its "
+                "parts), not on rotated copies or a workspace", what, D);
+  return COROPE_OK;
+}
+
 int launch_status(const char* what, hipError_t e) {
   if (e == hipSuccess) return COROPE_OK;
   return fail(COROPE_E_LAUNCH, "%s: HIP error %d (%s)", what, (int)e, hipGetErrorString(e));
@@ -86,7 +96,8 @@ int corope_amd_set_tile_rows(int rows) {
 int corope_rope_attn_check(int B, int H, int N, int D, int64_t freq_row_stride, float sm_scale, int backward) {
   (void)backward;
   if (B <= 0 || H <= 0 || N <= 0) return fail(COROPE_E_BADARG, "rope_attn: B, H, N must be positive (got %d, %d, %d)", B, H, N);
-  if (D != 64 && D != 128) return fail(COROPE_E_UNSUPPORTED, "rope_attn: head dim %d not built (64 and 128 are)", D);
+  if (D != 64 && D != 128 && D != 256)
+    return fail(COROPE_E_UNSUPPORTED, "rope_attn: head dim %d not built (64, 128 and 256 are)", D);
   if (freq_row_stride < D / 2 || freq_row_stride % 4 != 0)
     return fail(COROPE_E_BADARG, "rope_attn: freq_row_stride %lld must be >= D/2 and a multiple of 4", (long long)freq_row_stride);
   if (!(sm_scale > 0.f) || !std::isfinite(sm_scale)) return fail(COROPE_E_BADARG, "rope_attn: sm_scale must be positive and finite");
@@ -154,6 +165,10 @@ int rope_attn_fwd_impl(const char* what, const void* q, const void* k, const voi
   p.tile_kmax = tile_kmax;
   p.q_rot_out = static_cast<uint16_t*>(q_rot_out);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (workspace != nullptr || k_rot != nullptr) {
+    rc = rotated_copies_built(what, D);
+    if (rc) return rc;
+  }
   if (workspace != nullptr) {
     rc = check_ptrs(what, {workspace});
     if (rc) return rc;
@@ -276,6 +291,7 @@ int corope_rope_attn_fwd_train(const void* q, const void* k, const void* v, cons
                                int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
   if (rc) return rc;
+  if ((rc = rotated_copies_built("rope_attn_fwd_train", D))) return rc;
   rc = check_ptrs("rope_attn_fwd_train", {q, k, v, freqs_cos, freqs_sin, o, lse, q_rot, k_rot});
   if (rc) return rc;
   if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
@@ -290,6 +306,8 @@ int corope_rope_attn_fwd_train(const void* q, const void* k, const void* v, cons
 int corope_rope_rotate(const void* x, const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* y,
                        float* tile_max, int B, int H, int N, int D, float scale, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, 1.f, 0);
+  if (rc) return rc;
+  rc = rotated_copies_built("rope_rotate", D);
   if (rc) return rc;
   rc = check_ptrs("rope_rotate", {x, freqs_cos, freqs_sin, y});
   if (rc) return rc;
@@ -341,6 +359,7 @@ int bwd_dv_impl(const char* what, bool prerot, const void* q, const void* k, con
                 int D, float sm_scale, int causal, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
+  if (prerot && (rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q, k, d_o, lse, freqs_cos, freqs_sin, dv});
   if (rc) return rc;
   corope::BwdParams p = make_bwd(q, k, nullptr, nullptr, d_o, lse, nullptr, freqs_cos, freqs_sin, freq_row_stride,
@@ -354,6 +373,7 @@ int bwd_dk_impl(const char* what, bool prerot, const void* q, const void* k, con
                 int64_t freq_row_stride, void* dk, int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
+  if (prerot && (rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dk});
   if (rc) return rc;
   corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
@@ -369,6 +389,7 @@ int bwd_dq_impl(const char* what, bool prerot, const void* q, const void* k, con
                 const void* o = nullptr) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
+  if (prerot && (rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dq});
   if (rc) return rc;
   if (o != nullptr && !aligned16(o)) return fail(COROPE_E_ALIGN, "%s: pointer %p is not 16-byte aligned", what, o);
@@ -441,6 +462,7 @@ int corope_rope_attn_bwd_dkdv_prerotated(const void* q_rot, const void* k_rot, c
   const char* what = "rope_attn_bwd_dkdv_prerotated";
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
+  if ((rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, dk, dv});
   if (rc) return rc;
   corope::BwdParams p = make_bwd(q_rot, k_rot, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
@@ -482,6 +504,7 @@ int corope_rope_attn_bwd_prerotated(const void* q_rot, const void* k_rot, const 
   int rc = validate_bwd("rope_attn_bwd_prerotated", B, H, N, D, freq_row_stride, sm_scale,
                         {q_rot, k_rot, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv});
   if (rc) return rc;
+  if ((rc = rotated_copies_built("rope_attn_bwd_prerotated", D))) return rc;
   rc = corope_rope_attn_bwd_dq_prerotated(q_rot, k_rot, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, B,
                                           H, N, D, sm_scale, causal, stream);
   if (rc) return rc;
@@ -501,6 +524,7 @@ int corope_rope_attn_bwd_ws(const void* q, const void* k, const void* v, const v
   int rc = validate_bwd("rope_attn_bwd_ws", B, H, N, D, freq_row_stride, sm_scale,
                         {q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv, workspace});
   if (rc) return rc;
+  if ((rc = rotated_copies_built("rope_attn_bwd_ws", D))) return rc;
   if (workspace_bytes < 2 * bwd_ws_tensor_bytes(B, H, N, D))
     return fail(COROPE_E_BADARG, "rope_attn_bwd_ws: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
                 (long long)(2 * bwd_ws_tensor_bytes(B, H, N, D)));
@@ -526,6 +550,7 @@ int corope_rope_attn_fwd_gqa(const void* q, const void* k, const void* v, const 
   }
   int rc = corope_rope_attn_check(B, Hq, N, D, freq_row_stride, sm_scale, 0);
   if (rc) return rc;
+  if ((rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse, k_rot});
   if (rc) return rc;
   if (q_rot != nullptr && !aligned16(q_rot)) return fail(COROPE_E_ALIGN, "%s: q_rot %p is not 16-byte aligned", what, q_rot);
@@ -546,6 +571,7 @@ int corope_rope_attn_bwd_gqa(const void* q, const void* k, int prerotated, const
   if (Hkv <= 0 || Hq % Hkv != 0) return fail(COROPE_E_BADARG, "%s: Hq=%d is not a multiple of Hkv=%d", what, Hq, Hkv);
   int rc = corope_rope_attn_check(B, Hq, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
+  if (prerotated && (rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv});
   if (rc) return rc;
   rc = corope_rope_attn_bwd_preprocess(o, d_o, delta, B, Hq, N, D, stream);
@@ -601,6 +627,7 @@ int corope_rope_attn_bwd_f16(const void* q, const void* k, const void* v, const 
   corope::BwdParams p = make_bwd(q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, dk, dv, B, H, N,
                                  sm_scale);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (workspace != nullptr && (rc = rotated_copies_built(what, D))) return rc;
   if (workspace != nullptr) {
     // as corope_rope_attn_bwd_ws: q (scaled) and k are rotated once, the dQ kernel computes delta on its way, dK and dV
     // come from one kernel

@@ -130,6 +130,11 @@ __device__ __forceinline__ int kv_slab(int bh, int H, int Hkv) {
   return H == Hkv ? bh : (bh / H) * Hkv + (bh % H) / (H / Hkv);
 }
 
+// Waves per SIMD the attention kernels are built for: two up to D = 128 (256 registers per lane each); at D = 256 the
+// operand rows and accumulators of a wave need more than that, so one wave per SIMD, with 512.
+template <int D>
+constexpr int kWavesPerSimd = D > 128 ? 1 : 2;
+
 // ---- LDS tile layouts -----------------------------------------------------------------------------
 // Row-major tile [rows][D] of bf16 with PAD elements of padding per row.
 //   PAD = 8  (16 bytes): 16 consecutive rows read at the same column with 16-byte reads land in 16 different

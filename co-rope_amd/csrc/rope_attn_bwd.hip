@@ -61,7 +61,7 @@ struct DkdvCfg {
 
 // PREROT: Q and K come from copies that rope_rotate_kernel rotated beforehand (no table reads in the loop).
 template <int D, int NWAVES, int BLOCK_M, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
-__global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
+__global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<D>, kWavesPerSimd<D>))) void rope_attn_bwd_dkdv_kernel(BwdParams p) {
   constexpr int DO_PAD = DO_DK ? (DO_DV ? kDkdvBothWaysPad : 8) : 32;
   constexpr int Q_PAD = DO_DK ? kDkdvBothWaysPad : 8;
   constexpr bool V_LDS = DO_DV && DO_DK;
@@ -356,7 +356,7 @@ struct DqCfg {
 // block) items, the stream of K/V tiles runs on from item to item, and nothing at the change of items needs a workgroup
 // barrier (a wave's operand rows and its dQ rows go through an LDS tile of its own).
 template <int D, int NWAVES, int BLOCK_N, bool CAUSAL, bool PREROT>
-__global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<D>, kWavesPerSimd<D>))) void rope_attn_bwd_dq_kernel(BwdParams p) {
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
   constexpr int NT = Cfg::kThreads;
   constexpr int KC = D / 16, NDB = D / 32, NKB = BLOCK_N / 32;
@@ -535,8 +535,11 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
         const uint16_t* vrow = vs + RowTile<D>::off(kb * 32 + lq, 8 * lh);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
-          sacc = kc == 0 ? mfma32_from(*reinterpret_cast<const u32x4*>(krow), qb[0], msb)
-                         : mfma32(*reinterpret_cast<const u32x4*>(krow + 16 * kc), qb[kc], sacc);
+          // (mfma32_from is for builds whose accumulators stay in the registers it names: with one wave per SIMD the
+          // compiler keeps them in the other half of the register file and would copy the result there at once)
+          sacc = kc > 0 ? mfma32(*reinterpret_cast<const u32x4*>(krow + 16 * kc), qb[kc], sacc)
+                 : kWavesPerSimd<D> == 2 ? mfma32_from(*reinterpret_cast<const u32x4*>(krow), qb[0], msb)
+                                         : mfma32(*reinterpret_cast<const u32x4*>(krow), qb[0], msb);
 #pragma unroll
         for (int kc = 0; kc < KC; ++kc)
           dpacc = mfma32(*reinterpret_cast<const u32x4*>(vrow + 16 * kc), dob[kc], kc == 0 ? f32x16{0} : dpacc);
@@ -606,7 +609,7 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(2
 // ===================================================================================== launchers
 template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT, int NWAVES>
 static hipError_t launch_dkdv_waves(BwdParams p, hipStream_t stream) {
-  constexpr int BLOCK_M = 64;
+  constexpr int BLOCK_M = D > 128 ? 32 : 64;   // what fits the LDS beside the waves' own slots
   using Cfg = DkdvCfg<D, NWAVES, BLOCK_M, DO_DK ? (DO_DV ? kDkdvBothWaysPad : 8) : 32, DO_DK ? kDkdvBothWaysPad : 8>;
   auto kern = rope_attn_bwd_dkdv_kernel<D, NWAVES, BLOCK_M, CAUSAL, DO_DV, DO_DK, PREROT>;
   static std::atomic<uint64_t> lds_ok{0};
@@ -622,13 +625,17 @@ static hipError_t launch_dkdv_waves(BwdParams p, hipStream_t stream) {
 
 template <int D, bool CAUSAL, bool DO_DV, bool DO_DK, bool PREROT>
 static hipError_t launch_dkdv_cfg(const BwdParams& p, hipStream_t stream) {
-  return use_small_tiles(p.N, p.BH / p.H * p.Hkv) ? launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 4>(p, stream)
-                                                   : launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 8>(p, stream);
+  if constexpr (D > 128) {
+    return launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 4>(p, stream);   // 4 waves x 512 registers
+  } else {
+    return use_small_tiles(p.N, p.BH / p.H * p.Hkv) ? launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 4>(p, stream)
+                                                     : launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 8>(p, stream);
+  }
 }
 
 template <int D, bool CAUSAL, bool PREROT, int NWAVES>
 static hipError_t launch_dq_waves(BwdParams p, hipStream_t stream) {
-  constexpr int BLOCK_N = 64;
+  constexpr int BLOCK_N = D > 128 ? 32 : 64;   // what fits the LDS beside the waves' own tiles
   using Cfg = DqCfg<D, NWAVES, BLOCK_N>;
   auto kern = rope_attn_bwd_dq_kernel<D, NWAVES, BLOCK_N, CAUSAL, PREROT>;
   static std::atomic<uint64_t> lds_ok{0};
@@ -644,8 +651,12 @@ static hipError_t launch_dq_waves(BwdParams p, hipStream_t stream) {
 
 template <int D, bool CAUSAL, bool PREROT>
 static hipError_t launch_dq_cfg(const BwdParams& p, hipStream_t stream) {
-  return use_small_tiles(p.N, p.BH) ? launch_dq_waves<D, CAUSAL, PREROT, 4>(p, stream)
-                                    : launch_dq_waves<D, CAUSAL, PREROT, 8>(p, stream);
+  if constexpr (D > 128) {
+    return launch_dq_waves<D, CAUSAL, PREROT, 4>(p, stream);   // 4 waves x 512 registers
+  } else {
+    return use_small_tiles(p.N, p.BH) ? launch_dq_waves<D, CAUSAL, PREROT, 4>(p, stream)
+                                      : launch_dq_waves<D, CAUSAL, PREROT, 8>(p, stream);
+  }
 }
 
 // Dispatch on the run-time switches (head dim, causal, pre-rotated operands present).
@@ -653,10 +664,15 @@ template <bool DO_DV, bool DO_DK>
 static hipError_t launch_dkdv(const BwdParams& p, int D, bool causal, hipStream_t stream) {
   const bool pre = p.q_rot != nullptr && p.k_rot != nullptr;
 #define COROPE_DKDV(DD, CC, PP) launch_dkdv_cfg<DD, CC, DO_DV, DO_DK, PP>(p, stream)
+  if (D == 256) {   // separate dV and dK on the original operands only
+    if (pre || (DO_DV && DO_DK)) return hipErrorInvalidValue;
+    if constexpr (!(DO_DV && DO_DK)) return causal ? COROPE_DKDV(256, true, false) : COROPE_DKDV(256, false, false);
+  }
   if (D == 128) {
     if (pre) return causal ? COROPE_DKDV(128, true, true) : COROPE_DKDV(128, false, true);
     return causal ? COROPE_DKDV(128, true, false) : COROPE_DKDV(128, false, false);
   }
+  if (D != 64) return hipErrorInvalidValue;
   if (pre) return causal ? COROPE_DKDV(64, true, true) : COROPE_DKDV(64, false, true);
   return causal ? COROPE_DKDV(64, true, false) : COROPE_DKDV(64, false, false);
 #undef COROPE_DKDV
@@ -676,10 +692,15 @@ hipError_t launch_bwd_dk(const BwdParams& p, int D, bool causal, hipStream_t str
 
 hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream) {
   const bool pre = p.q_rot != nullptr && p.k_rot != nullptr;
+  if (D == 256) {
+    if (pre) return hipErrorInvalidValue;
+    return causal ? launch_dq_cfg<256, true, false>(p, stream) : launch_dq_cfg<256, false, false>(p, stream);
+  }
   if (D == 128) {
     if (pre) return causal ? launch_dq_cfg<128, true, true>(p, stream) : launch_dq_cfg<128, false, true>(p, stream);
     return causal ? launch_dq_cfg<128, true, false>(p, stream) : launch_dq_cfg<128, false, false>(p, stream);
   }
+  if (D != 64) return hipErrorInvalidValue;
   if (pre) return causal ? launch_dq_cfg<64, true, true>(p, stream) : launch_dq_cfg<64, false, true>(p, stream);
   return causal ? launch_dq_cfg<64, true, false>(p, stream) : launch_dq_cfg<64, false, false>(p, stream);
 }

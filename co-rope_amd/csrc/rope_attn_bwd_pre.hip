@@ -38,7 +38,11 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const uint16_t* __r
 
 hipError_t launch_bwd_preprocess(const BwdParams& p, int D, hipStream_t stream) {
   const int64_t rows = (int64_t)p.BH * p.N;
-  if (D == 128) {
+  if (D == 256) {
+    constexpr int per_block = (256 / 32) * 4;
+    hipLaunchKernelGGL(bwd_preprocess_kernel<256>, dim3((unsigned)((rows + per_block - 1) / per_block)), dim3(256), 0,
+                       stream, p.o, p.d_o, p.delta, rows);
+  } else if (D == 128) {
     constexpr int per_block = (256 / 16) * 4;
     hipLaunchKernelGGL(bwd_preprocess_kernel<128>, dim3((unsigned)((rows + per_block - 1) / per_block)), dim3(256), 0,
                        stream, p.o, p.d_o, p.delta, rows);

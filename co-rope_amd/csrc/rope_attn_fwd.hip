@@ -45,6 +45,7 @@ struct FwdCfg {
   static constexpr int kLoopBytes = kFwdStages * kStageBytes;
   static constexpr int kEpilogueBytes = NW * 32 * kAccTileStride<D> * 4;   // fp32 O rows of all waves on their way out
   static constexpr int kLdsBytes = kLoopBytes > kEpilogueBytes ? kLoopBytes : kEpilogueBytes;
+  static_assert(kLdsBytes <= 160 * 1024, "LDS of a compute unit");
 };
 
 // ---- online softmax with a lazily updated reference maximum -------------------------------------------------------
@@ -106,7 +107,7 @@ __device__ __forceinline__ float softmax_slow_half(const f32x16& sacc, u32x4 (&p
 // (two data-dependent branches per tile); the two-launch forward in rope_attn_fwd_pipe.hip gets the same guarantee
 // from key norms computed beforehand and has no such branch.
 template <int D, int BLOCK_N, bool CAUSAL, int NW>
-__global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void rope_attn_fwd_kernel(FwdParams p) {
+__global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<D>, kWavesPerSimd<D>))) void rope_attn_fwd_kernel(FwdParams p) {
   using Cfg = FwdCfg<D, BLOCK_N, NW>;
   static_assert(BLOCK_N == 64, "the slot schedule is written for two 32-key halves");
   constexpr int NT = Cfg::kThreads;
@@ -309,7 +310,10 @@ static hipError_t launch_fwd_cfg(const FwdParams& p, hipStream_t stream) {
 }
 
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream) {
+  // D = 256: four waves of 512 registers each, whatever the shape
+  if (D == 256) return causal ? launch_fwd_waves<256, 64, true, 4>(p, stream) : launch_fwd_waves<256, 64, false, 4>(p, stream);
   if (D == 128) return causal ? launch_fwd_cfg<128, 64, true>(p, stream) : launch_fwd_cfg<128, 64, false>(p, stream);
+  if (D != 64) return hipErrorInvalidValue;
   return causal ? launch_fwd_cfg<64, 64, true>(p, stream) : launch_fwd_cfg<64, 64, false>(p, stream);
 }
 

@@ -76,6 +76,7 @@ __global__ __launch_bounds__(kRotThreads) void rope_rotate_kernel(const uint16_t
 
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
                               float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale) {
+  if (D != 64 && D != 128) return hipErrorInvalidValue;
   const int n_tiles = (N + kRotRows - 1) / kRotRows;
   dim3 grid((unsigned)n_tiles * BH);   // one axis: the second grid axis stops at 65535 slabs
 #define COROPE_ROT(DD, SS)                                                                                             \

@@ -13,7 +13,10 @@ import torch
 
 from . import _lib
 
-_SUPPORTED_D = (64, 128)
+_SUPPORTED_D = (64, 128, 256)
+# 256 (the largest head dim of the reference, fused_rope_attn.py:661) is built for the kernels that take q and k as they
+# are: the single-launch forward and the dV, dK and dQ kernels that rotate while they stage, one wave per SIMD.
+_ROTATED_PATH_MAX_D = 128
 # Head dims of the reference (fused_rope_attn.py:661) below the kernels' own: run at D = 64 with each half of a row padded
 # with zeros (the rotation pairs column j with column j + D/2, so the halves must stay the starts of the new halves).
 _PADDED_D = (16, 32)
@@ -103,7 +106,7 @@ TRAIN_ROTATED_MIN_ND = 65536
 
 def use_rotated_path(N, D, training):
     """Whether the operator rotates the operands ahead of the attention kernels at this shape."""
-    return N >= TWO_LAUNCH_MIN_N or (training and N * D >= TRAIN_ROTATED_MIN_ND)
+    return D <= _ROTATED_PATH_MAX_D and (N >= TWO_LAUNCH_MIN_N or (training and N * D >= TRAIN_ROTATED_MIN_ND))
 
 
 def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, keep_rotated=False):

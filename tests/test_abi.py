@@ -45,7 +45,8 @@ def test_header_cites_reference_for_each_entry_point():
     ((0, 8, 128, 64, 64, 1.0, 0), -1),
     ((1, 8, -5, 64, 64, 1.0, 0), -1),
     ((1, 8, 128, 32, 32, 1.0, 0), -2),
-    ((1, 8, 128, 256, 256, 1.0, 0), -2),
+    ((1, 8, 128, 256, 256, 1.0, 0), 0),
+    ((1, 8, 128, 512, 256, 1.0, 0), -2),
     ((1, 8, 128, 64, 16, 1.0, 0), -1),      # table narrower than D/2
     ((1, 8, 128, 64, 66, 1.0, 0), -1),      # row stride not a multiple of 4 floats
     ((1, 8, 128, 64, 64, 0.0, 0), -1),

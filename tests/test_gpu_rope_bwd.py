@@ -277,3 +277,45 @@ def test_head_dims_below_the_kernels_own(pkg, B, H, N, D, causal):
         print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
         assert a.shape == b.shape and torch.isfinite(a).all(), name
         assert within_bar(a, b, TOL)[0], name
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,Hq,Hkv,N", [(1, 2, 2, 300), (2, 2, 2, 128), (1, 1, 1, 1), (1, 3, 3, 1100), (1, 4, 2, 260), (1, 40, 40, 200)])
+def test_head_dim_256(pkg, B, Hq, Hkv, N, causal):
+    """The largest head dim the reference admits (fused-rope/fused_rope_attn.py:661): single-launch forward and the dV, dK
+    and dQ kernels on the original operands, one wave per SIMD; ragged lengths, grouped-query K/V, more items than
+    compute units' worth of one round and fewer."""
+    D = 256
+    print(f"case D=256 B={B} Hq={Hq} Hkv={Hkv} N={N} causal={causal}", flush=True)
+    G = Hq // Hkv
+    q, g = (bf16_round(seeded((B, Hq, N, D), 70 + i)) for i in range(2))
+    k, v = (bf16_round(seeded((B, Hkv, N, D), 80 + i)) for i in range(2))
+    c, s = O.precompute_freqs_cis(D, N)
+    scale = 1 / math.sqrt(D)
+    o, dq, dk, dv = _gpu_fwd_bwd(pkg, q, k, v, g, causal, scale, c, s)
+    kx, vx = k.repeat_interleave(G, dim=1), v.repeat_interleave(G, dim=1)
+    ro, _, rdq, rdk, rdv, _ = O.rope_attn_fwd_bwd_blocked(q, kx, vx, g, causal, scale, c, s)
+    rdk, rdv = (t.reshape(B, Hkv, G, N, D).sum(2) for t in (rdk, rdv))
+    for name, a, b in (("O", o, ro), ("dQ", dq, rdq), ("dK", dk, rdk), ("dV", dv, rdv)):
+        err = (a - b).abs()
+        print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
+        assert a.shape == b.shape and torch.isfinite(a).all(), name
+        assert within_bar(a, b, TOL * (math.sqrt(G) if name in ("dK", "dV") else 1.0))[0], name
+
+
+def test_head_dim_256_has_no_rotated_copies(pkg):
+    """Entry points that work on rotated copies or a workspace refuse head dim 256 before any launch."""
+    B, H, N, D = 1, 1, 64, 256
+    dev = torch.device("cuda:0")
+    x = torch.zeros(B, H, N, D, device=dev, dtype=torch.bfloat16)
+    c, s = (t.to(dev) for t in O.precompute_freqs_cis(D, N))
+    with pytest.raises((ValueError, RuntimeError), match="original operands"):
+        pkg.rope_rotate(x, c, s)
+    lib = pkg._lib.load()
+    assert lib.corope_rope_attn_fwd_workspace_bytes(B, H, N, D) > 0   # the size query answers; the launch refuses
+    ws = torch.empty(lib.corope_rope_attn_fwd_workspace_bytes(B, H, N, D), device=dev, dtype=torch.uint8)
+    M = torch.empty(B, H, N, device=dev)
+    rc = lib.corope_rope_attn_fwd_ws(x.data_ptr(), x.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), c.stride(0),
+                                     x.data_ptr(), M.data_ptr(), B, H, N, D, 0.1, 1, ws.data_ptr(), ws.numel(),
+                                     torch.cuda.current_stream().cuda_stream)
+    assert rc != 0 and "original operands" in pkg._lib.last_error()
