@@ -7,7 +7,9 @@
  *
  * Conventions (all entry points)
  *   - tensors are device pointers to contiguous row-major (B, H, N, D) bf16 storage;
- *     D is 64 or 128; pointers are 16-byte aligned;
+ *     D is 64 or 128 (fused RoPE attention: also 256, in the entry points that take q and k as they
+ *     are -- those that work on rotated copies or a workspace return COROPE_E_UNSUPPORTED);
+ *     pointers are 16-byte aligned;
  *   - freqs_cos / freqs_sin are fp32 tables with one row per position; only columns
  *     [0, D/2) are read; `freq_row_stride` is the distance between rows in elements
  *     (D for the reference's duplicated-half (N, D) table);
