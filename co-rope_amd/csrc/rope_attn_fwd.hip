@@ -114,7 +114,8 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
   constexpr int KC = D / 16;        // contraction chunks of QK^T = MFMAs per S^T half
   constexpr int NDB = D / 32;       // 32-column blocks of O
   constexpr int NPV = 2 * NDB;      // MFMAs per PV half
-  constexpr int KA = 4;             // K operands in flight
+  constexpr int KA = D > 128 ? 2 : 4;       // K operands in flight
+  constexpr int NAV = D > 128 ? 4 : NDB;    // transposed V operands in flight
   constexpr int LSV = RowTile<D, Cfg::kVPad>::kStride;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -135,8 +136,12 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
   const int n_k_tiles = (N + BLOCK_N - 1) / BLOCK_N;
   const int n_tiles = CAUSAL ? min((m0 + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, n_k_tiles) : n_k_tiles;
 
-  RotStage<D, BLOCK_N, NT> kst;
-  CopyStage<D, BLOCK_N, NT, Cfg::kVPad> vst;
+  // SPLIT (D = 256, where registers are short): the staging registers hold half a tile (32 rows) at a time, and each
+  // half has half an iteration to land.
+  constexpr bool SPLIT = D > 128;
+  constexpr int SROWS = SPLIT ? BLOCK_N / 2 : BLOCK_N;
+  RotStage<D, SROWS, NT> kst;
+  CopyStage<D, SROWS, NT, Cfg::kVPad> vst;
   kst.load(kg, p.cos, p.sin, p.fstride, 0, N);
   vst.load(vg, 0, N);
 
@@ -152,6 +157,13 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
     qrows.park(qb, reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride, nullptr, 0, 0, p.qk_scale);
   }
   __syncthreads();   // the K and V buffers below overlap the tiles the waves just used
+  if constexpr (D > 128) {
+    // one wave per SIMD: the Q operand's home is the accumulator half of the register file (the matrix cores read their
+    // B operand from there as well); left to itself the register allocator keeps it in scratch memory and reloads a piece
+    // in front of every score product
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) asm volatile("" : "+a"(qb[kc]));
+  }
 
   constexpr float scale = 1.f;   // scores come out of the matrix cores in base-2 units
   f32x16 oacc[NDB];
@@ -169,6 +181,12 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
   // are clamped, which makes tiles past the end harmless to load and store.
   kst.store_rows(ks(0));
   vst.store_rows(vs(0));
+  if constexpr (SPLIT) {
+    kst.load(kg, p.cos, p.sin, p.fstride, SROWS, N);
+    vst.load(vg, SROWS, N);
+    kst.store_rows(ks(0) + RowTile<D>::off(SROWS, 0));
+    vst.store_rows(vs(0) + RowTile<D, Cfg::kVPad>::off(SROWS, 0));
+  }
   kst.load(kg, p.cos, p.sin, p.fstride, BLOCK_N, N);
   vst.load(vg, BLOCK_N, N);
   __syncthreads();
@@ -183,8 +201,17 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
     auto stage_next = [&]() {
       kst.store_rows(ks(t + 1));
       vst.store_rows(vs(t + 1));
-      kst.load(kg, p.cos, p.sin, p.fstride, n0 + 2 * BLOCK_N, N);
-      vst.load(vg, n0 + 2 * BLOCK_N, N);
+      const int next_rows = SPLIT ? n0 + BLOCK_N + SROWS : n0 + 2 * BLOCK_N;   // SPLIT: the other half of tile t+1
+      kst.load(kg, p.cos, p.sin, p.fstride, next_rows, N);
+      vst.load(vg, next_rows, N);
+    };
+    auto stage_second_half = [&]() {   // SPLIT only: second half of tile t+1 to LDS, first half of tile t+2 requested
+      if constexpr (SPLIT) {
+        kst.store_rows(ks(t + 1) + RowTile<D>::off(SROWS, 0));
+        vst.store_rows(vs(t + 1) + RowTile<D, Cfg::kVPad>::off(SROWS, 0));
+        kst.load(kg, p.cos, p.sin, p.fstride, n0 + 2 * BLOCK_N, N);
+        vst.load(vg, n0 + 2 * BLOCK_N, N);
+      }
     };
     auto k_operand = [&](int half, int kc) {
       return *reinterpret_cast<const u32x4*>(kt + RowTile<D>::off(half * 32, 16 * kc));
@@ -243,15 +270,16 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
         ms_ref = m_run * scale;
       }
       if (MASK) mask_scores(s1, 1);
-      u32x4 av[NDB];  // transposed V operands, one 16-key chunk ahead
+      u32x4 av[NAV];  // transposed V operands, NAV MFMAs ahead (one 16-key chunk up to D = 128)
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) av[db] = v_operand(0, db);
+      for (int db = 0; db < NAV; ++db) av[db] = v_operand(0, db);
       __builtin_amdgcn_sched_barrier(0);
       // ---- slot C: O^T += V^T P^T(half 0), softmax of half 1 between the MFMAs -----------------------------------
 #pragma unroll
       for (int i = 0; i < NPV; ++i) {
-        oacc[i % NDB] = mfma32(av[i % NDB], pb0[i / NDB], oacc[i % NDB]);
-        av[i % NDB] = i + NDB < NPV ? v_operand(0, i + NDB) : v_operand(1, i + NDB - NPV);
+        oacc[i % NDB] = mfma32(av[i % NAV], pb0[i / NDB], oacc[i % NDB]);
+        av[i % NAV] = i + NAV < NPV ? v_operand(0, i + NAV) : v_operand(1, i + NAV - NPV);
+        if (i == 0) stage_second_half();
         softmax_fast_piece(i, NPV, s1, pb1, lsum1, scale, ms_ref);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -266,8 +294,8 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
       // ---- slot D: O^T += V^T P^T(half 1) ------------------------------------------------------------------------
 #pragma unroll
       for (int i = 0; i < NPV; ++i) {
-        oacc[i % NDB] = mfma32(av[i % NDB], pb1[i / NDB], oacc[i % NDB]);
-        if (i + NDB < NPV) av[i % NDB] = v_operand(1, i + NDB);
+        oacc[i % NDB] = mfma32(av[i % NAV], pb1[i / NDB], oacc[i % NDB]);
+        if (i + NAV < NPV) av[i % NAV] = v_operand(1, i + NAV);
       }
     };
     // Tiles entirely above this wave's diagonal contribute nothing to it; the wave still stages its share.
@@ -277,6 +305,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
       run_tile(need_mask);
     } else {
       stage_next();
+      stage_second_half();
     }
     __syncthreads();
   }
