@@ -7,10 +7,18 @@ boundaries into a buffer ``bench.py --phase-trace`` hands them) and the stand-al
 (``csrc/mfma_rate.hip``: what the matrix pipes sustain on this machine)."""
 from __future__ import annotations
 
+import glob
 import os
 import subprocess
 import sys
+import tempfile
 from concurrent.futures import ThreadPoolExecutor
+
+try:
+    from .check_isa import check_asm_mfma
+except ImportError:   # run as a script
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from check_isa import check_asm_mfma
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
@@ -23,6 +31,9 @@ MFMA_RATE = os.path.join(LIBDIR, "mfma_rate")
 F16_SOURCES = ["rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip"]
 
 SOURCES = ["abi.hip", "rope_freqs.hip", "rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_fwd_pipe.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip", "corope_gqa_bwd.hip"]
+
+# sources with asm-issued matrix-core instructions: their generated assembly is checked (check_isa.py) in every variant
+ISA_CHECKED = {"rope_attn_fwd_pipe.hip", "rope_attn_bwd.hip"}
 
 # -packed-fp32-ops is switched off: packed fp32 VALU forms are not used by these kernels.
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-value",
@@ -40,11 +51,26 @@ def _hipcc():
 def _compile(src, extra, suffix=""):
     obj = os.path.join(LIBDIR, os.path.splitext(src)[0] + suffix + ".o")
     cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
-    r = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
+    if src not in ISA_CHECKED:
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        problems = []
+    else:   # the compiler's intermediate files, among them the device assembly, land in a directory of their own
+        with tempfile.TemporaryDirectory(prefix="corope_build_") as tmp:
+            r = subprocess.run(cmd + ["--save-temps"], capture_output=True, text=True, cwd=tmp)
+            problems = []
+            if r.returncode == 0:
+                asm = glob.glob(os.path.join(tmp, "*-hip-amdgcn-*.s"))
+                if not asm:
+                    raise RuntimeError(f"no device assembly of {src}{suffix} to check")
+                for path in asm:
+                    with open(path) as f:
+                        problems += check_asm_mfma(f.read(), src + suffix)
     err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    if problems:
+        raise RuntimeError("asm-issued matrix-core results touched too early:\n" + "\n".join(problems))
     return obj, err
 
 

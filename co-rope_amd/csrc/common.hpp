@@ -83,7 +83,9 @@ __device__ __forceinline__ uint32_t pack_elts(float lo, float hi) { return pack_
 // D = A * B + C with D in registers of its own (C stays intact): the form the score products start from, C holding minus
 // the reference value of the exponentials in every register.  Written as an asm statement because the compiler, given
 // the builtin, copies C into D first.  The only readers of D that may follow are further mfma32 that accumulate into it
-// (same registers as C and D: no wait states needed) -- the vector units must not read D before one of those has run.
+// (same registers as C and D: no wait states needed) -- the vector units must not touch D before one of those has run, and the
+// compiler, to which this statement is opaque, inserts no wait states behind it: the build checks the generated assembly
+// of every kernel for that (check_isa.py).
 __device__ __forceinline__ f32x16 mfma32_from(u32x4 a, u32x4 b, const f32x16& c) {
   f32x16 d;
 #ifdef COROPE_F16
