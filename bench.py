@@ -36,9 +36,9 @@ PEAK_HBM_GBS = 8000.0
 # benchmark (summary and commands: profiles/rope_attn_c3_hbm_traffic.md); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE
 # by 1.0, the factors a plain 1 GiB device copy gives for the same counters.
 HBM_TRAFFIC_BYTES = {
-    ("c3", "rope_attn_fwd"): int((307460 * 2.0 + 132096) * 1024),
-    ("c3", "rope_attn_bwd_dq"): int((402667 * 2.0 + 91136) * 1024),
-    ("c3", "rope_attn_bwd_dkdv"): int((315363 * 2.0 + 131072) * 1024),
+    ("c3", "rope_attn_fwd"): int((305561 * 2.0 + 132096) * 1024),
+    ("c3", "rope_attn_bwd_dq"): int((404872 * 2.0 + 91136) * 1024),
+    ("c3", "rope_attn_bwd_dkdv"): int((312964 * 2.0 + 131072) * 1024),
 }
 
 CONFIGS = {
