@@ -55,6 +55,7 @@ SIGNATURES = {
     "corope_gqa_bwd_workspace_bytes": (_L, [_I, _I, _I, _I, _I]),
     "corope_gqa_bwd_min_workspace_bytes": (_L, [_I, _I, _I, _I, _I]),
     "corope_gqa_bwd": (_I, [_P] * 8 + [_I] * 5 + [_F, _F, _P, _L, _P]),
+    "corope_gqa_bwd_f16": (_I, [_P] * 8 + [_I] * 5 + [_F, _F, _P, _L, _P]),
 }
 
 _lock = threading.Lock()

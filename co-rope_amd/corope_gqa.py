@@ -1,4 +1,4 @@
-"""Co-RoPE grouped-query attention forward behind the reference's call surface.
+"""Co-RoPE grouped-query attention (forward and backward, bfloat16 or float16) behind the reference's call surface.
 
 ``attention(q, k, v, causal, sm_scale, theta[, warp_specialize])`` mirrors the reference's
 ``_attention.apply`` (corope-exp/flash_attn_co_rope_gqa_triton.py:403-456, :580), including its validation
@@ -56,8 +56,6 @@ class _CoRopeGqaAttn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         q, k, v, o = ctx.saved_tensors
-        if q.dtype != torch.bfloat16:
-            raise ValueError("the Co-RoPE backward is built for bfloat16 tensors only (the forward also takes float16)")
         dq, dk, dv = corope_gqa_backward(q, k, v, grad_output, ctx.sm_scale, ctx.theta, out=o)
         return dq, dk, dv, None, None, None, None
 
@@ -109,9 +107,10 @@ def corope_gqa_backward(q, k, v, grad_output, sm_scale, theta, workspace=None, o
     have = workspace.numel() * workspace.element_size()
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     with torch.cuda.device(q.device):
-        rc = lib.corope_gqa_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o_ptr, d_o.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                                dv.data_ptr(), B, Hq, Hkv, N, D, float(sm_scale), float(theta), workspace.data_ptr(),
-                                have, torch.cuda.current_stream(q.device).cuda_stream)
+        bwd = lib.corope_gqa_bwd_f16 if q.dtype == torch.float16 else lib.corope_gqa_bwd
+        rc = bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o_ptr, d_o.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                 dv.data_ptr(), B, Hq, Hkv, N, D, float(sm_scale), float(theta), workspace.data_ptr(),
+                 have, torch.cuda.current_stream(q.device).cuda_stream)
     _lib.check(rc, "corope_gqa_bwd")
     return dq, dk, dv
 

@@ -722,18 +722,22 @@ int64_t corope_gqa_bwd_min_workspace_bytes(int B, int Hq, int Hkv, int N, int D)
   return 4 * corope::corope_gqa_bwd_workspace_floats(1, Hq / Hkv, 1, N, D);
 }
 
-int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk, void* dv,
-                   int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void* workspace,
-                   int64_t workspace_bytes, void* stream) {
+}  // extern "C" (reopened below)
+
+namespace {
+
+int corope_gqa_bwd_impl(const char* what, bool f16, const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                        void* dq, void* dk, void* dv, int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta,
+                        void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = corope_gqa_check(B, Hq, Hkv, N, D, sm_scale, theta);
   if (rc) return rc;
-  rc = check_ptrs("corope_gqa_bwd", {q, k, v, d_o, dq, dk, dv, workspace});
+  rc = check_ptrs(what, {q, k, v, d_o, dq, dk, dv, workspace});
   if (rc) return rc;
-  if (o != nullptr && !aligned16(o)) return fail(COROPE_E_ALIGN, "corope_gqa_bwd: pointer %p is not 16-byte aligned", o);
-  if ((int64_t)B * Hq > 65535) return fail(COROPE_E_UNSUPPORTED, "corope_gqa_bwd: B * Hq = %lld exceeds 65535", (long long)B * Hq);
+  if (o != nullptr && !aligned16(o)) return fail(COROPE_E_ALIGN, "%s: pointer %p is not 16-byte aligned", what, o);
+  if ((int64_t)B * Hq > 65535) return fail(COROPE_E_UNSUPPORTED, "%s: B * Hq = %lld exceeds 65535", what, (long long)B * Hq);
   const int64_t need = 4 * corope::corope_gqa_bwd_workspace_floats(1, Hq / Hkv, 1, N, D);
   if (workspace_bytes < need)
-    return fail(COROPE_E_BADARG, "corope_gqa_bwd: workspace of %lld bytes, at least %lld needed (one group's matrices)",
+    return fail(COROPE_E_BADARG, "%s: workspace of %lld bytes, at least %lld needed (one group's matrices)", what,
                 (long long)workspace_bytes, (long long)need);
   corope::CoropeBwdParams p{};
   p.q = static_cast<const uint16_t*>(q);
@@ -750,8 +754,29 @@ int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* o, c
   p.Hq = Hq;
   p.Hkv = Hkv;
   p.N = N;
-  return launch_status("corope_gqa_bwd", corope::launch_corope_gqa_bwd(p, D, static_cast<float*>(workspace), workspace_bytes / 4,
-                                                                       static_cast<hipStream_t>(stream)));
+  float* ws = static_cast<float*>(workspace);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return launch_status(what, f16 ? corope_f16::launch_corope_gqa_bwd(p, D, ws, workspace_bytes / 4, st)
+                                 : corope::launch_corope_gqa_bwd(p, D, ws, workspace_bytes / 4, st));
 }
+
+}  // namespace
+
+extern "C" {
+
+int corope_gqa_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk, void* dv,
+                   int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void* workspace,
+                   int64_t workspace_bytes, void* stream) {
+  return corope_gqa_bwd_impl("corope_gqa_bwd", false, q, k, v, o, d_o, dq, dk, dv, B, Hq, Hkv, N, D, sm_scale, theta, workspace,
+                             workspace_bytes, stream);
+}
+
+int corope_gqa_bwd_f16(const void* q, const void* k, const void* v, const void* o, const void* d_o, void* dq, void* dk,
+                       void* dv, int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void* workspace,
+                       int64_t workspace_bytes, void* stream) {
+  return corope_gqa_bwd_impl("corope_gqa_bwd_f16", true, q, k, v, o, d_o, dq, dk, dv, B, Hq, Hkv, N, D, sm_scale, theta,
+                             workspace, workspace_bytes, stream);
+}
+
 
 }  // extern "C"

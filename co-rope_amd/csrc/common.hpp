@@ -744,6 +744,7 @@ __device__ __forceinline__ float bf16_to_f(uint16_t x) { return __builtin_bit_ca
 __device__ __forceinline__ uint16_t f_to_bf16(float x) { return (uint16_t)(pack_bf16(x, 0.f) & 0xffffu); }
 __device__ __forceinline__ uint16_t f_to_f16(float x) { return (uint16_t)(pack_f16(x, 0.f) & 0xffffu); }
 __device__ __forceinline__ uint16_t f_to_elt(float x) { return (uint16_t)(pack_elts(x, 0.f) & 0xffffu); }
+__device__ __forceinline__ float elt_to_f(uint16_t x) { return elt_lo((uint32_t)x); }
 
 // f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
 // in the body, so register arrays indexed with it never look dynamically indexed to the optimiser.

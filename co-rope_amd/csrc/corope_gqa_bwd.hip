@@ -43,7 +43,7 @@
 #include "common.hpp"
 #include "kernels.hpp"
 
-namespace corope {
+namespace COROPE_NS {
 
 struct CoropeBwdFreqs {
   float turns[64];   // w_d / (2 pi): phase in revolutions per unit of delta (what v_sin_f32 / v_cos_f32 take)
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
       if (vr < G) {
         const u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + d0);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) val[e] = pack_f16(bf16_lo(raw[e]), bf16_hi(raw[e]));   // exact
+        for (int e = 0; e < 4; ++e) val[e] = pack_f16(elt_lo(raw[e]), elt_hi(raw[e]));   // exact
       } else if (vr < 2 * G) {
         const bool upper = d0 >= HALF;                       // columns of the second half take w q1, the first half -w q2
         const u32x4 src = *reinterpret_cast<const u32x4*>(qrow + (upper ? d0 - HALF : d0 + HALF));
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
         float x[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const float qv = e % 2 ? bf16_hi(src[e / 2]) : bf16_lo(src[e / 2]);
+          const float qv = e % 2 ? elt_hi(src[e / 2]) : elt_lo(src[e / 2]);
           x[e] = upper ? wr[e] * qv : -wr[e] * qv;
         }
         val = u32x4{pack_f16(x[0], x[1]), pack_f16(x[2], x[3]), pack_f16(x[4], x[5]), pack_f16(x[6], x[7])};
@@ -244,9 +244,9 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
     float acc = 0.f, sq = 0.f;
     const int64_t off = ((int64_t)(head0 + h) * N + i) * D;
     for (int d = lane; d < D; d += kWave) {
-      const float g_d = bf16_to_f(p.d_o[off + d]);
+      const float g_d = elt_to_f(p.d_o[off + d]);
       sq = __builtin_fmaf(g_d, g_d, sq);
-      if (p.o != nullptr) acc = __builtin_fmaf(bf16_to_f(p.o[off + d]), g_d, acc);
+      if (p.o != nullptr) acc = __builtin_fmaf(elt_to_f(p.o[off + d]), g_d, acc);
     }
     dref[h] = wave_sum(acc);
     int ex = 0;
@@ -320,8 +320,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
       for (int e = 0; e < 4; ++e) {
         const float x = __builtin_amdgcn_fractf(delta * fr.turns[d0 + e]);
         const float sn = __builtin_amdgcn_sinf(x), cs = __builtin_amdgcn_cosf(x);
-        const float k1 = e % 2 ? bf16_hi(w1[e / 2]) : bf16_lo(w1[e / 2]);
-        const float k2 = e % 2 ? bf16_hi(w2[e / 2]) : bf16_lo(w2[e / 2]);
+        const float k1 = e % 2 ? elt_hi(w1[e / 2]) : elt_lo(w1[e / 2]);
+        const float k2 = e % 2 ? elt_hi(w2[e / 2]) : elt_lo(w2[e / 2]);
         r1v[e] = __builtin_fmaf(cs, k1, sn * k2);
         r2v[e] = __builtin_fmaf(cs, k2, -(sn * k1));
       }
@@ -465,8 +465,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
       for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
-          const u32x2 w = {pack_bf16(dqa[db][4 * g4] * p.sm_scale, dqa[db][4 * g4 + 1] * p.sm_scale),
-                           pack_bf16(dqa[db][4 * g4 + 2] * p.sm_scale, dqa[db][4 * g4 + 3] * p.sm_scale)};
+          const u32x2 w = {pack_elts(dqa[db][4 * g4] * p.sm_scale, dqa[db][4 * g4 + 1] * p.sm_scale),
+                           pack_elts(dqa[db][4 * g4 + 2] * p.sm_scale, dqa[db][4 * g4 + 3] * p.sm_scale)};
           *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
         }
     }
@@ -580,11 +580,11 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_dq_leader_kernel(CoropeB
 #pragma unroll
     for (int x = 0; x < 8; ++x) {
       const float wv = (i < N && t + x <= i) ? (x < 4 ? w0[x] : w1[x - 4]) : 0.f;   // nothing beyond the diagonal is defined
-      hi[x] = bf16_to_f(f_to_bf16(wv));
+      hi[x] = elt_to_f(f_to_elt(wv));
       lo[x] = wv - hi[x];
     }
-    const u32x4 bhi = {pack_bf16(hi[0], hi[1]), pack_bf16(hi[2], hi[3]), pack_bf16(hi[4], hi[5]), pack_bf16(hi[6], hi[7])};
-    const u32x4 blo = {pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]), pack_bf16(lo[4], lo[5]), pack_bf16(lo[6], lo[7])};
+    const u32x4 bhi = {pack_elts(hi[0], hi[1]), pack_elts(hi[2], hi[3]), pack_elts(hi[4], hi[5]), pack_elts(hi[6], hi[7])};
+    const u32x4 blo = {pack_elts(lo[0], lo[1]), pack_elts(lo[2], lo[3]), pack_elts(lo[4], lo[5]), pack_elts(lo[6], lo[7])};
     if (t0 + STEP < t_end) fetch(t0 + STEP);
     __syncthreads();
     if (t0 <= iw + 31 && iw < N) {   // wave-uniform: some row of this wave sees a key of the step
@@ -604,8 +604,8 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_dq_leader_kernel(CoropeB
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         const f32x4 pv = *reinterpret_cast<const f32x4*>(part + db * 32 + 8 * g4 + 4 * hf);
-        const u32x2 w = {pack_bf16((acc[db][4 * g4] + pv[0]) * p.sm_scale, (acc[db][4 * g4 + 1] + pv[1]) * p.sm_scale),
-                         pack_bf16((acc[db][4 * g4 + 2] + pv[2]) * p.sm_scale, (acc[db][4 * g4 + 3] + pv[3]) * p.sm_scale)};
+        const u32x2 w = {pack_elts((acc[db][4 * g4] + pv[0]) * p.sm_scale, (acc[db][4 * g4 + 1] + pv[1]) * p.sm_scale),
+                         pack_elts((acc[db][4 * g4 + 2] + pv[2]) * p.sm_scale, (acc[db][4 * g4 + 3] + pv[3]) * p.sm_scale)};
         *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
       }
   }
@@ -666,8 +666,8 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_dv_kernel(CoropeBwdParam
     u32x4 bop[G];
 #pragma unroll
     for (int h = 0; h < G; ++h)
-      bop[h] = u32x4{pack_bf16(pnext[h][0], pnext[h][1]), pack_bf16(pnext[h][2], pnext[h][3]),
-                     pack_bf16(pnext[h][4], pnext[h][5]), pack_bf16(pnext[h][6], pnext[h][7])};
+      bop[h] = u32x4{pack_elts(pnext[h][0], pnext[h][1]), pack_elts(pnext[h][2], pnext[h][3]),
+                     pack_elts(pnext[h][4], pnext[h][5]), pack_elts(pnext[h][6], pnext[h][7])};
     const bool wave_on = i0 + ROWS - 1 >= jw && jw < N;
     if (i0 + ROWS < N) fetch(i0 + ROWS);
     __syncthreads();
@@ -685,7 +685,7 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_dv_kernel(CoropeBwdParam
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
-        const u32x2 w = {pack_bf16(acc[db][4 * g4], acc[db][4 * g4 + 1]), pack_bf16(acc[db][4 * g4 + 2], acc[db][4 * g4 + 3])};
+        const u32x2 w = {pack_elts(acc[db][4 * g4], acc[db][4 * g4 + 1]), pack_elts(acc[db][4 * g4 + 2], acc[db][4 * g4 + 3])};
         *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
       }
   }
@@ -813,9 +813,9 @@ __global__ __launch_bounds__(kDkWaves* kWave) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
           for (int h = 0; h < 8; ++h) {
             const float x = h < G ? trow[(2 + h) * kDkKeys + col] : 0.f;
-            dsv[h] = hf == 0 ? x : x - bf16_to_f(f_to_bf16(x));
+            dsv[h] = hf == 0 ? x : x - elt_to_f(f_to_elt(x));
           }
-          aop = u32x4{pack_bf16(dsv[0], dsv[1]), pack_bf16(dsv[2], dsv[3]), pack_bf16(dsv[4], dsv[5]), pack_bf16(dsv[6], dsv[7])};
+          aop = u32x4{pack_elts(dsv[0], dsv[1]), pack_elts(dsv[2], dsv[3]), pack_elts(dsv[4], dsv[5]), pack_elts(dsv[6], dsv[7])};
         }
         // delta and W of this lane's 16 keys: keys 8 n + 4 half + 0..3 for n = 0..3, as the accumulator rows are laid out
         f32x4 dl[4], wg[4];
@@ -830,7 +830,7 @@ __global__ __launch_bounds__(kDkWaves* kWave) __attribute__((amdgpu_waves_per_eu
         for (int np = 0; np < NP; ++np) {
           const u32x4 bq1 = *reinterpret_cast<const u32x4*>(qT + (r * D + 32 * np + col) * 8);
           const u32x4 bq2 = *reinterpret_cast<const u32x4*>(qT + (r * D + 32 * (NP + np) + col) * 8);
-          const float ql1 = bf16_lo(bq1[0]), ql2 = bf16_lo(bq2[0]);
+          const float ql1 = elt_lo(bq1[0]), ql2 = elt_lo(bq2[0]);
           const f32x16 u1 = mfma32(aop, bq1, f32x16{0}), u2 = mfma32(aop, bq2, f32x16{0});
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
@@ -850,8 +850,8 @@ __global__ __launch_bounds__(kDkWaves* kWave) __attribute__((amdgpu_waves_per_eu
         uint16_t* op = p.dk + ((int64_t)g * N + j) * D;
 #pragma unroll
         for (int np = 0; np < NP; ++np) {
-          op[32 * np + col] = f_to_bf16(dk1[np][e] * p.sm_scale);
-          op[32 * np + col + HALF] = f_to_bf16(dk2[np][e] * p.sm_scale);
+          op[32 * np + col] = f_to_elt(dk1[np][e] * p.sm_scale);
+          op[32 * np + col + HALF] = f_to_elt(dk2[np][e] * p.sm_scale);
         }
       }
     }
@@ -940,4 +940,4 @@ hipError_t launch_corope_gqa_bwd(const CoropeBwdParams& p, int D, float* workspa
   return hipSuccess;
 }
 
-}  // namespace corope
+}  // namespace COROPE_NS

@@ -202,4 +202,6 @@ hipError_t launch_bwd_dkdv_fused(const corope::BwdParams& p, int D, bool causal,
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
                               float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale);
 hipError_t launch_corope_gqa_fwd(const corope::CoropeParams& p, int D, hipStream_t stream);
+hipError_t launch_corope_gqa_bwd(const corope::CoropeBwdParams& p, int D, float* workspace, int64_t workspace_floats,
+                                 hipStream_t stream);
 }  // namespace corope_f16

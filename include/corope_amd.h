@@ -272,7 +272,7 @@ int corope_gqa_fwd(const void *q, const void *k, const void *v, void *o,
 
 /* The same forward on fp16 tensors, the dtype of the reference's kernel and of its comparison script
  * (corope-exp/flash_attn_co_rope_gqa_triton.py:406-456, compare_corope.py:18): fp16 q, k, v, o; same kernel built for
- * fp16 elements (leader logits, scores and P V all on fp16 matrix-core operands).  The backward is built for bf16 only. */
+ * fp16 elements (leader logits, scores and P V all on fp16 matrix-core operands).  The backward: corope_gqa_bwd_f16. */
 int corope_gqa_fwd_f16(const void *q, const void *k, const void *v, void *o,
                        int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta, void *stream);
 
@@ -301,6 +301,13 @@ int corope_gqa_bwd(const void *q, const void *k, const void *v, const void *o, c
                    void *dq, void *dk, void *dv,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta,
                    void *workspace, int64_t workspace_bytes, void *stream);
+
+/* The same for fp16 tensors, the dtype of the reference's callers (corope-exp/compare_corope.py:18): q, k, v, o, dO in and
+ * dq, dk, dv out are fp16, every matrix-core operand is fp16, the workspace is the same size. */
+int corope_gqa_bwd_f16(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+                       void *dq, void *dk, void *dv,
+                       int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta,
+                       void *workspace, int64_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -210,3 +210,28 @@ def test_corope_backward_does_not_depend_on_the_scale_of_dO(pkg, B, Hq, Hkv, N, 
         for name, a, b in zip(("dQ", "dK", "dV"), got, base):
             assert torch.isfinite(a).all(), (name, kexp)
             assert torch.equal(a, b * f), f"{name} at dO x 2^{kexp}: max rel diff {((a - b * f).abs() / (b.abs() * f + 1e-30)).max():.3e}"
+
+
+def _f16_round(x):
+    return x.to(torch.float16).float()
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,N,D", [(1, 4, 2, 32, 64), (1, 6, 2, 100, 64), (1, 8, 2, 130, 128), (2, 5, 1, 77, 128),
+                                           (1, 4, 1, 449, 128), (2, 4, 2, 64, 32)])
+def test_corope_backward_parity_fp16(pkg, B, Hq, Hkv, N, D):
+    """fp16 tensors, the dtype of the reference's callers (corope-exp/compare_corope.py:18), forward and backward: the same
+    kernels built for fp16 elements, against the oracle on the fp16-rounded inputs, at the bf16 bar (fp16 carries three
+    mantissa bits more)."""
+    print(f"case fp16 B={B} Hq={Hq} Hkv={Hkv} N={N} D={D}", flush=True)
+    q, k, v, d_o = (_f16_round(t) for t in _inputs(B, Hq, Hkv, N, D, seed=11))
+    scale = 1 / math.sqrt(D)
+    dev = torch.device("cuda:0")
+    qg, kg, vg = (t.to(dev, torch.float16).requires_grad_(True) for t in (q, k, v))
+    o = pkg.corope_attention(qg, kg, vg, True, scale, 10000.0)
+    o.backward(d_o.to(dev, torch.float16))
+    torch.cuda.synchronize()
+    assert all(t.grad.dtype == torch.float16 for t in (qg, kg, vg))
+    ro = C.corope_gqa_forward(q.double(), k.double(), v.double(), True, scale, 10000.0, torch.float64).float()
+    print(f"  O max-abs {(o.float().cpu() - ro).abs().max():.3e}", flush=True)
+    assert (o.float().cpu() - ro).abs().max() <= TOL
+    _compare([t.grad.float().cpu() for t in (qg, kg, vg)], _oracle_grads(q, k, v, d_o, scale, 10000.0), Hq // Hkv)
