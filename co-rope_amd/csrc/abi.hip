@@ -83,7 +83,7 @@ corope::BwdParams make_bwd(const void* q, const void* k, const void* v, const vo
 
 extern "C" {
 
-int corope_amd_version(void) { return 1; }
+int corope_amd_version(void) { return 2; }
 
 const char* corope_amd_last_error(void) { return g_err; }
 
@@ -593,9 +593,10 @@ int corope_rope_attn_bwd_gqa(const void* q, const void* k, int prerotated, const
 
 // ---- fp16 tensors (the reference's dtype): the same kernels built for fp16 elements -------------------------------------
 int corope_rope_attn_fwd_f16(const void* q, const void* k, const void* v, const float* freqs_cos, const float* freqs_sin,
-                             int64_t freq_row_stride, void* o, float* lse, int B, int H, int N, int D, float sm_scale,
-                             int causal, void* stream) {
+                             int64_t freq_row_stride, void* o, float* lse, int B, int H, int Hkv, int N, int D,
+                             float sm_scale, int causal, void* stream) {
   const char* what = "rope_attn_fwd_f16";
+  if (Hkv <= 0 || H % Hkv != 0) return fail(COROPE_E_BADARG, "%s: H=%d is not a multiple of Hkv=%d", what, H, Hkv);
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
   if (rc) return rc;
   rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse});
@@ -612,20 +613,23 @@ int corope_rope_attn_fwd_f16(const void* q, const void* k, const void* v, const 
   p.qk_scale = sm_scale * kLog2e;
   p.N = N;
   p.BH = B * H;
-  p.H = p.Hkv = H;
+  p.H = H;
+  p.Hkv = Hkv;
   return launch_status(what, corope_f16::launch_rope_attn_fwd(p, D, causal != 0, static_cast<hipStream_t>(stream)));
 }
 
 int corope_rope_attn_bwd_f16(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                              float* delta, const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* dq,
-                             void* dk, void* dv, int B, int H, int N, int D, float sm_scale, int causal, void* workspace,
-                             int64_t workspace_bytes, void* stream) {
+                             void* dk, void* dv, int B, int H, int Hkv, int N, int D, float sm_scale, int causal,
+                             void* workspace, int64_t workspace_bytes, void* stream) {
   const char* what = "rope_attn_bwd_f16";
+  if (Hkv <= 0 || H % Hkv != 0) return fail(COROPE_E_BADARG, "%s: H=%d is not a multiple of Hkv=%d", what, H, Hkv);
   int rc = validate_bwd(what, B, H, N, D, freq_row_stride, sm_scale,
                         {q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv});
   if (rc) return rc;
   corope::BwdParams p = make_bwd(q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, dk, dv, B, H, N,
                                  sm_scale);
+  p.Hkv = Hkv;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (workspace != nullptr && (rc = rotated_copies_built(what, D))) return rc;
   if (workspace != nullptr) {
@@ -641,7 +645,7 @@ int corope_rope_attn_bwd_f16(const void* q, const void* k, const void* v, const 
     rc = launch_status(what, corope_f16::launch_rope_rotate(p.q, p.cos, p.sin, p.fstride, q_rot, nullptr, p.BH, N, D, st,
                                                             p.qk_scale));
     if (rc) return rc;
-    rc = launch_status(what, corope_f16::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, k_rot, nullptr, p.BH, N, D, st, 1.f));
+    rc = launch_status(what, corope_f16::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, k_rot, nullptr, B * Hkv, N, D, st, 1.f));
     if (rc) return rc;
     p.q = p.q_rot = q_rot;
     p.k = p.k_rot = k_rot;

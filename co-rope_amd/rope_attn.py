@@ -77,8 +77,6 @@ def _check_inputs(q, k, v, freqs_cos, freqs_sin):
         raise ValueError("fused RoPE attention runs on the GPU only: all tensors must be on a HIP device")
     if not (q.dtype == k.dtype == v.dtype and q.dtype in (torch.bfloat16, torch.float16)):
         raise ValueError(f"q, k, v must all be bfloat16 or all float16 (got {q.dtype}, {k.dtype}, {v.dtype})")
-    if q.dtype == torch.float16 and k.shape[1] != q.shape[1]:
-        raise ValueError("grouped-query attention (fewer key/value heads) is built for bfloat16 only")
     n = q.shape[2]
     for name, f in (("freqs_cos", freqs_cos), ("freqs_sin", freqs_sin)):
         if f.dim() != 2 or f.shape[0] < n or f.shape[1] < d // 2:
@@ -127,7 +125,7 @@ def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, k
         if q.dtype == torch.float16:
             # the reference's dtype: one launch, a true running maximum wherever a probability would leave fp16's range
             rc = lib.corope_rope_attn_fwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
-                                              fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, N, D, float(sm_scale),
+                                              fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, Hkv, N, D, float(sm_scale),
                                               int(bool(causal)), _stream_ptr(q))
             _lib.check(rc, "corope_rope_attn_fwd_f16")
         elif Hkv != H:   # grouped-query attention: one entry point covers the three forms
@@ -208,9 +206,9 @@ class _FusedRopeAttn(torch.autograd.Function):
                     ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
                 rc = lib.corope_rope_attn_bwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
                                                   M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0),
-                                                  dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, N, D, ctx.sm_scale,
-                                                  int(ctx.causal), ws.data_ptr() if ws is not None else None, nbytes,
-                                                  _stream_ptr(q))
+                                                  dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, k.shape[1], N, D,
+                                                  ctx.sm_scale, int(ctx.causal), ws.data_ptr() if ws is not None else None,
+                                                  nbytes, _stream_ptr(q))
             elif k.shape[1] != H:         # grouped-query attention
                 rc = lib.corope_rope_attn_bwd_gqa(q.data_ptr(), k.data_ptr(), int(ctx.rotated), v.data_ptr(), o.data_ptr(),
                                                   do.data_ptr(), M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(),

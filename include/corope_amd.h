@@ -231,16 +231,17 @@ int corope_rope_attn_bwd_ws(const void *q, const void *k, const void *v, const v
  * bf16 can hold); the backward is preprocess + dV + dK + dQ as in corope_rope_attn_bwd, or -- given a workspace of
  * corope_rope_attn_bwd_workspace_bytes (may be NULL) -- the rotation of q and k into it followed by the dQ and the fused
  * dK+dV kernel as in corope_rope_attn_bwd_ws, which is the faster form from N * D = 65536 on.  `delta` is (B,H,N) fp32 scratch.
+ * k, v, dk, dv have Hkv heads (H a multiple of Hkv; Hkv = H: the reference's form), as in the grouped-query entry points below.
  * Replaces _attention.forward / .backward (fused-rope/fused_rope_attn.py:655-777) for callers that keep the reference's dtype. */
 int corope_rope_attn_fwd_f16(const void *q, const void *k, const void *v,
                              const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
                              void *o, float *lse,
-                             int B, int H, int N, int D, float sm_scale, int causal, void *stream);
+                             int B, int H, int Hkv, int N, int D, float sm_scale, int causal, void *stream);
 int corope_rope_attn_bwd_f16(const void *q, const void *k, const void *v, const void *o, const void *d_o,
                              const float *lse, float *delta,
                              const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
                              void *dq, void *dk, void *dv,
-                             int B, int H, int N, int D, float sm_scale, int causal,
+                             int B, int H, int Hkv, int N, int D, float sm_scale, int causal,
                              void *workspace, int64_t workspace_bytes, void *stream);
 
 /* Grouped-query form of the operator: q (B,Hq,N,D), k and v (B,Hkv,N,D), Hq a multiple of Hkv; query head h reads

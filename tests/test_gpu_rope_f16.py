@@ -97,3 +97,29 @@ def test_fp16_large_scores_stay_finite(pkg):
         print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
         assert torch.isfinite(a).all(), name
         assert err.max() <= 0.15 and err.mean() <= 5e-3, name
+
+
+@pytest.mark.parametrize("rotated", [False, True])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,Hq,Hkv,N,D", [(1, 8, 2, 320, 128), (2, 4, 1, 200, 64), (1, 6, 3, 1024, 128)])
+def test_fp16_grouped_query(pkg, monkeypatch, B, Hq, Hkv, N, D, causal, rotated):
+    """fp16 tensors with fewer key/value heads, on the original operands and on rotated copies: against the oracle run on
+    k, v repeated over their groups, dK and dV summed back over the group (bar scaled by sqrt(G) for those two)."""
+    print(f"case fp16 gqa B={B} Hq={Hq} Hkv={Hkv} N={N} D={D} causal={causal} rotated={rotated}", flush=True)
+    monkeypatch.setattr(pkg.rope_attn, "TWO_LAUNCH_MIN_N", 1 if rotated else 1 << 30)
+    monkeypatch.setattr(pkg.rope_attn, "TRAIN_ROTATED_MIN_ND", 1 if rotated else 1 << 60)
+    G = Hq // Hkv
+    f16 = lambda t: t.to(torch.float16).float()
+    q, g = (f16(seeded((B, Hq, N, D), 50 + i)) for i in range(2))
+    k, v = (f16(seeded((B, Hkv, N, D), 60 + i)) for i in range(2))
+    c, s = O.precompute_freqs_cis(D, N)
+    scale = 1 / math.sqrt(D)
+    got = _gpu(pkg, q, k, v, g, causal, scale, c, s)
+    kx, vx = k.repeat_interleave(G, dim=1), v.repeat_interleave(G, dim=1)
+    ro, _, rdq, rdk, rdv, _ = O.rope_attn_fwd_bwd_blocked(q, kx, vx, g, causal, scale, c, s)
+    rdk, rdv = (t.reshape(B, Hkv, G, N, D).sum(2) for t in (rdk, rdv))
+    for name, a, b in zip(("O", "dQ", "dK", "dV"), got, (ro, rdq, rdk, rdv)):
+        err = (a - b).abs()
+        print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e}")
+        assert a.shape == b.shape and torch.isfinite(a).all(), name
+        assert err.max() <= 2e-2 * (math.sqrt(G) if name in ("dK", "dV") else 1.0), name
