@@ -94,17 +94,17 @@ def _freq_table(f):
     return f
 
 
-# Sequences at least this long take the two-launch forward (K rotated once into a scratch buffer, then attention on
-# the rotated copy); shorter ones the single launch, where every K tile is rotated by few query blocks anyway.
+# Shapes from which the operator rotates its operands ahead of the attention kernels: K once into a scratch buffer for
+# the forward (every K tile is otherwise rotated again by each query block of its head), and, when a gradient will be asked
+# for, q and k once for the backward (fused dK+dV, no tables in its loops).  Measured crossover on MI355X, the same for both:
+# N * D = 65536 (N = 512 at D = 128, N = 1024 at D = 64); below it every kernel rotates its own tiles.
 TWO_LAUNCH_MIN_N = 1024
-# When a gradient will be asked for, the rotated copies also feed the backward (fused dK+dV, no tables in its loops), which
-# pays off earlier: from N * D >= this (N = 512 at D = 128, N = 1024 at D = 64; measured crossover on MI355X).
 TRAIN_ROTATED_MIN_ND = 65536
 
 
 def use_rotated_path(N, D, training):
     """Whether the operator rotates the operands ahead of the attention kernels at this shape."""
-    return D <= _ROTATED_PATH_MAX_D and (N >= TWO_LAUNCH_MIN_N or (training and N * D >= TRAIN_ROTATED_MIN_ND))
+    return D <= _ROTATED_PATH_MAX_D and (N >= TWO_LAUNCH_MIN_N or N * D >= TRAIN_ROTATED_MIN_ND)
 
 
 def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, keep_rotated=False):
