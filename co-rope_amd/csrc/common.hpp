@@ -69,6 +69,21 @@ __device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
 __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) { return mfma32_f16(a, b, c); }
 #endif
 
+// D(16x16) += A(16x32) * B(32x16): half the matrix-pipe time of the 32x32x16 form, for products that need few rows.
+//   A operand: lane l holds row (l % 16), contraction slots 8*(l / 16) .. +7
+//   B operand: lane l holds column (l % 16), contraction slots 8*(l / 16) .. +7
+//   D/C      : lane l holds column (l % 16); register i holds row 4*(l / 16) + i
+__device__ __forceinline__ f32x4 mfma16_f16(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+#ifdef COROPE_F16
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) { return mfma16_f16(a, b, c); }
+#else
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+#endif
+
 // ---- the element type of the attention kernels: two elements per 32-bit word, element 0 in the low half -------------
 #ifdef COROPE_F16
 __device__ __forceinline__ float elt_lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }

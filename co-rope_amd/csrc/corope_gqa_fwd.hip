@@ -21,8 +21,9 @@
 //
 // Mapping: one wave (= one workgroup) per (batch, kv head, query row), longest rows first; lane = key inside a 64-key
 // chunk.  Per chunk: the contiguous 64 x D block of K is fetched with whole cache lines per instruction and parked in
-// the LDS tile -> logits (MFMA, results moved back to lane = key with v_permlane32_swap) -> gate, scan over the lanes,
-// delta -> each lane rotates its own key row in place -> scores (MFMA) -> online softmax against a wave-uniform
+// the LDS tile -> logits (16x16x32 MFMA, every lane finds its key's logit in its own registers) -> gate, scan over the lanes,
+// delta -> each lane rotates its own key row in place -> scores (32x32x16 MFMA, rows moved back to lane = key with
+// v_permlane32_swap) -> online softmax against a wave-uniform
 // reference value per head (moved to the running maximum only when a score rises well above it) -> the block of V
 // replaces the rotated keys in the tile -> O accumulation (MFMA).  A wave's LDS instructions
 // execute in order, so the kernel needs no barriers; global loads for the next step are issued one step ahead.
@@ -57,7 +58,9 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
   const float scale2 = p.sm_scale * 1.4426950408889634f;               // scores in the base-2 domain
 
   // A operand of the score product, constant over the row: lane (vr, hf) holds columns 16 ks + 8 hf .. + 7 of q^vr as fp16
-  // for vr < G, zeros otherwise.  The logit product takes the leader's row in bf16 from LDS.
+  // for vr < G, zeros otherwise.  The logit product takes the leader's row in the element type from LDS.
+  // (This product stays on 32x32x16: with rows m of a 16x16x32 A operand holding head m % 4, which also needs no exchange
+  // between lanes, the kernel was 3.7 % slower at G = 4, D = 128 -- unlike the logit product below.)
   u32x4 aop[D / 16];
   {
     const uint16_t* qrow = p.q + ((int64_t)(head0 + (vr < G ? vr : 0)) * N + i) * D + 8 * hf;
@@ -113,26 +116,32 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
 #pragma unroll
     for (int h = 0; h < G; ++h) out[h] = (h / 4) % 2 ? hi_rows[4 * (h / 8) + h % 4] : lo_rows[4 * (h / 8) + h % 4];
   };
-  auto leader_times_tile = [&](f32x16& c0, f32x16& c1) __attribute__((always_inline)) {   // bf16: K as parked
-    c0 = f32x16{0};
-    c1 = f32x16{0};
+  // Leader logits of the 64 keys (K as parked): a 1 x D by D x 64 product, run as 16x16x32 products with the leader's row in
+  // every row of A.  All rows of a result block are then equal, block kb holds keys 16 kb .. 16 kb + 15 in the lanes with
+  // that l % 16, so every lane finds its own key's logit in block (lane / 16) of its own registers.
+  auto leader_logit = [&]() __attribute__((always_inline)) {
+    const int r = lane / 16, c = lane % 16;
+    f32x4 acc[4];
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) {
-      // every row of the A operand is the leader's row (a broadcast read): all result rows then hold the logits, and no
-      // lane needs a zero operand
-      const u32x4 a = *reinterpret_cast<const u32x4*>(ql + 16 * ks + 8 * hf);
-      c0 = mfma32(a, *reinterpret_cast<const u32x4*>(tile + vr * KS + 16 * ks + 8 * hf), c0);
-      c1 = mfma32(a, *reinterpret_cast<const u32x4*>(tile + (32 + vr) * KS + 16 * ks + 8 * hf), c1);
+    for (int kb = 0; kb < 4; ++kb) acc[kb] = f32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int ks = 0; ks < D / 32; ++ks) {
+      const u32x4 a = *reinterpret_cast<const u32x4*>(ql + 32 * ks + 8 * r);   // a broadcast read per 16 lanes
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb)
+        acc[kb] = mfma16(a, *reinterpret_cast<const u32x4*>(tile + (16 * kb + c) * KS + 32 * ks + 8 * r), acc[kb]);
     }
+    return r == 0 ? acc[0][0] : r == 1 ? acc[1][0] : r == 2 ? acc[2][0] : acc[3][0];
   };
-  auto heads_times_tile = [&](f32x16& c0, f32x16& c1) __attribute__((always_inline)) {    // fp16: the rotated keys
-    c0 = f32x16{0};
-    c1 = f32x16{0};
+  // scores of the G heads against the rotated keys (fp16) -> this lane's key: sc[h]
+  auto scores_of_key = [&](float (&sc)[G]) __attribute__((always_inline)) {
+    f32x16 c0 = f32x16{0}, c1 = f32x16{0};
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
       c0 = mfma32_f16(aop[ks], *reinterpret_cast<const u32x4*>(tile + vr * KS + 16 * ks + 8 * hf), c0);
       c1 = mfma32_f16(aop[ks], *reinterpret_cast<const u32x4*>(tile + (32 + vr) * KS + 16 * ks + 8 * hf), c1);
     }
+    rows_of_key(c0, c1, sc);
   };
 
   // oacc[db][4 g4 + e]: column 32 db + 8 g4 + 4 hf + e of head `vr`'s output row (lanes with vr >= G idle)
@@ -163,11 +172,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     lds_order();                  // (also orders the one-time write of the leader's row before its first read)
 
     // leader logits (row 0 of the product), gates, delta
-    f32x16 c0, c1;
-    leader_times_tile(c0, c1);
-    float lg[G];
-    rows_of_key(c0, c1, lg);
-    const float z = valid ? 1.f / (1.f + __expf(-lg[0] * p.sm_scale)) : 0.f;   // gates beyond the diagonal do not count
+    const float lg0 = leader_logit();
+    const float z = valid ? 1.f / (1.f + __expf(-lg0 * p.sm_scale)) : 0.f;   // gates beyond the diagonal do not count
     const float zpre = wave_prefix_sum(z), ztot = wave_last(zpre);
     const float delta = carry + (ztot - zpre);   // gates strictly to the right of this key, up to the diagonal
     carry += ztot;
@@ -201,9 +207,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     lds_order();
 
     // scores of every head, online softmax
-    heads_times_tile(c0, c1);
     float sc[G];
-    rows_of_key(c0, c1, sc);
+    scores_of_key(sc);
     // The reference value m_run[h] of the exponentials only has to keep them in range, it need not be the running
     // maximum: it moves (to the exact maximum so far, with the usual rescaling) only when some score of the chunk lies
     // more than kLazyMargin above it, which after the first chunks of a row is rare.  The common case then costs one
