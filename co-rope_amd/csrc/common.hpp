@@ -699,6 +699,19 @@ __device__ __forceinline__ void store_rows_via_lds(const f32x16 (&acc)[D / 32], 
   lds_order();
 }
 
+// A operand of mfma16 (16 rows m x 32 contraction slots) read transposed from a row-major tile T[k][m]: lane l gets
+// T[kbase + 8*(l / 16) + j][m0 + l % 16] for slots j = 0..7 (two transposing reads of 4 contraction rows each).
+__device__ __forceinline__ u32x4 load_a_trans16(const uint16_t* tile, int stride, int kbase, int m0) {
+  typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+  const int l = threadIdx.x % kWave;
+  const int g = l / 16, s = l % 16;
+  const uint16_t* p = tile + (kbase + 8 * g + s / 4) * stride + m0 + 4 * (s % 4);
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * stride));
+  u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
+  return u32x4{a[0], a[1], b[0], b[1]};
+}
+
 // Natural-order variant of load_a_trans: slot j of lane-half h <-> k = kbase + 8*h + j.
 __device__ __forceinline__ u32x4 load_a_trans_natural(const uint16_t* tile, int stride, int kbase, int m0) {
   typedef __attribute__((address_space(3))) s16x4* lds_ptr;

@@ -39,7 +39,7 @@ struct CoropeFreqs {
 template <int D, int G>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void corope_gqa_fwd_kernel(CoropeParams p,
                                                                                                        CoropeFreqs fr) {
-  constexpr int HALF = D / 2, KS = D + 8, WS = kWave + 8, NDB = D / 32, PIECES = D / 8;
+  constexpr int HALF = D / 2, KS = D + 8, WS = kWave + 8, PIECES = D / 8;
   constexpr int NI = 4 * ((G - 1) / 8 + 1);                            // accumulator registers that hold rows < G
   __shared__ __attribute__((aligned(16))) uint16_t tile[kWave * KS];   // [key][d]: K (bf16), then rotated K (fp16), then V (bf16)
   __shared__ __attribute__((aligned(16))) uint16_t ql[D];              // the leader's query row (bf16)
@@ -144,10 +144,14 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     rows_of_key(c0, c1, sc);
   };
 
-  // oacc[db][4 g4 + e]: column 32 db + 8 g4 + 4 hf + e of head `vr`'s output row (lanes with vr >= G idle)
-  f32x16 oacc[NDB];
+  // O^T += V^T P^T as 16x16x32 products (16 output columns x 16 heads per block, of which G are used: half the matrix-pipe
+  // time and half the accumulator registers of the 32x32x16 form).  oacc[db][e]: column 16 db + 4 (lane / 16) + e of head
+  // lane % 16's output row (lanes with lane % 16 >= G idle).
+  constexpr int NOB = D / 16;
+  const int oh = lane % 16, og = lane / 16;
+  f32x4 oacc[NOB];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) oacc[db] = f32x16{0};
+  for (int db = 0; db < NOB; ++db) oacc[db] = f32x4{0, 0, 0, 0};
   float m_run[G], l_run[G];   // running maximum (wave-uniform, base-2 domain) and this lane's sum of 2^(s - m)
 #pragma unroll
   for (int h = 0; h < G; ++h) {
@@ -229,12 +233,12 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
         const float a = fast_exp2(m_run[h] - m_new);
         m_run[h] = m_new;
         l_run[h] *= a;
-        al = vr == h ? a : al;
+        al = oh == h ? a : al;
       }
 #pragma unroll
-      for (int db = 0; db < NDB; ++db)
+      for (int db = 0; db < NOB; ++db)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) oacc[db][e] *= al;
+        for (int e = 0; e < 4; ++e) oacc[db][e] *= al;
     }
 #pragma unroll
     for (int h = 0; h < G; ++h) {
@@ -246,11 +250,11 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
     if (c > 0) fetch_block(kbase, c - 1, std::false_type{});  // K of the next chunk
     lds_order();
 #pragma unroll
-    for (int ks = 0; ks < kWave / 16; ++ks) {
+    for (int ks = 0; ks < kWave / 32; ++ks) {   // 32 keys per product
       u32x4 bop = u32x4{0, 0, 0, 0};
-      if (vr < G) bop = *reinterpret_cast<const u32x4*>(wts + vr * WS + 16 * ks + 8 * hf);
+      if (oh < G) bop = *reinterpret_cast<const u32x4*>(wts + oh * WS + 32 * ks + 8 * og);
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) oacc[db] = mfma32(load_a_trans_natural(tile, KS, 16 * ks, 32 * db), bop, oacc[db]);
+      for (int db = 0; db < NOB; ++db) oacc[db] = mfma16(load_a_trans16(tile, KS, 32 * ks, 16 * db), bop, oacc[db]);
     }
     lds_order();
   }
@@ -259,18 +263,15 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2))) void
 #pragma unroll
   for (int h = 0; h < G; ++h) {
     const float l = wave_sum(l_run[h]);
-    inv_l = vr == h ? (l > 0.f ? 1.f / l : 0.f) : inv_l;   // same guard as the reference's epilogue (:343-345)
+    inv_l = oh == h ? (l > 0.f ? 1.f / l : 0.f) : inv_l;   // same guard as the reference's epilogue (:343-345)
   }
-  if (vr < G) {
-    uint16_t* op = p.o + ((int64_t)(head0 + vr) * N + i) * D;
+  if (oh < G) {
+    uint16_t* op = p.o + ((int64_t)(head0 + oh) * N + i) * D;
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
-#pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const u32x2 w = {pack_elts(oacc[db][4 * g4] * inv_l, oacc[db][4 * g4 + 1] * inv_l),
-                         pack_elts(oacc[db][4 * g4 + 2] * inv_l, oacc[db][4 * g4 + 3] * inv_l)};
-        *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
-      }
+    for (int db = 0; db < NOB; ++db) {
+      const u32x2 w = {pack_elts(oacc[db][0] * inv_l, oacc[db][1] * inv_l), pack_elts(oacc[db][2] * inv_l, oacc[db][3] * inv_l)};
+      *reinterpret_cast<u32x2*>(op + db * 16 + 4 * og) = w;
+    }
   }
 }
 
