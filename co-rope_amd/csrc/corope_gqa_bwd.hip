@@ -217,11 +217,14 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
   // ---- right to left: gates, delta, raw scores, dS/ddelta, softmax statistics, dq sums --------------------------------
   // dq^h = c sum_j dS_j kt_j = c (sum_j e_j dP_j kt_j - Delta sum_j e_j kt_j) / L with e_j = exp(s_j - m): both sums are
   // accumulated on the matrix cores as rows 2h and 2h + 1 of W (virtual rows x keys) times Kt (keys x d), rescaled
-  // flash-attention style when the row's running maximum m moves.  dqa[db][4g + e] belongs to virtual row `vr` and
-  // column 32 db + 8 g + 4 hf + e.
-  f32x16 dqa[NDB];
+  // flash-attention style when the row's running maximum m moves.  The 2G <= 16 virtual rows are the columns of 16x16x32
+  // products (half the matrix-pipe time and accumulator registers of the 32x32x16 form, whose other 16 columns would be
+  // idle): dqa[db][e] belongs to virtual row `qv` = lane % 16 and column 16 db + 4 (lane / 16) + e.
+  constexpr int NQB = D / 16;
+  const int qv = lane % 16, qg = lane / 16;
+  f32x4 dqa[NQB];
 #pragma unroll
-  for (int db = 0; db < NDB; ++db) dqa[db] = f32x16{0};
+  for (int db = 0; db < NQB; ++db) dqa[db] = f32x4{0, 0, 0, 0};
   float m_run[G], l_run[G], pd_run[G];   // running maximum (wave-uniform); per lane: sum of exp(s - m), of exp(s - m) dP
 #pragma unroll
   for (int h = 0; h < G; ++h) {
@@ -389,12 +392,12 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
         m_run[h] = m_new;
         l_run[h] *= a;
         pd_run[h] *= a;
-        al = (vr / 2 == h && vr < 2 * G) ? a : al;
+        al = qv / 2 == h ? a : al;
       }
 #pragma unroll
-      for (int db = 0; db < NDB; ++db)
+      for (int db = 0; db < NQB; ++db)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) dqa[db][e] *= al;
+        for (int e = 0; e < 4; ++e) dqa[db][e] *= al;
     }
 #pragma unroll
     for (int h = 0; h < G; ++h) {
@@ -411,11 +414,11 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
     }
     lds_order();   // rotated keys and weights are in LDS
 #pragma unroll
-    for (int ks = 0; ks < kWave / 16; ++ks) {
+    for (int ks = 0; ks < kWave / 32; ++ks) {   // 32 keys per product
       u32x4 bop = u32x4{0, 0, 0, 0};
-      if (vr < 2 * G) bop = *reinterpret_cast<const u32x4*>(wts + vr * WS + 16 * ks + 8 * hf);
+      if (qv < 2 * G) bop = *reinterpret_cast<const u32x4*>(wts + qv * WS + 32 * ks + 8 * qg);
 #pragma unroll
-      for (int db = 0; db < NDB; ++db) dqa[db] = mfma32_f16(load_a_trans_natural(kt, KS, 16 * ks, 32 * db), bop, dqa[db]);
+      for (int db = 0; db < NQB; ++db) dqa[db] = mfma16_f16(load_a_trans16(kt, KS, 32 * ks, 16 * db), bop, dqa[db]);
     }
     lds_order();   // ... and consumed: the next chunk may overwrite them
   }
@@ -436,39 +439,33 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 5
     int my_exp = 0;
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-      my_inv = vr / 2 == h ? inv_l[h] : my_inv;
-      my_dsum = vr / 2 == h ? dsum[h] - dref[h] : my_dsum;
-      my_exp = vr / 2 == h ? w_exp[h] : my_exp;
+      my_inv = qv / 2 == h ? inv_l[h] : my_inv;
+      my_dsum = qv / 2 == h ? dsum[h] - dref[h] : my_dsum;
+      my_exp = qv / 2 == h ? w_exp[h] : my_exp;
     }
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
+    for (int db = 0; db < NQB; ++db)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
+      for (int e = 0; e < 4; ++e) {
         const float other = __shfl_xor(dqa[db][e], 1);
-        if (vr < 2 * G) dqa[db][e] = (ldexpf(dqa[db][e], my_exp) - my_dsum * other) * my_inv;
+        if (qv < 2 * G) dqa[db][e] = (ldexpf(dqa[db][e], my_exp) - my_dsum * other) * my_inv;
       }
   }
   // dq of the heads 1..G-1 is final; the leader's still lacks the gate path W K, which a separate plain matrix product
   // adds (corope_bwd_dq_leader_kernel): its row goes to the workspace in fp32, unscaled
-  if (vr < 2 * G && vr % 2 == 0) {
-    if (vr == 0) {
+  if (qv < 2 * G && qv % 2 == 0) {
+    if (qv == 0) {
       float* op = ws.dql(g, N, D) + (int64_t)i * D;
 #pragma unroll
-      for (int db = 0; db < NDB; ++db)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4)
-          *reinterpret_cast<f32x4*>(op + db * 32 + 8 * g4 + 4 * hf) =
-              f32x4{dqa[db][4 * g4], dqa[db][4 * g4 + 1], dqa[db][4 * g4 + 2], dqa[db][4 * g4 + 3]};
+      for (int db = 0; db < NQB; ++db) *reinterpret_cast<f32x4*>(op + db * 16 + 4 * qg) = dqa[db];
     } else {
-      uint16_t* op = p.dq + ((int64_t)(head0 + vr / 2) * N + i) * D;
+      uint16_t* op = p.dq + ((int64_t)(head0 + qv / 2) * N + i) * D;
 #pragma unroll
-      for (int db = 0; db < NDB; ++db)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          const u32x2 w = {pack_elts(dqa[db][4 * g4] * p.sm_scale, dqa[db][4 * g4 + 1] * p.sm_scale),
-                           pack_elts(dqa[db][4 * g4 + 2] * p.sm_scale, dqa[db][4 * g4 + 3] * p.sm_scale)};
-          *reinterpret_cast<u32x2*>(op + db * 32 + 8 * g4 + 4 * hf) = w;
-        }
+      for (int db = 0; db < NQB; ++db) {
+        const u32x2 w = {pack_elts(dqa[db][0] * p.sm_scale, dqa[db][1] * p.sm_scale),
+                         pack_elts(dqa[db][2] * p.sm_scale, dqa[db][3] * p.sm_scale)};
+        *reinterpret_cast<u32x2*>(op + db * 16 + 4 * qg) = w;
+      }
     }
   }
 
