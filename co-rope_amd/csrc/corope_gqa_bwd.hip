@@ -160,7 +160,7 @@ __global__ __launch_bounds__(4 * kWave) void corope_bwd_rowdot_kernel(const uint
 // the rotated key then runs on the matrix cores: the raw scores q^h . kt and their derivatives with respect to delta
 // (rows [-w q2, w q1] . kt) as one (2G x D) x (D x 64 keys) product, and the dq sums as (weights x keys) x (keys x D).
 template <int D, int G>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(D * G > 512 ? 1 : 2, D * G > 512 ? 1 : 2))) void corope_bwd_scores_kernel(CoropeBwdParams p, CoropeBwdWs ws, CoropeBwdFreqs fr) {
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void corope_bwd_scores_kernel(CoropeBwdParams p, CoropeBwdWs ws, CoropeBwdFreqs fr) {
   constexpr int HALF = D / 2;
   constexpr int KS = D + 8, WS = kWave + 8, NVR = 2 * G, NDB = D / 32;
   constexpr int NI = 4 * ((2 * G - 1) / 8 + 1);                       // accumulator registers that hold rows < 2G
