@@ -235,3 +235,25 @@ def test_corope_backward_parity_fp16(pkg, B, Hq, Hkv, N, D):
     print(f"  O max-abs {(o.float().cpu() - ro).abs().max():.3e}", flush=True)
     assert (o.float().cpu() - ro).abs().max() <= TOL
     _compare([t.grad.float().cpu() for t in (qg, kg, vg)], _oracle_grads(q, k, v, d_o, scale, 10000.0), Hq // Hkv)
+
+
+@pytest.mark.parametrize("kexp", [-8, 5])
+def test_corope_backward_fp16_scaled_upstream_gradient(pkg, kexp):
+    """fp16 tensors with an upstream gradient of 2^-8 and 2^5 times unit size (fp16's own range leaves room for little
+    more): the gradients stay finite and match the oracle at the bar scaled by the same factor."""
+    B, Hq, Hkv, N, D = 1, 4, 2, 130, 64
+    f = 2.0 ** kexp
+    q, k, v, d_o = (_f16_round(t) for t in _inputs(B, Hq, Hkv, N, D, seed=11))
+    d_o = _f16_round(d_o * f)
+    scale = 1 / math.sqrt(D)
+    dev = torch.device("cuda:0")
+    qg, kg, vg = (t.to(dev, torch.float16).requires_grad_(True) for t in (q, k, v))
+    pkg.corope_attention(qg, kg, vg, True, scale, 10000.0).backward(d_o.to(dev, torch.float16))
+    torch.cuda.synchronize()
+    ref = _oracle_grads(q, k, v, d_o, scale, 10000.0)
+    G = Hq // Hkv
+    for name, t, b, bar in zip(("dQ", "dK", "dV"), (qg, kg, vg), ref, (TOL, TOL * math.sqrt(G), TOL * math.sqrt(G))):
+        a = t.grad.float().cpu()
+        err = (a - b).abs().max()
+        print(f"  {name} at dO x 2^{kexp}: max-abs {err:.3e} (bar {bar * f:.3e}, max |ref| {b.abs().max():.3e})", flush=True)
+        assert torch.isfinite(a).all() and err <= bar * f, name
