@@ -31,10 +31,10 @@ MFMA_RATE = os.path.join(LIBDIR, "mfma_rate")
 F16_SOURCES = ["rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip",
                "corope_gqa_bwd.hip"]
 
-SOURCES = ["abi.hip", "rope_freqs.hip", "rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_fwd_pipe.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip", "corope_gqa_bwd.hip"]
+SOURCES = ["abi.hip", "rope_freqs.hip", "rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_fwd_pipe.hip", "rope_attn_fwd_pipe64.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip", "corope_gqa_bwd.hip"]
 
 # sources with asm-issued matrix-core instructions: their generated assembly is checked (check_isa.py) in every variant
-ISA_CHECKED = {"rope_attn_fwd_pipe.hip", "rope_attn_bwd.hip"}
+ISA_CHECKED = {"rope_attn_fwd_pipe.hip", "rope_attn_fwd_pipe64.hip", "rope_attn_bwd.hip"}
 
 # -packed-fp32-ops is switched off: packed fp32 VALU forms are not used by these kernels.
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-value",

@@ -4,6 +4,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 
 #include "kernels.hpp"
 
@@ -13,7 +14,10 @@ namespace corope { uint64_t* g_trace_buf = nullptr; }
 extern "C" void corope_debug_trace(void* buf) { corope::g_trace_buf = static_cast<uint64_t*>(buf); }
 #endif
 
-namespace corope { std::atomic<int> g_tile_rows{0}; }
+namespace corope {
+std::atomic<int> g_tile_rows{0};
+std::atomic<int> g_fwd_wave_rows{[] { const char* e = getenv("COROPE_AMD_FWD_WAVE_ROWS"); return e ? atoi(e) : 0; }()};
+}
 
 namespace {
 

@@ -74,6 +74,9 @@ inline int device_cu_count() {
 // number fewer than the compute units takes the 128-row form, which doubles the items and halves the time the heaviest
 // of them runs; `g_tile_rows` (0 = by shape, 128, 256) overrides the rule for tests and tuning.
 extern std::atomic<int> g_tile_rows;
+// Query rows per wave of the two-launch forward at D = 128 with 256-row items: 32 (8 waves, two per SIMD) or 64 (4 waves,
+// one per SIMD, every LDS fragment feeding two MFMAs); 0 = the default.
+extern std::atomic<int> g_fwd_wave_rows;
 inline bool use_small_tiles(int n_rows, int slabs) {
   const int forced = g_tile_rows.load(std::memory_order_relaxed);
   if (forced == 128) return true;
@@ -175,6 +178,8 @@ using namespace corope;
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
                               float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale = 1.f);
 hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream);  // needs k_rot
+// the same with 64 query rows per wave, one wave per SIMD (D = 128)
+hipError_t launch_rope_attn_fwd_prerotated_rows64(const FwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_preprocess(const BwdParams& p, int D, hipStream_t stream);
 hipError_t launch_bwd_dv(const BwdParams& p, int D, bool causal, hipStream_t stream);

@@ -472,6 +472,8 @@ static hipError_t launch_pipe_cfg(const FwdParams& p, hipStream_t stream) {
 
 hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream) {
   if (D != 64 && D != 128) return hipErrorInvalidValue;
+  if (D == 128 && !use_small_tiles(p.N, p.BH) && g_fwd_wave_rows.load(std::memory_order_relaxed) == 64)
+    return launch_rope_attn_fwd_prerotated_rows64(p, D, causal, stream);
   if (D == 128) return causal ? launch_pipe_cfg<128, true>(p, stream) : launch_pipe_cfg<128, false>(p, stream);
   return causal ? launch_pipe_cfg<64, true>(p, stream) : launch_pipe_cfg<64, false>(p, stream);
 }
