@@ -8,7 +8,7 @@ rotation FLOPs not counted), the roofline of the dominant kernel from per-launch
 oracle timed on the host cores as a baseline.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--no-cpu-baseline]
-                    [--parity] [--data normal|sink] [--phase-trace] [--sweep [--lanes]]
+                    [--parity | --no-parity] [--data normal|sink] [--phase-trace] [--sweep [--lanes] [--flush]]
 
 (c3 is the metric shape and the default; c2/c4 are the other RoPE-attention shapes; c5 is the Co-RoPE GQA forward,
 with its backward timed beside it.)  --parity adds per-tensor errors against the CPU oracle to the line (outside the
@@ -107,9 +107,10 @@ def sample_rows(N, n, torch, seed=1):
     return torch.unique(torch.cat([r, torch.tensor([0, 1, 63, 64, N // 2, N - 2, N - 1]).clamp(0, N - 1)]))
 
 
-def rope_parity(pkg, cfg_name, q, k, v, do, cos, sin, scale, fwd_only, torch):
+def rope_parity(pkg, cfg_name, q, k, v, do, cos, sin, scale, fwd_only, torch, quick=False):
     """Per-tensor errors of the HIP path against the fp32 CPU oracle on the same bf16-rounded inputs: O (and the row
-    statistic) on sampled rows of every head, dQ / dK / dV on whole heads (all of them at C2, 8 at C3)."""
+    statistic) on sampled rows of every head, dQ / dK / dV on whole heads (all of them at C2, 8 at C3).  ``quick``: the
+    sample every run of the benchmark carries in its line (32 rows of every head, 2 whole heads: seconds of host time)."""
     from oracle import rope_attn_oracle as O
     B, H, N, D = q.shape
     dev = torch.device("cuda:0")
@@ -119,14 +120,16 @@ def rope_parity(pkg, cfg_name, q, k, v, do, cos, sin, scale, fwd_only, torch):
         o.backward(do.to(dev, torch.bfloat16))
     torch.cuda.synchronize()
     o = o.detach().float().cpu()
-    rows = sample_rows(N, 128 if N <= 8192 else 48, torch)
+    rows = sample_rows(N, 25 if quick else (128 if N <= 8192 else 48), torch)
     c, s = cos.float().cpu(), sin.float().cpu()
     ro, _ = O.rope_attn_forward_blocked(q, k, v, True, scale, c, s, rows=rows)
     out = {"bar": "max-abs <= 2e-2 against the fp32 oracle (one bf16 ulp of the reference value where that is larger)",
            "O": dict(err_stats(o[:, :, rows], ro, torch), sample=f"{rows.numel()} rows x {B * H} heads")}
     if not fwd_only:
         heads = [(b, h) for b in range(B) for h in range(H)]
-        if len(heads) > 32:
+        if quick:
+            heads = [heads[len(heads) // 3], heads[-1]]
+        elif len(heads) > 32:
             heads = heads[:: len(heads) // 8][:8]
         acc = {n: ([], []) for n in ("dQ", "dK", "dV")}
         for (b, h) in heads:
@@ -215,36 +218,90 @@ SWEEP = [(4, 8, 512, 64, "Small-512"), (4, 8, 1024, 64, "Small-1K"), (2, 8, 2048
          (1, 16, 32768, 128, "Long-32K"), (1, 8, 65536, 128, "Long-64K"), (1, 4, 131072, 128, "Long-128K")]
 
 
+def sweep_protocol(N):
+    """(warm-up, measurement) in milliseconds for a sequence length: the reference harness's table
+    (fused-rope/bench_compare.py:390-401), whose timer takes both as durations, not counts."""
+    if N >= 262144:
+        return 20, 30
+    if N >= 131072:
+        return 25, 50
+    if N >= 65536:
+        return 50, 100
+    if N >= 32768:
+        return 50, 150
+    if N >= 8192:
+        return 100, 200
+    return 100, 300
+
+
+def timed_reps(fn, N, torch, flush_buf=None):
+    """(median, min, max) ms of fn over repetitions timed one by one with HIP events, as the reference harness's timer does
+    (fused-rope/bench_compare.py:30-58): the duration of one call is estimated from 5 calls, then warm-up and measurement
+    run for the durations sweep_protocol gives (the warm-up never shorter than SETTLE_SECONDS of sustained load, so that
+    every shape and lane is timed at settled clocks, like the headline line).  flush_buf: a buffer larger than every cache,
+    overwritten by a fill kernel before each timed call (that timer's cold-cache protocol); None: calls back to back."""
+    warm_ms, rep_ms = sweep_protocol(N)
+    fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    est = max(e0.elapsed_time(e1) / 5, 1e-3)
+    n_warm = max(1, int(max(warm_ms, SETTLE_SECONDS * 1e3) / est))
+    n_rep = max(5, min(1000, int(rep_ms / est)))
+    for _ in range(n_warm):
+        fn()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_rep)]
+    for a, b in evs:
+        if flush_buf is not None:
+            flush_buf.zero_()
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    t = sorted(a.elapsed_time(b) for a, b in evs)
+    return statistics.median(t), t[0], t[-1]
+
+
 def bench_sweep(args):
-    """Forward and backward-only times (median of HIP-event timings, backward with the forward graph retained, as the
-    reference's harness does) for the reference's 19 shapes; one JSON line per shape."""
+    """Forward and backward-only times (HIP-event timings, backward with the forward graph retained, as the reference's
+    harness does) for the reference's 19 shapes; one JSON line per shape: median / min / max of back-to-back calls at
+    settled clocks and, with --flush, of calls that each start on flushed caches."""
     import torch
     pkg = importlib.import_module("corope_amd")
     dev = torch.device("cuda:0")
+    flush_buf = torch.empty(512 << 20, dtype=torch.uint8, device=dev) if args.flush else None
     for (B, H, N, D, name) in SWEEP:
         g = torch.Generator().manual_seed(0)
         q, k, v, do = (torch.randn(B, H, N, D, generator=g).to(dev, torch.bfloat16) for _ in range(4))
         cos, sin = pkg.rope_freqs_device(D, N, 10000.0, device=dev)
         q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
-        reps = 30 if N <= 16384 else 8
+        stats = {}
 
-        def timed(fn):
-            for _ in range(3):
-                fn()
-            evs = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
-            evs[0].record()
-            for i in range(reps):
-                fn()
-                evs[i + 1].record()
-            torch.cuda.synchronize()
-            return statistics.median(evs[i].elapsed_time(evs[i + 1]) for i in range(reps))
+        def timed(fn, key=None):
+            med, lo, hi = timed_reps(fn, N, torch)
+            if key is not None:
+                stats[key + "_min_ms"], stats[key + "_max_ms"] = round(lo, 4), round(hi, 4)
+                if flush_buf is not None:
+                    fm, fl, fh = timed_reps(fn, N, torch, flush_buf)
+                    stats[key + "_flushed_ms"] = round(fm, 4)
+                    stats[key + "_flushed_min_ms"], stats[key + "_flushed_max_ms"] = round(fl, 4), round(fh, 4)
+            return med
 
-        f_ms = timed(lambda: pkg.attention(q, k, v, True, 0.5, cos, sin))
+        f_ms = timed(lambda: pkg.attention(q, k, v, True, 0.5, cos, sin), "fwd")
         o = pkg.attention(q, k, v, True, 0.5, cos, sin)
-        b_ms = timed(lambda: o.backward(do, retain_graph=True))
+
+        def clear_grads():   # otherwise every call after the first also runs three accumulate-into-.grad kernels
+            q.grad = k.grad = v.grad = None
+
+        b_ms = timed(lambda: (clear_grads(), o.backward(do, retain_graph=True)), "bwd")
         ff, fb = attention_flops(B, H, N, D, "fwd"), attention_flops(B, H, N, D, "bwd")
         row = {"config": name, "B": B, "H": H, "N": N, "D": D, "fwd_ms": round(f_ms, 4),
                "fwd_tflops": round(ff / f_ms * 1e-9, 1), "bwd_ms": round(b_ms, 4), "bwd_tflops": round(fb / b_ms * 1e-9, 1)}
+        row.update(stats)
         if args.lanes:
             # the reference harness's comparison lanes (fused-rope/bench_compare.py:98-260), on this GPU:
             #   unfused = a separate rotation pass over q and k, then the same attention kernels with identity tables
@@ -257,7 +314,11 @@ def bench_sweep(args):
             kr = pkg.rope_rotate(kd, cos, sin).requires_grad_(True)
             uf_ms = rot_ms + timed(lambda: pkg.attention(qr, kr, v, True, 0.5, one, zero))
             ou = pkg.attention(qr, kr, v, True, 0.5, one, zero)
-            ub_ms = rot_ms + timed(lambda: ou.backward(do, retain_graph=True))
+
+            def clear_rot_grads():
+                qr.grad = kr.grad = v.grad = None
+
+            ub_ms = rot_ms + timed(lambda: (clear_rot_grads(), ou.backward(do, retain_graph=True)))
             row.update({"unfused_fwd_ms": round(uf_ms, 4), "unfused_bwd_ms": round(ub_ms, 4),
                         "fwd_speedup_vs_unfused": round(uf_ms / f_ms, 3), "bwd_speedup_vs_unfused": round(ub_ms / b_ms, 3),
                         "calc_sim_vs_unfused": round(calc_sim(o.detach(), ou.detach()), 8)})
@@ -265,7 +326,7 @@ def bench_sweep(args):
                 sdpa = torch.nn.functional.scaled_dot_product_attention
                 sf_ms = rot_ms + timed(lambda: sdpa(qr, kr, v, is_causal=True, scale=0.5))
                 osd = sdpa(qr, kr, v, is_causal=True, scale=0.5)
-                sb_ms = rot_ms + timed(lambda: osd.backward(do, retain_graph=True))
+                sb_ms = rot_ms + timed(lambda: (clear_rot_grads(), osd.backward(do, retain_graph=True)))
                 row.update({"sdpa_fwd_ms": round(sf_ms, 4), "sdpa_bwd_ms": round(sb_ms, 4),
                             "fwd_speedup_vs_sdpa": round(sf_ms / f_ms, 3), "bwd_speedup_vs_sdpa": round(sb_ms / b_ms, 3)})
                 del osd
@@ -510,8 +571,11 @@ def main():
                     help="time the reference harness's 19 shapes instead (one JSON line per shape)")
     ap.add_argument("--lanes", action="store_true",
                     help="with --sweep: also time the unfused lanes (separate rotation + identity-table attention, PyTorch SDPA)")
+    ap.add_argument("--flush", action="store_true",
+                    help="with --sweep: also time every call on flushed caches (a 512 MiB buffer overwritten before each call)")
     ap.add_argument("--parity", action="store_true",
-                    help="after the timed region, add per-tensor errors against the CPU oracle to the line")
+                    help="the larger parity sample (the line always carries per-tensor errors against the CPU oracle on a small one)")
+    ap.add_argument("--no-parity", action="store_true", help="leave the per-tensor errors out of the line")
     ap.add_argument("--data", default="normal", choices=["normal", "sink"],
                     help="synthetic inputs: N(0,1), or attention-sink-like keys (see make_inputs)")
     ap.add_argument("--phase-trace", action="store_true",
@@ -656,7 +720,7 @@ def main():
     fwd_ms = avg["rope_attn_fwd"] + avg.get("rope_rotate_k", 0.0)
     fwd_tf = alg["rope_attn_fwd"] / (fwd_ms * 1e-3) * 1e-12
     out = {
-        "metric": "RoPE-attn fwd+bwd TFLOPS & % bf16 MFMA peak, B2 H32 N4096 D128 causal",
+        "metric": f"RoPE-attn {'fwd' if fwd_only else 'fwd+bwd'} TFLOPS & % bf16 MFMA peak, B{B} H{H} N{N} D{D} causal",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "settle_steps": settle_steps,
@@ -691,8 +755,10 @@ def main():
         out["fwd_ms_by_data"] = {args.data: round(forward_ms(pkg, q.detach(), k.detach(), v.detach(), cos, sin, scale, torch), 4),
                                  "normal": round(forward_ms(pkg, *(t.to(dev, torch.bfloat16) for t in (hq, hk, hv)), cos, sin,
                                                             scale, torch), 4)}
-    if args.parity:
-        out["parity"] = rope_parity(pkg, args.config, host[0], host[1], host[2], host[3], cos, sin, scale, fwd_only, torch)
+    # per-tensor errors against the CPU oracle, outside the timed region (--parity: the larger sample; --no-parity: none)
+    if not args.no_parity:
+        out["parity"] = rope_parity(pkg, args.config, host[0], host[1], host[2], host[3], cos, sin, scale, fwd_only, torch,
+                                    quick=not args.parity)
     out["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline()
     print(json.dumps(out))
 

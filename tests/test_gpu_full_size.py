@@ -123,7 +123,9 @@ def test_corope_long_hot_rows(pkg):
 
 def test_c5_corope_backward(pkg):
     """B2 Hq32 Hkv8 N4096 D128 Co-RoPE backward: dQ of sampled rows against autograd through the row-sampled oracle
-    (a query row's output depends on no other query row), and two size-independent identities for dK and dV:
+    (a query row's output depends on no other query row), dK and dV of one group's last 1024 keys against autograd through
+    the oracle over the query rows that see them (rows before key j contribute nothing to key j: causal, and the mileage
+    of a row sums gates of keys up to the row itself), and two size-independent identities for dK and dV as a whole:
     sum_j dv_j = sum_{h,i} dO^h_i per group (softmax rows sum to one), and sum q.dq = sum k.dk per group (scores and
     gates depend on q and k only through products q.k, so scaling q up and k down by the same factor changes nothing)."""
     import importlib
@@ -148,6 +150,20 @@ def test_c5_corope_backward(pkg):
     print(f"  C5 dQ max-abs {err.max():.3e} mean-abs {err.mean():.3e} on {rows.numel()} rows x {B * Hq} heads "
           f"(max |ref| {ref_dq[:, :, rows].abs().max():.3f})", flush=True)
     assert err.max() <= TOL
+
+    # one whole group's last keys: every query row that sees them, 64 rows at a time
+    b, kv, first = B - 1, Hkv // 2, N - 1024
+    qs, dos = q[b:b + 1, kv * G:(kv + 1) * G], d_o[b:b + 1, kv * G:(kv + 1) * G]
+    kx, vx = (t[b:b + 1, kv:kv + 1].clone().requires_grad_(True) for t in (k, v))
+    for r0 in range(first, N, 64):
+        blk = C.corope_gqa_forward_rows(qs[:, :, :r0 + 64], kx[:, :, :r0 + 64], vx[:, :, :r0 + 64], True, scale, 10000.0,
+                                        torch.arange(r0, r0 + 64), torch.float32, row_block=64)
+        blk.backward(dos[:, :, r0:r0 + 64])
+    for name, got, ref in (("dK", dk, kx.grad), ("dV", dv, vx.grad)):
+        err = (got[b, kv, first:] - ref[0, 0, first:]).abs()
+        print(f"  C5 {name} max-abs {err.max():.3e} mean-abs {err.mean():.3e} on the last {N - first} keys of group "
+              f"(batch {b}, kv head {kv}) (max |ref| {ref[0, 0, first:].abs().max():.3f})", flush=True)
+        assert err.max() <= TOL * math.sqrt(G), name     # sums over the group's G heads
 
     ulp = 2.0 ** -9
     dv_sum, do_sum = dv.double().sum(2), d_o.double().view(B, Hkv, G, N, D).sum((2, 3))
