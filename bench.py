@@ -9,6 +9,7 @@ oracle timed on the host cores as a baseline.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--no-cpu-baseline]
                     [--parity | --no-parity] [--data normal|sink] [--phase-trace] [--sweep [--lanes] [--flush]]
+                    [--mfma-rate]
 
 (c3 is the metric shape and the default; c2/c4 are the other RoPE-attention shapes; c5 is the Co-RoPE GQA forward,
 with its backward timed beside it.)  --parity adds per-tensor errors against the CPU oracle to the line (outside the
@@ -465,13 +466,10 @@ def bench_phase_trace(args):
     import numpy as np
     import torch
     pkg = importlib.import_module("corope_amd")
-    path = os.path.join(os.path.dirname(pkg._lib.LIB_PATH), "libcorope_amd_trace.so")
-    if not os.path.exists(path):
-        sys.exit(f"bench.py: {path} not found (python co-rope_amd/build.py makes it)")
-    lib = ctypes.CDLL(path)
-    for n, (r, a) in pkg._lib.SIGNATURES.items():
-        getattr(lib, n).restype, getattr(lib, n).argtypes = r, a
-    lib.corope_debug_trace.argtypes, lib.corope_debug_trace.restype = [ctypes.c_void_p], None
+    try:
+        lib = pkg._lib.load_trace()
+    except pkg._lib.CoRopeLibraryError as e:
+        sys.exit(f"bench.py: {e}")
     dev = torch.device("cuda:0")
     cfg = CONFIGS[args.config]
     B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
@@ -582,6 +580,9 @@ def main():
                     help="split the attention kernels of the chosen RoPE config into phases (trace build of the library)")
     ap.add_argument("--trace-dump", default=None, metavar="DIR",
                     help="with --phase-trace: also save the raw stamps of every kernel (one row of 16 per item) as .npy files there")
+    ap.add_argument("--mfma-rate", action="store_true",
+                    help="build (if stale) and run bench_mfma_rate.hip: what the matrix pipes sustain on this machine, by operand "
+                         "source, instruction shape and accompanying vector work (markdown tables)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
@@ -589,6 +590,12 @@ def main():
         sys.exit("bench.py: this build runs on ONE GPU (every (batch, head) is independent, so the path would shard over "
                  "batch x heads without any exchange); run it with --gpus 1")
 
+    if args.mfma_rate:
+        import subprocess
+        src, exe = os.path.join(ROOT, "bench_mfma_rate.hip"), os.path.join(ROOT, "bench_mfma_rate")
+        if not os.path.exists(exe) or os.path.getmtime(exe) < os.path.getmtime(src):
+            importlib.import_module("corope_amd.build").build_program(src, exe)
+        return sys.exit(subprocess.run([exe]).returncode)
     if args.copy_calibration:
         import torch
         a = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda:0").normal_()

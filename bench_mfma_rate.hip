@@ -1,0 +1,477 @@
+// Measurement program beside bench.py (not part of the library): what the gfx950 matrix pipes sustain on this machine,
+// and what a wave can do beside them.  `python bench.py --mfma-rate` builds it (hipcc) and runs it.  Four tables:
+//
+// 1. Loops of nothing but 32x32x16 bf16 MFMAs on all 256 CUs (8 waves each), with the A operand either held in registers
+//    or fetched from LDS as a fresh 1 KB fragment that feeds R MFMAs, on all-zero operands and on N(0,1) operands rounded
+//    to bf16.  Every run also measures the shader clock it ran at (core-clock counter against the constant 100 MHz
+//    counter), so the table shows how far the power management lowers the clock under the switching activity of real
+//    data: the figure to read the attention kernels' fractions of the published 2.5 PFLOP/s against.
+// 2. The same kind of loop on N(0,1) data by instruction shape (32x32x16 against 16x16x32), number of accumulators and
+//    number of distinct operand sets, at one and at two waves per SIMD.
+// 3. How many independent vector instructions of the SAME wave hide under one MFMA (one wave per SIMD, all-zero operands,
+//    so at the full clock), with the accumulator and / or the B operand in the accumulation half of the register file.
+// 4. The steady-state tile loop of the forward in its form with 64 query rows per wave, one wave per SIMD
+//    (csrc/rope_attn_fwd_pipe64.hip) without any data-dependent control flow, feature by feature: MFMAs alone, + LDS
+//    operand reads, + softmax, + barrier, + staging of the next K/V tile.
+#include "co-rope_amd/csrc/common.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+using namespace corope;
+
+constexpr int kSrcWords = 65536;   // 16-byte words of operand data
+
+template <int R, bool FROM_LDS>
+__global__ __launch_bounds__(512) void mfma_loop(const u32x4* src, float* out, unsigned long long* clocks, int iters) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  u32x4* tile = reinterpret_cast<u32x4*>(smem);   // 64 KB: 4096 x 16 B
+  for (int e = threadIdx.x; e < 4096; e += 512) tile[e] = src[(blockIdx.x * 4096 + e) % kSrcWords];
+  __syncthreads();
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  u32x4 b[R];
+  f32x16 acc[R];
+  for (int r = 0; r < R; ++r) {
+    b[r] = src[(threadIdx.x * 7 + r * 13) % kSrcWords];
+    acc[r] = f32x16{0};
+  }
+  u32x4 areg = src[(threadIdx.x * 3) % kSrcWords];
+  const unsigned long long c0 = __builtin_readcyclecounter(), t0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int f = 0; f < 16; ++f) {
+      u32x4 a = areg;
+      if (FROM_LDS) a = tile[((wave * 16 + f + it) % 64) * 64 + lane];   // 1 KB per wave per fragment, conflict-free
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b[r]),
+                                                         acc[r], 0, 0, 0);
+    }
+  }
+  float s = 0;
+  for (int r = 0; r < R; ++r)
+    for (int i = 0; i < 16; ++i) s += acc[r][i];
+  out[blockIdx.x * 512 + threadIdx.x] = s;
+  if (threadIdx.x == 0) {
+    clocks[2 * blockIdx.x] = __builtin_readcyclecounter() - c0;
+    clocks[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - t0;
+  }
+}
+
+struct Result {
+  double tflops, ghz;
+};
+
+template <int R, bool L>
+Result run(const u32x4* src, float* out, unsigned long long* clocks, int iters) {
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(mfma_loop<R, L>), hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+  hipEvent_t e0, e1;
+  (void)hipEventCreate(&e0);
+  (void)hipEventCreate(&e1);
+  for (int w = 0; w < 3; ++w) hipLaunchKernelGGL((mfma_loop<R, L>), dim3(256), dim3(512), 65536, 0, src, out, clocks, iters);
+  (void)hipEventRecord(e0);
+  for (int w = 0; w < 10; ++w) hipLaunchKernelGGL((mfma_loop<R, L>), dim3(256), dim3(512), 65536, 0, src, out, clocks, iters);
+  (void)hipEventRecord(e1);
+  (void)hipEventSynchronize(e1);
+  float ms = 0;
+  (void)hipEventElapsedTime(&ms, e0, e1);
+  ms /= 10;
+  std::vector<unsigned long long> h(512);
+  (void)hipMemcpy(h.data(), clocks, h.size() * 8, hipMemcpyDeviceToHost);
+  double ghz = 0;
+  for (int i = 0; i < 256; ++i) ghz += (double)h[2 * i] / ((double)h[2 * i + 1] * 10.0) / 256;   // cycles per ns
+  const double flop = 256.0 * 8 * iters * 16 * R * 32768.0;
+  return {flop / (ms * 1e-3) * 1e-12, ghz};
+}
+
+static unsigned gauss_bf16_bits() {   // N(0,1) rounded to bf16 (Box-Muller)
+  float u1 = (rand() + 1.0f) / ((float)RAND_MAX + 2.0f), u2 = rand() / (float)RAND_MAX;
+  float g = sqrtf(-2.f * logf(u1)) * cosf(6.2831853f * u2);
+  unsigned bits;
+  memcpy(&bits, &g, 4);
+  return (bits + 0x8000u) >> 16;
+}
+
+int table1() {
+  u32x4* src;
+  float* out;
+  unsigned long long* clocks;
+  if (hipMalloc(&src, kSrcWords * 16) != hipSuccess || hipMalloc(&out, 256 * 512 * 4) != hipSuccess ||
+      hipMalloc(&clocks, 512 * 8) != hipSuccess) {
+    fprintf(stderr, "mfma_rate: no HIP device\n");
+    return 1;
+  }
+  const int iters = 2000;
+  printf("## 1. MFMA-only loops, 256 CUs x 8 waves\n\n| operands | A operand | MFMAs per fragment | TFLOP/s | of 2500 | shader clock GHz |\n|---|---|---|---|---|---|\n");
+  for (int gaussian = 0; gaussian < 2; ++gaussian) {
+    std::vector<unsigned> h(kSrcWords * 4, 0u);
+    srand(1);
+    auto gauss_bf16 = [&]() {   // N(0,1) rounded to bf16 (Box-Muller)
+      float u1 = (rand() + 1.0f) / ((float)RAND_MAX + 2.0f), u2 = rand() / (float)RAND_MAX;
+      float g = sqrtf(-2.f * logf(u1)) * cosf(6.2831853f * u2);
+      unsigned bits;
+      memcpy(&bits, &g, 4);
+      return (bits + 0x8000u) >> 16;
+    };
+    if (gaussian)
+      for (auto& x : h) x = gauss_bf16() | (gauss_bf16() << 16);
+    (void)hipMemcpy(src, h.data(), h.size() * 4, hipMemcpyHostToDevice);
+    for (int i = 0; i < 3; ++i) run<2, true>(src, out, clocks, iters);   // a long warm-up so that the clocks settle
+    const char* name = gaussian ? "N(0,1) bf16" : "all zero";
+    Result r;
+    r = run<1, true>(src, out, clocks, iters);
+    printf("| %s | LDS | 1 | %.0f | %.3f | %.2f |\n", name, r.tflops, r.tflops / 2500, r.ghz);
+    r = run<2, true>(src, out, clocks, iters);
+    printf("| %s | LDS | 2 | %.0f | %.3f | %.2f |\n", name, r.tflops, r.tflops / 2500, r.ghz);
+    r = run<4, true>(src, out, clocks, iters);
+    printf("| %s | LDS | 4 | %.0f | %.3f | %.2f |\n", name, r.tflops, r.tflops / 2500, r.ghz);
+    r = run<2, false>(src, out, clocks, iters);
+    printf("| %s | registers | - (2 accumulators) | %.0f | %.3f | %.2f |\n", name, r.tflops, r.tflops / 2500, r.ghz);
+    r = run<4, false>(src, out, clocks, iters);
+    printf("| %s | registers | - (4 accumulators) | %.0f | %.3f | %.2f |\n", name, r.tflops, r.tflops / 2500, r.ghz);
+  }
+  return hipGetLastError() == hipSuccess ? 0 : 1;
+}
+
+// ---- 2. instruction shape, accumulators, operand sets (N(0,1) data, operands in registers) -------------------------------
+namespace t2 {
+template <int SHAPE, int NACC, int NOPS>
+__global__ __launch_bounds__(512) void loop(const u32x4* src, float* out, int iters) {
+  u32x4 a[NOPS], b[NOPS];
+  for (int i = 0; i < NOPS; ++i) {
+    a[i] = src[(threadIdx.x * 7 + i * 131) % kSrcWords];
+    b[i] = src[(threadIdx.x * 3 + i * 977 + 5) % kSrcWords];
+  }
+  f32x16 acc32[NACC];
+  f32x4 acc16[NACC * 2];
+  for (int i = 0; i < NACC; ++i) acc32[i] = f32x16{0};
+  for (int i = 0; i < NACC * 2; ++i) acc16[i] = f32x4{0};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      if (SHAPE == 32) {
+        acc32[u % NACC] = mfma32(a[u % NOPS], b[(u / 2) % NOPS], acc32[u % NACC]);
+      } else {   // two 16x16x32 products = the FLOPs of one 32x32x16
+        acc16[(2 * u) % (2 * NACC)] = mfma16(a[u % NOPS], b[(u / 2) % NOPS], acc16[(2 * u) % (2 * NACC)]);
+        acc16[(2 * u + 1) % (2 * NACC)] = mfma16(b[u % NOPS], a[(u / 2) % NOPS], acc16[(2 * u + 1) % (2 * NACC)]);
+      }
+    }
+  }
+  float s = 0;
+  for (int n = 0; n < NACC; ++n)
+    for (int i = 0; i < 16; ++i) s += acc32[n][i];
+  for (int n = 0; n < 2 * NACC; ++n)
+    for (int i = 0; i < 4; ++i) s += acc16[n][i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+template <int SHAPE, int NACC, int NOPS>
+void run(int threads, const u32x4* src, float* out) {
+  const int iters = 3000;
+  for (int w = 0; w < 4; ++w) hipLaunchKernelGGL((loop<SHAPE, NACC, NOPS>), dim3(256), dim3(threads), 0, 0, src, out, iters);
+  hipEvent_t e0, e1;
+  (void)hipEventCreate(&e0);
+  (void)hipEventCreate(&e1);
+  (void)hipEventRecord(e0);
+  for (int w = 0; w < 10; ++w) hipLaunchKernelGGL((loop<SHAPE, NACC, NOPS>), dim3(256), dim3(threads), 0, 0, src, out, iters);
+  (void)hipEventRecord(e1);
+  (void)hipEventSynchronize(e1);
+  float ms = 0;
+  (void)hipEventElapsedTime(&ms, e0, e1);
+  ms /= 10;
+  printf("| %s | %d | %d | %d | %.0f |\n", SHAPE == 32 ? "32x32x16" : "16x16x32", NACC * (SHAPE == 32 ? 1 : 2), NOPS, threads / 256,
+         256.0 * (threads / 64) * iters * 16 * 32768.0 / (ms * 1e-3) * 1e-12);
+}
+void table(const u32x4* src, float* out) {
+  printf("\n## 2. MFMA-only loops on N(0,1) bf16 operands held in registers, by instruction shape\n\n"
+         "| shape | accumulators in turn | operand sets in turn | waves per SIMD | TFLOP/s |\n|---|---|---|---|---|\n");
+  for (int threads : {256, 512}) {
+    run<32, 1, 1>(threads, src, out);
+    run<32, 4, 1>(threads, src, out);
+    run<32, 4, 8>(threads, src, out);
+    run<16, 1, 1>(threads, src, out);
+    run<16, 4, 1>(threads, src, out);
+    run<16, 4, 8>(threads, src, out);
+  }
+}
+}  // namespace t2
+
+// ---- 3. vector instructions of the same wave under an MFMA, by where the MFMA's operands live ---------------------------
+namespace t3 {
+template <int K, int ACC, int BA>   // K vector instructions per MFMA; ACC: C/D in the accumulation half; BA: B operand there
+__global__ __launch_bounds__(256) void loop(const u32x4* src, float* out, int iters) {
+  u32x4 a = src[threadIdx.x], b = src[threadIdx.x + 512];
+  if (BA) asm volatile("" : "=a"(b) : "0"(b));
+  f32x16 acc[2];
+  for (int i = 0; i < 2; ++i) {
+    acc[i] = f32x16{0};
+    if (ACC) asm volatile("" : "=a"(acc[i]) : "0"(acc[i]));
+  }
+  float x[8];
+  for (int i = 0; i < 8; ++i) x[i] = (float)threadIdx.x * 0.001f + i;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      if (ACC && BA) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc[u % 2]) : "v"(a), "a"(b));
+      if (ACC && !BA) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc[u % 2]) : "v"(a), "v"(b));
+      if (!ACC && BA) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc[u % 2]) : "v"(a), "a"(b));
+      if (!ACC && !BA) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc[u % 2]) : "v"(a), "v"(b));
+#pragma unroll
+      for (int k = 0; k < K; ++k) x[k % 8] = x[k % 8] * 1.0001f + 0.5f;   // independent of the MFMAs and of each other
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  float s = 0;
+  for (int n = 0; n < 2; ++n) {
+    if (ACC) asm volatile("" : "=v"(acc[n]) : "0"(acc[n]));
+    for (int i = 0; i < 16; ++i) s += acc[n][i];
+  }
+  for (int i = 0; i < 8; ++i) s += x[i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+template <int K, int ACC, int BA>
+double run(const u32x4* src, float* out) {
+  const int iters = 2000;
+  hipLaunchKernelGGL((loop<K, ACC, BA>), dim3(256), dim3(256), 0, 0, src, out, iters);
+  hipEvent_t e0, e1;
+  (void)hipEventCreate(&e0);
+  (void)hipEventCreate(&e1);
+  (void)hipEventRecord(e0);
+  hipLaunchKernelGGL((loop<K, ACC, BA>), dim3(256), dim3(256), 0, 0, src, out, iters);
+  (void)hipEventRecord(e1);
+  (void)hipEventSynchronize(e1);
+  float ms = 0;
+  (void)hipEventElapsedTime(&ms, e0, e1);
+  return ms * 1e6 / (iters * 16.0);   // ns per MFMA
+}
+template <int K>
+void row(const u32x4* src, float* out) {
+  printf("| %d | %.1f | %.1f | %.1f | %.1f |\n", K, run<K, 0, 0>(src, out), run<K, 1, 0>(src, out), run<K, 0, 1>(src, out), run<K, 1, 1>(src, out));
+}
+void table(const u32x4* zeros, float* out) {
+  printf("\n## 3. One wave per SIMD, all-zero operands: ns per MFMA (13.3 = the matrix pipe alone at 2.4 GHz) with K independent\n"
+         "vector multiply-adds of the same wave behind every MFMA\n\n"
+         "| K | C/D and B in vector registers | C/D in accumulation registers | B in accumulation registers | both |\n|---|---|---|---|---|\n");
+  row<0>(zeros, out);
+  row<2>(zeros, out);
+  row<4>(zeros, out);
+  row<6>(zeros, out);
+  row<8>(zeros, out);
+  row<12>(zeros, out);
+}
+}  // namespace t3
+
+// ---- 4. the tile loop of the forward with 64 query rows per wave, feature by feature -------------------------------------
+namespace t4 {
+__device__ __forceinline__ void softmax_half(int j, int e, const f32x16& sacc, u32x4 (&pb)[2], float& lsum, float& keep) {
+  asm volatile("" : "+v"(lsum));
+  const float pr = fast_exp2(sacc[2 * j + e]);
+  lsum += pr;
+  if (e == 0) {
+    keep = pr;
+    asm volatile("" : "+v"(keep), "+v"(lsum));
+  } else {
+    uint32_t w = pack_elts(keep, pr);
+    asm volatile("" : "+v"(w), "+v"(lsum));
+    pb[j / 4][j % 4] = w;
+  }
+}
+__device__ __forceinline__ f32x16 mfma32_from_aq(u32x4 a, const u32x4& b, const f32x16& c) {
+  f32x16 d;
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
+  return d;
+}
+__device__ __forceinline__ void mfma32_acc_aq(f32x16& d, u32x4 a, const u32x4& b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+}
+
+// F bits: 1 softmax, 2 LDS operand reads, 4 staging (global -> registers -> LDS), 8 barrier per tile.  NB: blocks of 32 rows
+// per wave (2: the form of rope_attn_fwd_pipe64.hip in its steady state; 1: the same wave with its second block alone).
+template <int F, int NB>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void tile_loop(const uint16_t* kg, const uint16_t* vg, float* out, int n_tiles) {
+  constexpr int D = 128, M = 8, NDB = 4, RING = 4, NT = 256, BLOCK_N = 64, ROWS = 4096;
+  constexpr int kKBytes = RowTile<D>::bytes(64), kVBytes = RowTile<D, 32>::bytes(64);
+  constexpr int LSV = RowTile<D, 32>::kStride;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int lane = threadIdx.x % 64, lq = lane % 32, lh = lane / 32;
+  CopyStage<D, 64, NT, 8> kst;
+  CopyStage<D, 64, NT, 32> vst;
+  constexpr int kVBase = 2 * kKBytes;
+  int koff_cur = 0, koff_next = kKBytes;
+  int voff_prev = kVBase + 2 * kVBytes, voff_cur = kVBase, voff_next = kVBase + kVBytes;
+  auto rotate_buffers = [&]() __attribute__((always_inline)) {
+    int k = koff_cur; koff_cur = koff_next; koff_next = k;
+    int v = voff_prev; voff_prev = voff_cur; voff_cur = voff_next; voff_next = v;
+    koff_cur = __builtin_amdgcn_readfirstlane(koff_cur); koff_next = __builtin_amdgcn_readfirstlane(koff_next);
+    voff_prev = __builtin_amdgcn_readfirstlane(voff_prev); voff_cur = __builtin_amdgcn_readfirstlane(voff_cur);
+    voff_next = __builtin_amdgcn_readfirstlane(voff_next);
+  };
+  auto lds_at = [&](uint32_t byte_off) { return reinterpret_cast<uint16_t*>(smem + byte_off); };
+  const uint32_t k_lane_off = RowTile<D>::off(lq, 8 * lh) * 2;
+  const uint32_t v_lane_off = a_trans_lane_offset(LSV) * 2;
+  int l_tile = 0;
+  const uint16_t* kgb = kg + (size_t)(blockIdx.x % 64) * ROWS * D;
+  const uint16_t* vgb = vg + (size_t)(blockIdx.x % 64) * ROWS * D;
+  auto stage_next = [&]() __attribute__((always_inline)) {
+    int ko = koff_next, vo = voff_next;
+    asm volatile("" : "+s"(ko), "+s"(vo));
+    kst.store_rows(lds_at(ko));
+    vst.store_rows(lds_at(vo));
+    l_tile = (l_tile + 1) & 63;
+    kst.load(kgb, l_tile * BLOCK_N, ROWS);
+    vst.load(vgb, l_tile * BLOCK_N, ROWS);
+  };
+  kst.load(kgb, 0, ROWS);
+  vst.load(vgb, 0, ROWS);
+  kst.store_rows(lds_at(koff_cur));
+  vst.store_rows(lds_at(voff_cur));
+  kst.store_rows(lds_at(koff_next));
+  vst.store_rows(lds_at(voff_next));
+  vst.store_rows(lds_at(voff_prev));
+  kst.load(kgb, 64, ROWS);
+  vst.load(vgb, 64, ROWS);
+  u32x4 qa[2][M];
+  for (int b = 0; b < 2; ++b)
+    for (int kc = 0; kc < M; ++kc) {
+      u32x4 x = *reinterpret_cast<const u32x4*>(kgb + (size_t)(lq + 32 * b) * D + 16 * kc + 8 * lh);
+      asm volatile("" : "=a"(qa[b][kc]) : "0"(x));
+    }
+  __syncthreads();
+  f32x16 oacc[2][NDB];
+  for (int b = 0; b < 2; ++b)
+    for (int i = 0; i < NDB; ++i) oacc[b][i] = f32x16{0};
+  float lsum[2] = {0.f, 0.f}, keep[2] = {0.f, 0.f};
+  f32x16 msb[2], s1[2], t0[2];
+  for (int b = 0; b < 2; ++b)
+    for (int i = 0; i < 16; ++i) {
+      float x = -30.f;
+      asm volatile("" : "+v"(x));
+      msb[b][i] = x;
+      s1[b][i] = -1.f;
+      t0[b][i] = -1.f;
+    }
+  u32x4 pb0[2][2], pb1[2][2];
+  for (int b = 0; b < 2; ++b)
+    for (int i = 0; i < 2; ++i) pb0[b][i] = pb1[b][i] = u32x4{0, 0, 0, 0};
+  constexpr int FIRST = NB == 2 ? 0 : 1;
+
+  for (int t = 0; t < n_tiles; ++t) {
+    uint32_t k_lane = k_lane_off + koff_cur, vt = v_lane_off + voff_cur, vprev = v_lane_off + voff_prev;
+    asm volatile("" : "+v"(k_lane), "+v"(vt), "+v"(vprev));
+    auto k_operand = [&](int half, int kc) { return *reinterpret_cast<const u32x4*>(lds_at(k_lane) + RowTile<D>::off(half * 32, 16 * kc)); };
+    auto v_operand = [&](uint32_t v_lane, int half, int i) { return load_a_trans_at(lds_at(v_lane), LSV, half * 32 + 16 * (i / NDB), (i % NDB) * 32); };
+    auto operand = [&](int n) {
+      const int slot = n / M, i = n % M;
+      return slot == 0 ? k_operand(0, i) : slot == 1 ? v_operand(vprev, 1, i) : slot == 2 ? k_operand(1, i) : v_operand(vt, 0, i);
+    };
+    constexpr int TOTAL = 4 * M;
+    u32x4 ring[RING];
+#pragma unroll
+    for (int n = 0; n < RING; ++n) ring[n] = operand(n);
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<TOTAL>([&](auto n_c) __attribute__((always_inline)) {
+      constexpr int n = decltype(n_c)::value;
+      constexpr int slot = n / M, i = n % M;
+      static_for<2>([&](auto b_c) __attribute__((always_inline)) {
+        constexpr int b = decltype(b_c)::value;
+        if constexpr (b >= FIRST) {
+          const u32x4 frag = ring[n % RING];
+          if (slot == 0) { if (i == 0) t0[b] = mfma32_from_aq(frag, qa[b][i], msb[b]); else mfma32_acc_aq(t0[b], frag, qa[b][i]); }
+          if (slot == 1) oacc[b][i % NDB] = mfma32(frag, pb1[b][i / NDB], oacc[b][i % NDB]);
+          if (slot == 2) { if (i == 0) s1[b] = mfma32_from_aq(frag, qa[b][i], msb[b]); else mfma32_acc_aq(s1[b], frag, qa[b][i]); }
+          if (slot == 3) oacc[b][i % NDB] = mfma32(frag, pb0[b][i / NDB], oacc[b][i % NDB]);
+          if (b == 1) {
+            if ((F & 2) && n + RING < TOTAL) ring[n % RING] = operand(n + RING);
+            if ((F & 4) && n == 0) stage_next();
+          }
+          if (i == 0) { if (FIRST == 0) asm volatile("s_nop 1"); else asm volatile("s_nop 7"); }
+          if (F & 1) {
+#pragma unroll
+            for (int hh = (i == 0 ? 0 : i - 1); hh < (i == 0 ? 0 : i == M - 1 ? 8 : i); ++hh) {
+              const int j = hh / 2, e = hh % 2;
+              if (slot == 0) softmax_half(4 + j, e, s1[b], pb1[b], lsum[b], keep[b]);
+              if (slot == 1) softmax_half(j, e, t0[b], pb0[b], lsum[b], keep[b]);
+              if (slot == 2) softmax_half(4 + j, e, t0[b], pb0[b], lsum[b], keep[b]);
+              if (slot == 3) softmax_half(j, e, s1[b], pb1[b], lsum[b], keep[b]);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+    });
+    rotate_buffers();
+    if (F & 8) __syncthreads();
+  }
+  float s = lsum[0] + lsum[1];
+  for (int b = 0; b < 2; ++b) {
+    for (int i = 0; i < NDB; ++i)
+      for (int e = 0; e < 16; ++e) s += oacc[b][i][e];
+    for (int e = 0; e < 16; ++e) s += t0[b][e] + s1[b][e];
+    for (int i = 0; i < 2; ++i)
+      for (int e = 0; e < 4; ++e) s += (float)(pb0[b][i][e] + pb1[b][i][e]);
+  }
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+template <int F, int NB>
+void run(const uint16_t* k, const uint16_t* v, float* out) {
+  constexpr int lds = 2 * RowTile<128>::bytes(64) + 3 * RowTile<128, 32>::bytes(64);
+  auto kern = tile_loop<F, NB>;
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  const int n_tiles = 400;
+  for (int w = 0; w < 3; ++w) hipLaunchKernelGGL(kern, dim3(256), dim3(256), lds, 0, k, v, out, n_tiles);
+  hipEvent_t e0, e1;
+  (void)hipEventCreate(&e0);
+  (void)hipEventCreate(&e1);
+  (void)hipEventRecord(e0);
+  for (int w = 0; w < 5; ++w) hipLaunchKernelGGL(kern, dim3(256), dim3(256), lds, 0, k, v, out, n_tiles);
+  (void)hipEventRecord(e1);
+  (void)hipEventSynchronize(e1);
+  float ms = 0;
+  (void)hipEventElapsedTime(&ms, e0, e1);
+  ms /= 5;
+  printf("| %d | %s | %s | %s | %s | %.3f | %.0f |\n", 32 * NB, (F & 2) ? "yes" : "no", (F & 1) ? "yes" : "no", (F & 8) ? "yes" : "no",
+         (F & 4) ? "yes" : "no", ms * 1e3 / n_tiles, 1024.0 * n_tiles * 32 * NB * 32768.0 / (ms * 1e-3) * 1e-12);
+}
+
+void table(const uint16_t* k, const uint16_t* v, float* out) {
+  printf("\n## 4. Tile loop of the forward with one wave per SIMD (256 x 64 scores per workgroup and tile at D = 128), N(0,1) keys\n\n"
+         "| query rows per wave | LDS operand reads | softmax | barrier per tile | staging of the next tile | us per tile | TFLOP/s executed |\n"
+         "|---|---|---|---|---|---|---|\n");
+  run<0, 2>(k, v, out);
+  run<2, 2>(k, v, out);
+  run<2 + 1, 2>(k, v, out);
+  run<2 + 1 + 8, 2>(k, v, out);
+  run<2 + 1 + 8 + 4, 2>(k, v, out);
+  run<2 + 1 + 8 + 4, 1>(k, v, out);
+}
+}  // namespace t4
+
+int main() {
+  if (table1() != 0) return 1;
+  u32x4* src;
+  float* out;
+  uint16_t *k, *v;
+  const size_t n = (size_t)64 * 4096 * 128;
+  if (hipMalloc(&src, kSrcWords * 16) != hipSuccess || hipMalloc(&out, 256 * 512 * 4) != hipSuccess ||
+      hipMalloc(&k, n * 2) != hipSuccess || hipMalloc(&v, n * 2) != hipSuccess)
+    return 1;
+  std::vector<unsigned> h(kSrcWords * 4);
+  srand(1);
+  for (auto& x : h) x = gauss_bf16_bits() | (gauss_bf16_bits() << 16);
+  (void)hipMemcpy(src, h.data(), h.size() * 4, hipMemcpyHostToDevice);
+  t2::table(src, out);
+  (void)hipMemset(src, 0, kSrcWords * 16);
+  t3::table(src, out);
+  std::vector<uint16_t> hk(n);
+  for (auto& x : hk) x = (uint16_t)gauss_bf16_bits();
+  (void)hipMemcpy(k, hk.data(), n * 2, hipMemcpyHostToDevice);
+  for (auto& x : hk) x = (uint16_t)gauss_bf16_bits();
+  (void)hipMemcpy(v, hk.data(), n * 2, hipMemcpyHostToDevice);
+  t4::table(k, v, out);
+  return hipGetLastError() == hipSuccess ? 0 : 1;
+}

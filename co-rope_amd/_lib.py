@@ -10,7 +10,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libcorope_amd.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # status codes of include/corope_amd.h
 OK, E_BADARG, E_UNSUPPORTED, E_ALIGN, E_LAUNCH = 0, -1, -2, -3, -4
@@ -21,7 +21,6 @@ _P, _I, _F, _L = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_int64
 SIGNATURES = {
     "corope_amd_version": (_I, []),
     "corope_amd_last_error": (ctypes.c_char_p, []),
-    "corope_amd_set_tile_rows": (_I, [_I]),
     "corope_rope_attn_check": (_I, [_I, _I, _I, _I, _L, _F, _I]),
     "corope_gqa_check": (_I, [_I, _I, _I, _I, _I, _F, _F]),
     "corope_rope_freqs": (_I, [_P, _P, _I, _I, _I, _L, _I, _F, _P]),
@@ -89,6 +88,48 @@ def load():
             raise CoRopeLibraryError(f"{LIB_PATH} has ABI version {lib.corope_amd_version()}, expected {ABI_VERSION}")
         _lib = lib
     return _lib
+
+
+TRACE_LIB_PATH = os.path.join(_HERE, "lib", "libcorope_amd_trace.so")
+_trace_lib = None
+
+
+def load_trace():
+    """The measurement build of the library (same kernels with time stamps compiled in; made by build.py beside the shipped
+    one): every entry point of the shipped library plus ``corope_debug_trace(buf)`` and
+    ``corope_debug_set_forms(tile_rows, fwd_wave_rows)``, which forces kernel forms for the tests."""
+    global _trace_lib
+    if _trace_lib is None:
+        if not os.path.exists(TRACE_LIB_PATH):
+            raise CoRopeLibraryError(f"{TRACE_LIB_PATH} not found: `python co-rope_amd/build.py` makes it")
+        lib = ctypes.CDLL(TRACE_LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        lib.corope_debug_trace.restype, lib.corope_debug_trace.argtypes = None, [_P]
+        lib.corope_debug_set_forms.restype, lib.corope_debug_set_forms.argtypes = _I, [_I, _I]
+        _trace_lib = lib
+    return _trace_lib
+
+
+class using:
+    """Context in which ``load()`` hands out `lib` (e.g. the measurement build) instead of the shipped library."""
+
+    def __init__(self, lib):
+        self.lib, self.prev = lib, None
+
+    def __enter__(self):
+        global _lib
+        load()
+        with _lock:
+            self.prev, _lib = _lib, self.lib
+        return self.lib
+
+    def __exit__(self, *exc):
+        global _lib
+        with _lock:
+            _lib = self.prev
+        return False
 
 
 def last_error():

@@ -3,8 +3,8 @@
 Run as ``python co-rope_amd/build.py`` or call ``build()``; the result lands in
 ``co-rope_amd/lib/libcorope_amd.so`` and is what ``_lib.load()`` opens.  Beside it, for measurement only:
 ``libcorope_amd_trace.so`` (the same sources with -DCOROPE_TRACE: the attention kernels stamp a clock at their phase
-boundaries into a buffer ``bench.py --phase-trace`` hands them) and the stand-alone program ``mfma_rate``
-(``csrc/mfma_rate.hip``: what the matrix pipes sustain on this machine)."""
+boundaries into a buffer ``bench.py --phase-trace`` hands them, and a call forces kernel forms for the tests).
+``build_program`` compiles a stand-alone HIP program with the same flags (``bench.py --mfma-rate`` uses it)."""
 from __future__ import annotations
 
 import glob
@@ -15,17 +15,16 @@ import tempfile
 from concurrent.futures import ThreadPoolExecutor
 
 try:
-    from .check_isa import check_asm_mfma
+    from .check_isa import ASM_MFMA_IN_SOURCE, check_asm_mfma
 except ImportError:   # run as a script
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-    from check_isa import check_asm_mfma
+    from check_isa import ASM_MFMA_IN_SOURCE, check_asm_mfma
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libcorope_amd.so")
 TRACE_LIB = os.path.join(LIBDIR, "libcorope_amd_trace.so")
-MFMA_RATE = os.path.join(LIBDIR, "mfma_rate")
 
 # compiled a second time with -DCOROPE_F16 (fp16 elements, namespace corope_f16)
 F16_SOURCES = ["rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip",
@@ -33,8 +32,14 @@ F16_SOURCES = ["rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_bwd_pre.hip", 
 
 SOURCES = ["abi.hip", "rope_freqs.hip", "rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_fwd_pipe.hip", "rope_attn_fwd_pipe64.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip", "corope_gqa_bwd.hip"]
 
-# sources with asm-issued matrix-core instructions: their generated assembly is checked (check_isa.py) in every variant
-ISA_CHECKED = {"rope_attn_fwd_pipe.hip", "rope_attn_fwd_pipe64.hip", "rope_attn_bwd.hip"}
+
+
+def isa_checked(src):
+    """Whether a source issues matrix-core instructions from asm statements (itself or through the helpers of common.hpp):
+    the generated assembly of every variant of such a source is checked (check_isa.py)."""
+    with open(os.path.join(CSRC, src)) as f:
+        return ASM_MFMA_IN_SOURCE.search(f.read()) is not None
+
 
 # -packed-fp32-ops is switched off: packed fp32 VALU forms are not used by these kernels.
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-value",
@@ -53,7 +58,7 @@ def _compile(src, extra, suffix=""):
     obj = os.path.join(LIBDIR, os.path.splitext(src)[0] + suffix + ".o")
     cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     noise = "is not a recognized feature for this target"
-    if src not in ISA_CHECKED:
+    if not isa_checked(src):
         r = subprocess.run(cmd, capture_output=True, text=True)
         problems = []
     else:   # the compiler's intermediate files, among them the device assembly, land in a directory of their own
@@ -84,12 +89,11 @@ def _link(objs, out, shared=True):
 
 
 def build(verbose=False, extra_flags=(), extras=True):
-    """Compiles every source.  ``extras``: also the trace variant of the library and the mfma_rate program."""
+    """Compiles every source.  ``extras``: also the trace variant of the library."""
     os.makedirs(LIBDIR, exist_ok=True)
     jobs = [(s, list(extra_flags), "") for s in SOURCES] + [(s, list(extra_flags) + ["-DCOROPE_F16"], ".f16") for s in F16_SOURCES]
     if extras:
         jobs += [(s, j[1] + ["-DCOROPE_TRACE"], j[2] + ".trace") for j in list(jobs) for s in [j[0]]]
-        jobs += [("mfma_rate.hip", [], "")]
     with ThreadPoolExecutor(max_workers=8) as ex:
         results = list(ex.map(lambda j: _compile(*j), jobs))
     if verbose:
@@ -100,8 +104,16 @@ def build(verbose=False, extra_flags=(), extras=True):
     _link([o for o, _ in results[:n]], LIB)
     if extras:
         _link([o for o, _ in results[n:2 * n]], TRACE_LIB)
-        _link([results[2 * n][0]], MFMA_RATE, shared=False)
     return LIB
+
+
+def build_program(source, out):
+    """Compiles one stand-alone HIP program (a measurement tool beside bench.py) for gfx950."""
+    flags = [f for f in HIPCC_FLAGS if f != "-fPIC"]
+    r = subprocess.run([_hipcc(), *flags, "-I", os.path.dirname(HERE), source, "-o", out], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {source}:\n{r.stderr}")
+    return out
 
 
 if __name__ == "__main__":

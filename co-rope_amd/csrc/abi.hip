@@ -5,6 +5,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <initializer_list>
 
 #include "kernels.hpp"
 
@@ -15,9 +16,34 @@ extern "C" void corope_debug_trace(void* buf) { corope::g_trace_buf = static_cas
 #endif
 
 namespace corope {
-std::atomic<int> g_tile_rows{0};
-std::atomic<int> g_fwd_wave_rows{[] { const char* e = getenv("COROPE_AMD_FWD_WAVE_ROWS"); return e ? atoi(e) : 0; }()};
+namespace {
+// An environment variable that must hold one of `allowed` (anything else, or unset: 0 = the library's own choice).
+int env_choice(const char* name, std::initializer_list<int> allowed) {
+  const char* e = getenv(name);
+  if (e == nullptr) return 0;
+  const int v = atoi(e);
+  for (int a : allowed)
+    if (v == a) return v;
+  return 0;
 }
+}  // namespace
+// Kernel forms are picked by shape.  For diagnostics two environment variables, read ONCE when the library is loaded,
+// override the pick for the whole process: COROPE_AMD_TILE_ROWS (128 or 256 rows per workgroup item) and
+// COROPE_AMD_FWD_WAVE_ROWS (32 or 64 query rows per wave in the two-launch forward at D = 128).  The shipped library has
+// no call that changes them afterwards; the measurement build (libcorope_amd_trace.so) has one, for the tests.
+std::atomic<int> g_tile_rows{env_choice("COROPE_AMD_TILE_ROWS", {128, 256})};
+std::atomic<int> g_fwd_wave_rows{env_choice("COROPE_AMD_FWD_WAVE_ROWS", {32, 64})};
+}  // namespace corope
+
+#ifdef COROPE_TRACE
+extern "C" int corope_debug_set_forms(int tile_rows, int fwd_wave_rows) {
+  if ((tile_rows != 0 && tile_rows != 128 && tile_rows != 256) || (fwd_wave_rows != 0 && fwd_wave_rows != 32 && fwd_wave_rows != 64))
+    return COROPE_E_BADARG;
+  corope::g_tile_rows.store(tile_rows);
+  corope::g_fwd_wave_rows.store(fwd_wave_rows);
+  return COROPE_OK;
+}
+#endif
 
 namespace {
 
@@ -87,15 +113,9 @@ corope::BwdParams make_bwd(const void* q, const void* k, const void* v, const vo
 
 extern "C" {
 
-int corope_amd_version(void) { return 2; }
+int corope_amd_version(void) { return 3; }
 
 const char* corope_amd_last_error(void) { return g_err; }
-
-int corope_amd_set_tile_rows(int rows) {
-  if (rows != 0 && rows != 128 && rows != 256) return fail(COROPE_E_BADARG, "set_tile_rows: %d is not 0, 128 or 256", rows);
-  corope::g_tile_rows.store(rows);
-  return COROPE_OK;
-}
 
 int corope_rope_attn_check(int B, int H, int N, int D, int64_t freq_row_stride, float sm_scale, int backward) {
   (void)backward;

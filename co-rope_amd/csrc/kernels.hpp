@@ -72,7 +72,7 @@ inline int device_cu_count() {
 
 // Rows per workgroup of the attention kernels: 256 (8 waves) or 128 (4 waves).  By shape: a launch whose 256-row items
 // number fewer than the compute units takes the 128-row form, which doubles the items and halves the time the heaviest
-// of them runs; `g_tile_rows` (0 = by shape, 128, 256) overrides the rule for tests and tuning.
+// of them runs; `g_tile_rows` (0 = by shape, 128, 256; set from the environment when the library is loaded) overrides the rule.
 extern std::atomic<int> g_tile_rows;
 // Query rows per wave of the two-launch forward at D = 128 with 256-row items: 32 (8 waves, two per SIMD) or 64 (4 waves,
 // one per SIMD, every LDS fragment feeding two MFMAs); 0 = the default.

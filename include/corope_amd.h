@@ -42,10 +42,10 @@ int corope_amd_version(void);
 /* Text of the last error raised on the calling thread ("" if none). */
 const char *corope_amd_last_error(void);
 
-/* Rows per workgroup of the RoPE attention kernels: 0 = chosen by shape (256, or 128 when a launch would otherwise have
- * fewer than two workgroups per CU -- the reference picks its tile sizes per shape too, fused-rope/fused_rope_attn.py:
- * 163-183), 128 or 256 = forced, for tests and tuning.  Process-wide; results do not depend on it beyond rounding. */
-int corope_amd_set_tile_rows(int rows);
+/* No entry point changes how later calls run: kernel forms (rows per workgroup item, rows per wave) are picked per call
+ * from the shape, as the reference picks its tile sizes per shape (fused-rope/fused_rope_attn.py:163-183).  For diagnostics
+ * the environment variables COROPE_AMD_TILE_ROWS (128 | 256) and COROPE_AMD_FWD_WAVE_ROWS (32 | 64), read once when the
+ * library is loaded, override the pick for the whole process; results do not depend on them beyond rounding. */
 
 /* Argument check only (no HIP call): what corope_rope_attn_fwd/bwd would return for these sizes. */
 int corope_rope_attn_check(int B, int H, int N, int D, int64_t freq_row_stride, float sm_scale, int backward);

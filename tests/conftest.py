@@ -27,11 +27,27 @@ def pkg():
 @pytest.fixture(params=[128, 256])
 def tile_rows(request, pkg):
     """Runs the test once with 128-row (4-wave) and once with 256-row (8-wave) workgroups of the RoPE attention kernels,
-    whatever the library would pick for the shape."""
-    lib = pkg._lib.load()
-    assert lib.corope_amd_set_tile_rows(request.param) == 0
-    yield request.param
-    assert lib.corope_amd_set_tile_rows(0) == 0
+    whatever the library would pick for the shape.  The shipped library has no call that forces a form; its measurement
+    build (same kernels, time stamps compiled in) has, so the test runs on that one."""
+    lib = pkg._lib.load_trace()
+    with pkg._lib.using(lib):
+        assert lib.corope_debug_set_forms(request.param, 0) == 0
+        try:
+            yield request.param
+        finally:
+            assert lib.corope_debug_set_forms(0, 0) == 0
+
+
+@pytest.fixture
+def rows64(pkg):
+    """256-row items and 64 query rows per wave (one wave per SIMD) in the two-launch forward at D = 128."""
+    lib = pkg._lib.load_trace()
+    with pkg._lib.using(lib):
+        assert lib.corope_debug_set_forms(256, 64) == 0
+        try:
+            yield 64
+        finally:
+            assert lib.corope_debug_set_forms(0, 0) == 0
 
 
 @pytest.fixture(scope="session")

@@ -136,11 +136,14 @@ def test_composite_entry_points_check_every_argument_before_the_first_launch(pkg
     assert rc == -2 and "scratch" in pkg._lib.last_error()
 
 
-def test_tile_rows_knob(pkg):
+def test_no_entry_point_changes_later_calls(pkg):
+    """The shipped library exports nothing that forces kernel forms (its measurement build does, for the tests)."""
     lib = pkg._lib.load()
-    assert lib.corope_amd_set_tile_rows(128) == 0 and lib.corope_amd_set_tile_rows(256) == 0
-    assert lib.corope_amd_set_tile_rows(64) == -1 and "tile_rows" in pkg._lib.last_error()
-    assert lib.corope_amd_set_tile_rows(0) == 0
+    for name in ("corope_amd_set_tile_rows", "corope_debug_set_forms", "corope_debug_trace"):
+        assert not hasattr(lib, name), name
+    trace = pkg._lib.load_trace()
+    assert trace.corope_debug_set_forms(64, 0) == -1 and trace.corope_debug_set_forms(0, 48) == -1
+    assert trace.corope_debug_set_forms(128, 64) == 0 and trace.corope_debug_set_forms(0, 0) == 0
 
 
 def test_grouped_query_argument_checks(pkg):

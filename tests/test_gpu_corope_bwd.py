@@ -156,6 +156,32 @@ def test_corope_backward_caller_workspace_and_reuse(pkg):
         mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4, workspace=ws[: one // 4 - 1])
 
 
+def test_corope_backward_keeps_its_own_workspace_between_calls(pkg, monkeypatch):
+    """Without a caller's workspace the operator uses one buffer per device, sized by the shape and a cap alone: the second
+    call allocates nothing new, a smaller cap walks the groups in passes with the same gradients, release frees it."""
+    import importlib
+    mod = importlib.import_module("corope_amd.corope_gqa")
+    dev = torch.device("cuda:0")
+    B, Hq, Hkv, N, D = 2, 6, 3, 70, 64
+    q, k, v, d_o = (t.to(dev, torch.bfloat16) for t in _inputs(B, Hq, Hkv, N, D, seed=5))
+    mod.release_backward_workspace()
+    a = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4)
+    ws = mod._workspaces[dev.index]
+    assert ws.numel() == mod.backward_workspace_bytes(B, Hq, Hkv, N, D)
+    b = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4)
+    assert mod._workspaces[dev.index].data_ptr() == ws.data_ptr()
+    one = mod.backward_min_workspace_bytes(B, Hq, Hkv, N, D)
+    mod.release_backward_workspace(dev)
+    assert dev.index not in mod._workspaces
+    monkeypatch.setattr(mod, "BACKWARD_WORKSPACE_CAP_BYTES", 2 * one + 5)
+    c = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4)
+    assert mod._workspaces[dev.index].numel() == 2 * one
+    torch.cuda.synchronize()
+    for x, y, z in zip(a, b, c):
+        assert torch.equal(x, y) and torch.equal(x, z)
+    mod.release_backward_workspace()
+
+
 def test_corope_random_shapes_forward_and_backward(pkg):
     """A seeded sweep over batch, group size, head dim, ragged lengths, temperature and rotation base: forward and
     backward in one go, each tensor against the dense oracle with the bar of conftest.within_bar (2e-2, or one bf16 step
