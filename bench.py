@@ -275,9 +275,12 @@ def bench_sweep(args):
     pkg = importlib.import_module("corope_amd")
     dev = torch.device("cuda:0")
     flush_buf = torch.empty(512 << 20, dtype=torch.uint8, device=dev) if args.flush else None
-    for (B, H, N, D, name) in SWEEP:
+    dtype = torch.float16 if args.dtype == "fp16" else torch.bfloat16
+    pkg.rope_attn.FP16_TRAINING_FORWARD = args.fp16_forward
+    shapes = [s for s in SWEEP if args.only is None or s[4] in args.only.split(",")]
+    for (B, H, N, D, name) in shapes:
         g = torch.Generator().manual_seed(0)
-        q, k, v, do = (torch.randn(B, H, N, D, generator=g).to(dev, torch.bfloat16) for _ in range(4))
+        q, k, v, do = (torch.randn(B, H, N, D, generator=g).to(dev, dtype) for _ in range(4))
         cos, sin = pkg.rope_freqs_device(D, N, 10000.0, device=dev)
         q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
         stats = {}
@@ -300,7 +303,7 @@ def bench_sweep(args):
 
         b_ms = timed(lambda: (clear_grads(), o.backward(do, retain_graph=True)), "bwd")
         ff, fb = attention_flops(B, H, N, D, "fwd"), attention_flops(B, H, N, D, "bwd")
-        row = {"config": name, "B": B, "H": H, "N": N, "D": D, "fwd_ms": round(f_ms, 4),
+        row = {"config": name, "B": B, "H": H, "N": N, "D": D, "dtype": args.dtype, "fwd_ms": round(f_ms, 4),
                "fwd_tflops": round(ff / f_ms * 1e-9, 1), "bwd_ms": round(b_ms, 4), "bwd_tflops": round(fb / b_ms * 1e-9, 1)}
         row.update(stats)
         if args.lanes:
@@ -569,6 +572,10 @@ def main():
                     help="time the reference harness's 19 shapes instead (one JSON line per shape)")
     ap.add_argument("--lanes", action="store_true",
                     help="with --sweep: also time the unfused lanes (separate rotation + identity-table attention, PyTorch SDPA)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"], help="with --sweep: element type of q, k, v, dO")
+    ap.add_argument("--fp16-forward", default="exact", choices=["exact", "fast"],
+                    help="with --sweep --dtype fp16: rope_attn.FP16_TRAINING_FORWARD (the forward of a differentiated call)")
+    ap.add_argument("--only", default=None, help="with --sweep: comma-separated names of the shapes to run")
     ap.add_argument("--flush", action="store_true",
                     help="with --sweep: also time every call on flushed caches (a 512 MiB buffer overwritten before each call)")
     ap.add_argument("--parity", action="store_true",

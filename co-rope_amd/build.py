@@ -27,7 +27,7 @@ LIB = os.path.join(LIBDIR, "libcorope_amd.so")
 TRACE_LIB = os.path.join(LIBDIR, "libcorope_amd_trace.so")
 
 # compiled a second time with -DCOROPE_F16 (fp16 elements, namespace corope_f16)
-F16_SOURCES = ["rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip",
+F16_SOURCES = ["rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_fwd_pipe.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip",
                "corope_gqa_bwd.hip"]
 
 SOURCES = ["abi.hip", "rope_freqs.hip", "rope_rotate.hip", "rope_attn_fwd.hip", "rope_attn_fwd_pipe.hip", "rope_attn_fwd_pipe64.hip", "rope_attn_bwd_pre.hip", "rope_attn_bwd.hip", "corope_gqa_fwd.hip", "corope_gqa_bwd.hip"]

@@ -617,14 +617,15 @@ int corope_rope_attn_bwd_gqa(const void* q, const void* k, int prerotated, const
 
 // ---- fp16 tensors (the reference's dtype): the same kernels built for fp16 elements -------------------------------------
 int corope_rope_attn_fwd_f16(const void* q, const void* k, const void* v, const float* freqs_cos, const float* freqs_sin,
-                             int64_t freq_row_stride, void* o, float* lse, int B, int H, int Hkv, int N, int D,
-                             float sm_scale, int causal, void* stream) {
+                             int64_t freq_row_stride, void* o, float* lse, void* q_rot, void* k_rot, float* tile_kmax, int B,
+                             int H, int Hkv, int N, int D, float sm_scale, int causal, void* stream) {
   const char* what = "rope_attn_fwd_f16";
   if (Hkv <= 0 || H % Hkv != 0) return fail(COROPE_E_BADARG, "%s: H=%d is not a multiple of Hkv=%d", what, H, Hkv);
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
   if (rc) return rc;
   rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse});
   if (rc) return rc;
+  if (k_rot == nullptr && q_rot != nullptr) return fail(COROPE_E_BADARG, "%s: q_rot without k_rot", what);
   corope::FwdParams p{};
   p.q = static_cast<const uint16_t*>(q);
   p.k = static_cast<const uint16_t*>(k);
@@ -639,13 +640,29 @@ int corope_rope_attn_fwd_f16(const void* q, const void* k, const void* v, const 
   p.BH = B * H;
   p.H = H;
   p.Hkv = Hkv;
-  return launch_status(what, corope_f16::launch_rope_attn_fwd(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (k_rot == nullptr) return launch_status(what, corope_f16::launch_rope_attn_fwd(p, D, causal != 0, st));
+  // two launches: K rotated once into k_rot (with the largest key norm of every 64-key tile), then the attention kernel
+  // on it, which leaves its rotated, scaled Q rows in q_rot if asked to (the operands of a backward on rotated copies)
+  if ((rc = rotated_copies_built(what, D))) return rc;
+  rc = check_ptrs(what, {k_rot});
+  if (rc) return rc;
+  if (q_rot != nullptr && !aligned16(q_rot)) return fail(COROPE_E_ALIGN, "%s: q_rot %p is not 16-byte aligned", what, q_rot);
+  if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
+    return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "%s: tile_kmax %p is null or misaligned", what, (const void*)tile_kmax);
+  rc = launch_status(what, corope_f16::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, static_cast<uint16_t*>(k_rot), tile_kmax,
+                                                          B * Hkv, N, D, st, 1.f));
+  if (rc) return rc;
+  p.k_rot = static_cast<const uint16_t*>(k_rot);
+  p.tile_kmax = tile_kmax;
+  p.q_rot_out = static_cast<uint16_t*>(q_rot);
+  return launch_status(what, corope_f16::launch_rope_attn_fwd_prerotated(p, D, causal != 0, st));
 }
 
-int corope_rope_attn_bwd_f16(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
-                             float* delta, const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* dq,
-                             void* dk, void* dv, int B, int H, int Hkv, int N, int D, float sm_scale, int causal,
-                             void* workspace, int64_t workspace_bytes, void* stream) {
+int corope_rope_attn_bwd_f16(const void* q, const void* k, int prerotated, const void* v, const void* o, const void* d_o,
+                             const float* lse, float* delta, const float* freqs_cos, const float* freqs_sin,
+                             int64_t freq_row_stride, void* dq, void* dk, void* dv, int B, int H, int Hkv, int N, int D,
+                             float sm_scale, int causal, void* workspace, int64_t workspace_bytes, void* stream) {
   const char* what = "rope_attn_bwd_f16";
   if (Hkv <= 0 || H % Hkv != 0) return fail(COROPE_E_BADARG, "%s: H=%d is not a multiple of Hkv=%d", what, H, Hkv);
   int rc = validate_bwd(what, B, H, N, D, freq_row_stride, sm_scale,
@@ -655,10 +672,17 @@ int corope_rope_attn_bwd_f16(const void* q, const void* k, const void* v, const 
                                  sm_scale);
   p.Hkv = Hkv;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (workspace != nullptr && (rc = rotated_copies_built(what, D))) return rc;
+  if ((workspace != nullptr || prerotated) && (rc = rotated_copies_built(what, D))) return rc;
+  if (prerotated) {
+    // q, k are the rotated copies a two-launch forward kept: the dQ kernel computes delta on its way, dK and dV come
+    // from one kernel
+    mark_prerotated(p, true);
+    rc = launch_status(what, corope_f16::launch_bwd_dq(p, D, causal != 0, st));
+    if (rc) return rc;
+    return launch_status(what, corope_f16::launch_bwd_dkdv_fused(p, D, causal != 0, st));
+  }
   if (workspace != nullptr) {
-    // as corope_rope_attn_bwd_ws: q (scaled) and k are rotated once, the dQ kernel computes delta on its way, dK and dV
-    // come from one kernel
+    // as corope_rope_attn_bwd_ws: q (scaled) and k are rotated once, then as above
     if (!aligned16(workspace)) return fail(COROPE_E_ALIGN, "%s: pointer %p is not 16-byte aligned", what, workspace);
     const int64_t each = bwd_ws_tensor_bytes(B, H, N, D);
     if (workspace_bytes < 2 * each)

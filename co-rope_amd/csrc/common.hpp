@@ -47,11 +47,12 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 //   A operand: lane l holds row (l % 32), contraction slots 8*(l / 32) .. +7
 //   B operand: lane l holds column (l % 32), contraction slots 8*(l / 32) .. +7
 //   D/C      : lane l holds column (l % 32); register i holds row 8*(i / 4) + 4*(l / 32) + (i % 4)
-#ifndef COROPE_F16
-__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+__device__ __forceinline__ f32x16 mfma32_bf16(u32x4 a, u32x4 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
                                                  0, 0, 0);
 }
+#ifndef COROPE_F16
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) { return mfma32_bf16(a, b, c); }
 #endif
 
 // The same tile shape with fp16 operands (11 significant bits instead of 8).

@@ -199,6 +199,7 @@ hipError_t launch_rope_freqs(float* cosp, float* sinp, int n_pos, int D, int wid
 // fp16 matrix-core operands, fp16 outputs; same parameter blocks.
 namespace corope_f16 {
 hipError_t launch_rope_attn_fwd(const corope::FwdParams& p, int D, bool causal, hipStream_t stream);
+hipError_t launch_rope_attn_fwd_prerotated(const corope::FwdParams& p, int D, bool causal, hipStream_t stream);  // needs k_rot
 hipError_t launch_bwd_preprocess(const corope::BwdParams& p, int D, hipStream_t stream);
 hipError_t launch_bwd_dv(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_dk(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);

@@ -59,6 +59,27 @@ struct FwdPipeCfg {
   static_assert(kLdsBytes <= 160 * 1024, "LDS of a compute unit");
 };
 
+// P^T is a bf16 operand in both builds (its unnormalised values span up to 2^kPipeMargin, more binary orders than fp16
+// has), so the product O^T += V^T P^T is a bf16 product in both: in the fp16 build the V tile is converted to bf16 while
+// it is staged (fp16's 11 significant bits become 8: the same rounding P itself carries).
+#ifdef COROPE_F16
+__device__ __forceinline__ u32x4 v_operand_format(u32x4 x) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) x[w] = pack_bf16(elt_lo(x[w]), elt_hi(x[w]));
+  return x;
+}
+#else
+__device__ __forceinline__ u32x4 v_operand_format(u32x4 x) { return x; }
+#endif
+template <class Stage, class Tile>
+__device__ __forceinline__ void store_v_rows(const Stage& st, uint16_t* lds, Tile) {
+#pragma unroll
+  for (int it = 0; it < Stage::kIters; ++it) {
+    const int u = threadIdx.x + it * (Stage::kUnits / Stage::kIters);
+    *reinterpret_cast<u32x4*>(lds + Tile::off(u / Stage::kChunks, (u % Stage::kChunks) * 8)) = v_operand_format(st.x[it]);
+  }
+}
+
 // One exponential pair of a 32-key half: scores 2j, 2j+1 of the lane (already relative to the reference value, base-2
 // units) -> one bf16x2 word of the P^T operand.
 __device__ __forceinline__ void softmax_pair(int j, const f32x16& sacc, u32x4 (&pb)[2], float& lsum) {
@@ -67,7 +88,7 @@ __device__ __forceinline__ void softmax_pair(int j, const f32x16& sacc, u32x4 (&
   float p1 = fast_exp2(sacc[2 * j + 1]);
   // plain adds: the bf16 dot-product instruction would do this in one op but stalls the MFMA pipe
   lsum += p0 + p1;
-  uint32_t w = pack_elts(p0, p1);
+  uint32_t w = pack_bf16(p0, p1);
   asm volatile("" : "+v"(w), "+v"(lsum));   // ... and ends here, between the two MFMAs it is written between
   pb[j / 4][j % 4] = w;
 }
@@ -166,7 +187,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
     int ko = koff_next, vo = voff_next;
     asm volatile("" : "+s"(ko), "+s"(vo));
     kst.store_rows(lds_at(ko));
-    vst.store_rows(lds_at(vo));
+    store_v_rows(vst, lds_at(vo), RowTile<D, Cfg::kVPad>{});
     load_next_tile();
   };
 
@@ -203,7 +224,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
   request_q(item);
   take_q(item);
   kst.store_rows(lds_at(koff_cur));
-  vst.store_rows(lds_at(voff_cur));
+  store_v_rows(vst, lds_at(voff_cur), RowTile<D, Cfg::kVPad>{});
   load_next_tile();
   __syncthreads();
 
@@ -275,7 +296,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
 #pragma unroll
       for (int j = 4; j < 8; ++j) softmax_pair(j, s1, pb1, lsum);
 #pragma unroll
-      for (int i = 0; i < M; ++i) oacc[i % NDB] = mfma32(v_operand(vp_lane, 1, i), pb1[i / NDB], oacc[i % NDB]);
+      for (int i = 0; i < M; ++i) oacc[i % NDB] = mfma32_bf16(v_operand(vp_lane, 1, i), pb1[i / NDB], oacc[i % NDB]);
     };
 
     // the Q operands and the first 64 key-norm maxima have landed before the loop on every path: left to their first use,
@@ -333,9 +354,9 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
           constexpr int slot = n / M, i = n % M;
           // MFMA
           if (slot == 0) t0 = i == 0 ? mfma32_from(ring[n % RING], qb[i], msb) : mfma32(ring[n % RING], qb[i], t0);
-          if (slot == 1) oacc[i % NDB] = mfma32(ring[n % RING], pb1[i / NDB], oacc[i % NDB]);
+          if (slot == 1) oacc[i % NDB] = mfma32_bf16(ring[n % RING], pb1[i / NDB], oacc[i % NDB]);
           if (slot == 2) s1 = i == 0 ? mfma32_from(ring[n % RING], qb[i], msb) : mfma32(ring[n % RING], qb[i], s1);
-          if (slot == 3) oacc[i % NDB] = mfma32(ring[n % RING], pb0[i / NDB], oacc[i % NDB]);
+          if (slot == 3) oacc[i % NDB] = mfma32_bf16(ring[n % RING], pb0[i / NDB], oacc[i % NDB]);
           if (n + RING < TOTAL) ring[n % RING] = operand(n + RING);
           if (n == 0) stage_next();
           // softmax on the side: four exponential pairs per slot
@@ -472,8 +493,10 @@ static hipError_t launch_pipe_cfg(const FwdParams& p, hipStream_t stream) {
 
 hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream) {
   if (D != 64 && D != 128) return hipErrorInvalidValue;
+#ifndef COROPE_F16
   if (D == 128 && !use_small_tiles(p.N, p.BH) && g_fwd_wave_rows.load(std::memory_order_relaxed) == 64)
     return launch_rope_attn_fwd_prerotated_rows64(p, D, causal, stream);
+#endif
   if (D == 128) return causal ? launch_pipe_cfg<128, true>(p, stream) : launch_pipe_cfg<128, false>(p, stream);
   return causal ? launch_pipe_cfg<64, true>(p, stream) : launch_pipe_cfg<64, false>(p, stream);
 }

@@ -5,8 +5,8 @@ like the reference's ``attention = _attention.apply`` (fused-rope/fused_rope_att
 accepted and ignored (it selects a Triton code path there).  ``fused_rope_attn`` is a keyword-friendly wrapper.
 
 Forward and backward run hand-written gfx950 kernels through the C ABI in ``include/corope_amd.h``; there is no
-other implementation behind this module.  Tensors are bfloat16 (the fast paths) or float16 (the reference's dtype,
-fused_rope_attn.py:236; same kernels built for fp16 elements, single-launch forward)."""
+other implementation behind this module.  Tensors are bfloat16 or float16 (the reference's dtype, fused_rope_attn.py:236;
+the same kernel sources built for fp16 elements)."""
 from __future__ import annotations
 
 import torch
@@ -102,6 +102,15 @@ TWO_LAUNCH_MIN_N = 1024
 TRAIN_ROTATED_MIN_ND = 65536
 
 
+# fp16 tensors, forward of a call that will be differentiated: "exact" = the single-launch forward, which keeps P and V in
+# fp16 (O within 1.2e-2 of the fp32 oracle at the reference's verification temperature sm_scale = 0.5, gradients within its
+# 0.15 / 5e-3 thresholds); "fast" = the two-launch forward (bf16 probabilities against a V converted to bf16 on its way
+# into LDS: as fast as with bf16 tensors, 1.5x faster than "exact" at B2 H32 N4096 D128, O within one bf16 ulp), whose O
+# carries bf16's rounding of V into delta = rowsum(O * dO) and through it into dQ and dK: up to 0.24 there instead of 0.05.
+# A forward that will not be differentiated always takes the fast form.
+FP16_TRAINING_FORWARD = "exact"
+
+
 def use_rotated_path(N, D, training):
     """Whether the operator rotates the operands ahead of the attention kernels at this shape."""
     return D <= _ROTATED_PATH_MAX_D and (N >= TWO_LAUNCH_MIN_N or N * D >= TRAIN_ROTATED_MIN_ND)
@@ -123,11 +132,22 @@ def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, k
     Hkv = k.shape[1]
     with _on_device(q):
         if q.dtype == torch.float16:
-            # the reference's dtype: one launch, a true running maximum wherever a probability would leave fp16's range
+            # the reference's dtype: the same two forms (the two-launch one with bf16 probabilities against a V converted
+            # to bf16 on its way into LDS); one entry point covers them, grouped-query K/V included
+            if keep_rotated and FP16_TRAINING_FORWARD != "fast":
+                two_launch = False
+            q_rot = torch.empty_like(q) if (two_launch and keep_rotated) else None
+            k_rot = torch.empty_like(k) if two_launch else None
+            kmax = torch.empty((B, Hkv, (N + 63) // 64), device=q.device, dtype=torch.float32) if two_launch else None
             rc = lib.corope_rope_attn_fwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
-                                              fc.stride(0), o.data_ptr(), M.data_ptr(), B, H, Hkv, N, D, float(sm_scale),
-                                              int(bool(causal)), _stream_ptr(q))
+                                              fc.stride(0), o.data_ptr(), M.data_ptr(),
+                                              q_rot.data_ptr() if q_rot is not None else None,
+                                              k_rot.data_ptr() if k_rot is not None else None,
+                                              kmax.data_ptr() if kmax is not None else None, B, H, Hkv, N, D,
+                                              float(sm_scale), int(bool(causal)), _stream_ptr(q))
             _lib.check(rc, "corope_rope_attn_fwd_f16")
+            if q_rot is not None:
+                rotated = (q_rot, k_rot)
         elif Hkv != H:   # grouped-query attention: one entry point covers the three forms
             q_rot = torch.empty_like(q) if (two_launch and keep_rotated) else None
             k_rot = torch.empty_like(k) if two_launch else None
@@ -177,7 +197,7 @@ class _FusedRopeAttn(torch.autograd.Function):
         # when a gradient will be asked for, the forward keeps its rotated q and k for the backward and the originals
         # are not saved (the reference saves q and k, fused_rope_attn.py:718, and re-rotates them in its backward)
         o, M, fc, fs, rotated = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin,
-                                         keep_rotated=any(ctx.needs_input_grad[:3]) and q.dtype == torch.bfloat16)
+                                         keep_rotated=any(ctx.needs_input_grad[:3]))
         ctx.rotated = rotated is not None
         if ctx.rotated:
             ctx.save_for_backward(rotated[0], rotated[1], v, o, M, fc, fs)
@@ -201,10 +221,10 @@ class _FusedRopeAttn(torch.autograd.Function):
         with _on_device(q):
             if q.dtype == torch.float16:
                 ws, nbytes = None, 0
-                if use_rotated_path(N, D, training=True):   # rotate q and k once, then the kernels on the rotated copies
+                if not ctx.rotated and use_rotated_path(N, D, training=True):   # rotate q and k once, then the kernels on the copies
                     nbytes = lib.corope_rope_attn_bwd_workspace_bytes(B, H, N, D)
                     ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
-                rc = lib.corope_rope_attn_bwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(),
+                rc = lib.corope_rope_attn_bwd_f16(q.data_ptr(), k.data_ptr(), int(ctx.rotated), v.data_ptr(), o.data_ptr(), do.data_ptr(),
                                                   M.data_ptr(), delta.data_ptr(), fc.data_ptr(), fs.data_ptr(), fc.stride(0),
                                                   dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, k.shape[1], N, D,
                                                   ctx.sm_scale, int(ctx.causal), ws.data_ptr() if ws is not None else None,

@@ -224,20 +224,26 @@ int corope_rope_attn_bwd_ws(const void *q, const void *k, const void *v, const v
                             void *workspace, int64_t workspace_bytes, void *stream);
 
 /* The operator on fp16 tensors -- the only dtype of the reference's kernels (fused-rope/fused_rope_attn.py:236,
- * verification.py:14): q, k, v, o, d_o, dq, dk, dv are fp16, the matrix cores take fp16 operands, everything else (tables,
- * lse, delta, accumulation) is fp32 as above.  Same kernels as the bf16 entry points built for the other element type:
- * the forward is corope_rope_attn_fwd's single launch with a true running maximum per 32-key half whenever a
- * probability would leave fp16's range (the two-launch forward carries unnormalised probabilities up to 2^64, which only
- * bf16 can hold); the backward is preprocess + dV + dK + dQ as in corope_rope_attn_bwd, or -- given a workspace of
+ * verification.py:14): q, k, v, o, d_o, dq, dk, dv are fp16, the score products take fp16 operands, everything else
+ * (tables, lse, delta, accumulation) is fp32 as above.  Same kernel sources as the bf16 entry points built for the other
+ * element type.
+ * Forward: k_rot == NULL: corope_rope_attn_fwd's single launch, with a true running maximum per 32-key half whenever a
+ * probability would leave fp16's range.  k_rot != NULL ((B,Hkv,N,D) fp16 scratch, with tile_kmax (B,Hkv,ceil(N/64)) fp32):
+ * the two-launch form as in corope_rope_attn_fwd_train / _gqa -- K rotated once into k_rot, then the pipelined attention
+ * kernel, in which the unnormalised probabilities (up to 2^64: more binary orders than fp16 has) are bf16 and V is
+ * converted to bf16 on its way into LDS, so that P V is a bf16 product; q_rot ((B,H,N,D) fp16, may be NULL) receives the
+ * rotated Q times sm_scale*log2(e), and (q_rot, k_rot) are then the operands of a backward with prerotated = 1.
+ * Backward: prerotated = 1: q, k are those rotated copies (dQ kernel, which computes delta on its way, then the fused dK+dV
+ * kernel); else preprocess + dV + dK + dQ as in corope_rope_attn_bwd, or -- given a workspace of
  * corope_rope_attn_bwd_workspace_bytes (may be NULL) -- the rotation of q and k into it followed by the dQ and the fused
- * dK+dV kernel as in corope_rope_attn_bwd_ws, which is the faster form from N * D = 65536 on.  `delta` is (B,H,N) fp32 scratch.
+ * dK+dV kernel as in corope_rope_attn_bwd_ws, the faster form from N * D = 65536 on.  `delta` is (B,H,N) fp32 scratch.
  * k, v, dk, dv have Hkv heads (H a multiple of Hkv; Hkv = H: the reference's form), as in the grouped-query entry points below.
  * Replaces _attention.forward / .backward (fused-rope/fused_rope_attn.py:655-777) for callers that keep the reference's dtype. */
 int corope_rope_attn_fwd_f16(const void *q, const void *k, const void *v,
                              const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
-                             void *o, float *lse,
+                             void *o, float *lse, void *q_rot, void *k_rot, float *tile_kmax,
                              int B, int H, int Hkv, int N, int D, float sm_scale, int causal, void *stream);
-int corope_rope_attn_bwd_f16(const void *q, const void *k, const void *v, const void *o, const void *d_o,
+int corope_rope_attn_bwd_f16(const void *q, const void *k, int prerotated, const void *v, const void *o, const void *d_o,
                              const float *lse, float *delta,
                              const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
                              void *dq, void *dk, void *dv,
