@@ -182,21 +182,33 @@ def test_grouped_query_parity(pkg, monkeypatch, tile_rows, B, Hq, Hkv, N, D, cau
 @pytest.mark.parametrize("B,H,N,D", [(2, 4, 512, 64), (1, 8, 1024, 128), (4, 16, 2048, 64)])
 def test_backward_parity_verification_script_cases(pkg, monkeypatch, B, H, N, D, causal, two_launch):
     """The six cases of the reference's verification script (fused-rope/verification.py:153-161) at its sm_scale = 0.5,
-    backward.  The script's gradient thresholds (verification.py:116: max < 0.15 and mean < 5e-3 per tensor) are written
-    for fp16 tensors.  bf16 carries three mantissa bits fewer (8x coarser), and at this temperature (logits with a
-    standard deviation of 4 at D = 64 and 5.7 at D = 128) the rounding of the rotated q and k alone moves single
-    probabilities by 1-2 %, which is what the error of dQ and dK (values up to 29; one bf16 ulp there is 0.125) consists
-    of.  Bar for bf16: 4x the script's thresholds; measured: 0.3x to 2.5x of them."""
+    backward, on bf16 tensors.  The script's gradient thresholds (verification.py:116: max < 0.15 and mean < 5e-3 per
+    tensor) are written for fp16 tensors, which this operator meets as they stand (test_gpu_rope_f16.py).  The reference
+    rounds the rotated q and k to the tensors' 16-bit type before the score product (fused_rope_attn.py:96-99); with bf16
+    that rounding alone (8 significant bits, logits with a standard deviation of 4 at D = 64 and 5.7 at D = 128) moves
+    single probabilities by 1-2 %.  Asserted here against the oracle evaluated on q, k rotated and rounded at that point:
+    max < 0.25, mean < 6e-3 (measured: up to 0.235 / 5.4e-3).  What is left there comes, in this order, from delta =
+    rowsum(O * dO) taken from the bf16 output O (0.10 / 3e-3 by itself at D = 128), the rounding of dS (0.05 / 1.7e-3), of
+    the gradients themselves (values up to 29: 0.06 / 1.5e-3) and of P (0.03 / 6e-4) -- bf16's 8 bits where the script's
+    dtype has 11.  Against the oracle in fp32 throughout (printed): up to 0.32 / 1.2e-2."""
     print(f"case B={B} H={H} N={N} D={D} causal={causal} sm_scale=0.5 two_launch={two_launch}", flush=True)
     _force_path(monkeypatch, pkg, two_launch)
     q, k, v, g, c, s = _case(B, H, N, D)
     o, dq, dk, dv = _gpu_fwd_bwd(pkg, q, k, v, g, causal, 0.5, c, s)
     ro, _, rdq, rdk, rdv, _ = O.rope_attn_fwd_bwd_blocked(q, k, v, g, causal, 0.5, c, s)
-    for name, a, b in (("O", o, ro), ("dQ", dq, rdq), ("dK", dk, rdk), ("dV", dv, rdv)):
-        err = (a - b).abs()
-        print(f"  {name}: max-abs {err.max():.3e} mean-abs {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
+    # the same with the rotated operands rounded where the kernels (and the reference's) round them: the rotated q carries
+    # sm_scale * log2(e) into its rounding; gradients with respect to the rotated operands are rotated back
+    cc = 0.5 * math.log2(math.e)
+    qr, kr = bf16_round(O.apply_rotary_emb(q, c, s) * cc) / cc, bf16_round(O.apply_rotary_emb(k, c, s))
+    po, _, pdq, pdk, pdv, _ = O.rope_attn_fwd_bwd_blocked(qr, kr, v, g, causal, 0.5, torch.ones_like(c), torch.zeros_like(s))
+    pdq, pdk = O.apply_rotary_emb(pdq, c, -s), O.apply_rotary_emb(pdk, c, -s)
+    for name, a, b, pb in (("O", o, ro, po), ("dQ", dq, rdq, pdq), ("dK", dk, rdk, pdk), ("dV", dv, rdv, pdv)):
+        err, perr = (a - b).abs(), (a - pb).abs()
+        print(f"  {name}: against rounded rotated q, k: max-abs {perr.max():.3e} mean-abs {perr.mean():.3e}; "
+              f"against fp32 throughout: {err.max():.3e} / {err.mean():.3e} (|ref| max {b.abs().max():.2f})")
         assert torch.isfinite(a).all(), name
-        assert err.max() < 4 * 0.15 and err.mean() < 4 * 5e-3, name
+        assert perr.max() < 0.25 and perr.mean() < 6e-3, name
+        assert err.max() < 0.4 and err.mean() < 1.5e-2, name
 
 
 @pytest.mark.parametrize("causal", [True, False])
