@@ -9,7 +9,7 @@ oracle timed on the host cores as a baseline.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--no-cpu-baseline]
                     [--parity | --no-parity] [--data normal|sink] [--phase-trace] [--sweep [--lanes] [--flush]]
-                    [--mfma-rate]
+                    [--mfma-rate] [--hbm-passes]
 
 (c3 is the metric shape and the default; c2/c4 are the other RoPE-attention shapes; c5 is the Co-RoPE GQA forward,
 with its backward timed beside it.)  --parity adds per-tensor errors against the CPU oracle to the line (outside the
@@ -34,12 +34,17 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak used for every "fracti
 PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE on this
-# benchmark (summary and commands: profiles/rope_attn_c3_hbm_traffic.md); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE
+# benchmark (summary and commands: profiles/rope_attn_c3_c4_hbm_traffic.md); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE
 # by 1.0, the factors a plain 1 GiB device copy gives for the same counters.
 HBM_TRAFFIC_BYTES = {
     ("c3", "rope_attn_fwd"): int((305561 * 2.0 + 132096) * 1024),
     ("c3", "rope_attn_bwd_dq"): int((404872 * 2.0 + 91136) * 1024),
     ("c3", "rope_attn_bwd_dkdv"): int((312964 * 2.0 + 131072) * 1024),
+    ("c4", "rope_attn_fwd"): int((1073484 * 2.0 + 243220) * 1024),
+    # Co-RoPE at C5 (profiles/corope_gqa_c5_hbm_traffic.md): the forward kernel; the backward's six launches together
+    ("c5", "corope_gqa_fwd"): int((70416 * 2.0 + 65536) * 1024),
+    ("c5", "corope_gqa_bwd"): int(((2 * 22429 + 701939 + 48483 + 226967 + 298542) * 2.0
+                                   + (2 * 188709 + 1422980 + 2364 + 2341 + 2341)) * 1024),
 }
 
 CONFIGS = {
@@ -431,20 +436,73 @@ def bench_corope(args):
            "sincos_pairs_per_s": round(pairs / (kms * 1e-3), 1), "kernel_ms": round(kms, 4),
            "roofline": {"bound": "valu", "kernel": "corope_gqa_fwd", "achieved": round(fwd_instr / (kms * 1e-3) * 1e-12, 3),
                         "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T issue slots/s",
-                        "frac": round(fwd_instr / (kms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4), "traffic": None},
+                        "frac": round(fwd_instr / (kms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4),
+                        "traffic": HBM_TRAFFIC_BYTES[("c5", "corope_gqa_fwd")]},
            "backward": {"ms": round(bms, 4), "steps": bsteps, "workspace_gib": round(ws_bytes / 2**30, 2), "ms_by_workspace": by_workspace,
                         "sincos_pairs_per_s": round(2 * pairs / (bms * 1e-3), 1),
                         "tflops_attention_equivalent": round(2.5 * flops / (bms * 1e-3) * 1e-12, 2),
                         "roofline": {"bound": "valu", "kernel": "corope_gqa_bwd (6 launches)",
                                      "achieved": round(bwd_instr / (bms * 1e-3) * 1e-12, 3),
                                      "peak": round(256 * 4 * 16 * 2.4e9 * 1e-12, 3), "unit": "T issue slots/s",
-                                     "frac": round(bwd_instr / (bms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4), "traffic": None}},
+                                     "frac": round(bwd_instr / (bms * 1e-3) / (256 * 4 * 16 * 2.4e9), 4),
+                                     "traffic": HBM_TRAFFIC_BYTES[("c5", "corope_gqa_bwd")]}},
            "cpu_baseline": None}
     if args.parity:
         torch.cuda.synchronize()
         out["parity"] = corope_parity(pkg, q.float().cpu(), k.float().cpu(), v.float().cpu(), do.float().cpu(), o.float().cpu(),
                                       tuple(t.float().cpu() for t in (dq, dk, dv)), scale, 10000.0, torch)
     print(json.dumps(out))
+
+
+def bench_hbm_passes(args):
+    """The two HBM-bound passes of the chosen RoPE shape (rotation of K with per-tile norms; delta = rowsum(O * dO)) beside a
+    plain device copy of the same tensor, each timed two ways: back to back (operands largely resident in the 256 MB
+    last-level cache from the previous call) and with a 1 GiB buffer overwritten before every call (nothing resident).
+    Inside a training step the passes run between those two extremes.  Prints a markdown table."""
+    import torch
+    pkg = importlib.import_module("corope_amd")
+    lib = pkg._lib.load()
+    dev = torch.device("cuda:0")
+    cfg = CONFIGS[args.config]
+    B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
+    k, o, do, _ = (t.to(dev, torch.bfloat16) for t in make_inputs(B, H, N, D, "normal", torch))
+    c, s = pkg.precompute_freqs_cis(D, N, 10000.0, device=dev)
+    kr = torch.empty_like(k)
+    kmax = torch.empty(B, H, (N + 63) // 64, device=dev, dtype=torch.float32)
+    delta = torch.empty(B, H, N, device=dev, dtype=torch.float32)
+    st = torch.cuda.current_stream().cuda_stream
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    ops = [("plain copy of one tensor (torch copy_)", lambda: kr.copy_(k), 2 * k.numel() * 2),
+           ("rope_rotate_k (read K, write rotated K + tile norms)",
+            lambda: lib.corope_rope_rotate(k.data_ptr(), c.data_ptr(), s.data_ptr(), c.stride(0), kr.data_ptr(), kmax.data_ptr(),
+                                           B, H, N, D, 1.0, st), 2 * k.numel() * 2 + kmax.numel() * 4),
+           ("rope_attn_bwd_preprocess (read O and dO, write delta)",
+            lambda: lib.corope_rope_attn_bwd_preprocess(o.data_ptr(), do.data_ptr(), delta.data_ptr(), B, H, N, D, st),
+            2 * k.numel() * 2 + delta.numel() * 4)]
+    print(f"Workload: {cfg['name']}\n\n| pass | bytes | back to back: us | GB/s | of 8 TB/s | caches flushed before every call: us | GB/s | of 8 TB/s |\n"
+          "|---|---|---|---|---|---|---|---|")
+    for name, fn, by in ops:
+        for _ in range(50):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(300):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        warm = e0.elapsed_time(e1) / 300
+        ts = []
+        for _ in range(40):
+            flush.zero_()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1))
+        cold = statistics.median(ts)
+        print(f"| {name} | {by / 1e6:.1f} MB | {warm * 1e3:.1f} | {by / warm * 1e-6:.0f} | {by / warm * 1e-6 / PEAK_HBM_GBS:.2f} | "
+              f"{cold * 1e3:.1f} | {by / cold * 1e-6:.0f} | {by / cold * 1e-6 / PEAK_HBM_GBS:.2f} |")
 
 
 def forward_ms(pkg, q, k, v, cos, sin, scale, torch, reps=100):
@@ -587,6 +645,9 @@ def main():
                     help="split the attention kernels of the chosen RoPE config into phases (trace build of the library)")
     ap.add_argument("--trace-dump", default=None, metavar="DIR",
                     help="with --phase-trace: also save the raw stamps of every kernel (one row of 16 per item) as .npy files there")
+    ap.add_argument("--hbm-passes", action="store_true",
+                    help="time the rotation and dO.O passes of the chosen RoPE shape beside a plain device copy, with warm and "
+                         "with flushed caches (markdown table)")
     ap.add_argument("--mfma-rate", action="store_true",
                     help="build (if stale) and run bench_mfma_rate.hip: what the matrix pipes sustain on this machine, by operand "
                          "source, instruction shape and accompanying vector work (markdown tables)")
@@ -617,6 +678,8 @@ def main():
         return bench_corope(args)
     if args.phase_trace:
         return bench_phase_trace(args)
+    if args.hbm_passes:
+        return bench_hbm_passes(args)
     import torch
     pkg = importlib.import_module("corope_amd")
     lib = pkg._lib.load()
