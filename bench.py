@@ -691,7 +691,8 @@ def main():
     host = make_inputs(B, H, N, D, args.data, torch)
     q, k, v, do = (t.to(dev, torch.bfloat16) for t in host)
     cos, sin = pkg.precompute_freqs_cis(D, N, 10000.0, device=dev)
-    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    if not fwd_only:
+        q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
 
     def step():
         o = pkg.attention(q, k, v, True, scale, cos, sin)
