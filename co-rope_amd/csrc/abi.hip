@@ -714,7 +714,7 @@ int corope_rope_attn_bwd_f16(const void* q, const void* k, int prerotated, const
 int corope_rope_freqs(float* freqs_cos, float* freqs_sin, int n_pos, int D, int width, int64_t freq_row_stride, int pos0,
                       float theta, void* stream) {
   if (n_pos <= 0 || D <= 0 || D % 2 != 0) return fail(COROPE_E_BADARG, "rope_freqs: n_pos must be positive and D even");
-  if (D > 128) return fail(COROPE_E_UNSUPPORTED, "rope_freqs: head dim %d exceeds 128", D);
+  if (D > 256) return fail(COROPE_E_UNSUPPORTED, "rope_freqs: head dim %d exceeds 256", D);
   if (width != D && width != D / 2) return fail(COROPE_E_BADARG, "rope_freqs: width must be D or D/2 (got %d)", width);
   if (freq_row_stride < width) return fail(COROPE_E_BADARG, "rope_freqs: row stride smaller than the row");
   if (pos0 < 0 || !(theta > 0.f) || !std::isfinite(theta)) return fail(COROPE_E_BADARG, "rope_freqs: bad pos0 or theta");

@@ -10,7 +10,7 @@
 namespace corope {
 
 struct InvFreqs {
-  float w[64];  // theta^(-2i/D), evaluated on the host with the reference's fp32 expression
+  float w[128];  // theta^(-2i/D), evaluated on the host with the reference's fp32 expression
 };
 
 __global__ __launch_bounds__(256) void rope_freqs_kernel(float* __restrict__ cosp, float* __restrict__ sinp, int n_pos,

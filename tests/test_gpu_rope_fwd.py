@@ -122,7 +122,7 @@ def test_deterministic(pkg):
 def test_device_freq_tables_match_the_oracle(pkg):
     """The library's own table kernel against the oracle's precompute_freqs_cis: fp32 angles are formed the same way;
     the device's cosf/sinf may differ from the host's by a few ulp."""
-    for D, N, theta in ((128, 4096, 10000.0), (64, 777, 500.0)):
+    for D, N, theta in ((128, 4096, 10000.0), (64, 777, 500.0), (256, 300, 10000.0)):
         c, s = pkg.rope_freqs_device(D, N, theta, device="cuda:0")
         rc, rs = O.precompute_freqs_cis(D, N, theta)
         assert c.shape == (N, D) and (c.cpu() - rc).abs().max() < 2e-6 and (s.cpu() - rs).abs().max() < 2e-6
