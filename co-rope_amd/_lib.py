@@ -47,6 +47,7 @@ SIGNATURES = {
     "corope_rope_attn_bwd_ws": (_I, [_P] * 9 + [_L, _P, _P, _P, _I, _I, _I, _I, _F, _I, _P, _L, _P]),
     "corope_rope_attn_fwd_f16": (_I, [_P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P]),
     "corope_rope_attn_bwd_f16": (_I, [_P, _P, _I] + [_P] * 7 + [_L, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _L, _P]),
+    "corope_rope_attn_fwd_strided": (_I, [_P] * 8 + [_L] + [_P] * 5 + [_I] * 5 + [_F, _I, _I, _P]),
     "corope_rope_attn_fwd_gqa": (_I, [_P] * 5 + [_L] + [_P] * 5 + [_I] * 5 + [_F, _I, _P]),
     "corope_rope_attn_bwd_gqa": (_I, [_P, _P, _I] + [_P] * 7 + [_L, _P, _P, _P] + [_I] * 5 + [_F, _I, _P]),
     "corope_gqa_fwd": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P]),

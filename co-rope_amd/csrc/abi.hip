@@ -185,6 +185,7 @@ int rope_attn_fwd_impl(const char* what, const void* q, const void* k, const voi
   p.BH = B * H;
   p.H = H;
   p.Hkv = Hkv > 0 ? Hkv : H;
+  p.contiguous(D);
   p.k_rot = static_cast<const uint16_t*>(k_rot);
   p.tile_kmax = tile_kmax;
   p.q_rot_out = static_cast<uint16_t*>(q_rot_out);
@@ -640,6 +641,7 @@ int corope_rope_attn_fwd_f16(const void* q, const void* k, const void* v, const 
   p.BH = B * H;
   p.H = H;
   p.Hkv = Hkv;
+  p.contiguous(D);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (k_rot == nullptr) return launch_status(what, corope_f16::launch_rope_attn_fwd(p, D, causal != 0, st));
   // two launches: K rotated once into k_rot (with the largest key norm of every 64-key tile), then the attention kernel
@@ -651,7 +653,7 @@ int corope_rope_attn_fwd_f16(const void* q, const void* k, const void* v, const 
   if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
     return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "%s: tile_kmax %p is null or misaligned", what, (const void*)tile_kmax);
   rc = launch_status(what, corope_f16::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, static_cast<uint16_t*>(k_rot), tile_kmax,
-                                                          B * Hkv, N, D, st, 1.f));
+                                                          B * Hkv, N, D, st, 1.f, 1, 0, 0, 0));
   if (rc) return rc;
   p.k_rot = static_cast<const uint16_t*>(k_rot);
   p.tile_kmax = tile_kmax;
@@ -691,9 +693,9 @@ int corope_rope_attn_bwd_f16(const void* q, const void* k, int prerotated, const
     uint16_t* q_rot = static_cast<uint16_t*>(workspace);
     uint16_t* k_rot = reinterpret_cast<uint16_t*>(static_cast<char*>(workspace) + each);
     rc = launch_status(what, corope_f16::launch_rope_rotate(p.q, p.cos, p.sin, p.fstride, q_rot, nullptr, p.BH, N, D, st,
-                                                            p.qk_scale));
+                                                            p.qk_scale, 1, 0, 0, 0));
     if (rc) return rc;
-    rc = launch_status(what, corope_f16::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, k_rot, nullptr, B * Hkv, N, D, st, 1.f));
+    rc = launch_status(what, corope_f16::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, k_rot, nullptr, B * Hkv, N, D, st, 1.f, 1, 0, 0, 0));
     if (rc) return rc;
     p.q = p.q_rot = q_rot;
     p.k = p.k_rot = k_rot;
@@ -709,6 +711,66 @@ int corope_rope_attn_bwd_f16(const void* q, const void* k, int prerotated, const
   rc = launch_status(what, corope_f16::launch_bwd_dk(p, D, causal != 0, st));
   if (rc) return rc;
   return launch_status(what, corope_f16::launch_bwd_dq(p, D, causal != 0, st));
+}
+
+int corope_rope_attn_fwd_strided(const void* q, const int64_t* q_strides, const void* k, const int64_t* k_strides, const void* v,
+                                 const int64_t* v_strides, const float* freqs_cos, const float* freqs_sin,
+                                 int64_t freq_row_stride, void* o, float* lse, void* q_rot, void* k_rot, float* tile_kmax, int B,
+                                 int H, int Hkv, int N, int D, float sm_scale, int causal, int fp16, void* stream) {
+  const char* what = "rope_attn_fwd_strided";
+  if (Hkv <= 0 || H % Hkv != 0) return fail(COROPE_E_BADARG, "%s: H=%d is not a multiple of Hkv=%d", what, H, Hkv);
+  int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
+  if (rc) return rc;
+  rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse});
+  if (rc) return rc;
+  if (q_strides == nullptr || k_strides == nullptr || v_strides == nullptr) return fail(COROPE_E_BADARG, "%s: null strides", what);
+  for (const int64_t* st : {q_strides, k_strides, v_strides}) {
+    // rows start on 16-byte boundaries and one (batch, head) slice stays below 4 GiB (32-bit offsets inside it)
+    if (st[2] < D || st[0] < 0 || st[1] < 0 || st[0] % 8 != 0 || st[1] % 8 != 0 || st[2] % 8 != 0)
+      return fail(COROPE_E_BADARG, "%s: strides (%lld, %lld, %lld) must be non-negative multiples of 8 elements, rows at least D apart",
+                  what, (long long)st[0], (long long)st[1], (long long)st[2]);
+    if ((int64_t)N * st[2] * 2 >= ((int64_t)1 << 32) || st[2] >= ((int64_t)1 << 30))
+      return fail(COROPE_E_UNSUPPORTED, "%s: one (batch, head) slice spans 4 GiB or more at row stride %lld", what, (long long)st[2]);
+  }
+  if (k_rot == nullptr && q_rot != nullptr) return fail(COROPE_E_BADARG, "%s: q_rot without k_rot", what);
+  corope::FwdParams p{};
+  p.q = static_cast<const uint16_t*>(q);
+  p.k = static_cast<const uint16_t*>(k);
+  p.v = static_cast<const uint16_t*>(v);
+  p.cos = freqs_cos;
+  p.sin = freqs_sin;
+  p.o = static_cast<uint16_t*>(o);
+  p.lse = lse;
+  p.fstride = freq_row_stride;
+  p.qk_scale = sm_scale * kLog2e;
+  p.N = N;
+  p.BH = B * H;
+  p.H = H;
+  p.Hkv = Hkv;
+  p.q_sb = q_strides[0], p.q_sh = q_strides[1], p.q_sn = (int)q_strides[2];
+  p.k_sb = k_strides[0], p.k_sh = k_strides[1], p.k_sn = (int)k_strides[2];
+  p.v_sb = v_strides[0], p.v_sh = v_strides[1], p.v_sn = (int)v_strides[2];
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (k_rot == nullptr)
+    return launch_status(what, fp16 ? corope_f16::launch_rope_attn_fwd(p, D, causal != 0, st)
+                                    : corope::launch_rope_attn_fwd(p, D, causal != 0, st));
+  if ((rc = rotated_copies_built(what, D))) return rc;
+  rc = check_ptrs(what, {k_rot});
+  if (rc) return rc;
+  if (q_rot != nullptr && !aligned16(q_rot)) return fail(COROPE_E_ALIGN, "%s: q_rot %p is not 16-byte aligned", what, q_rot);
+  if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
+    return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "%s: tile_kmax %p is null or misaligned", what, (const void*)tile_kmax);
+  uint16_t* kr = static_cast<uint16_t*>(k_rot);
+  rc = launch_status(what, fp16 ? corope_f16::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, kr, tile_kmax, B * Hkv, N, D, st, 1.f,
+                                                                 Hkv, p.k_sb, p.k_sh, p.k_sn)
+                                : corope::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, kr, tile_kmax, B * Hkv, N, D, st, 1.f, Hkv,
+                                                             p.k_sb, p.k_sh, p.k_sn));
+  if (rc) return rc;
+  p.k_rot = kr;
+  p.tile_kmax = tile_kmax;
+  p.q_rot_out = static_cast<uint16_t*>(q_rot);
+  return launch_status(what, fp16 ? corope_f16::launch_rope_attn_fwd_prerotated(p, D, causal != 0, st)
+                                  : corope::launch_rope_attn_fwd_prerotated(p, D, causal != 0, st));
 }
 
 int corope_rope_freqs(float* freqs_cos, float* freqs_sin, int n_pos, int D, int width, int64_t freq_row_stride, int pos0,

@@ -190,15 +190,17 @@ struct RotStage {
   float out_scale = 1.f;
 
   // src: first row of the (n, D) bf16 matrix; row0: first tile row; rows >= n_rows are clamped.
+  // row_bytes: bytes between rows of src (D * 2 for a contiguous matrix)
   __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float* __restrict__ cosp,
-                                       const float* __restrict__ sinp, int64_t fstride, int row0, int n_rows) {
+                                       const float* __restrict__ sinp, int64_t fstride, int row0, int n_rows,
+                                       uint32_t row_bytes = D * 2) {
 #pragma unroll
     for (int it = 0; it < kIters; ++it) {
       int u = threadIdx.x + it * NT;
       if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
       int r = u / kChunks, ch = u % kChunks;
       int row = min(row0 + r, n_rows - 1);
-      const uint16_t* p = byte_offset(src, (uint32_t)row * (D * 2) + ch * 16);
+      const uint16_t* p = byte_offset(src, (uint32_t)row * row_bytes + ch * 16);
       x1[it] = *reinterpret_cast<const u32x4*>(p);
       x2[it] = *reinterpret_cast<const u32x4*>(p + D / 2);
       const uint32_t foff = ((uint32_t)row * (uint32_t)fstride + ch * 8) * 4;
@@ -252,13 +254,13 @@ struct CopyStage {
   static constexpr int kIters = (kUnits + NT - 1) / NT;
   u32x4 x[kIters];
 
-  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, int row0, int n_rows) {
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ src, int row0, int n_rows, uint32_t row_bytes = D * 2) {
 #pragma unroll
     for (int it = 0; it < kIters; ++it) {
       int u = threadIdx.x + it * NT;
       if (kUnits % NT != 0 && u >= kUnits) u = kUnits - 1;
       int row = min(row0 + u / kChunks, n_rows - 1);
-      x[it] = *reinterpret_cast<const u32x4*>(byte_offset(src, (uint32_t)row * (D * 2) + (u % kChunks) * 16));
+      x[it] = *reinterpret_cast<const u32x4*>(byte_offset(src, (uint32_t)row * row_bytes + (u % kChunks) * 16));
     }
   }
   __device__ __forceinline__ void store_rows(uint16_t* lds) const {
@@ -279,8 +281,8 @@ template <int D, int ROWS, int NT, bool SCALED, int PAD>
 struct RopeStage<D, ROWS, NT, true, SCALED, PAD> : CopyStage<D, ROWS, NT, PAD> {
   float out_scale = 1.f;   // unused: the copy was scaled when it was rotated
   __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float*, const float*, int64_t, int row0,
-                                       int n_rows) {
-    CopyStage<D, ROWS, NT, PAD>::load(src, row0, n_rows);
+                                       int n_rows, uint32_t row_bytes = D * 2) {
+    CopyStage<D, ROWS, NT, PAD>::load(src, row0, n_rows, row_bytes);
   }
 };
 
@@ -394,11 +396,11 @@ struct WaveRows<D, false> {
   static constexpr int IT = 32 / RPI;
   u32x4 x[IT];
   __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float*, const float*, int64_t, int row0,
-                                       int n_rows, int l = threadIdx.x % kWave) {
+                                       int n_rows, int l = threadIdx.x % kWave, uint32_t row_bytes = D * 2) {
 #pragma unroll
     for (int i = 0; i < IT; ++i)
       x[i] = *reinterpret_cast<const u32x4*>(
-          byte_offset(src, (uint32_t)min(row0 + RPI * i + l / CPR, n_rows - 1) * (D * 2) + (l % CPR) * 16));
+          byte_offset(src, (uint32_t)min(row0 + RPI * i + l / CPR, n_rows - 1) * row_bytes + (l % CPR) * 16));
   }
   __device__ __forceinline__ void park(u32x4 (&out)[D / 16], uint16_t* wave_tile, uint16_t* = nullptr, int = 0, int = 0,
                                        float = 1.f) {
@@ -426,11 +428,11 @@ struct WaveRows<D, true> {
   // per-lane address parts are recomputed per item instead of being kept in registers across the whole loop)
   __device__ __forceinline__ void load(const uint16_t* __restrict__ src, const float* __restrict__ cosp,
                                        const float* __restrict__ sinp, int64_t fstride, int row0, int n_rows,
-                                       int l = threadIdx.x % kWave) {
+                                       int l = threadIdx.x % kWave, uint32_t row_bytes = D * 2) {
 #pragma unroll
     for (int i = 0; i < IT; ++i) {
       const int row = min(row0 + RPI * i + l / UPR, n_rows - 1), u = l % UPR;
-      const uint16_t* xp = byte_offset(src, (uint32_t)row * (D * 2) + u * 16);
+      const uint16_t* xp = byte_offset(src, (uint32_t)row * row_bytes + u * 16);
       x1[i] = *reinterpret_cast<const u32x4*>(xp);
       x2[i] = *reinterpret_cast<const u32x4*>(xp + D / 2);
       const uint32_t foff = ((uint32_t)row * (uint32_t)fstride + u * 8) * 4;

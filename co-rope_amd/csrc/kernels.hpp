@@ -111,6 +111,21 @@ struct FwdParams {
   int H, Hkv;        // query heads and key/value heads per batch (grouped-query attention when Hkv < H; k, v, k_rot and
                      // tile_kmax then have B * Hkv slabs and query head h reads key/value head h / (H / Hkv))
   int num_m_blocks;  // filled in by the launcher
+  // Layout of q, k, v (the forward only; o, lse, k_rot, q_rot_out are contiguous): elements between batches, heads and
+  // rows; the last dimension is contiguous.  contiguous(D) fills in (B, H, N, D) row-major.
+  int64_t q_sb, q_sh, k_sb, k_sh, v_sb, v_sh;
+  int q_sn, k_sn, v_sn;
+  void contiguous(int D) {
+    q_sn = k_sn = v_sn = D;
+    q_sh = k_sh = v_sh = (int64_t)N * D;
+    q_sb = (int64_t)H * N * D;
+    k_sb = v_sb = (int64_t)Hkv * N * D;
+  }
+#if defined(__HIPCC__)
+  __device__ __forceinline__ const uint16_t* q_slab(int bh) const { return q + (bh / H) * q_sb + (bh % H) * q_sh; }
+  __device__ __forceinline__ const uint16_t* k_slab(int kvs) const { return k + (kvs / Hkv) * k_sb + (kvs % Hkv) * k_sh; }
+  __device__ __forceinline__ const uint16_t* v_slab(int kvs) const { return v + (kvs / Hkv) * v_sb + (kvs % Hkv) * v_sh; }
+#endif
 };
 
 struct BwdParams {
@@ -175,8 +190,10 @@ namespace COROPE_NS {
 using namespace corope;
 
 // y = out_scale * rotated x for a (BH, N, D) tensor; tile_max (may be null) receives [BH][ceil(N / 64)] largest row norms.
+// (x_sb, x_sh, x_sn: elements between batches, heads and rows of x, with H heads per batch; 0, 0, 0: contiguous)
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
-                              float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale = 1.f);
+                              float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale = 1.f, int H = 1,
+                              int64_t x_sb = 0, int64_t x_sh = 0, int x_sn = 0);
 hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream);  // needs k_rot
 // the same with 64 query rows per wave, one wave per SIMD (D = 128)
 hipError_t launch_rope_attn_fwd_prerotated_rows64(const FwdParams& p, int D, bool causal, hipStream_t stream);
@@ -206,7 +223,8 @@ hipError_t launch_bwd_dk(const corope::BwdParams& p, int D, bool causal, hipStre
 hipError_t launch_bwd_dq(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_dkdv_fused(const corope::BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
-                              float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale);
+                              float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale, int H, int64_t x_sb,
+                              int64_t x_sh, int x_sn);
 hipError_t launch_corope_gqa_fwd(const corope::CoropeParams& p, int D, hipStream_t stream);
 hipError_t launch_corope_gqa_bwd(const corope::CoropeBwdParams& p, int D, float* workspace, int64_t workspace_floats,
                                  hipStream_t stream);

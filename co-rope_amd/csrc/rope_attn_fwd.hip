@@ -128,10 +128,11 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
   const int lq = lane % 32, lh = lane / 32;
   const int N = p.N;
 
-  const uint16_t* qg = p.q + (int64_t)bh * N * D;
+  const uint16_t* qg = p.q_slab(bh);
+  const uint32_t q_rb = (uint32_t)p.q_sn * 2, k_rb = (uint32_t)p.k_sn * 2, v_rb = (uint32_t)p.v_sn * 2;   // bytes between rows
   const int kvs = kv_slab(bh, p.H, p.Hkv);   // key/value slab of this query head
-  const uint16_t* kg = p.k + (int64_t)kvs * N * D;
-  const uint16_t* vg = p.v + (int64_t)kvs * N * D;
+  const uint16_t* kg = p.k_slab(kvs);
+  const uint16_t* vg = p.v_slab(kvs);
 
   const int n_k_tiles = (N + BLOCK_N - 1) / BLOCK_N;
   const int n_tiles = CAUSAL ? min((m0 + Cfg::kBlockM + BLOCK_N - 1) / BLOCK_N, n_k_tiles) : n_k_tiles;
@@ -142,8 +143,8 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
   constexpr int SROWS = SPLIT ? BLOCK_N / 2 : BLOCK_N;
   RotStage<D, SROWS, NT> kst;
   CopyStage<D, SROWS, NT, Cfg::kVPad> vst;
-  kst.load(kg, p.cos, p.sin, p.fstride, 0, N);
-  vst.load(vg, 0, N);
+  kst.load(kg, p.cos, p.sin, p.fstride, 0, N, k_rb);
+  vst.load(vg, 0, N, v_rb);
 
   // ---- Q rows of this wave: load, rotate, keep as the B operand (through a wave-private LDS tile, so that the
   // global loads touch whole row segments) ---------------------------------------------------------------------
@@ -151,7 +152,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
   u32x4 qb[KC];
   {
     WaveRows<D, true> qrows;
-    qrows.load(qg, p.cos, p.sin, p.fstride, m0 + wave * 32, N);
+    qrows.load(qg, p.cos, p.sin, p.fstride, m0 + wave * 32, N, threadIdx.x % kWave, q_rb);
     // the rotated Q rows carry sm_scale * log2(e), as in every other kernel of the operator: forward and backward then
     // see the same rounded operands, and the same scores
     qrows.park(qb, reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride, nullptr, 0, 0, p.qk_scale);
@@ -182,13 +183,13 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
   kst.store_rows(ks(0));
   vst.store_rows(vs(0));
   if constexpr (SPLIT) {
-    kst.load(kg, p.cos, p.sin, p.fstride, SROWS, N);
-    vst.load(vg, SROWS, N);
+    kst.load(kg, p.cos, p.sin, p.fstride, SROWS, N, k_rb);
+    vst.load(vg, SROWS, N, v_rb);
     kst.store_rows(ks(0) + RowTile<D>::off(SROWS, 0));
     vst.store_rows(vs(0) + RowTile<D, Cfg::kVPad>::off(SROWS, 0));
   }
-  kst.load(kg, p.cos, p.sin, p.fstride, BLOCK_N, N);
-  vst.load(vg, BLOCK_N, N);
+  kst.load(kg, p.cos, p.sin, p.fstride, BLOCK_N, N, k_rb);
+  vst.load(vg, BLOCK_N, N, v_rb);
   __syncthreads();
 
   const int wave_q_lo = m0 + wave * 32, wave_q_hi = wave_q_lo + 31;
@@ -202,15 +203,15 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
       kst.store_rows(ks(t + 1));
       vst.store_rows(vs(t + 1));
       const int next_rows = SPLIT ? n0 + BLOCK_N + SROWS : n0 + 2 * BLOCK_N;   // SPLIT: the other half of tile t+1
-      kst.load(kg, p.cos, p.sin, p.fstride, next_rows, N);
-      vst.load(vg, next_rows, N);
+      kst.load(kg, p.cos, p.sin, p.fstride, next_rows, N, k_rb);
+      vst.load(vg, next_rows, N, v_rb);
     };
     auto stage_second_half = [&]() {   // SPLIT only: second half of tile t+1 to LDS, first half of tile t+2 requested
       if constexpr (SPLIT) {
         kst.store_rows(ks(t + 1) + RowTile<D>::off(SROWS, 0));
         vst.store_rows(vs(t + 1) + RowTile<D, Cfg::kVPad>::off(SROWS, 0));
-        kst.load(kg, p.cos, p.sin, p.fstride, n0 + 2 * BLOCK_N, N);
-        vst.load(vg, n0 + 2 * BLOCK_N, N);
+        kst.load(kg, p.cos, p.sin, p.fstride, n0 + 2 * BLOCK_N, N, k_rb);
+        vst.load(vg, n0 + 2 * BLOCK_N, N, v_rb);
       }
     };
     auto k_operand = [&](int half, int kc) {

@@ -146,7 +146,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
     if (i >= total) return false;
     const int kvs = kv_slab(i % p.BH, p.H, p.Hkv);
     l_kg = p.k_rot + (int64_t)kvs * N * D;
-    l_vg = p.v + (int64_t)kvs * N * D;
+    l_vg = p.v_slab(kvs);
     l_tiles = tiles_of(p.num_m_blocks - 1 - i / p.BH);
     return true;
   };
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
       l_tile = 0;
     }   // else: past the last tile of the last item; the same tile is requested again and never used
     kst.load(l_kg, l_tile * BLOCK_N, N);
-    vst.load(l_vg, l_tile * BLOCK_N, N);
+    vst.load(l_vg, l_tile * BLOCK_N, N, (uint32_t)p.v_sn * 2);
   };
 
   // LDS ring: K buffers at [0, 2 * kKBytes), V buffers behind them.  The buffers rotate by renaming byte offsets (no
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
   auto request_q = [&](int i) __attribute__((always_inline)) {
     const int bh = i % p.BH, m0 = (p.num_m_blocks - 1 - i / p.BH) * Cfg::kBlockM;
     const int l = opaque_lane();
-    qrows.load(p.q + (int64_t)bh * N * D, p.cos, p.sin, p.fstride, m0 + rb * 32, N, l);
+    qrows.load(p.q_slab(bh), p.cos, p.sin, p.fstride, m0 + rb * 32, N, l, (uint32_t)p.q_sn * 2);
     kvec = reinterpret_cast<const uint32_t*>(p.tile_kmax)[(int64_t)kv_slab(bh, p.H, p.Hkv) * n_k_tiles + min(l, n_k_tiles - 1)];
   };
   auto take_q = [&](int i) __attribute__((always_inline)) {
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(2, 2)
   COROPE_ISTAMP(0);
   load_item(0);
   kst.load(l_kg, 0, N);
-  vst.load(l_vg, 0, N);
+  vst.load(l_vg, 0, N, (uint32_t)p.v_sn * 2);
   request_q(item);
   take_q(item);
   kst.store_rows(lds_at(koff_cur));

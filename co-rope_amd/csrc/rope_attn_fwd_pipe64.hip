@@ -146,7 +146,7 @@ __global__ __launch_bounds__(pipe64::Cfg<D>::kThreads) __attribute__((amdgpu_wav
     if (i >= total) return false;
     const int kvs = kv_slab(i % p.BH, p.H, p.Hkv);
     l_kg = p.k_rot + (int64_t)kvs * N * D;
-    l_vg = p.v + (int64_t)kvs * N * D;
+    l_vg = p.v_slab(kvs);
     l_tiles = tiles_of(p.num_m_blocks - 1 - i / p.BH);
     return true;
   };
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(pipe64::Cfg<D>::kThreads) __attribute__((amdgpu_wav
       l_tile = 0;
     }   // else: past the last tile of the last item; the same tile is requested again and never used
     kst.load(l_kg, l_tile * BLOCK_N, N);
-    vst.load(l_vg, l_tile * BLOCK_N, N);
+    vst.load(l_vg, l_tile * BLOCK_N, N, (uint32_t)p.v_sn * 2);
   };
 
   // LDS ring: K buffers at [0, 2 * kKBytes), V buffers behind them; the buffers rotate by renaming byte offsets.
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(pipe64::Cfg<D>::kThreads) __attribute__((amdgpu_wav
   auto request_q = [&](int i, auto b_c) __attribute__((always_inline)) {
     constexpr int b = decltype(b_c)::value;
     const int bh = i % p.BH, m0 = (p.num_m_blocks - 1 - i / p.BH) * C::kBlockM;
-    qrows[b].load(p.q + (int64_t)bh * N * D, p.cos, p.sin, p.fstride, m0 + rb[b] * 32, N, opaque_lane());
+    qrows[b].load(p.q_slab(bh), p.cos, p.sin, p.fstride, m0 + rb[b] * 32, N, opaque_lane(), (uint32_t)p.q_sn * 2);
   };
   auto request_kvec = [&](int i) __attribute__((always_inline)) {
     const int bh = i % p.BH;
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(pipe64::Cfg<D>::kThreads) __attribute__((amdgpu_wav
   COROPE_ISTAMP(0);
   load_item(0);
   kst.load(l_kg, 0, N);
-  vst.load(l_vg, 0, N);
+  vst.load(l_vg, 0, N, (uint32_t)p.v_sn * 2);
   request_q(item, B0{});
   request_q(item, B1{});
   request_kvec(item);

@@ -26,18 +26,19 @@ __global__ __launch_bounds__(kRotThreads) void rope_rotate_kernel(const uint16_t
                                                                   const float* __restrict__ cosp,
                                                                   const float* __restrict__ sinp, int64_t fstride,
                                                                   uint16_t* __restrict__ y, float* __restrict__ tile_max,
-                                                                  int N, int n_tiles, float out_scale) {
+                                                                  int N, int n_tiles, float out_scale, int H, int64_t x_sb,
+                                                                  int64_t x_sh, int x_sn) {
   using Stage = RotStage<D, kRotRows, kRotThreads, SCALED>;
   constexpr int kChunks = Stage::kChunks;
   __shared__ float wave_max[kRotThreads / kWave];
   const int tile = blockIdx.x % n_tiles, bh = blockIdx.x / n_tiles;
   const int row0 = tile * kRotRows;
-  const uint16_t* xg = x + (int64_t)bh * N * D;
+  const uint16_t* xg = x + (bh / H) * x_sb + (bh % H) * x_sh;   // the source may be a strided view; y is contiguous
   uint16_t* yg = y + (int64_t)bh * N * D;
 
   Stage st;
   st.out_scale = out_scale;
-  st.load(xg, cosp, sinp, fstride, row0, N);
+  st.load(xg, cosp, sinp, fstride, row0, N, (uint32_t)x_sn * 2);
   float best = 0.f;
 #pragma unroll
   for (int it = 0; it < Stage::kIters; ++it) {
@@ -75,13 +76,20 @@ __global__ __launch_bounds__(kRotThreads) void rope_rotate_kernel(const uint16_t
 }
 
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
-                              float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale) {
+                              float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale, int H, int64_t x_sb,
+                              int64_t x_sh, int x_sn) {
   if (D != 64 && D != 128) return hipErrorInvalidValue;
+  if (x_sn == 0) {   // contiguous (BH, N, D)
+    H = 1;
+    x_sb = (int64_t)N * D;
+    x_sh = 0;
+    x_sn = D;
+  }
   const int n_tiles = (N + kRotRows - 1) / kRotRows;
   dim3 grid((unsigned)n_tiles * BH);   // one axis: the second grid axis stops at 65535 slabs
 #define COROPE_ROT(DD, SS)                                                                                             \
   hipLaunchKernelGGL((rope_rotate_kernel<DD, SS>), grid, dim3(kRotThreads), 0, stream, x, cosp, sinp, fstride, y, tile_max, \
-                     N, n_tiles, out_scale)
+                     N, n_tiles, out_scale, H, x_sb, x_sh, x_sn)
   if (D == 128) {
     if (out_scale == 1.f) COROPE_ROT(128, false); else COROPE_ROT(128, true);
   } else {

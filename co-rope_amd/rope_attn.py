@@ -9,6 +9,8 @@ other implementation behind this module.  Tensors are bfloat16 or float16 (the r
 the same kernel sources built for fp16 elements)."""
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -116,22 +118,56 @@ def use_rotated_path(N, D, training):
     return D <= _ROTATED_PATH_MAX_D and (N >= TWO_LAUNCH_MIN_N or N * D >= TRAIN_ROTATED_MIN_ND)
 
 
+def _view_strides(t):
+    """(batch, head, row) strides in elements if the kernels can read t where it lies -- last dimension contiguous, rows
+    16-byte aligned and at least D apart, as the reference's forward reads q and k through their strides
+    (fused_rope_attn.py:709-710) -- else None."""
+    sb, sh, sn, sd = t.stride()
+    d = t.shape[-1]
+    if sd != 1 or sn < d or min(sb, sh) < 0 or sb % 8 or sh % 8 or sn % 8 or t.data_ptr() % 16 or t.shape[2] * sn * 2 >= 1 << 32:
+        return None
+    return (ctypes.c_int64 * 3)(sb, sh, sn)
+
+
 def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, keep_rotated=False):
     """Runs the forward kernels; returns (o, M, fc, fs, rotated) with the tables in the form the kernels were given.
-    ``rotated`` is (q_rot, k_rot) when ``keep_rotated`` was asked for and the two-launch path ran, else None."""
+    ``rotated`` is (q_rot, k_rot) when ``keep_rotated`` was asked for and the two-launch path ran, else None.
+    q, k, v may be strided views (a (B, N, H, D) tensor seen as (B, H, N, D), a slice of a fused projection): they are read
+    where they lie when their layout allows it, else copied."""
     lib = _lib.load()
     fc, fs = _freq_table(freqs_cos), _freq_table(freqs_sin)
     if fc.stride(0) != fs.stride(0):
         fc, fs = fc.contiguous(), fs.contiguous()
     B, H, N, D = q.shape
-    o = torch.empty_like(q)
+    strides = None
+    if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+        strides = tuple(_view_strides(t) for t in (q, k, v))
+        if any(st is None for st in strides) or D > _ROTATED_PATH_MAX_D:
+            q, k, v, strides = q.contiguous(), k.contiguous(), v.contiguous(), None
+    o = torch.empty(q.shape, device=q.device, dtype=q.dtype)
     M = torch.empty((B, H, N), device=q.device, dtype=torch.float32)
     if two_launch is None:
         two_launch = use_rotated_path(N, D, training=keep_rotated)
     rotated = None
     Hkv = k.shape[1]
     with _on_device(q):
-        if q.dtype == torch.float16:
+        if strides is not None:
+            fp16 = q.dtype == torch.float16
+            if fp16 and keep_rotated and FP16_TRAINING_FORWARD != "fast":
+                two_launch = False
+            q_rot = torch.empty(q.shape, device=q.device, dtype=q.dtype) if (two_launch and keep_rotated) else None
+            k_rot = torch.empty(k.shape, device=q.device, dtype=q.dtype) if two_launch else None
+            kmax = torch.empty((B, Hkv, (N + 63) // 64), device=q.device, dtype=torch.float32) if two_launch else None
+            rc = lib.corope_rope_attn_fwd_strided(q.data_ptr(), strides[0], k.data_ptr(), strides[1], v.data_ptr(), strides[2],
+                                                  fc.data_ptr(), fs.data_ptr(), fc.stride(0), o.data_ptr(), M.data_ptr(),
+                                                  q_rot.data_ptr() if q_rot is not None else None,
+                                                  k_rot.data_ptr() if k_rot is not None else None,
+                                                  kmax.data_ptr() if kmax is not None else None, B, H, Hkv, N, D,
+                                                  float(sm_scale), int(bool(causal)), int(fp16), _stream_ptr(q))
+            _lib.check(rc, "corope_rope_attn_fwd_strided")
+            if q_rot is not None:
+                rotated = (q_rot, k_rot)
+        elif q.dtype == torch.float16:
             # the reference's dtype: the same two forms (the two-launch one with bf16 probabilities against a V converted
             # to bf16 on its way into LDS); one entry point covers them, grouped-query K/V included
             if keep_rotated and FP16_TRAINING_FORWARD != "fast":
@@ -192,17 +228,18 @@ class _FusedRopeAttn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, causal, sm_scale, freqs_cos, freqs_sin, warp_specialize=True):
         _check_inputs(q, k, v, freqs_cos, freqs_sin)
-        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         B, H, N, D = q.shape
+        training = any(ctx.needs_input_grad[:3])
+        if training:
+            v = v.contiguous()         # the backward kernels read v row-major; q and k they read as the forward left them
         # when a gradient will be asked for, the forward keeps its rotated q and k for the backward and the originals
         # are not saved (the reference saves q and k, fused_rope_attn.py:718, and re-rotates them in its backward)
-        o, M, fc, fs, rotated = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin,
-                                         keep_rotated=any(ctx.needs_input_grad[:3]))
+        o, M, fc, fs, rotated = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, keep_rotated=training)
         ctx.rotated = rotated is not None
         if ctx.rotated:
             ctx.save_for_backward(rotated[0], rotated[1], v, o, M, fc, fs)
         else:
-            ctx.save_for_backward(q, k, v, o, M, fc, fs)
+            ctx.save_for_backward(q.contiguous(), k.contiguous(), v.contiguous(), o, M, fc, fs)
         ctx.sm_scale = float(sm_scale)
         ctx.HEAD_DIM = D
         ctx.causal = bool(causal)
@@ -282,7 +319,6 @@ def rope_attn_forward_with_lse(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, 
     """Forward only, returning (O, M) where M is the saved base-2 log-sum-exp statistic (B, H, N) fp32.
     ``two_launch`` forces (True / False) or leaves to the length rule (None) the choice of forward path."""
     _check_inputs(q, k, v, freqs_cos, freqs_sin)
-    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     o, M, _, _, _ = _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch)
     return o, M
 

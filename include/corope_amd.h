@@ -250,6 +250,18 @@ int corope_rope_attn_bwd_f16(const void *q, const void *k, int prerotated, const
                              int B, int H, int Hkv, int N, int D, float sm_scale, int causal,
                              void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The forward on q, k, v that are strided views: `*_strides` = elements between batches, heads and rows of the
+ * (B, H or Hkv, N, D) tensor (the last dimension contiguous; every stride a multiple of 8 elements, rows at least D apart) --
+ * e.g. (N*H*D, D, H*D) for a (B, N, H, D) tensor viewed as (B, H, N, D).  The reference's forward kernel takes the strides
+ * of q and k the same way (fused-rope/fused_rope_attn.py:709-710; its V and O go through contiguous descriptors, :245-251);
+ * o, lse and the optional scratch are contiguous.  k_rot == NULL: single launch; k_rot != NULL: the two-launch form as
+ * in corope_rope_attn_fwd_gqa (q_rot may be NULL); fp16 != 0: fp16 tensors as in corope_rope_attn_fwd_f16, else bf16. */
+int corope_rope_attn_fwd_strided(const void *q, const int64_t *q_strides, const void *k, const int64_t *k_strides,
+                                 const void *v, const int64_t *v_strides,
+                                 const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,
+                                 void *o, float *lse, void *q_rot, void *k_rot, float *tile_kmax,
+                                 int B, int H, int Hkv, int N, int D, float sm_scale, int causal, int fp16, void *stream);
+
 /* Grouped-query form of the operator: q (B,Hq,N,D), k and v (B,Hkv,N,D), Hq a multiple of Hkv; query head h reads
  * key/value head h / (Hq/Hkv); dk and dv (B,Hkv,N,D) are sums over the query heads of their group (the key block's
  * workgroup sweeps all of them, no atomics).  The reference's RoPE operator requires Hq == Hkv

@@ -252,3 +252,18 @@ def test_missing_library_fails_loudly(pkg, monkeypatch):
     monkeypatch.setattr(pkg._lib, "LIB_PATH", "/nonexistent/libcorope_amd.so")
     with pytest.raises(pkg._lib.CoRopeLibraryError):
         pkg._lib.load()
+
+
+def test_strided_forward_argument_checks(pkg):
+    """Strides are checked before any launch: multiples of 8 elements, rows at least D apart, slices below 4 GiB."""
+    import ctypes
+    lib = pkg._lib.load()
+    ok = 4096
+    arr = lambda *x: (ctypes.c_int64 * 3)(*x)
+    good = arr(8 * 64 * 100, 64, 8 * 64)
+    tail = (ok, ok, 64, ok, ok, None, None, None, 1, 8, 8, 100, 64, 1.0, 1, 0, None)
+    for bad in (arr(8 * 64 * 100, 64, 32), arr(8 * 64 * 100, 60, 8 * 64), arr(-512, 64, 512), arr(0, 0, 1 << 31)):
+        rc = lib.corope_rope_attn_fwd_strided(ok, bad, ok, good, ok, good, *tail)
+        assert rc in (-1, -2) and "stride" in pkg._lib.last_error(), list(bad)
+    assert lib.corope_rope_attn_fwd_strided(ok, None, ok, good, ok, good, *tail) == -1
+    assert lib.corope_rope_attn_fwd_strided(ok, good, ok, good, ok + 2, good, *tail) == -3

@@ -226,3 +226,33 @@ def test_two_launch_softmax_modes(pkg, tile_rows, case, causal):
     # (an output that is the small remainder of cancelling terms carries the absolute error of those terms: half the
     # parity bar as the fixed part)
     assert ((o - o1).abs() <= (3e-2 if hot else 1e-2) + o.abs() / 64).all() and (M - M1).abs().max() * LN2 <= (1e-2 if hot else 1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,Hkv,N,D", [(2, 4, 4, 300, 64), (1, 8, 2, 1100, 128), (2, 3, 3, 1024, 128)])
+def test_strided_views_are_read_where_they_lie(pkg, B, H, Hkv, N, D, dtype):
+    """q, k, v as slices of one fused (B, N, Hq + 2 Hkv, D) projection seen as (B, H, N, D) -- the layout a model hands
+    over -- give bit for bit what their contiguous copies give, forward (both forms) and backward, and no copy of q or k
+    is made on the way (the reference's forward reads q and k through their strides too, fused_rope_attn.py:709-710)."""
+    dev = torch.device("cuda:0")
+    fused = seeded((B, N, H + 2 * Hkv, D), 5).to(dev, dtype)
+    q, k, v = (fused[:, :, a:b].transpose(1, 2) for a, b in ((0, H), (H, H + Hkv), (H + Hkv, H + 2 * Hkv)))
+    assert not q.is_contiguous() and q.shape == (B, H, N, D)
+    c, s = (t.to(dev) for t in O.precompute_freqs_cis(D, N))
+    scale = 1 / math.sqrt(D)
+    for two_launch in (False, True):
+        o1, m1 = pkg.rope_attn_forward_with_lse(q, k, v, True, scale, c, s, two_launch)
+        o2, m2 = pkg.rope_attn_forward_with_lse(q.contiguous(), k.contiguous(), v.contiguous(), True, scale, c, s, two_launch)
+        torch.cuda.synchronize()
+        assert o1.is_contiguous() and torch.equal(o1, o2) and torch.equal(m1, m2), two_launch
+    g = seeded((B, H, N, D), 9).to(dev, dtype)
+    grads = []
+    for views in (True, False):
+        f = fused.clone().requires_grad_(True)
+        qq, kk, vv = (f[:, :, a:b].transpose(1, 2) for a, b in ((0, H), (H, H + Hkv), (H + Hkv, H + 2 * Hkv)))
+        if not views:
+            qq, kk, vv = qq.contiguous(), kk.contiguous(), vv.contiguous()
+        pkg.attention(qq, kk, vv, True, scale, c, s).backward(g)
+        grads.append(f.grad)
+    torch.cuda.synchronize()
+    assert torch.equal(grads[0], grads[1])
