@@ -283,7 +283,11 @@ def bench_sweep(args):
     dtype = torch.float16 if args.dtype == "fp16" else torch.bfloat16
     pkg.rope_attn.FP16_TRAINING_FORWARD = args.fp16_forward
     shapes = [s for s in SWEEP if args.only is None or s[4] in args.only.split(",")]
+    if args.shape is not None:
+        B, H, N, D = (int(x) for x in args.shape.split(","))
+        shapes = [(B, H, N, D, f"B{B}-H{H}-N{N}-D{D}")]
     for (B, H, N, D, name) in shapes:
+        sm_scale = args.sm_scale if args.sm_scale is not None else 0.5   # the reference harness's value
         g = torch.Generator().manual_seed(0)
         q, k, v, do = (torch.randn(B, H, N, D, generator=g).to(dev, dtype) for _ in range(4))
         cos, sin = pkg.rope_freqs_device(D, N, 10000.0, device=dev)
@@ -300,15 +304,15 @@ def bench_sweep(args):
                     stats[key + "_flushed_min_ms"], stats[key + "_flushed_max_ms"] = round(fl, 4), round(fh, 4)
             return med
 
-        f_ms = timed(lambda: pkg.attention(q, k, v, True, 0.5, cos, sin), "fwd")
-        o = pkg.attention(q, k, v, True, 0.5, cos, sin)
+        f_ms = timed(lambda: pkg.attention(q, k, v, True, sm_scale, cos, sin), "fwd")
+        o = pkg.attention(q, k, v, True, sm_scale, cos, sin)
 
         def clear_grads():   # otherwise every call after the first also runs three accumulate-into-.grad kernels
             q.grad = k.grad = v.grad = None
 
         b_ms = timed(lambda: (clear_grads(), o.backward(do, retain_graph=True)), "bwd")
         ff, fb = attention_flops(B, H, N, D, "fwd"), attention_flops(B, H, N, D, "bwd")
-        row = {"config": name, "B": B, "H": H, "N": N, "D": D, "dtype": args.dtype, "fwd_ms": round(f_ms, 4),
+        row = {"config": name, "B": B, "H": H, "N": N, "D": D, "dtype": args.dtype, "sm_scale": sm_scale, "fwd_ms": round(f_ms, 4),
                "fwd_tflops": round(ff / f_ms * 1e-9, 1), "bwd_ms": round(b_ms, 4), "bwd_tflops": round(fb / b_ms * 1e-9, 1)}
         row.update(stats)
         if args.lanes:
@@ -321,8 +325,8 @@ def bench_sweep(args):
             rot_ms = timed(lambda: (pkg.rope_rotate(qd, cos, sin), pkg.rope_rotate(kd, cos, sin)))
             qr = pkg.rope_rotate(qd, cos, sin).requires_grad_(True)
             kr = pkg.rope_rotate(kd, cos, sin).requires_grad_(True)
-            uf_ms = rot_ms + timed(lambda: pkg.attention(qr, kr, v, True, 0.5, one, zero))
-            ou = pkg.attention(qr, kr, v, True, 0.5, one, zero)
+            uf_ms = rot_ms + timed(lambda: pkg.attention(qr, kr, v, True, sm_scale, one, zero))
+            ou = pkg.attention(qr, kr, v, True, sm_scale, one, zero)
 
             def clear_rot_grads():
                 qr.grad = kr.grad = v.grad = None
@@ -333,8 +337,8 @@ def bench_sweep(args):
                         "calc_sim_vs_unfused": round(calc_sim(o.detach(), ou.detach()), 8)})
             try:
                 sdpa = torch.nn.functional.scaled_dot_product_attention
-                sf_ms = rot_ms + timed(lambda: sdpa(qr, kr, v, is_causal=True, scale=0.5))
-                osd = sdpa(qr, kr, v, is_causal=True, scale=0.5)
+                sf_ms = rot_ms + timed(lambda: sdpa(qr, kr, v, is_causal=True, scale=sm_scale))
+                osd = sdpa(qr, kr, v, is_causal=True, scale=sm_scale)
                 sb_ms = rot_ms + timed(lambda: (clear_rot_grads(), osd.backward(do, retain_graph=True)))
                 row.update({"sdpa_fwd_ms": round(sf_ms, 4), "sdpa_bwd_ms": round(sb_ms, 4),
                             "fwd_speedup_vs_sdpa": round(sf_ms / f_ms, 3), "bwd_speedup_vs_sdpa": round(sb_ms / b_ms, 3)})
@@ -633,6 +637,8 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"], help="with --sweep: element type of q, k, v, dO")
     ap.add_argument("--fp16-forward", default="exact", choices=["exact", "fast"],
                     help="with --sweep --dtype fp16: rope_attn.FP16_TRAINING_FORWARD (the forward of a differentiated call)")
+    ap.add_argument("--sm-scale", type=float, default=None, help="with --sweep: softmax scale instead of the reference harness's 0.5")
+    ap.add_argument("--shape", default=None, help="with --sweep: one shape B,H,N,D of your own instead of the 19 (e.g. 2,16,4096,256)")
     ap.add_argument("--only", default=None, help="with --sweep: comma-separated names of the shapes to run")
     ap.add_argument("--flush", action="store_true",
                     help="with --sweep: also time every call on flushed caches (a 512 MiB buffer overwritten before each call)")

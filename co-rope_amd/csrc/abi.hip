@@ -69,16 +69,6 @@ int check_ptrs(const char* what, std::initializer_list<const void*> ptrs) {
   return COROPE_OK;
 }
 
-// Head dim 256 is built for the kernels that take q and k as they are (single-launch forward; dV, dK and dQ that rotate
-// while they stage): entry points that work on rotated copies say so instead of launching.
-int rotated_copies_built(const char* what, int D) {
-  if (D > 128)
-    return fail(COROPE_E_UNSUPPORTED,
-                "%s: head dim %d runs on the original operands only (corope_rope_attn_fwd, corope_rope_attn_bwd and its "
-                "parts), not on rotated copies or a workspace", what, D);
-  return COROPE_OK;
-}
-
 int launch_status(const char* what, hipError_t e) {
   if (e == hipSuccess) return COROPE_OK;
   return fail(COROPE_E_LAUNCH, "%s: HIP error %d (%s)", what, (int)e, hipGetErrorString(e));
@@ -190,10 +180,6 @@ int rope_attn_fwd_impl(const char* what, const void* q, const void* k, const voi
   p.tile_kmax = tile_kmax;
   p.q_rot_out = static_cast<uint16_t*>(q_rot_out);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (workspace != nullptr || k_rot != nullptr) {
-    rc = rotated_copies_built(what, D);
-    if (rc) return rc;
-  }
   if (workspace != nullptr) {
     rc = check_ptrs(what, {workspace});
     if (rc) return rc;
@@ -316,7 +302,6 @@ int corope_rope_attn_fwd_train(const void* q, const void* k, const void* v, cons
                                int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 0);
   if (rc) return rc;
-  if ((rc = rotated_copies_built("rope_attn_fwd_train", D))) return rc;
   rc = check_ptrs("rope_attn_fwd_train", {q, k, v, freqs_cos, freqs_sin, o, lse, q_rot, k_rot});
   if (rc) return rc;
   if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
@@ -331,8 +316,6 @@ int corope_rope_attn_fwd_train(const void* q, const void* k, const void* v, cons
 int corope_rope_rotate(const void* x, const float* freqs_cos, const float* freqs_sin, int64_t freq_row_stride, void* y,
                        float* tile_max, int B, int H, int N, int D, float scale, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, 1.f, 0);
-  if (rc) return rc;
-  rc = rotated_copies_built("rope_rotate", D);
   if (rc) return rc;
   rc = check_ptrs("rope_rotate", {x, freqs_cos, freqs_sin, y});
   if (rc) return rc;
@@ -384,7 +367,6 @@ int bwd_dv_impl(const char* what, bool prerot, const void* q, const void* k, con
                 int D, float sm_scale, int causal, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
-  if (prerot && (rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q, k, d_o, lse, freqs_cos, freqs_sin, dv});
   if (rc) return rc;
   corope::BwdParams p = make_bwd(q, k, nullptr, nullptr, d_o, lse, nullptr, freqs_cos, freqs_sin, freq_row_stride,
@@ -398,7 +380,6 @@ int bwd_dk_impl(const char* what, bool prerot, const void* q, const void* k, con
                 int64_t freq_row_stride, void* dk, int B, int H, int N, int D, float sm_scale, int causal, void* stream) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
-  if (prerot && (rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dk});
   if (rc) return rc;
   corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
@@ -414,7 +395,6 @@ int bwd_dq_impl(const char* what, bool prerot, const void* q, const void* k, con
                 const void* o = nullptr) {
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
-  if (prerot && (rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dq});
   if (rc) return rc;
   if (o != nullptr && !aligned16(o)) return fail(COROPE_E_ALIGN, "%s: pointer %p is not 16-byte aligned", what, o);
@@ -487,7 +467,6 @@ int corope_rope_attn_bwd_dkdv_prerotated(const void* q_rot, const void* k_rot, c
   const char* what = "rope_attn_bwd_dkdv_prerotated";
   int rc = corope_rope_attn_check(B, H, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
-  if ((rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q_rot, k_rot, v, d_o, lse, delta, freqs_cos, freqs_sin, dk, dv});
   if (rc) return rc;
   corope::BwdParams p = make_bwd(q_rot, k_rot, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
@@ -529,7 +508,6 @@ int corope_rope_attn_bwd_prerotated(const void* q_rot, const void* k_rot, const 
   int rc = validate_bwd("rope_attn_bwd_prerotated", B, H, N, D, freq_row_stride, sm_scale,
                         {q_rot, k_rot, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv});
   if (rc) return rc;
-  if ((rc = rotated_copies_built("rope_attn_bwd_prerotated", D))) return rc;
   rc = corope_rope_attn_bwd_dq_prerotated(q_rot, k_rot, v, o, d_o, lse, delta, freqs_cos, freqs_sin, freq_row_stride, dq, B,
                                           H, N, D, sm_scale, causal, stream);
   if (rc) return rc;
@@ -549,7 +527,6 @@ int corope_rope_attn_bwd_ws(const void* q, const void* k, const void* v, const v
   int rc = validate_bwd("rope_attn_bwd_ws", B, H, N, D, freq_row_stride, sm_scale,
                         {q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv, workspace});
   if (rc) return rc;
-  if ((rc = rotated_copies_built("rope_attn_bwd_ws", D))) return rc;
   if (workspace_bytes < 2 * bwd_ws_tensor_bytes(B, H, N, D))
     return fail(COROPE_E_BADARG, "rope_attn_bwd_ws: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
                 (long long)(2 * bwd_ws_tensor_bytes(B, H, N, D)));
@@ -575,7 +552,6 @@ int corope_rope_attn_fwd_gqa(const void* q, const void* k, const void* v, const 
   }
   int rc = corope_rope_attn_check(B, Hq, N, D, freq_row_stride, sm_scale, 0);
   if (rc) return rc;
-  if ((rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q, k, v, freqs_cos, freqs_sin, o, lse, k_rot});
   if (rc) return rc;
   if (q_rot != nullptr && !aligned16(q_rot)) return fail(COROPE_E_ALIGN, "%s: q_rot %p is not 16-byte aligned", what, q_rot);
@@ -596,7 +572,6 @@ int corope_rope_attn_bwd_gqa(const void* q, const void* k, int prerotated, const
   if (Hkv <= 0 || Hq % Hkv != 0) return fail(COROPE_E_BADARG, "%s: Hq=%d is not a multiple of Hkv=%d", what, Hq, Hkv);
   int rc = corope_rope_attn_check(B, Hq, N, D, freq_row_stride, sm_scale, 1);
   if (rc) return rc;
-  if (prerotated && (rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {q, k, v, o, d_o, lse, delta, freqs_cos, freqs_sin, dq, dk, dv});
   if (rc) return rc;
   rc = corope_rope_attn_bwd_preprocess(o, d_o, delta, B, Hq, N, D, stream);
@@ -646,7 +621,6 @@ int corope_rope_attn_fwd_f16(const void* q, const void* k, const void* v, const 
   if (k_rot == nullptr) return launch_status(what, corope_f16::launch_rope_attn_fwd(p, D, causal != 0, st));
   // two launches: K rotated once into k_rot (with the largest key norm of every 64-key tile), then the attention kernel
   // on it, which leaves its rotated, scaled Q rows in q_rot if asked to (the operands of a backward on rotated copies)
-  if ((rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {k_rot});
   if (rc) return rc;
   if (q_rot != nullptr && !aligned16(q_rot)) return fail(COROPE_E_ALIGN, "%s: q_rot %p is not 16-byte aligned", what, q_rot);
@@ -674,7 +648,6 @@ int corope_rope_attn_bwd_f16(const void* q, const void* k, int prerotated, const
                                  sm_scale);
   p.Hkv = Hkv;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if ((workspace != nullptr || prerotated) && (rc = rotated_copies_built(what, D))) return rc;
   if (prerotated) {
     // q, k are the rotated copies a two-launch forward kept: the dQ kernel computes delta on its way, dK and dV come
     // from one kernel
@@ -754,7 +727,6 @@ int corope_rope_attn_fwd_strided(const void* q, const int64_t* q_strides, const 
   if (k_rot == nullptr)
     return launch_status(what, fp16 ? corope_f16::launch_rope_attn_fwd(p, D, causal != 0, st)
                                     : corope::launch_rope_attn_fwd(p, D, causal != 0, st));
-  if ((rc = rotated_copies_built(what, D))) return rc;
   rc = check_ptrs(what, {k_rot});
   if (rc) return rc;
   if (q_rot != nullptr && !aligned16(q_rot)) return fail(COROPE_E_ALIGN, "%s: q_rot %p is not 16-byte aligned", what, q_rot);

@@ -664,9 +664,12 @@ template <bool DO_DV, bool DO_DK>
 static hipError_t launch_dkdv(const BwdParams& p, int D, bool causal, hipStream_t stream) {
   const bool pre = p.q_rot != nullptr && p.k_rot != nullptr;
 #define COROPE_DKDV(DD, CC, PP) launch_dkdv_cfg<DD, CC, DO_DV, DO_DK, PP>(p, stream)
-  if (D == 256) {   // separate dV and dK on the original operands only
-    if (pre || (DO_DV && DO_DK)) return hipErrorInvalidValue;
-    if constexpr (!(DO_DV && DO_DK)) return causal ? COROPE_DKDV(256, true, false) : COROPE_DKDV(256, false, false);
+  if (D == 256) {   // separate dV and dK only: the accumulators of both do not fit one wave
+    if (DO_DV && DO_DK) return hipErrorInvalidValue;
+    if constexpr (!(DO_DV && DO_DK)) {
+      if (pre) return causal ? COROPE_DKDV(256, true, true) : COROPE_DKDV(256, false, true);
+      return causal ? COROPE_DKDV(256, true, false) : COROPE_DKDV(256, false, false);
+    }
   }
   if (D == 128) {
     if (pre) return causal ? COROPE_DKDV(128, true, true) : COROPE_DKDV(128, false, true);
@@ -679,6 +682,10 @@ static hipError_t launch_dkdv(const BwdParams& p, int D, bool causal, hipStream_
 }
 
 hipError_t launch_bwd_dkdv_fused(const BwdParams& p, int D, bool causal, hipStream_t stream) {
+  if (D == 256) {   // two launches: the accumulators of dK and dV together do not fit a wave's registers at this head dim
+    if (hipError_t e = launch_dkdv<true, false>(p, D, causal, stream); e != hipSuccess) return e;
+    return launch_dkdv<false, true>(p, D, causal, stream);
+  }
   return launch_dkdv<true, true>(p, D, causal, stream);
 }
 
@@ -693,7 +700,7 @@ hipError_t launch_bwd_dk(const BwdParams& p, int D, bool causal, hipStream_t str
 hipError_t launch_bwd_dq(const BwdParams& p, int D, bool causal, hipStream_t stream) {
   const bool pre = p.q_rot != nullptr && p.k_rot != nullptr;
   if (D == 256) {
-    if (pre) return hipErrorInvalidValue;
+    if (pre) return causal ? launch_dq_cfg<256, true, true>(p, stream) : launch_dq_cfg<256, false, true>(p, stream);
     return causal ? launch_dq_cfg<256, true, false>(p, stream) : launch_dq_cfg<256, false, false>(p, stream);
   }
   if (D == 128) {

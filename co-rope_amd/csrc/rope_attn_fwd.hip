@@ -106,7 +106,9 @@ __device__ __forceinline__ float softmax_slow_half(const f32x16& sacc, u32x4 (&p
 // This kernel knows nothing about the keys in advance, so every half runs the fast pieces and is verified afterwards
 // (two data-dependent branches per tile); the two-launch forward in rope_attn_fwd_pipe.hip gets the same guarantee
 // from key norms computed beforehand and has no such branch.
-template <int D, int BLOCK_N, bool CAUSAL, int NW>
+// PREROT: the keys come from a copy that rope_rotate_kernel rotated beforehand (p.k_rot; no table reads and no rotation in
+// the loop), and the rotated, scaled query rows are also written to p.q_rot_out when that is given.
+template <int D, int BLOCK_N, bool CAUSAL, int NW, bool PREROT = false>
 __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<D>, kWavesPerSimd<D>))) void rope_attn_fwd_kernel(FwdParams p) {
   using Cfg = FwdCfg<D, BLOCK_N, NW>;
   static_assert(BLOCK_N == 64, "the slot schedule is written for two 32-key halves");
@@ -129,9 +131,9 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
   const int N = p.N;
 
   const uint16_t* qg = p.q_slab(bh);
-  const uint32_t q_rb = (uint32_t)p.q_sn * 2, k_rb = (uint32_t)p.k_sn * 2, v_rb = (uint32_t)p.v_sn * 2;   // bytes between rows
+  const uint32_t q_rb = (uint32_t)p.q_sn * 2, k_rb = PREROT ? D * 2 : (uint32_t)p.k_sn * 2, v_rb = (uint32_t)p.v_sn * 2;   // bytes between rows
   const int kvs = kv_slab(bh, p.H, p.Hkv);   // key/value slab of this query head
-  const uint16_t* kg = p.k_slab(kvs);
+  const uint16_t* kg = PREROT ? p.k_rot + (int64_t)kvs * N * D : p.k_slab(kvs);
   const uint16_t* vg = p.v_slab(kvs);
 
   const int n_k_tiles = (N + BLOCK_N - 1) / BLOCK_N;
@@ -141,7 +143,7 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
   // half has half an iteration to land.
   constexpr bool SPLIT = D > 128;
   constexpr int SROWS = SPLIT ? BLOCK_N / 2 : BLOCK_N;
-  RotStage<D, SROWS, NT> kst;
+  RopeStage<D, SROWS, NT, PREROT> kst;
   CopyStage<D, SROWS, NT, Cfg::kVPad> vst;
   kst.load(kg, p.cos, p.sin, p.fstride, 0, N, k_rb);
   vst.load(vg, 0, N, v_rb);
@@ -155,7 +157,8 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
     qrows.load(qg, p.cos, p.sin, p.fstride, m0 + wave * 32, N, threadIdx.x % kWave, q_rb);
     // the rotated Q rows carry sm_scale * log2(e), as in every other kernel of the operator: forward and backward then
     // see the same rounded operands, and the same scores
-    qrows.park(qb, reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride, nullptr, 0, 0, p.qk_scale);
+    qrows.park(qb, reinterpret_cast<uint16_t*>(smem) + wave * 32 * RowTile<D>::kStride,
+               PREROT && p.q_rot_out != nullptr ? p.q_rot_out + (int64_t)bh * N * D : nullptr, m0 + wave * 32, N, p.qk_scale);
   }
   __syncthreads();   // the K and V buffers below overlap the tiles the waves just used
   if constexpr (D > 128) {
@@ -321,10 +324,10 @@ __global__ __launch_bounds__(NW* kWave) __attribute__((amdgpu_waves_per_eu(kWave
 }
 
 // ---- host-side launch -----------------------------------------------------------------------------------------
-template <int D, int BLOCK_N, bool CAUSAL, int NW>
+template <int D, int BLOCK_N, bool CAUSAL, int NW, bool PREROT = false>
 static hipError_t launch_fwd_waves(FwdParams p, hipStream_t stream) {
   using Cfg = FwdCfg<D, BLOCK_N, NW>;
-  auto kern = rope_attn_fwd_kernel<D, BLOCK_N, CAUSAL, NW>;
+  auto kern = rope_attn_fwd_kernel<D, BLOCK_N, CAUSAL, NW, PREROT>;
   static std::atomic<uint64_t> lds_ok{0};
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), Cfg::kLdsBytes, lds_ok); e != hipSuccess) return e;
   p.num_m_blocks = (p.N + Cfg::kBlockM - 1) / Cfg::kBlockM;
@@ -345,6 +348,11 @@ hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStrea
   if (D == 128) return causal ? launch_fwd_cfg<128, 64, true>(p, stream) : launch_fwd_cfg<128, 64, false>(p, stream);
   if (D != 64) return hipErrorInvalidValue;
   return causal ? launch_fwd_cfg<64, 64, true>(p, stream) : launch_fwd_cfg<64, 64, false>(p, stream);
+}
+
+// Head dim 256 on a key copy rotated beforehand: the same kernel without the rotation in its loop.
+hipError_t launch_rope_attn_fwd_prerotated_d256(const FwdParams& p, bool causal, hipStream_t stream) {
+  return causal ? launch_fwd_waves<256, 64, true, 4, true>(p, stream) : launch_fwd_waves<256, 64, false, 4, true>(p, stream);
 }
 
 }  // namespace COROPE_NS

@@ -1,5 +1,6 @@
 // Fused half-layout-RoPE flash-attention forward for gfx950 on a K that rope_rotate_kernel rotated beforehand:
-// the form with 64 query rows per wave, one wave per SIMD.
+// the forms with one wave per SIMD -- 64 query rows per wave at head dim 128 (first part of the file), 32 query rows per
+// wave at head dim 256 (second part).
 //
 // Device counterpart of the reference's _attn_fwd / _attn_fwd_inner (fused-rope/fused_rope_attn.py:222-320, :48-138).
 // Same mathematics, MFMA operand layouts, softmax bookkeeping (lazy reference value against per-tile key-norm bounds)
@@ -498,6 +499,382 @@ __global__ __launch_bounds__(pipe64::Cfg<D>::kThreads) __attribute__((amdgpu_wav
   }
 }
 
+// ================================================================================ head dim 256
+// The same one-wave-per-SIMD form for head dim 256: a workgroup is 4 waves of 32 query rows (128-row items); a wave's Q
+// operand (64 registers) and O accumulators (128) live in the accumulation half of its 512 registers.  K and V tiles are 32
+// keys, so that a ring of 2 K + 3 V buffers and the waves' private tiles fit the LDS (151 KB), and a tile is what a 32-key
+// half is above: with 16 MFMAs per product a wave spends two slots on every tile,
+//
+//     slot A:  S(t)  = K(t) Q^T              |  softmax of S(t-1), second half   -> P(t-1)
+//     slot B:  O^T  += V(t-1)^T P(t-1)       |  softmax of S(t), first half
+//
+// one exponential half pair behind every second MFMA.  At the end of a tile the eight scores per lane that its softmax
+// still needs and the finished half of its P^T operand are moved to registers of their own (12 vector moves).
+namespace pipe64 {
+struct Cfg256 {
+  static constexpr int kD = 256;
+  static constexpr int kWaves = 4;
+  static constexpr int kThreads = kWaves * kWave;
+  static constexpr int kBlockM = kWaves * 32;
+  static constexpr int kBlockN = 32;
+  static constexpr int kVPad = 32;
+  static constexpr int kKBytes = RowTile<kD>::bytes(kBlockN);
+  static constexpr int kVBytes = RowTile<kD, kVPad>::bytes(kBlockN);
+  static constexpr int kKStages = 2, kVStages = 3;
+  static constexpr int kRingBytes = kKStages * kKBytes + kVStages * kVBytes;
+  static constexpr int kLdsBytes = kRingBytes + kWaves * WaveTile<kD>::kBytes;
+  static_assert(kLdsBytes <= 160 * 1024, "LDS of a compute unit");
+};
+}  // namespace pipe64
+
+template <bool CAUSAL>
+__global__ __launch_bounds__(pipe64::Cfg256::kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void rope_attn_fwd_pipe256_kernel(FwdParams p) {
+  using namespace pipe64;
+  using C = Cfg256;
+  constexpr int D = C::kD;
+  constexpr int BLOCK_N = C::kBlockN;
+  constexpr int NT = C::kThreads;
+  constexpr int M = D / 16;         // MFMAs per slot: contraction chunks of S^T = (16-key steps) x (32-column blocks) of PV
+  constexpr int NDB = D / 32;       // 32-column blocks of O
+  constexpr int RING = 4;           // LDS fragments in flight
+  constexpr int LSV = RowTile<D, C::kVPad>::kStride;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int lq = lane % 32, lh = lane / 32;
+  const int N = p.N;
+  [[maybe_unused]] constexpr int TT = (C::kWaves - 1) * kWave;   // stamping thread: first lane of the wave with the item's last rows
+  uint8_t* const wave_tile = smem + C::kRingBytes + wave * WaveTile<D>::kBytes;
+
+  // ---- the workgroup's list of items --------------------------------------------------------------------------------
+  const ItemList items;
+  const int total = p.num_m_blocks * p.BH;
+  auto item_at = [&](int r) { return items.at(r); };   // position in the heaviest-first order; >= total: none
+  const int n_k_tiles = (N + BLOCK_N - 1) / BLOCK_N;
+  const int n_norm_tiles = (N + 63) / 64;              // the rotation pass leaves one key-norm maximum per 64 keys
+  auto tiles_of = [&](int mb) {
+    return CAUSAL ? min((mb * C::kBlockM + C::kBlockM + BLOCK_N - 1) / BLOCK_N, n_k_tiles) : n_k_tiles;
+  };
+
+  // ---- the stream of K/V tiles: a cursor two tiles ahead of the tile being consumed -----------------------------------
+  CopyStage<D, BLOCK_N, NT, 8> kst;
+  CopyStage<D, BLOCK_N, NT, C::kVPad> vst;
+  int l_round = 0, l_tile = 0, l_tiles;
+  const uint16_t *l_kg, *l_vg;
+  auto load_item = [&](int r) {    // false: no such item
+    const int i = item_at(r);
+    if (i >= total) return false;
+    const int kvs = kv_slab(i % p.BH, p.H, p.Hkv);
+    l_kg = p.k_rot + (int64_t)kvs * N * D;
+    l_vg = p.v_slab(kvs);
+    l_tiles = tiles_of(p.num_m_blocks - 1 - i / p.BH);
+    return true;
+  };
+  auto load_next_tile = [&]() __attribute__((always_inline)) {   // moves the cursor on and requests that tile
+    if (l_tile + 1 < l_tiles) {
+      ++l_tile;
+    } else if (load_item(l_round + 1)) {
+      ++l_round;
+      l_tile = 0;
+    }   // else: past the last tile of the last item; the same tile is requested again and never used
+    kst.load(l_kg, l_tile * BLOCK_N, N);
+    vst.load(l_vg, l_tile * BLOCK_N, N, (uint32_t)p.v_sn * 2);
+  };
+
+  // LDS ring: K buffers at [0, 2 * kKBytes), V buffers behind them; the buffers rotate by renaming byte offsets.
+  constexpr int kVBase = C::kKStages * C::kKBytes;
+  int koff_cur = 0, koff_next = C::kKBytes;
+  int voff_prev = kVBase + 2 * C::kVBytes, voff_cur = kVBase, voff_next = kVBase + C::kVBytes;
+  auto rotate_buffers = [&]() __attribute__((always_inline)) {
+    int k = koff_cur; koff_cur = koff_next; koff_next = k;
+    int v = voff_prev; voff_prev = voff_cur; voff_cur = voff_next; voff_next = v;
+    koff_cur = __builtin_amdgcn_readfirstlane(koff_cur); koff_next = __builtin_amdgcn_readfirstlane(koff_next);
+    voff_prev = __builtin_amdgcn_readfirstlane(voff_prev); voff_cur = __builtin_amdgcn_readfirstlane(voff_cur);
+    voff_next = __builtin_amdgcn_readfirstlane(voff_next);
+  };
+  auto lds_at = [&](uint32_t byte_off) { return reinterpret_cast<uint16_t*>(smem + byte_off); };
+  const uint32_t k_lane_off = RowTile<D>::off(lq, 8 * lh) * 2;
+  const uint32_t v_lane_off = a_trans_lane_offset(LSV) * 2;
+  auto stage_next = [&]() __attribute__((always_inline)) {
+    int ko = koff_next, vo = voff_next;
+    asm volatile("" : "+s"(ko), "+s"(vo));
+    kst.store_rows(lds_at(ko));
+    vst.store_rows(lds_at(vo));
+    load_next_tile();
+  };
+
+  // ---- Q rows of an item: load, rotate, scale, keep as the B operand; the largest key norms of the item's first tiles
+  WaveRows<D, true> qrows;
+  u32x4 qb[M];   // as loaded (vector half of the register file): for the norm bound, then moved over into ...
+  u32x4 qa[M];   // ... the accumulation half, where the score products read them
+  uint32_t kvec;   // lane i: bit pattern of the largest rotated-key norm of keys [64 (kvec_base + i), + 64)
+  auto opaque_lane = [&]() __attribute__((always_inline)) {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    return l;
+  };
+  auto request_q = [&](int i) __attribute__((always_inline)) {
+    const int bh = i % p.BH, m0 = (p.num_m_blocks - 1 - i / p.BH) * C::kBlockM;
+    qrows.load(p.q_slab(bh), p.cos, p.sin, p.fstride, m0 + wave * 32, N, opaque_lane(), (uint32_t)p.q_sn * 2);
+  };
+  auto request_kvec = [&](int i) __attribute__((always_inline)) {
+    const int bh = i % p.BH;
+    kvec = reinterpret_cast<const uint32_t*>(p.tile_kmax)[(int64_t)kv_slab(bh, p.H, p.Hkv) * n_norm_tiles + min(opaque_lane(), n_norm_tiles - 1)];
+  };
+  auto take_q = [&](int i) __attribute__((always_inline)) {
+    const int bh = i % p.BH, m0 = (p.num_m_blocks - 1 - i / p.BH) * C::kBlockM;
+    park_rotated_rows<D>(qrows, qb, wave_tile, p.q_rot_out != nullptr ? p.q_rot_out + (int64_t)bh * N * D : nullptr,
+                         m0 + wave * 32, N, p.qk_scale, opaque_lane());
+  };
+
+  // ---- first item: nothing to hide its prologue behind ----------------------------------------------------------------
+  int item = item_at(0);
+  COROPE_ISTAMP(0);
+  load_item(0);
+  kst.load(l_kg, 0, N);
+  vst.load(l_vg, 0, N, (uint32_t)p.v_sn * 2);
+  request_q(item);
+  request_kvec(item);
+  take_q(item);
+  kst.store_rows(lds_at(koff_cur));
+  vst.store_rows(lds_at(voff_cur));
+  load_next_tile();
+  __syncthreads();
+
+  for (int round = 0;; ++round) {
+    const int bh = item % p.BH, mb = p.num_m_blocks - 1 - item / p.BH;
+    const int m0 = mb * C::kBlockM;
+    const int n_tiles = tiles_of(mb);
+    const uint32_t* tile_kmax_bits = reinterpret_cast<const uint32_t*>(p.tile_kmax) + (int64_t)kv_slab(bh, p.H, p.Hkv) * n_norm_tiles;
+    COROPE_ISTAMP(1);
+
+    // Largest |q_r| (scaled: base-2 units) of the wave's rows, a little generous: times the largest key norm of a tile it
+    // bounds the tile's scores.
+    float q_bound_wave;
+    {
+      float ss = 0.f;
+#pragma unroll
+      for (int kc = 0; kc < M; ++kc)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          float x0 = elt_lo(qb[kc][w]), x1 = elt_hi(qb[kc][w]);
+          ss += x0 * x0 + x1 * x1;
+        }
+      q_bound_wave = __builtin_sqrtf(wave_max(half_sum(ss))) * 1.01f;
+#pragma unroll
+      for (int kc = 0; kc < M; ++kc) qa[kc] = to_acc_half(qb[kc]);
+    }
+
+    f32x16 oacc[NDB];
+#pragma unroll
+    for (int i = 0; i < NDB; ++i) oacc[i] = f32x16{0};
+    float m_run = -INFINITY;    // reference value of the exponentials (this lane's query), base-2 units
+    float m_true = -INFINITY;   // largest score seen by the reference moves
+    float l_run = 0.f;          // this lane's share of the denominator up to the last move of the reference
+    float lsum = 0.f;           // ... and since then
+    float keep = 0.f;           // first probability of the pair in flight
+    f32x16 msb = f32x16{0};     // -m_run in every register: the accumulator the score MFMAs start from
+    f32x16 s;                   // scores of the tile
+    float s_prev[8];            // scores 8..15 of the lane in the tile before it (the half whose softmax is still to come)
+    u32x4 pb[2];                // P^T operand of the tile: the first half of its softmax fills pb[0]
+    u32x4 pb_prev[2];           // ... of the tile before it: pb_prev[0] taken over from pb[0], pb_prev[1] from s_prev
+
+    const int wave_q_lo = m0 + wave * 32;
+    const int key_limit = CAUSAL ? wave_q_lo + lq : N - 1;   // last key this lane's query attends to
+    const int t_last = __builtin_amdgcn_readfirstlane(CAUSAL ? min(n_tiles - 1, (wave_q_lo + 31) / BLOCK_N) : n_tiles - 1);
+    const int norm_last = (t_last * BLOCK_N) / 64;
+
+    // Reference value that puts every tile this wave will see within the margin.
+    float lift_target;
+    {
+      uint32_t kall = lane <= norm_last ? kvec : 0u;   // non-negative floats order like their bit patterns
+      for (int tb = kWave; tb <= norm_last; tb += kWave) {
+        const int tt = tb + lane;
+        kall = max(kall, tt <= norm_last ? tile_kmax_bits[tt] : 0u);
+      }
+      lift_target = q_bound_wave * wave_max(__builtin_bit_cast(float, kall)) - kMargin;
+    }
+    uint32_t thr_bits = 0;
+    int kvec_base = 0;
+
+    auto v_operand = [&](uint32_t v_lane, int i) {   // MFMA i of a PV slot: output block i % NDB, 16-key step i / NDB
+      return load_a_trans_at(lds_at(v_lane), LSV, 16 * (i / NDB), (i % NDB) * 32);
+    };
+    // Second half of the softmax of the previous tile, pair j (0..3), element e: from s_prev into pb_prev[1].
+    auto softmax_prev = [&](int j, int e) __attribute__((always_inline)) {
+      asm volatile("" : "+v"(lsum));
+      const float pr = fast_exp2(s_prev[2 * j + e]);
+      lsum += pr;
+      if (e == 0) {
+        keep = pr;
+        asm volatile("" : "+v"(keep), "+v"(lsum));
+      } else {
+        uint32_t w = pack_elts(keep, pr);
+        asm volatile("" : "+v"(w), "+v"(lsum));
+        pb_prev[1][j] = w;
+      }
+    };
+    // Takes the previous tile (first half of its softmax done) out of the pipeline: rest of its softmax, then its PV product
+    // (its V tile is the previous one of the ring).
+    auto drain = [&]() __attribute__((always_inline)) {
+      uint32_t vp_lane = v_lane_off + voff_prev;
+      asm volatile("" : "+v"(vp_lane));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        softmax_prev(j, 0);
+        softmax_prev(j, 1);
+      }
+#pragma unroll
+      for (int i = 0; i < M; ++i) oacc[i % NDB] = mfma32(v_operand(vp_lane, i), pb_prev[i / NDB], oacc[i % NDB]);
+    };
+
+#pragma unroll
+    for (int kc = 0; kc < M; ++kc) asm volatile("" ::"a"(qa[kc]));
+    asm volatile("" ::"v"(kvec));
+    COROPE_ISTAMP(2);
+#ifdef COROPE_TRACE
+    COROPE_ISTAMP_ID(n_tiles);
+    const uint64_t clk0 = __builtin_readcyclecounter();
+    uint64_t exact_passes = 0;
+#endif
+
+    auto tile_step = [&](int t, bool need_mask) __attribute__((always_inline)) {
+      const int n0 = t * BLOCK_N;
+#ifdef COROPE_TRACE
+      if (t == 1) COROPE_ISTAMP(3);
+      if (n0 == m0) COROPE_ISTAMP(4);
+#endif
+      uint32_t k_lane = k_lane_off + koff_cur, vprev = v_lane_off + (t == 0 ? voff_cur : voff_prev);
+      asm volatile("" : "+v"(k_lane), "+v"(vprev));
+      auto k_operand = [&](int kc) { return *reinterpret_cast<const u32x4*>(lds_at(k_lane) + RowTile<D>::off(0, 16 * kc)); };
+      auto mask_scores = [&](f32x16& sacc) __attribute__((always_inline)) {
+        int rel = key_limit - n0 - 4 * lh;
+        asm volatile("" : "+v"(rel));
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (8 * (i / 4) + i % 4 > rel) sacc[i] = -INFINITY;
+      };
+
+      auto run_tile = [&](const bool MASK) __attribute__((always_inline)) {
+        auto operand = [&](int n) { return n < M ? k_operand(n) : v_operand(vprev, n - M); };
+        constexpr int TOTAL = 2 * M;
+        u32x4 ring[RING];
+#pragma unroll
+        for (int n = 0; n < RING; ++n) ring[n] = operand(n);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<TOTAL>([&](auto n_c) __attribute__((always_inline)) {
+          constexpr int n = decltype(n_c)::value;
+          constexpr int slot = n / M, i = n % M;
+          const u32x4 frag = ring[n % RING];
+          if (slot == 0) { if (i == 0) s = mfma32_from_aq(frag, qa[i], msb); else mfma32_acc_aq(s, frag, qa[i]); }
+          if (slot == 1) oacc[i % NDB] = mfma32(frag, pb_prev[i / NDB], oacc[i % NDB]);
+          if (n + RING < TOTAL) ring[n % RING] = operand(n + RING);
+          if (n == 0) stage_next();
+          // The scores a slot's softmax reads were completed by an asm statement, behind which the compiler inserts no wait
+          // states: nothing reads them behind MFMA 0 of the next slot, which waits a little instead.
+          if (i == 0) asm volatile("s_nop 7");
+          if (slot == 1 && i == 1 && MASK) mask_scores(s);
+          if (i % 2 == 1) {
+            const int hh = i / 2, j = hh / 2, e = hh % 2;
+            if (slot == 0) softmax_prev(j, e);                          // S(t-1), second half
+            if (slot == 1) softmax_half(j, e, s, pb, lsum, keep);       // S(t), first half
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        // the tile becomes the previous one: the scores its softmax still needs and the half of its P^T that exists move over
+        // (vector moves of matrix-core results: the last score MFMA lies a whole slot back)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s_prev[i] = s[8 + i];
+        pb_prev[0] = pb[0];
+      };
+
+      // ---- does the reference have to move before this tile? ------------------------------------------------------
+      const int nt = n0 / 64;   // the 64-key block whose norm maximum bounds this tile
+      if (nt - kvec_base == kWave) {
+        kvec_base = nt;
+        kvec = tile_kmax_bits[min(nt + lane, n_norm_tiles - 1)];
+        asm volatile("" ::"v"(kvec));
+      }
+      const uint32_t kmax_bits = __builtin_amdgcn_readlane(kvec, nt - kvec_base);
+      if (t == 0 || kmax_bits > thr_bits) {
+#ifdef COROPE_TRACE
+        ++exact_passes;
+#endif
+        if (t > 0) drain();
+        f32x16 r = f32x16{0};
+#pragma unroll
+        for (int kc = 0; kc < M; ++kc) r = mfma32(k_operand(kc), from_acc_half(qa[kc]), r);
+        if (need_mask) mask_scores(r);
+        float mt = r[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) mt = fmaxf(mt, r[i]);
+        m_true = fmaxf(m_true, half_max(mt));
+        const float m_new = fmaxf(m_run, fmaxf(m_true, fminf(lift_target, m_true + kLift)));
+        const float alpha = fast_exp2(m_run - m_new);   // m_new is finite: every row sees key 0 of tile 0
+        l_run = (l_run + lsum) * alpha;
+        lsum = 0.f;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
+        m_run = m_new;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float x = -m_new;
+          asm volatile("" : "+v"(x));   // sixteen values of their own
+          msb[i] = x;
+        }
+        // nothing is pending now: all-masked previous scores and a zero P make the pending half of the tile body a no-op
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s_prev[i] = -INFINITY;
+        pb_prev[0] = pb_prev[1] = u32x4{0, 0, 0, 0};
+        const float m_min = -wave_max(-m_run);
+        const float thr = (m_min + kMargin) / q_bound_wave;
+        thr_bits = __builtin_amdgcn_readfirstlane(thr > 0.f ? __builtin_bit_cast(uint32_t, thr) : 0u);
+      }
+      run_tile(need_mask);
+      rotate_buffers();
+      __syncthreads();
+    };
+
+    for (int t = 0; t <= t_last; ++t) {
+      const bool need_mask = (CAUSAL && t * BLOCK_N + BLOCK_N - 1 > wave_q_lo) || (!CAUSAL && t * BLOCK_N + BLOCK_N > N);
+      tile_step(t, need_mask);
+    }
+
+    // The next item's Q rows are requested as soon as the registers of this item's Q rows are free.  (After the last item
+    // its own rows are requested once more and never used.)
+    const int next_item = item_at(round + 1);
+    const bool has_next = next_item < total;
+    request_q(has_next ? next_item : item);
+    request_kvec(has_next ? next_item : item);
+    drain();
+    COROPE_ISTAMP(5);
+#ifdef COROPE_TRACE
+    if (p.trace != nullptr && threadIdx.x == TT) {
+      p.trace[(int64_t)item * 16 + 7] = __builtin_readcyclecounter() - clk0;
+      p.trace[(int64_t)item * 16 + 13] = exact_passes;
+    }
+#endif
+    // of the tiles entirely above this wave's diagonal it only stages its share
+    for (int t = t_last + 1; t < n_tiles; ++t) {
+      stage_next();
+      rotate_buffers();
+      __syncthreads();
+    }
+    {
+      const float l_tot = half_sum(l_run + lsum);
+      store_rows_via_wave_tile<D>(oacc, p.o + (int64_t)bh * N * D, wave_q_lo, N, 1.f / l_tot, wave_tile, opaque_lane());
+      if (wave_q_lo + lq < N && lh == 0) p.lse[(int64_t)bh * N + wave_q_lo + lq] = m_run + fast_log2(l_tot);
+    }
+    COROPE_ISTAMP(6);
+    if (!has_next) break;
+    item = next_item;
+    COROPE_ISTAMP(0);
+    take_q(item);
+  }
+}
+
 // ---- host-side launch -----------------------------------------------------------------------------------------
 template <int D, bool CAUSAL>
 static hipError_t launch_pipe64(FwdParams p, hipStream_t stream) {
@@ -519,6 +896,27 @@ static hipError_t launch_pipe64(FwdParams p, hipStream_t stream) {
 hipError_t launch_rope_attn_fwd_prerotated_rows64(const FwdParams& p, int D, bool causal, hipStream_t stream) {
   if (D != 128) return hipErrorInvalidValue;
   return causal ? launch_pipe64<128, true>(p, stream) : launch_pipe64<128, false>(p, stream);
+}
+
+template <bool CAUSAL>
+static hipError_t launch_pipe256(FwdParams p, hipStream_t stream) {
+  using C = pipe64::Cfg256;
+  auto kern = rope_attn_fwd_pipe256_kernel<CAUSAL>;
+  static std::atomic<uint64_t> lds_ok{0};
+  if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), C::kLdsBytes, lds_ok); e != hipSuccess) return e;
+  p.num_m_blocks = (p.N + C::kBlockM - 1) / C::kBlockM;
+#ifdef COROPE_TRACE
+  p.trace = g_trace_buf;
+#endif
+  const int64_t n_items = (int64_t)p.num_m_blocks * p.BH;
+  const int64_t cus = device_cu_count();
+  dim3 grid((unsigned)(n_items < cus ? n_items : cus));
+  hipLaunchKernelGGL(kern, grid, dim3(C::kThreads), C::kLdsBytes, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_rope_attn_fwd_prerotated_pipe256(const FwdParams& p, bool causal, hipStream_t stream) {
+  return causal ? launch_pipe256<true>(p, stream) : launch_pipe256<false>(p, stream);
 }
 
 }  // namespace COROPE_NS

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(kRotThreads) void rope_rotate_kernel(const uint16_t
 hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float* sinp, int64_t fstride, uint16_t* y,
                               float* tile_max, int BH, int N, int D, hipStream_t stream, float out_scale, int H, int64_t x_sb,
                               int64_t x_sh, int x_sn) {
-  if (D != 64 && D != 128) return hipErrorInvalidValue;
+  if (D != 64 && D != 128 && D != 256) return hipErrorInvalidValue;
   if (x_sn == 0) {   // contiguous (BH, N, D)
     H = 1;
     x_sb = (int64_t)N * D;
@@ -90,7 +90,9 @@ hipError_t launch_rope_rotate(const uint16_t* x, const float* cosp, const float*
 #define COROPE_ROT(DD, SS)                                                                                             \
   hipLaunchKernelGGL((rope_rotate_kernel<DD, SS>), grid, dim3(kRotThreads), 0, stream, x, cosp, sinp, fstride, y, tile_max, \
                      N, n_tiles, out_scale, H, x_sb, x_sh, x_sn)
-  if (D == 128) {
+  if (D == 256) {
+    if (out_scale == 1.f) COROPE_ROT(256, false); else COROPE_ROT(256, true);
+  } else if (D == 128) {
     if (out_scale == 1.f) COROPE_ROT(128, false); else COROPE_ROT(128, true);
   } else {
     if (out_scale == 1.f) COROPE_ROT(64, false); else COROPE_ROT(64, true);

@@ -16,9 +16,9 @@ import torch
 from . import _lib
 
 _SUPPORTED_D = (64, 128, 256)
-# 256 (the largest head dim of the reference, fused_rope_attn.py:661) is built for the kernels that take q and k as they
-# are: the single-launch forward and the dV, dK and dQ kernels that rotate while they stage, one wave per SIMD.
-_ROTATED_PATH_MAX_D = 128
+# 256 (the largest head dim of the reference, fused_rope_attn.py:661) runs one wave per SIMD: the single-launch forward
+# kernel (on a rotated key copy from the rotated path's lengths on) and separate dQ, dV and dK kernels.
+_ROTATED_PATH_MAX_D = 256
 # Head dims of the reference (fused_rope_attn.py:661) below the kernels' own: run at D = 64 with each half of a row padded
 # with zeros (the rotation pairs column j with column j + D/2, so the halves must stay the starts of the new halves).
 _PADDED_D = (16, 32)

@@ -291,14 +291,16 @@ def test_head_dims_below_the_kernels_own(pkg, B, H, N, D, causal):
         assert within_bar(a, b, TOL)[0], name
 
 
+@pytest.mark.parametrize("two_launch", [False, True])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,Hq,Hkv,N", [(1, 2, 2, 300), (2, 2, 2, 128), (1, 1, 1, 1), (1, 3, 3, 1100), (1, 4, 2, 260), (1, 40, 40, 200)])
-def test_head_dim_256(pkg, B, Hq, Hkv, N, causal):
-    """The largest head dim the reference admits (fused-rope/fused_rope_attn.py:661): single-launch forward and the dV, dK
-    and dQ kernels on the original operands, one wave per SIMD; ragged lengths, grouped-query K/V, more items than
-    compute units' worth of one round and fewer."""
+def test_head_dim_256(pkg, monkeypatch, B, Hq, Hkv, N, causal, two_launch):
+    """The largest head dim the reference admits (fused-rope/fused_rope_attn.py:661), one wave per SIMD: the single-launch
+    forward kernel and separate dQ, dV and dK kernels, on the original operands and (two_launch) on copies rotated
+    beforehand; ragged lengths, grouped-query K/V, more items than compute units' worth of one round and fewer."""
     D = 256
-    print(f"case D=256 B={B} Hq={Hq} Hkv={Hkv} N={N} causal={causal}", flush=True)
+    print(f"case D=256 B={B} Hq={Hq} Hkv={Hkv} N={N} causal={causal} two_launch={two_launch}", flush=True)
+    _force_path(monkeypatch, pkg, two_launch)
     G = Hq // Hkv
     q, g = (bf16_round(seeded((B, Hq, N, D), 70 + i)) for i in range(2))
     k, v = (bf16_round(seeded((B, Hkv, N, D), 80 + i)) for i in range(2))
@@ -315,22 +317,34 @@ def test_head_dim_256(pkg, B, Hq, Hkv, N, causal):
         assert within_bar(a, b, TOL * (math.sqrt(G) if name in ("dK", "dV") else 1.0))[0], name
 
 
-def test_head_dim_256_has_no_rotated_copies(pkg):
-    """Entry points that work on rotated copies or a workspace refuse head dim 256 before any launch."""
-    B, H, N, D = 1, 1, 64, 256
+def test_head_dim_256_rotated_copies(pkg):
+    """Head dim 256 through the entry points that work on rotated copies: the rotation pass against the oracle's rotation,
+    and the forward with a workspace bit-equal to the forward on rotated copies made by hand."""
+    B, H, N, D = 1, 2, 200, 256
     dev = torch.device("cuda:0")
-    x = torch.zeros(B, H, N, D, device=dev, dtype=torch.bfloat16)
-    c, s = (t.to(dev) for t in O.precompute_freqs_cis(D, N))
-    with pytest.raises((ValueError, RuntimeError), match="original operands"):
-        pkg.rope_rotate(x, c, s)
+    q, k, v = (bf16_round(seeded((B, H, N, D), 60 + i)) for i in range(3))
+    c, s = O.precompute_freqs_cis(D, N)
+    qd, kd, vd = (t.to(dev, torch.bfloat16) for t in (q, k, v))
+    cd, sd = c.to(dev), s.to(dev)
+    kr, kmax = pkg.rope_rotate(kd, cd, sd, with_tile_max=True)
+    ref = O.apply_rotary_emb(k, c, s)
+    assert ((kr.float().cpu() - ref).abs() <= ref.abs() / 128 + 1e-6).all()     # one bf16 ulp (fused multiply-adds)
     lib = pkg._lib.load()
-    assert lib.corope_rope_attn_fwd_workspace_bytes(B, H, N, D) > 0   # the size query answers; the launch refuses
+    st = torch.cuda.current_stream().cuda_stream
     ws = torch.empty(lib.corope_rope_attn_fwd_workspace_bytes(B, H, N, D), device=dev, dtype=torch.uint8)
-    M = torch.empty(B, H, N, device=dev)
-    rc = lib.corope_rope_attn_fwd_ws(x.data_ptr(), x.data_ptr(), x.data_ptr(), c.data_ptr(), s.data_ptr(), c.stride(0),
-                                     x.data_ptr(), M.data_ptr(), B, H, N, D, 0.1, 1, ws.data_ptr(), ws.numel(),
-                                     torch.cuda.current_stream().cuda_stream)
-    assert rc != 0 and "original operands" in pkg._lib.last_error()
+    o1, o2 = torch.empty_like(qd), torch.empty_like(qd)
+    M1, M2 = torch.empty(B, H, N, device=dev), torch.empty(B, H, N, device=dev)
+    rc = lib.corope_rope_attn_fwd_ws(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), cd.data_ptr(), sd.data_ptr(), cd.stride(0),
+                                     o1.data_ptr(), M1.data_ptr(), B, H, N, D, 0.0625, 1, ws.data_ptr(), ws.numel(), st)
+    assert rc == 0, pkg._lib.last_error()
+    rc = lib.corope_rope_attn_fwd_prerotated(qd.data_ptr(), kr.data_ptr(), kmax.data_ptr(), vd.data_ptr(), cd.data_ptr(),
+                                             sd.data_ptr(), cd.stride(0), o2.data_ptr(), M2.data_ptr(), None, B, H, N, D,
+                                             0.0625, 1, st)
+    assert rc == 0, pkg._lib.last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2) and torch.equal(M1, M2)
+    ro = O.rope_attn_forward(q, k, v, True, 0.0625, c, s)[0]
+    assert within_bar(o1.float().cpu(), ro, TOL)[0]
 
 
 def test_seeded_sweep_over_shapes_and_paths(pkg, monkeypatch):

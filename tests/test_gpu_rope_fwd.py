@@ -180,13 +180,49 @@ def test_rotate_pass_with_more_slabs_than_a_grid_axis(pkg):
     assert torch.allclose(tm.cpu()[..., 0], y.norm(dim=-1).amax(-1), rtol=1e-5, atol=0)
 
 
+SOFTMAX_MODE_CASES = ["large_norms", "outlier_keys", "growing_scores", "tiny_scores", "huge_norms_hot"]
+
+
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("case", ["large_norms", "outlier_keys", "growing_scores", "tiny_scores", "huge_norms_hot"])
+@pytest.mark.parametrize("case", SOFTMAX_MODE_CASES)
 def test_two_launch_softmax_modes(pkg, tile_rows, case, causal):
     """Inputs that push tiles of the two-launch forward onto each of its softmax modes: the per-tile score bound
     (query norm x largest key norm of the tile) decides, so large norms, a few huge keys, and scores that keep
     growing along the sequence all force the exact mode on some tiles while others stay on the unchecked one."""
-    B, H, N, D = 1, 2, 640, 128
+    _softmax_modes(pkg, case, causal, 128)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("case", SOFTMAX_MODE_CASES)
+def test_two_launch_softmax_modes_head_dim_256(pkg, case, causal):
+    """The same at head dim 256, whose two-launch forward is a kernel of its own (one wave per SIMD, 32-key tiles)."""
+    _softmax_modes(pkg, case, causal, 256)
+
+
+def test_head_dim_256_long_sequence(pkg):
+    """More than 64 x 64 keys at head dim 256: the forward's lane-held vector of key-norm maxima is refilled on the way, and an
+    outlier key sits behind the refill.  Sampled rows of both heads against the oracle, two-launch against single-launch."""
+    B, H, N, D = 1, 2, 4500, 256
+    q, k, v = _inputs(B, H, N, D, seed=77)
+    k[:, :, 4200] *= 6
+    k = bf16_round(k)
+    c, s = O.precompute_freqs_cis(D, N)
+    scale = 1 / math.sqrt(D)
+    print("case D=256 long sequence", flush=True)
+    o, M = _run(pkg, q, k, v, True, scale, c, s, True)
+    o1, M1 = _run(pkg, q, k, v, True, scale, c, s, False)
+    rows = torch.cat([torch.arange(0, N, 97), torch.arange(4090, 4230), torch.arange(N - 40, N)]).unique()
+    ro, rl = O.rope_attn_forward_blocked(q, k, v, True, scale, c, s, rows=rows)
+    for name, got, lse in (("two-launch", o, M), ("single", o1, M1)):
+        err = (got[:, :, rows] - ro).abs()
+        print(f"  {name}: O max-abs {err.max():.3e} mean-abs {err.mean():.3e}")
+        assert torch.isfinite(got).all() and err.max() <= TOL
+        assert ((lse[:, :, rows] * LN2 - rl).abs() <= 2e-2 + rl.abs() / 128).all()
+    assert ((o - o1).abs() <= 1e-2 + o.abs() / 64).all()
+
+
+def _softmax_modes(pkg, case, causal, D):
+    B, H, N = 1, 2, 640
     q, k, v = _inputs(B, H, N, D, seed=31)
     scale = 1 / math.sqrt(D)
     if case == "large_norms":
@@ -205,7 +241,7 @@ def test_two_launch_softmax_modes(pkg, tile_rows, case, causal):
         # has to move on most tiles and must not be lifted out of reach of the scores that actually occur
         q, k, scale = bf16_round(q * 1.8), bf16_round(k * 1.8), 0.5
     c, s = O.precompute_freqs_cis(D, N)
-    print(f"case modes {case} causal={causal}", flush=True)
+    print(f"case modes {case} causal={causal} D={D}", flush=True)
     o, M = _run(pkg, q, k, v, causal, scale, c, s, True)
     o1, M1 = _run(pkg, q, k, v, causal, scale, c, s, False)
     ro, rl = O.rope_attn_forward_blocked(q, k, v, causal, scale, c, s)
@@ -229,7 +265,7 @@ def test_two_launch_softmax_modes(pkg, tile_rows, case, causal):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("B,H,Hkv,N,D", [(2, 4, 4, 300, 64), (1, 8, 2, 1100, 128), (2, 3, 3, 1024, 128)])
+@pytest.mark.parametrize("B,H,Hkv,N,D", [(2, 4, 4, 300, 64), (1, 8, 2, 1100, 128), (2, 3, 3, 1024, 128), (1, 4, 2, 700, 256)])
 def test_strided_views_are_read_where_they_lie(pkg, B, H, Hkv, N, D, dtype):
     """q, k, v as slices of one fused (B, N, Hq + 2 Hkv, D) projection seen as (B, H, N, D) -- the layout a model hands
     over -- give bit for bit what their contiguous copies give, forward (both forms) and backward, and no copy of q or k
