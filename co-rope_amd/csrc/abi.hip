@@ -624,8 +624,8 @@ int corope_rope_attn_fwd_f16(const void* q, const void* k, const void* v, const 
   rc = check_ptrs(what, {k_rot});
   if (rc) return rc;
   if (q_rot != nullptr && !aligned16(q_rot)) return fail(COROPE_E_ALIGN, "%s: q_rot %p is not 16-byte aligned", what, q_rot);
-  if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
-    return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "%s: tile_kmax %p is null or misaligned", what, (const void*)tile_kmax);
+  // tile_kmax null: the attention kernel is the single-launch one on the rotated copy (probabilities in fp16 against an fp16 V)
+  if (reinterpret_cast<uintptr_t>(tile_kmax) & 3u) return fail(COROPE_E_ALIGN, "%s: tile_kmax %p is misaligned", what, (const void*)tile_kmax);
   rc = launch_status(what, corope_f16::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, static_cast<uint16_t*>(k_rot), tile_kmax,
                                                           B * Hkv, N, D, st, 1.f, 1, 0, 0, 0));
   if (rc) return rc;
@@ -730,8 +730,9 @@ int corope_rope_attn_fwd_strided(const void* q, const int64_t* q_strides, const 
   rc = check_ptrs(what, {k_rot});
   if (rc) return rc;
   if (q_rot != nullptr && !aligned16(q_rot)) return fail(COROPE_E_ALIGN, "%s: q_rot %p is not 16-byte aligned", what, q_rot);
-  if (tile_kmax == nullptr || (reinterpret_cast<uintptr_t>(tile_kmax) & 3u))
-    return fail(tile_kmax ? COROPE_E_ALIGN : COROPE_E_BADARG, "%s: tile_kmax %p is null or misaligned", what, (const void*)tile_kmax);
+  // tile_kmax null: the attention kernel is the single-launch one on the rotated copy (no lazy reference value; for fp16
+  // tensors: probabilities in fp16 against an fp16 V)
+  if (reinterpret_cast<uintptr_t>(tile_kmax) & 3u) return fail(COROPE_E_ALIGN, "%s: tile_kmax %p is misaligned", what, (const void*)tile_kmax);
   uint16_t* kr = static_cast<uint16_t*>(k_rot);
   rc = launch_status(what, fp16 ? corope_f16::launch_rope_rotate(p.k, p.cos, p.sin, p.fstride, kr, tile_kmax, B * Hkv, N, D, st, 1.f,
                                                                  Hkv, p.k_sb, p.k_sh, p.k_sn)

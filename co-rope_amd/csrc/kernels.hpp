@@ -200,8 +200,8 @@ hipError_t launch_rope_attn_fwd_prerotated_rows64(const FwdParams& p, int D, boo
 // head dim 256 (bf16): 32 query rows per wave, one wave per SIMD, 32-key tiles
 hipError_t launch_rope_attn_fwd_prerotated_pipe256(const FwdParams& p, bool causal, hipStream_t stream);
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream);
-// head dim 256 on a rotated key copy (p.k_rot): the single-launch kernel without the rotation in its loop
-hipError_t launch_rope_attn_fwd_prerotated_d256(const FwdParams& p, bool causal, hipStream_t stream);
+// the single-launch kernel on a rotated key copy (p.k_rot; no key norms needed): no rotation in its loop
+hipError_t launch_rope_attn_fwd_single_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_preprocess(const BwdParams& p, int D, hipStream_t stream);
 hipError_t launch_bwd_dv(const BwdParams& p, int D, bool causal, hipStream_t stream);
 hipError_t launch_bwd_dk(const BwdParams& p, int D, bool causal, hipStream_t stream);

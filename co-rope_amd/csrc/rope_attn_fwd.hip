@@ -336,10 +336,10 @@ static hipError_t launch_fwd_waves(FwdParams p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int D, int BLOCK_N, bool CAUSAL>
+template <int D, int BLOCK_N, bool CAUSAL, bool PREROT = false>
 static hipError_t launch_fwd_cfg(const FwdParams& p, hipStream_t stream) {
-  return use_small_tiles(p.N, p.BH) ? launch_fwd_waves<D, BLOCK_N, CAUSAL, 4>(p, stream)
-                                    : launch_fwd_waves<D, BLOCK_N, CAUSAL, 8>(p, stream);
+  return use_small_tiles(p.N, p.BH) ? launch_fwd_waves<D, BLOCK_N, CAUSAL, 4, PREROT>(p, stream)
+                                    : launch_fwd_waves<D, BLOCK_N, CAUSAL, 8, PREROT>(p, stream);
 }
 
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream) {
@@ -350,9 +350,13 @@ hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStrea
   return causal ? launch_fwd_cfg<64, 64, true>(p, stream) : launch_fwd_cfg<64, 64, false>(p, stream);
 }
 
-// Head dim 256 on a key copy rotated beforehand: the same kernel without the rotation in its loop.
-hipError_t launch_rope_attn_fwd_prerotated_d256(const FwdParams& p, bool causal, hipStream_t stream) {
-  return causal ? launch_fwd_waves<256, 64, true, 4, true>(p, stream) : launch_fwd_waves<256, 64, false, 4, true>(p, stream);
+// The same kernel on a key copy rotated beforehand (p.k_rot): no rotation and no table reads in its loop; it needs no key
+// norms, and keeps the softmax bookkeeping of the single launch (probabilities in the tensors' own 16-bit type).
+hipError_t launch_rope_attn_fwd_single_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream) {
+  if (D == 256) return causal ? launch_fwd_waves<256, 64, true, 4, true>(p, stream) : launch_fwd_waves<256, 64, false, 4, true>(p, stream);
+  if (D == 128) return causal ? launch_fwd_cfg<128, 64, true, true>(p, stream) : launch_fwd_cfg<128, 64, false, true>(p, stream);
+  if (D != 64) return hipErrorInvalidValue;
+  return causal ? launch_fwd_cfg<64, 64, true, true>(p, stream) : launch_fwd_cfg<64, 64, false, true>(p, stream);
 }
 
 }  // namespace COROPE_NS

@@ -492,11 +492,13 @@ static hipError_t launch_pipe_cfg(const FwdParams& p, hipStream_t stream) {
 }
 
 hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream) {
+  // without key-norm maxima: the kernel that needs none
+  if (p.tile_kmax == nullptr) return launch_rope_attn_fwd_single_prerotated(p, D, causal, stream);
 #ifndef COROPE_F16
-  if (D == 256 && p.tile_kmax != nullptr && g_fwd_wave_rows.load(std::memory_order_relaxed) != 32)
+  if (D == 256 && g_fwd_wave_rows.load(std::memory_order_relaxed) != 32)
     return launch_rope_attn_fwd_prerotated_pipe256(p, causal, stream);
 #endif
-  if (D == 256) return launch_rope_attn_fwd_prerotated_d256(p, causal, stream);
+  if (D == 256) return launch_rope_attn_fwd_single_prerotated(p, D, causal, stream);
   if (D != 64 && D != 128) return hipErrorInvalidValue;
 #ifndef COROPE_F16
   if (D == 128 && !use_small_tiles(p.N, p.BH) && g_fwd_wave_rows.load(std::memory_order_relaxed) == 64)

@@ -104,12 +104,12 @@ TWO_LAUNCH_MIN_N = 1024
 TRAIN_ROTATED_MIN_ND = 65536
 
 
-# fp16 tensors, forward of a call that will be differentiated: "exact" = the single-launch forward, which keeps P and V in
-# fp16 (O within 1.2e-2 of the fp32 oracle at the reference's verification temperature sm_scale = 0.5, gradients within its
-# 0.15 / 5e-3 thresholds); "fast" = the two-launch forward (bf16 probabilities against a V converted to bf16 on its way
-# into LDS: as fast as with bf16 tensors, 1.5x faster than "exact" at B2 H32 N4096 D128, O within one bf16 ulp), whose O
-# carries bf16's rounding of V into delta = rowsum(O * dO) and through it into dQ and dK: up to 0.24 there instead of 0.05.
-# A forward that will not be differentiated always takes the fast form.
+# fp16 tensors, forward of a call that will be differentiated: "exact" = the single-launch kernel's bookkeeping, which
+# keeps P and V in fp16 (O within 1.2e-2 of the fp32 oracle at the reference's verification temperature sm_scale = 0.5,
+# gradients within its 0.15 / 5e-3 thresholds), from the rotated path's lengths on run on a key copy rotated beforehand;
+# "fast" = the pipelined forward (bf16 probabilities against a V converted to bf16 on its way into LDS: as fast as with
+# bf16 tensors, O within one bf16 ulp), whose O carries bf16's rounding of V into delta = rowsum(O * dO) and through it
+# into dQ and dK: up to 0.24 there instead of 0.05.  A forward that will not be differentiated always takes the fast form.
 FP16_TRAINING_FORWARD = "exact"
 
 
@@ -153,11 +153,11 @@ def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, k
     with _on_device(q):
         if strides is not None:
             fp16 = q.dtype == torch.float16
-            if fp16 and keep_rotated and FP16_TRAINING_FORWARD != "fast":
-                two_launch = False
+            # fp16 with gradients: P and V stay fp16 (no key-norm maxima: the single-launch kernel, on the rotated copy)
+            exact = fp16 and keep_rotated and FP16_TRAINING_FORWARD != "fast"
             q_rot = torch.empty(q.shape, device=q.device, dtype=q.dtype) if (two_launch and keep_rotated) else None
             k_rot = torch.empty(k.shape, device=q.device, dtype=q.dtype) if two_launch else None
-            kmax = torch.empty((B, Hkv, (N + 63) // 64), device=q.device, dtype=torch.float32) if two_launch else None
+            kmax = torch.empty((B, Hkv, (N + 63) // 64), device=q.device, dtype=torch.float32) if (two_launch and not exact) else None
             rc = lib.corope_rope_attn_fwd_strided(q.data_ptr(), strides[0], k.data_ptr(), strides[1], v.data_ptr(), strides[2],
                                                   fc.data_ptr(), fs.data_ptr(), fc.stride(0), o.data_ptr(), M.data_ptr(),
                                                   q_rot.data_ptr() if q_rot is not None else None,
@@ -168,13 +168,13 @@ def _forward(q, k, v, causal, sm_scale, freqs_cos, freqs_sin, two_launch=None, k
             if q_rot is not None:
                 rotated = (q_rot, k_rot)
         elif q.dtype == torch.float16:
-            # the reference's dtype: the same two forms (the two-launch one with bf16 probabilities against a V converted
-            # to bf16 on its way into LDS); one entry point covers them, grouped-query K/V included
-            if keep_rotated and FP16_TRAINING_FORWARD != "fast":
-                two_launch = False
+            # the reference's dtype: one entry point covers the forms, grouped-query K/V included.  With key-norm maxima: the
+            # pipelined kernel (bf16 probabilities against a V converted to bf16 on its way into LDS); without, for a forward
+            # with gradients: the single-launch kernel on the rotated copy, P and V in fp16
+            exact = keep_rotated and FP16_TRAINING_FORWARD != "fast"
             q_rot = torch.empty_like(q) if (two_launch and keep_rotated) else None
             k_rot = torch.empty_like(k) if two_launch else None
-            kmax = torch.empty((B, Hkv, (N + 63) // 64), device=q.device, dtype=torch.float32) if two_launch else None
+            kmax = torch.empty((B, Hkv, (N + 63) // 64), device=q.device, dtype=torch.float32) if (two_launch and not exact) else None
             rc = lib.corope_rope_attn_fwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), fc.data_ptr(), fs.data_ptr(),
                                               fc.stride(0), o.data_ptr(), M.data_ptr(),
                                               q_rot.data_ptr() if q_rot is not None else None,

@@ -232,6 +232,8 @@ int corope_rope_attn_bwd_ws(const void *q, const void *k, const void *v, const v
  * kernel, in which the unnormalised probabilities (up to 2^64: more binary orders than fp16 has) are bf16 and V is
  * converted to bf16 on its way into LDS, so that P V is a bf16 product; q_rot ((B,H,N,D) fp16, may be NULL) receives the
  * rotated Q times sm_scale*log2(e), and (q_rot, k_rot) are then the operands of a backward with prerotated = 1.
+ * k_rot != NULL with tile_kmax == NULL: K is rotated once into k_rot and the single-launch kernel runs on the copy, without
+ * the rotation in its loop and with its own bookkeeping -- P and V stay fp16, as in the reference -- and q_rot as above.
  * Backward: prerotated = 1: q, k are those rotated copies (dQ kernel, which computes delta on its way, then the fused dK+dV
  * kernel); else preprocess + dV + dK + dQ as in corope_rope_attn_bwd, or -- given a workspace of
  * corope_rope_attn_bwd_workspace_bytes (may be NULL) -- the rotation of q and k into it followed by the dQ and the fused
@@ -254,7 +256,8 @@ int corope_rope_attn_bwd_f16(const void *q, const void *k, int prerotated, const
  * e.g. (N*H*D, D, H*D) for a (B, N, H, D) tensor viewed as (B, H, N, D).  The reference's forward kernel takes the strides
  * of q and k the same way (fused-rope/fused_rope_attn.py:709-710; its V and O go through contiguous descriptors, :245-251);
  * o, lse and the optional scratch are contiguous.  k_rot == NULL: single launch; k_rot != NULL: the two-launch form as
- * in corope_rope_attn_fwd_gqa (q_rot may be NULL); fp16 != 0: fp16 tensors as in corope_rope_attn_fwd_f16, else bf16. */
+ * in corope_rope_attn_fwd_gqa (q_rot may be NULL; tile_kmax == NULL: the single-launch kernel on the rotated copy, as in
+ * corope_rope_attn_fwd_f16); fp16 != 0: fp16 tensors as in corope_rope_attn_fwd_f16, else bf16. */
 int corope_rope_attn_fwd_strided(const void *q, const int64_t *q_strides, const void *k, const int64_t *k_strides,
                                  const void *v, const int64_t *v_strides,
                                  const float *freqs_cos, const float *freqs_sin, int64_t freq_row_stride,

@@ -38,8 +38,9 @@ def _gpu(pkg, q, k, v, g, causal, scale, c, s):
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,N,D", [(2, 4, 512, 64), (1, 8, 1024, 128), (4, 16, 2048, 64)])
 def test_fp16_verification_script_cases(pkg, monkeypatch, B, H, N, D, causal, path):
-    """path: the kernels the operator picks by shape for a call that is differentiated (single-launch forward, which keeps P
-    and V in fp16; from N * D = 65536 on the backward on rotated copies); "fast": rope_attn.FP16_TRAINING_FORWARD = "fast"
+    """path: the kernels the operator picks by shape for a call that is differentiated (the single-launch forward kernel,
+    which keeps P and V in fp16 -- from N * D = 65536 on it runs on a key copy rotated beforehand and leaves the rotated q
+    and k for the backward); "fast": rope_attn.FP16_TRAINING_FORWARD = "fast"
     (K rotated once, the pipelined forward with bf16 probabilities against a V converted to bf16 on its way into LDS, the
     backward on the rotated copies the forward kept); or, forced, every kernel on the original operands.  The fast form
     carries bf16's rounding of V into O (bar: one bf16 ulp of the reference value where |O| >= 2.56, as for bf16 tensors)
