@@ -112,6 +112,63 @@ __device__ __forceinline__ f32x16 mfma32_from(u32x4 a, u32x4 b, const f32x16& c)
   return d;
 }
 
+// With one wave per SIMD (head dim 256) the compiler gives every MFMA it selects its accumulator in the accumulation half
+// of the register file, and a product whose result the vector units read next (scores, dP) then costs a copy per element
+// each way.  The same products as asm statements with every operand in the vector half: mfma32_zero_v starts a chain from
+// zero, mfma32_acc_v accumulates in place, and mfma32_settle behind the last of a chain waits the 12 states after which the
+// vector units may touch the result (the compiler inserts none behind an asm statement; check_isa.py verifies).
+__device__ __forceinline__ f32x16 mfma32_zero_v(u32x4 a, u32x4 b) {
+  f32x16 d;
+#ifdef COROPE_F16
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+#else
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+#endif
+  return d;
+}
+__device__ __forceinline__ void mfma32_acc_v(f32x16& d, u32x4 a, u32x4 b) {
+#ifdef COROPE_F16
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+#else
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+#endif
+}
+// ... and with the B operand in the accumulation half (where a wave's per-item operand rows live when it has 512 registers):
+// Score products with the query operand in the accumulation half of the register file (the matrix cores read A and B
+// operands from either half; the vector units only the other one, which the scores, probabilities and staging fill).
+// As asm statements: the compiler, given the builtin, copies such an operand over before every use.  `from`: the result
+// lands in registers of its own, C stays intact; `acc`: accumulates in place.  The compiler inserts no wait states behind
+// an asm statement: the first vector instruction that reads the scores follows at least two further MFMAs (or one and
+// an explicit s_nop) behind the last of these, which the build checks in the generated assembly (check_isa.py).
+// mfma32_zero_aq starts a chain from zero.
+__device__ __forceinline__ f32x16 mfma32_from_aq(u32x4 a, const u32x4& b, const f32x16& c) {
+  f32x16 d;
+#ifdef COROPE_F16
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
+#else
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
+#endif
+  return d;
+}
+__device__ __forceinline__ void mfma32_acc_aq(f32x16& d, u32x4 a, const u32x4& b) {
+#ifdef COROPE_F16
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+#else
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+#endif
+}
+__device__ __forceinline__ f32x16 mfma32_zero_aq(u32x4 a, const u32x4& b) {
+  f32x16 d;
+#ifdef COROPE_F16
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+#else
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+#endif
+  return d;
+}
+
+__device__ __forceinline__ void mfma32_settle(f32x16& d) { asm volatile("s_nop 7\n\ts_nop 3" : "+v"(d)); }
+
 // Row index (0..31) held by accumulator register i of lane-half h in a 32x32 MFMA result.
 __device__ __forceinline__ constexpr int acc_row(int i, int h) { return 8 * (i / 4) + 4 * h + (i % 4); }
 

@@ -246,16 +246,21 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(k
         }
         const uint16_t* qrow = qs + RowTile<D, Q_PAD>::off(qb * 32 + lq, 8 * lh);
         const uint16_t* dorow = dos + RowTile<D, DO_PAD>::off(qb * 32 + lq, 8 * lh);
+        constexpr bool V_FORM = kWavesPerSimd<D> == 1;   // see mfma32_acc_v
 #pragma unroll
-        for (int kc = 0; kc < KC; ++kc)
-          sacc = mfma32(*reinterpret_cast<const u32x4*>(qrow + 16 * kc), kb[kc], sacc);
+        for (int kc = 0; kc < KC; ++kc) {
+          const u32x4 a = *reinterpret_cast<const u32x4*>(qrow + 16 * kc);
+          if constexpr (V_FORM) mfma32_acc_v(sacc, a, kb[kc]); else sacc = mfma32(a, kb[kc], sacc);
+        }
         if constexpr (DO_DK) {
 #pragma unroll
-          for (int kc = 0; kc < KC; ++kc)
-            dpacc = mfma32(*reinterpret_cast<const u32x4*>(dorow + 16 * kc),
-                           V_LDS ? *reinterpret_cast<const u32x4*>(vrows + RowTile<D>::off(lq, 8 * lh + 16 * kc)) : vb[V_LDS ? 0 : kc],
-                           dpacc);
+          for (int kc = 0; kc < KC; ++kc) {
+            const u32x4 a = *reinterpret_cast<const u32x4*>(dorow + 16 * kc);
+            const u32x4 b = V_LDS ? *reinterpret_cast<const u32x4*>(vrows + RowTile<D>::off(lq, 8 * lh + 16 * kc)) : vb[V_LDS ? 0 : kc];
+            if constexpr (V_FORM) mfma32_acc_v(dpacc, a, b); else dpacc = mfma32(a, b, dpacc);
+          }
         }
+        if constexpr (V_FORM) mfma32_settle(DO_DK ? dpacc : sacc);
 
         // Causal mask on the raw scores, under a wave-uniform branch of its own (written into the exponential loop it
         // is turned into compare + select on every tile).  Register i holds query mq0 + 8*(i/4) + 4*lh + i%4; the
@@ -297,6 +302,16 @@ __global__ __launch_bounds__(NWAVES* kWave) __attribute__((amdgpu_waves_per_eu(k
         // without the causal branches the two blocks of a tile are one stretch of code: kept apart, or the scheduler
         // interleaves them and needs both blocks' score registers at once
         if constexpr (!CAUSAL) __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (kWavesPerSimd<D> == 1) {
+        // one wave per SIMD: the accumulators' home is the accumulation half of the register file, where the MFMAs the
+        // compiler selects update them; said here, or it carries them round the loop in the other half and copies all of
+        // them over and back on every tile
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+          if constexpr (DO_DV) asm volatile("" : "+a"(dvacc[db]));
+          if constexpr (DO_DK) asm volatile("" : "+a"(dkacc[db]));
+        }
       }
       store_tile(cur ^ 1);
       cur ^= 1;

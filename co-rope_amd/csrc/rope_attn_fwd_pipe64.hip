@@ -68,29 +68,6 @@ __device__ __forceinline__ void softmax_half(int j, int e, const f32x16& sacc, u
   }
 }
 
-// Score products with the query operand in the accumulation half of the register file (the matrix cores read A and B
-// operands from either half; the vector units only the other one, which the scores, probabilities and staging fill).
-// As asm statements: the compiler, given the builtin, copies such an operand over before every use.  `from`: the result
-// lands in registers of its own, C stays intact; `acc`: accumulates in place.  The compiler inserts no wait states behind
-// an asm statement: the first vector instruction that reads the scores follows at least two further MFMAs (or one and
-// an explicit s_nop) behind the last of these, which the build checks in the generated assembly (check_isa.py).
-__device__ __forceinline__ f32x16 mfma32_from_aq(u32x4 a, const u32x4& b, const f32x16& c) {
-  f32x16 d;
-#ifdef COROPE_F16
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
-#else
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "a"(b), "v"(c));
-#endif
-  return d;
-}
-__device__ __forceinline__ void mfma32_acc_aq(f32x16& d, u32x4 a, const u32x4& b) {
-#ifdef COROPE_F16
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
-#else
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
-#endif
-}
-
 // A 16-byte operand moved into / out of the accumulation half of the register file, explicitly: values that only ever meet
 // "a" constraints afterwards stay there.
 __device__ __forceinline__ u32x4 to_acc_half(const u32x4& x) {
