@@ -697,7 +697,9 @@ static hipError_t launch_dkdv(const BwdParams& p, int D, bool causal, hipStream_
 }
 
 hipError_t launch_bwd_dkdv_fused(const BwdParams& p, int D, bool causal, hipStream_t stream) {
-  if (D == 256) {   // two launches: the accumulators of dK and dV together do not fit a wave's registers at this head dim
+  if (D == 256) {
+    if (p.q_rot != nullptr && p.k_rot != nullptr)   // on rotated copies: fused, both sets of accumulators in the accumulation registers
+      return causal ? launch_dkdv_cfg<256, true, true, true, true>(p, stream) : launch_dkdv_cfg<256, false, true, true, true>(p, stream);
     if (hipError_t e = launch_dkdv<true, false>(p, D, causal, stream); e != hipSuccess) return e;
     return launch_dkdv<false, true>(p, D, causal, stream);
   }

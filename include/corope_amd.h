@@ -7,7 +7,7 @@
  *
  * Conventions (all entry points)
  *   - tensors are device pointers to contiguous row-major (B, H, N, D) bf16 storage;
- *     D is 64 or 128 (fused RoPE attention: also 256; there the fused dK+dV entry point makes two launches);
+ *     D is 64 or 128 (fused RoPE attention: also 256);
  *     pointers are 16-byte aligned;
  *   - freqs_cos / freqs_sin are fp32 tables with one row per position; only columns
  *     [0, D/2) are read; `freq_row_stride` is the distance between rows in elements
