@@ -36,7 +36,7 @@ _ADDEND_ANY = 16
 _OPERAND_WAIT = 2
 _MFMA = re.compile(r"^\s*v_mfma_\w+\s+([va]\[\d+:\d+\])\s*,\s*([^,]+),\s*([^,]+),\s*(\S+)")
 #: source text that issues a matrix-core instruction from an asm statement, or calls a helper that does
-ASM_MFMA_IN_SOURCE = re.compile(r"\bmfma32_(from|acc)\w*\s*\(|asm[^;]*\"v_mfma")
+ASM_MFMA_IN_SOURCE = re.compile(r"\bmfma32_(from|acc|zero)\w*\s*\(|asm[^;]*\"v_mfma")
 
 
 def _regs(text):
