@@ -347,6 +347,34 @@ def test_head_dim_256_rotated_copies(pkg):
     assert within_bar(o1.float().cpu(), ro, TOL)[0]
 
 
+@pytest.mark.parametrize("B,H,N,D", [(1, 2, 300, 64), (2, 2, 520, 128), (1, 2, 300, 256)])
+def test_backward_with_workspace_matches_the_operator(pkg, monkeypatch, B, H, N, D):
+    """corope_rope_attn_bwd_ws (q and k rotated into a caller's workspace, then the kernels on the copies) gives the
+    gradients of the operator's own backward on the rotated copies its forward kept, bit for bit."""
+    print(f"case bwd_ws B={B} H={H} N={N} D={D}", flush=True)
+    _force_path(monkeypatch, pkg, True)
+    q, k, v, g, c, s = _case(B, H, N, D)
+    scale = 1 / math.sqrt(D)
+    dev = torch.device("cuda:0")
+    qd, kd, vd = (t.to(dev, torch.bfloat16).requires_grad_(True) for t in (q, k, v))
+    gd, cd, sd = g.to(dev, torch.bfloat16), c.to(dev), s.to(dev)
+    o = pkg.attention(qd, kd, vd, True, scale, cd, sd)
+    o.backward(gd)
+    M = pkg.rope_attn_forward_with_lse(qd.detach(), kd.detach(), vd.detach(), True, scale, cd, sd, two_launch=True)[1]
+    lib = pkg._lib.load()
+    ws = torch.empty(lib.corope_rope_attn_bwd_workspace_bytes(B, H, N, D), device=dev, dtype=torch.uint8)
+    delta = torch.empty(B, H, N, device=dev)
+    dq, dk, dv = (torch.full_like(qd, float("nan")) for _ in range(3))
+    rc = lib.corope_rope_attn_bwd_ws(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(), gd.data_ptr(), M.data_ptr(),
+                                     delta.data_ptr(), cd.data_ptr(), sd.data_ptr(), cd.stride(0), dq.data_ptr(), dk.data_ptr(),
+                                     dv.data_ptr(), B, H, N, D, scale, 1, ws.data_ptr(), ws.numel(),
+                                     torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, pkg._lib.last_error()
+    torch.cuda.synchronize()
+    for name, a, b in (("dQ", dq, qd.grad), ("dK", dk, kd.grad), ("dV", dv, vd.grad)):
+        assert torch.equal(a, b), f"{name}: {(a.float() - b.float()).abs().max().item():.3e}"
+
+
 def test_seeded_sweep_over_shapes_and_paths(pkg, monkeypatch):
     """Forty seeded draws over head dim (16 .. 256), batch, heads, grouped-query sharing, ragged lengths, causal or not,
     bf16 or fp16, temperature, and the choice of path (the operator's own, all kernels on rotated copies, none): forward
