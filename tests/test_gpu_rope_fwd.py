@@ -292,3 +292,37 @@ def test_strided_views_are_read_where_they_lie(pkg, B, H, Hkv, N, D, dtype):
         grads.append(f.grad)
     torch.cuda.synchronize()
     assert torch.equal(grads[0], grads[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,Hkv,N,D", [(2, 4, 4, 300, 64), (1, 4, 2, 1100, 128), (1, 2, 2, 333, 256), (8, 40, 40, 128, 64)])
+def test_single_launch_kernel_on_a_rotated_key_copy(pkg, B, H, Hkv, N, D, causal, dtype):
+    """corope_rope_attn_fwd_strided with a place for the rotated K and none for key-norm maxima: the rotation pass, then the
+    single-launch kernel on the copy.  Same rounding points as the single launch on the original K, so O and LSE are equal
+    bit for bit, and the rotated q and k it leaves equal the rotation pass's (checked for bf16)."""
+    print(f"case prerot-single B={B} H={H} Hkv={Hkv} N={N} D={D} causal={causal} {dtype}", flush=True)
+    dev = torch.device("cuda:0")
+    q = seeded((B, H, N, D), 21).to(dev, dtype)
+    k, v = (seeded((B, Hkv, N, D), 22 + i).to(dev, dtype) for i in range(2))
+    c, s = (t.to(dev) for t in O.precompute_freqs_cis(D, N))
+    scale = 1 / math.sqrt(D)
+    lib = pkg._lib.load()
+    import ctypes
+    st3 = lambda t: (ctypes.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+    outs = []
+    for with_copy in (False, True):
+        o, M = torch.empty_like(q), torch.empty(B, H, N, device=dev)
+        q_rot, k_rot = (torch.empty_like(q), torch.empty_like(k)) if with_copy else (None, None)
+        rc = lib.corope_rope_attn_fwd_strided(q.data_ptr(), st3(q), k.data_ptr(), st3(k), v.data_ptr(), st3(v), c.data_ptr(),
+                                              s.data_ptr(), c.stride(0), o.data_ptr(), M.data_ptr(),
+                                              q_rot.data_ptr() if with_copy else None, k_rot.data_ptr() if with_copy else None,
+                                              None, B, H, Hkv, N, D, scale, int(causal), int(dtype == torch.float16),
+                                              torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, pkg._lib.last_error()
+        outs.append((o, M, q_rot, k_rot))
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    if dtype == torch.bfloat16:   # (the Python wrapper of the rotation pass takes bf16 only)
+        assert torch.equal(outs[1][3], pkg.rope_rotate(k, c, s))
+        assert torch.equal(outs[1][2], pkg.rope_rotate(q, c, s, scale=scale * math.log2(math.e)))
