@@ -561,7 +561,7 @@ def bench_phase_trace(args):
         for n, f in launches:
             assert f() == 0, n
     torch.cuda.synchronize()
-    n_wg = B * H * ((N + 255) // 256)
+    n_wg = B * H * ((N + 127) // 128)     # room for the forms with 128-row items as well
     bufs = {n: torch.zeros(n_wg * 16, dtype=torch.int64, device=dev) for n, _ in launches[1:]}
     for rep in range(3):         # the traced step sits between untraced ones
         for n, f in launches:

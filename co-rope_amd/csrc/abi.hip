@@ -29,15 +29,15 @@ int env_choice(const char* name, std::initializer_list<int> allowed) {
 }  // namespace
 // Kernel forms are picked by shape.  For diagnostics two environment variables, read ONCE when the library is loaded,
 // override the pick for the whole process: COROPE_AMD_TILE_ROWS (128 or 256 rows per workgroup item) and
-// COROPE_AMD_FWD_WAVE_ROWS (32 or 64 query rows per wave in the two-launch forward at D = 128).  The shipped library has
+// COROPE_AMD_FWD_WAVE_ROWS (32 or 64 query rows per wave, or 128: 128-row items with two workgroups per compute unit, in the two-launch forward at D = 128).  The shipped library has
 // no call that changes them afterwards; the measurement build (libcorope_amd_trace.so) has one, for the tests.
 std::atomic<int> g_tile_rows{env_choice("COROPE_AMD_TILE_ROWS", {128, 256})};
-std::atomic<int> g_fwd_wave_rows{env_choice("COROPE_AMD_FWD_WAVE_ROWS", {32, 64})};
+std::atomic<int> g_fwd_wave_rows{env_choice("COROPE_AMD_FWD_WAVE_ROWS", {32, 64, 128})};
 }  // namespace corope
 
 #ifdef COROPE_TRACE
 extern "C" int corope_debug_set_forms(int tile_rows, int fwd_wave_rows) {
-  if ((tile_rows != 0 && tile_rows != 128 && tile_rows != 256) || (fwd_wave_rows != 0 && fwd_wave_rows != 32 && fwd_wave_rows != 64))
+  if ((tile_rows != 0 && tile_rows != 128 && tile_rows != 256) || (fwd_wave_rows != 0 && fwd_wave_rows != 32 && fwd_wave_rows != 64 && fwd_wave_rows != 128))
     return COROPE_E_BADARG;
   corope::g_tile_rows.store(tile_rows);
   corope::g_fwd_wave_rows.store(fwd_wave_rows);

@@ -199,6 +199,8 @@ hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causa
 hipError_t launch_rope_attn_fwd_prerotated_rows64(const FwdParams& p, int D, bool causal, hipStream_t stream);
 // head dim 256 (bf16): 32 query rows per wave, one wave per SIMD, 32-key tiles
 hipError_t launch_rope_attn_fwd_prerotated_pipe256(const FwdParams& p, bool causal, hipStream_t stream);
+// head dim 128 in that form (128-row items, 32-key tiles), two workgroups per compute unit
+hipError_t launch_rope_attn_fwd_prerotated_pipe32x2(const FwdParams& p, bool causal, hipStream_t stream);
 hipError_t launch_rope_attn_fwd(const FwdParams& p, int D, bool causal, hipStream_t stream);
 // the single-launch kernel on a rotated key copy (p.k_rot; no key norms needed): no rotation in its loop
 hipError_t launch_rope_attn_fwd_single_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream);

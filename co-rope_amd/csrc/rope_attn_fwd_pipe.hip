@@ -501,6 +501,8 @@ hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causa
   if (D == 256) return launch_rope_attn_fwd_single_prerotated(p, D, causal, stream);
   if (D != 64 && D != 128) return hipErrorInvalidValue;
 #ifndef COROPE_F16
+  if (D == 128 && g_fwd_wave_rows.load(std::memory_order_relaxed) == 128)
+    return launch_rope_attn_fwd_prerotated_pipe32x2(p, causal, stream);
   if (D == 128 && !use_small_tiles(p.N, p.BH) && g_fwd_wave_rows.load(std::memory_order_relaxed) == 64)
     return launch_rope_attn_fwd_prerotated_rows64(p, D, causal, stream);
 #endif

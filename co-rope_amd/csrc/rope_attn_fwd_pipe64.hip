@@ -485,11 +485,14 @@ __global__ __launch_bounds__(pipe64::Cfg<D>::kThreads) __attribute__((amdgpu_wav
 //     slot A:  S(t)  = K(t) Q^T              |  softmax of S(t-1), second half   -> P(t-1)
 //     slot B:  O^T  += V(t-1)^T P(t-1)       |  softmax of S(t), first half
 //
-// one exponential half pair behind every second MFMA.  At the end of a tile the eight scores per lane that its softmax
+// the eight exponential half pairs of a slot spread over its MFMAs.  At the end of a tile the eight scores per lane that its softmax
 // still needs and the finished half of its P^T operand are moved to registers of their own (12 vector moves).
 namespace pipe64 {
-struct Cfg256 {
-  static constexpr int kD = 256;
+template <int D_>
+struct Cfg32 {
+  static constexpr int kD = D_;
+  // head dim 256: one wave per SIMD (512 registers each); 128: two, i.e. two workgroups per compute unit
+  static constexpr int kWavesPerSimd = D_ > 128 ? 1 : 2;
   static constexpr int kWaves = 4;
   static constexpr int kThreads = kWaves * kWave;
   static constexpr int kBlockM = kWaves * 32;
@@ -500,14 +503,16 @@ struct Cfg256 {
   static constexpr int kKStages = 2, kVStages = 3;
   static constexpr int kRingBytes = kKStages * kKBytes + kVStages * kVBytes;
   static constexpr int kLdsBytes = kRingBytes + kWaves * WaveTile<kD>::kBytes;
-  static_assert(kLdsBytes <= 160 * 1024, "LDS of a compute unit");
+  static_assert(kWavesPerSimd * kLdsBytes <= 160 * 1024, "LDS of a compute unit");
 };
+using Cfg256 = Cfg32<256>;
 }  // namespace pipe64
 
-template <bool CAUSAL>
-__global__ __launch_bounds__(pipe64::Cfg256::kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void rope_attn_fwd_pipe256_kernel(FwdParams p) {
+template <int D_, bool CAUSAL>
+__global__ __launch_bounds__(pipe64::Cfg32<D_>::kThreads)
+    __attribute__((amdgpu_waves_per_eu(pipe64::Cfg32<D_>::kWavesPerSimd, pipe64::Cfg32<D_>::kWavesPerSimd))) void rope_attn_fwd_pipe32_kernel(FwdParams p) {
   using namespace pipe64;
-  using C = Cfg256;
+  using C = Cfg32<D_>;
   constexpr int D = C::kD;
   constexpr int BLOCK_N = C::kBlockN;
   constexpr int NT = C::kThreads;
@@ -751,8 +756,10 @@ __global__ __launch_bounds__(pipe64::Cfg256::kThreads) __attribute__((amdgpu_wav
           // states: nothing reads them behind MFMA 0 of the next slot, which waits a little instead.
           if (i == 0) asm volatile("s_nop 7");
           if (slot == 1 && i == 1 && MASK) mask_scores(s);
-          if (i % 2 == 1) {
-            const int hh = i / 2, j = hh / 2, e = hh % 2;
+          // the slot's eight half pairs, spread over its MFMAs 1 .. M-1
+#pragma unroll
+          for (int hh = (i == 0 ? 0 : (i - 1) * 8 / (M - 1)); hh < (i == 0 ? 0 : i * 8 / (M - 1)); ++hh) {
+            const int j = hh / 2, e = hh % 2;
             if (slot == 0) softmax_prev(j, e);                          // S(t-1), second half
             if (slot == 1) softmax_half(j, e, s, pb, lsum, keep);       // S(t), first half
           }
@@ -875,10 +882,10 @@ hipError_t launch_rope_attn_fwd_prerotated_rows64(const FwdParams& p, int D, boo
   return causal ? launch_pipe64<128, true>(p, stream) : launch_pipe64<128, false>(p, stream);
 }
 
-template <bool CAUSAL>
-static hipError_t launch_pipe256(FwdParams p, hipStream_t stream) {
-  using C = pipe64::Cfg256;
-  auto kern = rope_attn_fwd_pipe256_kernel<CAUSAL>;
+template <int D, bool CAUSAL>
+static hipError_t launch_pipe32(FwdParams p, hipStream_t stream) {
+  using C = pipe64::Cfg32<D>;
+  auto kern = rope_attn_fwd_pipe32_kernel<D, CAUSAL>;
   static std::atomic<uint64_t> lds_ok{0};
   if (hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kern), C::kLdsBytes, lds_ok); e != hipSuccess) return e;
   p.num_m_blocks = (p.N + C::kBlockM - 1) / C::kBlockM;
@@ -886,14 +893,19 @@ static hipError_t launch_pipe256(FwdParams p, hipStream_t stream) {
   p.trace = g_trace_buf;
 #endif
   const int64_t n_items = (int64_t)p.num_m_blocks * p.BH;
-  const int64_t cus = device_cu_count();
-  dim3 grid((unsigned)(n_items < cus ? n_items : cus));
+  const int64_t slots = (int64_t)device_cu_count() * C::kWavesPerSimd;   // workgroups resident at once
+  dim3 grid((unsigned)(n_items < slots ? n_items : slots));
   hipLaunchKernelGGL(kern, grid, dim3(C::kThreads), C::kLdsBytes, stream, p);
   return hipGetLastError();
 }
 
 hipError_t launch_rope_attn_fwd_prerotated_pipe256(const FwdParams& p, bool causal, hipStream_t stream) {
-  return causal ? launch_pipe256<true>(p, stream) : launch_pipe256<false>(p, stream);
+  return causal ? launch_pipe32<256, true>(p, stream) : launch_pipe32<256, false>(p, stream);
+}
+
+// Head dim 128 in the same form, two workgroups of four waves per compute unit.
+hipError_t launch_rope_attn_fwd_prerotated_pipe32x2(const FwdParams& p, bool causal, hipStream_t stream) {
+  return causal ? launch_pipe32<128, true>(p, stream) : launch_pipe32<128, false>(p, stream);
 }
 
 }  // namespace COROPE_NS

@@ -43,7 +43,7 @@ const char *corope_amd_last_error(void);
 
 /* No entry point changes how later calls run: kernel forms (rows per workgroup item, rows per wave) are picked per call
  * from the shape, as the reference picks its tile sizes per shape (fused-rope/fused_rope_attn.py:163-183).  For diagnostics
- * the environment variables COROPE_AMD_TILE_ROWS (128 | 256) and COROPE_AMD_FWD_WAVE_ROWS (32 | 64), read once when the
+ * the environment variables COROPE_AMD_TILE_ROWS (128 | 256) and COROPE_AMD_FWD_WAVE_ROWS (32 | 64 | 128), read once when the
  * library is loaded, override the pick for the whole process; results do not depend on them beyond rounding. */
 
 /* Argument check only (no HIP call): what corope_rope_attn_fwd/bwd would return for these sizes. */

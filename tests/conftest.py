@@ -38,14 +38,15 @@ def tile_rows(request, pkg):
             assert lib.corope_debug_set_forms(0, 0) == 0
 
 
-@pytest.fixture
-def rows64(pkg):
-    """256-row items and 64 query rows per wave (one wave per SIMD) in the two-launch forward at D = 128."""
+@pytest.fixture(params=[64, 128])
+def alt_forward_form(pkg, request):
+    """The two measured alternatives to the shipped two-launch forward at D = 128: 64 query rows per wave with one wave
+    per SIMD (64), and 128-row items on 32-key tiles with two workgroups per compute unit (128)."""
     lib = pkg._lib.load_trace()
     with pkg._lib.using(lib):
-        assert lib.corope_debug_set_forms(256, 64) == 0
+        assert lib.corope_debug_set_forms(256 if request.param == 64 else 0, request.param) == 0
         try:
-            yield 64
+            yield request.param
         finally:
             assert lib.corope_debug_set_forms(0, 0) == 0
 

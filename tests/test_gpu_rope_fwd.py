@@ -56,11 +56,12 @@ def test_forward_parity(pkg, tile_rows, B, H, N, D, causal, two_launch):
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,N,D,std,scale", [(1, 8, 1024, 128, 1.0, None), (1, 3, 333, 128, 1.0, None), (1, 2, 257, 128, 1.0, None),
                                                (2, 2, 1500, 128, 1.0, None), (1, 2, 640, 128, 1.8, 0.5)])
-def test_forward_parity_with_64_rows_per_wave(pkg, rows64, B, H, N, D, std, scale, causal):
-    """The two-launch forward in its form with 64 query rows per wave, one wave per SIMD (an opt-in form: slower than the
-    8 x 32 one at the benchmark shape): same bar as test_forward_parity; the last case is the hot, large-norm one of
-    test_two_launch_softmax_modes, where the reference value of the exponentials has to move on most tiles."""
-    print(f"case rows64 B={B} H={H} N={N} D={D} causal={causal} std={std}", flush=True)
+def test_forward_parity_of_the_alternative_forms(pkg, alt_forward_form, B, H, N, D, std, scale, causal):
+    """The two-launch forward in its opt-in forms (both slower than the 8 x 32 one at the benchmark shape): 64 query rows per
+    wave with one wave per SIMD, and 128-row items on 32-key tiles with two workgroups per compute unit.  Same bar as
+    test_forward_parity; the last case is the hot, large-norm one of test_two_launch_softmax_modes, where the reference value
+    of the exponentials has to move on most tiles."""
+    print(f"case form {alt_forward_form} B={B} H={H} N={N} D={D} causal={causal} std={std}", flush=True)
     q, k, v = _inputs(B, H, N, D, seed=31, std=std)
     c, s = O.precompute_freqs_cis(D, N)
     hot = scale is not None
