@@ -77,17 +77,25 @@ extern std::atomic<int> g_tile_rows;
 // Query rows per wave of the two-launch forward at D = 128 with 256-row items: 32 (8 waves, two per SIMD) or 64 (4 waves,
 // one per SIMD, every LDS fragment feeding two MFMAs); 0 = the default.
 extern std::atomic<int> g_fwd_wave_rows;
-inline bool use_small_tiles(int n_rows, int slabs) {
+// Whether two 4-wave workgroups of lds_bytes each fit a compute unit (the attention kernels are compiled for two waves
+// per SIMD).
+constexpr bool fits_twice(int lds_bytes) { return 2 * lds_bytes <= 160 * 1024; }
+// small_lds_bytes: LDS of the kernel's 4-wave form.  Where two of those fit a compute unit, 128-row items pay as long as
+// the 256-row items make fewer than two rounds (measured at D = 64: +15 % with one item per compute unit, +4 % with one
+// and a half, -3 % with two); where only one fits, as long as they make less than one.
+inline bool use_small_tiles(int n_rows, int slabs, int small_lds_bytes = 160 * 1024) {
   const int forced = g_tile_rows.load(std::memory_order_relaxed);
   if (forced == 128) return true;
   if (forced == 256) return false;
-  return (int64_t)((n_rows + 255) / 256) * slabs < device_cu_count();
+  return (int64_t)((n_rows + 255) / 256) * slabs < (int64_t)device_cu_count() * (fits_twice(small_lds_bytes) ? 2 : 1);
 }
 
 // Workgroups of a persistent launch: one per compute unit -- two where two fit (4-wave workgroups whose LDS leaves room
-// for a second one: the attention kernels are compiled for two waves per SIMD) -- or one per item if those are fewer.
+// for a second one) -- or one per item if those are fewer.  (Letting the two workgroups of a compute unit take its rounds in
+// turn, so that every compute unit gets the same total, was measured and not kept: what counts is that both stay busy at the
+// same time -- at one and a half rounds it cost 15 %, at exactly one it gained 3 %.)
 inline unsigned persistent_grid(int64_t n_items, int waves, int lds_bytes) {
-  const int per_cu = (waves <= 4 && 2 * lds_bytes <= 160 * 1024) ? 2 : 1;
+  const int per_cu = (waves <= 4 && fits_twice(lds_bytes)) ? 2 : 1;
   const int64_t slots = (int64_t)device_cu_count() * per_cu;
   return (unsigned)(n_items < slots ? n_items : slots);
 }

@@ -643,7 +643,8 @@ static hipError_t launch_dkdv_cfg(const BwdParams& p, hipStream_t stream) {
   if constexpr (D > 128) {
     return launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 4>(p, stream);   // 4 waves x 512 registers
   } else {
-    return use_small_tiles(p.N, p.BH / p.H * p.Hkv) ? launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 4>(p, stream)
+    using Small = DkdvCfg<D, 4, 64, DO_DK ? (DO_DV ? kDkdvBothWaysPad : 8) : 32, DO_DK ? kDkdvBothWaysPad : 8>;
+    return use_small_tiles(p.N, p.BH / p.H * p.Hkv, Small::kLdsBytes) ? launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 4>(p, stream)
                                                      : launch_dkdv_waves<D, CAUSAL, DO_DV, DO_DK, PREROT, 8>(p, stream);
   }
 }
@@ -669,7 +670,7 @@ static hipError_t launch_dq_cfg(const BwdParams& p, hipStream_t stream) {
   if constexpr (D > 128) {
     return launch_dq_waves<D, CAUSAL, PREROT, 4>(p, stream);   // 4 waves x 512 registers
   } else {
-    return use_small_tiles(p.N, p.BH) ? launch_dq_waves<D, CAUSAL, PREROT, 4>(p, stream)
+    return use_small_tiles(p.N, p.BH, DqCfg<D, 4, 64>::kLdsBytes) ? launch_dq_waves<D, CAUSAL, PREROT, 4>(p, stream)
                                       : launch_dq_waves<D, CAUSAL, PREROT, 8>(p, stream);
   }
 }

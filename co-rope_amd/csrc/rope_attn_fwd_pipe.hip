@@ -488,7 +488,8 @@ static hipError_t launch_pipe_waves(FwdParams p, hipStream_t stream) {
 
 template <int D, bool CAUSAL>
 static hipError_t launch_pipe_cfg(const FwdParams& p, hipStream_t stream) {
-  return use_small_tiles(p.N, p.BH) ? launch_pipe_waves<D, CAUSAL, 4>(p, stream) : launch_pipe_waves<D, CAUSAL, 8>(p, stream);
+  return use_small_tiles(p.N, p.BH, FwdPipeCfg<D, 4>::kLdsBytes) ? launch_pipe_waves<D, CAUSAL, 4>(p, stream)
+                                                                  : launch_pipe_waves<D, CAUSAL, 8>(p, stream);
 }
 
 hipError_t launch_rope_attn_fwd_prerotated(const FwdParams& p, int D, bool causal, hipStream_t stream) {

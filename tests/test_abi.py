@@ -267,3 +267,14 @@ def test_strided_forward_argument_checks(pkg):
         assert rc in (-1, -2) and "stride" in pkg._lib.last_error(), list(bad)
     assert lib.corope_rope_attn_fwd_strided(ok, None, ok, good, ok, good, *tail) == -1
     assert lib.corope_rope_attn_fwd_strided(ok, good, ok, good, ok + 2, good, *tail) == -3
+
+
+def test_alias_names_the_same_modules():
+    """``corope_amd`` is an alias of the package in the directory ``co-rope_amd``: importing a submodule through either
+    name gives the one module object whose globals the package's functions read (a second copy would have thresholds
+    and switches of its own, and setting them would change nothing)."""
+    from importlib import import_module
+    pkg = import_module("corope_amd")
+    for sub in ("rope_attn", "corope_gqa", "_lib", "freqs"):
+        assert import_module("corope_amd." + sub) is import_module("co-rope_amd." + sub) is getattr(pkg, sub), sub
+    assert pkg.attention.__globals__ is pkg.rope_attn.__dict__

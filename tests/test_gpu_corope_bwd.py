@@ -130,8 +130,7 @@ def test_corope_backward_caller_workspace_and_reuse(pkg):
     """A caller-owned workspace filled with garbage gives the same gradients, whether it holds every group's matrices
     (one pass), some of them (the groups are walked in passes of as many as fit) or a single group's; one that cannot
     hold a single group's is refused."""
-    import importlib
-    mod = importlib.import_module("corope_amd.corope_gqa")
+    mod = pkg.corope_gqa
     dev = torch.device("cuda:0")
     B, Hq, Hkv, N, D = 2, 6, 3, 70, 64
     q, k, v, d_o = (t.to(dev, torch.bfloat16) for t in _inputs(B, Hq, Hkv, N, D, seed=3))
@@ -159,8 +158,7 @@ def test_corope_backward_caller_workspace_and_reuse(pkg):
 def test_corope_backward_keeps_its_own_workspace_between_calls(pkg, monkeypatch):
     """Without a caller's workspace the operator uses one buffer per device, sized by the shape and a cap alone: the second
     call allocates nothing new, a smaller cap walks the groups in passes with the same gradients, release frees it."""
-    import importlib
-    mod = importlib.import_module("corope_amd.corope_gqa")
+    mod = pkg.corope_gqa
     dev = torch.device("cuda:0")
     B, Hq, Hkv, N, D = 2, 6, 3, 70, 64
     q, k, v, d_o = (t.to(dev, torch.bfloat16) for t in _inputs(B, Hq, Hkv, N, D, seed=5))
@@ -219,8 +217,7 @@ def test_corope_backward_does_not_depend_on_the_scale_of_dO(pkg, B, Hq, Hkv, N, 
     """Upstream gradients of a mean-reduced loss (1e-6 and below) and unnormalised ones (1e3): the backward is linear in
     dO, and a power-of-two factor commutes with every rounding in it (the fp16 weights of the dQ sums are normalised per
     row by a power of two of |dO_i|), so grad(2^k dO) == 2^k grad(dO) bit for bit -- and both match the oracle."""
-    import importlib
-    mod = importlib.import_module("corope_amd.corope_gqa")
+    mod = pkg.corope_gqa
     dev = torch.device("cuda:0")
     q, k, v, d_o = _inputs(B, Hq, Hkv, N, D, seed=11)
     scale = 1 / math.sqrt(D)

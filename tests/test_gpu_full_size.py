@@ -128,8 +128,7 @@ def test_c5_corope_backward(pkg):
     of a row sums gates of keys up to the row itself), and two size-independent identities for dK and dV as a whole:
     sum_j dv_j = sum_{h,i} dO^h_i per group (softmax rows sum to one), and sum q.dq = sum k.dk per group (scores and
     gates depend on q and k only through products q.k, so scaling q up and k down by the same factor changes nothing)."""
-    import importlib
-    mod = importlib.import_module("corope_amd.corope_gqa")
+    mod = pkg.corope_gqa
     B, Hq, Hkv, N, D = 2, 32, 8, 4096, 128
     G = Hq // Hkv
     dev = torch.device("cuda:0")
