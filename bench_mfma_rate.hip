@@ -11,7 +11,7 @@
 // 3. How many independent vector instructions of the SAME wave hide under one MFMA (one wave per SIMD, all-zero operands,
 //    so at the full clock), with the accumulator and / or the B operand in the accumulation half of the register file.
 // 4. The steady-state tile loop of the forward in its form with 64 query rows per wave, one wave per SIMD
-//    (csrc/rope_attn_fwd_pipe64.hip) without any data-dependent control flow, feature by feature: MFMAs alone, + LDS
+//    (csrc/rope_attn_fwd_pipe_acc.hip) without any data-dependent control flow, feature by feature: MFMAs alone, + LDS
 //    operand reads, + softmax, + barrier, + staging of the next K/V tile.
 // 5. The same tile with 8 waves of 32 rows (two per SIMD), compiler-scheduled, built on 32x32x16 and on 16x16x32 MFMAs.
 #include "co-rope_amd/csrc/common.hpp"
@@ -291,7 +291,7 @@ __device__ __forceinline__ void mfma32_acc_aq(f32x16& d, u32x4 a, const u32x4& b
 }
 
 // F bits: 1 softmax, 2 LDS operand reads, 4 staging (global -> registers -> LDS), 8 barrier per tile.  NB: blocks of 32 rows
-// per wave (2: the form of rope_attn_fwd_pipe64.hip in its steady state; 1: the same wave with its second block alone).
+// per wave (2: the form of rope_attn_fwd_pipe_acc.hip in its steady state; 1: the same wave with its second block alone).
 template <int F, int NB>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void tile_loop(const uint16_t* kg, const uint16_t* vg, float* out, int n_tiles) {
   constexpr int D = 128, M = 8, NDB = 4, RING = 4, NT = 256, BLOCK_N = 64, ROWS = 4096;

@@ -1,7 +1,7 @@
 """Build-time check of the places where the kernels rely on something the compiler does not know.
 
 Some matrix-core instructions are issued from asm statements (``mfma32_from`` in csrc/common.hpp: a result in registers of
-its own; the score products of csrc/rope_attn_fwd_pipe64.hip: an operand in the accumulation half of the register file).
+its own; the score products of csrc/rope_attn_fwd_pipe_acc.hip: an operand in the accumulation half of the register file).
 The compiler inserts the wait states the instruction set asks for around a matrix-core instruction only for instructions
 it selected itself: to it an asm statement is opaque.  ``check_asm_mfma`` verifies on the generated assembly, for every
 such statement of every kernel:

@@ -1,6 +1,8 @@
 // Fused half-layout-RoPE flash-attention forward for gfx950 on a K that rope_rotate_kernel rotated beforehand:
-// the forms with one wave per SIMD -- 64 query rows per wave at head dim 128 (first part of the file), 32 query rows per
-// wave at head dim 256 (second part).
+// the forms that keep the Q operand and the O accumulators in the accumulation half of the register file and issue
+// their score products as asm statements -- 64 query rows per wave, one wave per SIMD, at head dim 128 (first part of the
+// file: a measured alternative), and 32 query rows per wave on 32-key tiles (second part: the forward of head dim 256, one
+// wave per SIMD; at head dim 128, two workgroups per compute unit, another measured alternative).
 //
 // Device counterpart of the reference's _attn_fwd / _attn_fwd_inner (fused-rope/fused_rope_attn.py:222-320, :48-138).
 // Same mathematics, MFMA operand layouts, softmax bookkeeping (lazy reference value against per-tile key-norm bounds)

@@ -61,5 +61,5 @@ def test_operand_written_right_in_front_is_reported():
 def test_sources_with_asm_matrix_instructions_are_found():
     build = importlib.import_module("co-rope_amd.build")
     checked = {s for s in build.SOURCES if build.isa_checked(s)}
-    assert {"rope_attn_fwd_pipe.hip", "rope_attn_fwd_pipe64.hip", "rope_attn_bwd.hip"} <= checked
+    assert {"rope_attn_fwd_pipe.hip", "rope_attn_fwd_pipe_acc.hip", "rope_attn_bwd.hip"} <= checked
     assert "rope_rotate.hip" not in checked and "abi.hip" not in checked
