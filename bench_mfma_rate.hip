@@ -1,5 +1,5 @@
 // Measurement program beside bench.py (not part of the library): what the gfx950 matrix pipes sustain on this machine,
-// and what a wave can do beside them.  `python bench.py --mfma-rate` builds it (hipcc) and runs it.  Five tables:
+// and what a wave can do beside them.  `python bench.py --mfma-rate` builds it (hipcc) and runs it.  Six tables:
 //
 // 1. Loops of nothing but 32x32x16 bf16 MFMAs on all 256 CUs (8 waves each), with the A operand either held in registers
 //    or fetched from LDS as a fresh 1 KB fragment that feeds R MFMAs, on all-zero operands and on N(0,1) operands rounded
@@ -14,6 +14,10 @@
 //    (csrc/rope_attn_fwd_pipe_acc.hip) without any data-dependent control flow, feature by feature: MFMAs alone, + LDS
 //    operand reads, + softmax, + barrier, + staging of the next K/V tile.
 // 5. The same tile with 8 waves of 32 rows (two per SIMD), compiler-scheduled, built on 32x32x16 and on 16x16x32 MFMAs.
+// 6. What it would cost to sum dQ over key blocks in memory (a backward in one kernel: 5 matrix products per tile instead
+//    of the 7 of the dQ + dK/dV pair, but every 256-key block then adds a 64 x 128 fp32 tile to each 64-query tile at or
+//    below it): those adds alone, as fp32 atomics, as plain read-modify-writes and as plain stores, in the pattern of
+//    B2 H32 N4096 D128 causal (1.14 GB of tiles per launch onto 134 MB).
 #include "co-rope_amd/csrc/common.hpp"
 
 #include <hip/hip_runtime.h>
@@ -638,6 +642,73 @@ void table(uint16_t* k, uint16_t* v, float* out, size_t n) {
 }
 }  // namespace t5
 
+// ---------------------------------------------------------------------------------------------------------------------
+// Table 6: accumulating dQ tiles in memory.
+namespace t6 {
+constexpr int kHeads = 64, kKeyBlocks = 16, kQueryTiles = 64, kTileFloats = 64 * 128;
+
+// 256 workgroups of 8 waves; workgroup w serves head (w % 8) + 8 (w / 32) with four of its 16 key blocks (two heavy, two
+// light: 136 tile adds each).  A wave adds its 32 x 32 block of the tile as 16 instructions of 64 consecutive floats.
+template <int MODE>
+__global__ __launch_bounds__(512) void accumulate(float* __restrict__ acc) {
+  const int wg = blockIdx.x, j = wg / 8, head = wg % 8 + 8 * (j / 4), m = j % 4;
+  const int blocks[4] = {m, 7 - m, 8 + m, 15 - m};
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  for (int it = 0; it < 4; ++it) {
+    for (int qt = blocks[it] * 4; qt < kQueryTiles; ++qt) {
+      float* p = acc + ((size_t)(head * kQueryTiles + qt) * 8 + wave) * 1024 + lane;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        if (MODE == 0) unsafeAtomicAdd(p + r * 64, 1.0f);   // global_atomic_add_f32, no return value
+        else if (MODE == 1) p[r * 64] += 1.0f;              // not a valid sum between workgroups: the traffic only
+        else p[r * 64] = 1.0f;
+      }
+    }
+  }
+}
+
+template <int MODE>
+void run(float* acc, const char* what) {
+  const size_t n = (size_t)kHeads * kQueryTiles * kTileFloats;
+  for (int w = 0; w < 3; ++w) hipLaunchKernelGGL(accumulate<MODE>, dim3(256), dim3(512), 0, 0, acc);
+  (void)hipMemset(acc, 0, n * 4);
+  hipEvent_t e0, e1;
+  (void)hipEventCreate(&e0);
+  (void)hipEventCreate(&e1);
+  const int reps = 10;
+  (void)hipEventRecord(e0);
+  for (int w = 0; w < reps; ++w) hipLaunchKernelGGL(accumulate<MODE>, dim3(256), dim3(512), 0, 0, acc);
+  (void)hipEventRecord(e1);
+  (void)hipEventSynchronize(e1);
+  float ms = 0;
+  (void)hipEventElapsedTime(&ms, e0, e1);
+  ms /= reps;
+  long wrong = -1;
+  if (MODE != 1) {
+    std::vector<float> h(n);
+    (void)hipMemcpy(h.data(), acc, n * 4, hipMemcpyDeviceToHost);
+    wrong = 0;
+    for (size_t i = 0; i < n; ++i) {
+      const int qt = (int)(i / kTileFloats) % kQueryTiles;
+      wrong += h[i] != (MODE == 0 ? (float)(reps * (qt / 4 + 1)) : 1.0f);
+    }
+  }
+  const double bytes = 256.0 * 136 * kTileFloats * 4;
+  printf("| %s | %.3f | %.2f | %s |\n", what, ms, bytes / (ms * 1e-3) * 1e-12, wrong < 0 ? "not checked" : wrong == 0 ? "exact" : "WRONG");
+}
+
+void table() {
+  float* acc;
+  if (hipMalloc(&acc, (size_t)kHeads * kQueryTiles * kTileFloats * 4) != hipSuccess) return;
+  printf("\n## 6. Adding the dQ tiles of a one-kernel backward to memory (B2 H32 N4096 D128 causal: 34816 tiles of 64 x 128 fp32, 1.14 GB, onto 134 MB)\n\n"
+         "| how | ms per launch | TB/s of tile bytes | sums |\n|---|---|---|---|\n");
+  run<0>(acc, "fp32 atomic add (global_atomic_add_f32)");
+  run<1>(acc, "plain load, add, store");
+  run<2>(acc, "plain store");
+  (void)hipFree(acc);
+}
+}  // namespace t6
+
 int main() {
   if (table1() != 0) return 1;
   u32x4* src;
@@ -661,5 +732,6 @@ int main() {
   (void)hipMemcpy(v, hk.data(), n * 2, hipMemcpyHostToDevice);
   t4::table(k, v, out);
   t5::table(k, v, out, n);
+  t6::table();
   return hipGetLastError() == hipSuccess ? 0 : 1;
 }
