@@ -177,3 +177,75 @@ def test_c5_corope_backward(pkg):
     print(f"  C5 sum q.dq vs sum k.dk per group: max diff {float((lhs - rhs).abs().max()):.3e}, "
           f"|sum| up to {float(lhs.abs().max()):.3e}, bound min {float(bound.min()):.3e}", flush=True)
     assert ((lhs - rhs).abs() <= bound + 2e-3 * lhs.abs()).all()
+
+
+def test_tensors_of_more_than_2_31_elements(pkg):
+    """B66 H128 N2048 D128: 8448 (batch, head) slabs, 2.2e9 elements (4.4 GB) per tensor, so the offsets of the last slabs
+    do not fit 32 bits.  The first slab, one in the middle and the last two are held against the oracle, forward and
+    backward, and against the same slabs run on their own."""
+    B, H, N, D = 66, 128, 2048, 128
+    dev = torch.device("cuda:0")
+    assert B * H * N * D > 2 ** 31
+    gen = torch.Generator(device=dev).manual_seed(7)
+    qd, kd, vd, gd = (torch.randn((B, H, N, D), device=dev, dtype=torch.bfloat16, generator=gen) for _ in range(4))
+    c, s = O.precompute_freqs_cis(D, N)
+    cd, sd = c.to(dev), s.to(dev)
+    scale = 1 / math.sqrt(D)
+    for t in (qd, kd, vd):
+        t.requires_grad_(True)
+    out = pkg.attention(qd, kd, vd, True, scale, cd, sd)
+    out.backward(gd)
+    torch.cuda.synchronize()
+    for (b, h) in ((0, 0), (32, 65), (65, 126), (65, 127)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        q, k, v, g = (t.detach()[sl].float().cpu() for t in (qd, kd, vd, gd))
+        ro, _, rdq, rdk, rdv, _ = O.rope_attn_fwd_bwd_blocked(q, k, v, g, True, scale, c, s)
+        q1, k1, v1 = (t.detach()[sl].clone().requires_grad_(True) for t in (qd, kd, vd))
+        o1 = pkg.attention(q1, k1, v1, True, scale, cd, sd)
+        o1.backward(gd[sl].clone())
+        for name, a, r, alone in (("O", out.detach()[sl], ro, o1.detach()), ("dQ", qd.grad[sl], rdq, q1.grad),
+                                  ("dK", kd.grad[sl], rdk, k1.grad), ("dV", vd.grad[sl], rdv, v1.grad)):
+            ok, err = within_bar(a.float().cpu(), r, TOL)[:2]
+            d_alone = (a.float() - alone.float()).abs().max().item()
+            print(f"  slab ({b},{h}) {name}: max-abs {err:.3e} against the oracle, {d_alone:.1e} against the slab alone", flush=True)
+            assert ok, (b, h, name)
+            assert d_alone <= 2e-2, (b, h, name)
+
+
+def test_corope_tensors_of_more_than_2_31_elements(pkg):
+    """Co-RoPE at B66 Hq128 Hkv32 N2048 D128: q, O, dO and dQ hold 2.2e9 elements each, so the offsets of the last heads do
+    not fit 32 bits (and the backward walks its workspace in slices of groups).  The first group, one in the middle and
+    the last are held against the same groups run on their own, forward and backward, and sampled rows of the last
+    group's output against the oracle."""
+    mod = pkg.corope_gqa
+    B, Hq, Hkv, N, D = 66, 128, 32, 2048, 128
+    G = Hq // Hkv
+    dev = torch.device("cuda:0")
+    assert B * Hq * N * D > 2 ** 31
+    gen = torch.Generator(device=dev).manual_seed(11)
+    qd, gd = (torch.randn((B, Hq, N, D), device=dev, dtype=torch.bfloat16, generator=gen) for _ in range(2))
+    kd, vd = (torch.randn((B, Hkv, N, D), device=dev, dtype=torch.bfloat16, generator=gen) for _ in range(2))
+    scale = 1 / math.sqrt(D)
+    print("  launching the forward", flush=True)
+    out = pkg.corope_attention(qd, kd, vd, True, scale, 10000.0)
+    torch.cuda.synchronize()
+    print("  launching the backward", flush=True)
+    dq, dk, dv = mod.corope_gqa_backward(qd, kd, vd, gd, scale, 10000.0)
+    torch.cuda.synchronize()
+    for (b, kv) in ((0, 0), (31, 17), (B - 1, Hkv - 1)):
+        hs, sl = (slice(b, b + 1), slice(kv * G, (kv + 1) * G)), (slice(b, b + 1), slice(kv, kv + 1))
+        q1, g1, k1, v1 = qd[hs].clone(), gd[hs].clone(), kd[sl].clone(), vd[sl].clone()
+        o1 = pkg.corope_attention(q1, k1, v1, True, scale, 10000.0)
+        dq1, dk1, dv1 = mod.corope_gqa_backward(q1, k1, v1, g1, scale, 10000.0)
+        torch.cuda.synchronize()
+        for name, a, alone in (("O", out[hs], o1), ("dQ", dq[hs], dq1), ("dK", dk[sl], dk1), ("dV", dv[sl], dv1)):
+            d = (a.float() - alone.float()).abs().max().item()
+            print(f"  group ({b},{kv}) {name}: {d:.1e} against the group alone", flush=True)
+            assert torch.isfinite(a.float()).all() and d <= TOL, (b, kv, name)
+    rows = _rows(N, 5, 9)
+    hs, sl = (slice(B - 1, B), slice(Hq - G, Hq)), (slice(B - 1, B), slice(Hkv - 1, Hkv))
+    ref = C.corope_gqa_forward_rows(qd[hs].float().cpu(), kd[sl].float().cpu(), vd[sl].float().cpu(), True, scale, 10000.0,
+                                    rows, torch.float32, row_block=16)
+    err = (out[hs].float().cpu()[:, :, rows] - ref).abs().max().item()
+    print(f"  last group: O max-abs {err:.3e} against the oracle on {rows.numel()} rows", flush=True)
+    assert err <= TOL
