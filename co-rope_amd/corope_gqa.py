@@ -77,20 +77,22 @@ def backward_min_workspace_bytes(B, Hq, Hkv, N, D):
     return n
 
 
-# The backward's scratch when the caller brings none: one buffer per device, kept between calls and grown when a call needs
-# more, holding as many groups' matrices as fit BACKWARD_WORKSPACE_CAP_BYTES (never less than one group; all groups in one
-# pass is fastest: at B2 Hq32 Hkv8 N4096 D128 7.1 GiB and 14 ms, against 31 ms with a quarter of that).  The size depends
-# on the shape and the cap only, not on what else is resident.
+# The backward's scratch when the caller brings none: one buffer per device and stream, kept between calls and grown when
+# a call needs more, holding as many groups' matrices as fit BACKWARD_WORKSPACE_CAP_BYTES (never less than one group; all
+# groups in one pass is fastest: at B2 Hq32 Hkv8 N4096 D128 7.1 GiB and 14 ms, against 31 ms with a quarter of that).  The
+# size depends on the shape and the cap only, not on what else is resident.  Per stream, because calls on two streams of a
+# device may run at the same time and torch's allocator only orders a buffer's reuse on the stream it was allocated on.
 BACKWARD_WORKSPACE_CAP_BYTES = 8 << 30
-_workspaces = {}   # device index -> uint8 tensor
+_workspaces = {}   # (device index, stream handle) -> uint8 tensor
 
 
 def _cached_workspace(device, B, Hq, Hkv, N, D):
     one, full = backward_min_workspace_bytes(B, Hq, Hkv, N, D), backward_workspace_bytes(B, Hq, Hkv, N, D)
     want = min(full, max(1, BACKWARD_WORKSPACE_CAP_BYTES // one) * one)
-    ws = _workspaces.get(device.index)
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
     if ws is None or ws.numel() < want:
-        _workspaces.pop(device.index, None)
+        _workspaces.pop(key, None)
         ws = None                      # the old buffer goes back to the allocator before the larger one is asked for
         try:
             ws = torch.empty(want, dtype=torch.uint8, device=device)
@@ -103,7 +105,7 @@ def _cached_workspace(device, B, Hq, Hkv, N, D):
         if ws is None:
             raise MemoryError(f"Co-RoPE backward at B={B} Hq={Hq} Hkv={Hkv} N={N} D={D} needs at least {one} bytes of scratch "
                               f"(one key/value group; {full} for all groups in one pass) and {device} does not have them")
-        _workspaces[device.index] = ws
+        _workspaces[key] = ws
     return ws
 
 
@@ -112,7 +114,11 @@ def release_backward_workspace(device=None):
     if device is None:
         _workspaces.clear()
     else:
-        _workspaces.pop(torch.device(device).index, None)
+        index = torch.device(device).index
+        if index is None:
+            index = torch.cuda.current_device()
+        for key in [k for k in _workspaces if k[0] == index]:
+            del _workspaces[key]
 
 
 def corope_gqa_backward(q, k, v, grad_output, sm_scale, theta, workspace=None, out=None):
@@ -120,7 +126,7 @@ def corope_gqa_backward(q, k, v, grad_output, sm_scale, theta, workspace=None, o
 
     ``workspace`` may be a caller-owned uint8/float tensor of at least ``backward_min_workspace_bytes`` bytes (the groups
     are then processed in passes of as many as fit; ``backward_workspace_bytes`` holds them all); without one a buffer
-    cached per device is used (``BACKWARD_WORKSPACE_CAP_BYTES``, ``release_backward_workspace``); ``out`` the
+    cached per device and stream is used (``BACKWARD_WORKSPACE_CAP_BYTES``, ``release_backward_workspace``); ``out`` the
     forward's output for the same inputs (optional: it only steadies the rounding of dQ on sharply peaked rows)."""
     lib = _lib.load()
     B, Hq, N, D = q.shape

@@ -156,24 +156,25 @@ def test_corope_backward_caller_workspace_and_reuse(pkg):
 
 
 def test_corope_backward_keeps_its_own_workspace_between_calls(pkg, monkeypatch):
-    """Without a caller's workspace the operator uses one buffer per device, sized by the shape and a cap alone: the second
+    """Without a caller's workspace the operator uses one buffer per device and stream, sized by the shape and a cap alone: the second
     call allocates nothing new, a smaller cap walks the groups in passes with the same gradients, release frees it."""
     mod = pkg.corope_gqa
     dev = torch.device("cuda:0")
     B, Hq, Hkv, N, D = 2, 6, 3, 70, 64
     q, k, v, d_o = (t.to(dev, torch.bfloat16) for t in _inputs(B, Hq, Hkv, N, D, seed=5))
     mod.release_backward_workspace()
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
     a = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4)
-    ws = mod._workspaces[dev.index]
+    ws = mod._workspaces[key]
     assert ws.numel() == mod.backward_workspace_bytes(B, Hq, Hkv, N, D)
     b = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4)
-    assert mod._workspaces[dev.index].data_ptr() == ws.data_ptr()
+    assert mod._workspaces[key].data_ptr() == ws.data_ptr() and len(mod._workspaces) == 1
     one = mod.backward_min_workspace_bytes(B, Hq, Hkv, N, D)
     mod.release_backward_workspace(dev)
-    assert dev.index not in mod._workspaces
+    assert not mod._workspaces
     monkeypatch.setattr(mod, "BACKWARD_WORKSPACE_CAP_BYTES", 2 * one + 5)
     c = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4)
-    assert mod._workspaces[dev.index].numel() == 2 * one
+    assert mod._workspaces[key].numel() == 2 * one
     torch.cuda.synchronize()
     for x, y, z in zip(a, b, c):
         assert torch.equal(x, y) and torch.equal(x, z)
