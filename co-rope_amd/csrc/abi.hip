@@ -430,6 +430,11 @@ int corope_rope_attn_bwd_dkdv(const void* q, const void* k, const void* v, const
   int rc = validate_bwd("rope_attn_bwd_dkdv", B, H, N, D, freq_row_stride, sm_scale,
                         {q, k, v, d_o, lse, delta, freqs_cos, freqs_sin, dk, dv});
   if (rc) return rc;
+  if (D == 64) {   // both sets of accumulators and the rotation's table values fit a wave's registers: one launch
+    corope::BwdParams p = make_bwd(q, k, v, nullptr, d_o, lse, const_cast<float*>(delta), freqs_cos, freqs_sin,
+                                   freq_row_stride, nullptr, dk, dv, B, H, N, sm_scale);
+    return launch_status("rope_attn_bwd_dkdv", corope::launch_bwd_dkdv_fused(p, D, causal != 0, static_cast<hipStream_t>(stream)));
+  }
   rc = corope_rope_attn_bwd_dv(q, k, d_o, lse, freqs_cos, freqs_sin, freq_row_stride, dv, B, H, N, D, sm_scale, causal,
                                stream);
   if (rc) return rc;

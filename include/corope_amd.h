@@ -147,7 +147,8 @@ int corope_rope_attn_bwd_dk(const void *q, const void *k, const void *v, const v
                             void *dk,
                             int B, int H, int N, int D, float sm_scale, int causal, void *stream);
 
-/* dK and dV = corope_rope_attn_bwd_dv followed by corope_rope_attn_bwd_dk on the same stream.
+/* dK and dV: corope_rope_attn_bwd_dv followed by corope_rope_attn_bwd_dk on the same stream (head dim 64: one
+ * launch that computes both).
  * Replaces the _attn_bwd_dkdv half of _attn_bwd (reference fused-rope/fused_rope_attn.py:342-404,
  * :524-579) including the host-side K pre-scale (:746-748), which is folded into the kernels. */
 int corope_rope_attn_bwd_dkdv(const void *q, const void *k, const void *v, const void *d_o,
