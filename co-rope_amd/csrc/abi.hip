@@ -826,7 +826,6 @@ int corope_gqa_bwd_impl(const char* what, bool f16, const void* q, const void* k
   rc = check_ptrs(what, {q, k, v, d_o, dq, dk, dv, workspace});
   if (rc) return rc;
   if (o != nullptr && !aligned16(o)) return fail(COROPE_E_ALIGN, "%s: pointer %p is not 16-byte aligned", what, o);
-  if ((int64_t)B * Hq > 65535) return fail(COROPE_E_UNSUPPORTED, "%s: B * Hq = %lld exceeds 65535", what, (long long)B * Hq);
   const int64_t need = 4 * corope::corope_gqa_bwd_workspace_floats(1, Hq / Hkv, 1, N, D);
   if (workspace_bytes < need)
     return fail(COROPE_E_BADARG, "%s: workspace of %lld bytes, at least %lld needed (one group's matrices)", what,

@@ -913,7 +913,8 @@ hipError_t launch_corope_gqa_bwd(const CoropeBwdParams& p, int D, float* workspa
   }
   const int G = p.Hq / p.Hkv, n_groups = p.B * p.Hkv;
   const int64_t per_group = corope_gqa_bwd_workspace_floats(1, G, 1, p.N, D);
-  const int per_pass = (int)std::min<int64_t>(n_groups, workspace_floats / per_group);
+  // (a launch spreads the groups' heads over the third grid axis, which ends at 65535)
+  const int per_pass = (int)std::min<int64_t>(std::min<int64_t>(n_groups, 65535 / G), workspace_floats / per_group);
   if (per_pass < 1) return hipErrorInvalidValue;
   for (int g0 = 0; g0 < n_groups; g0 += per_pass) {
     const int gc = std::min(per_pass, n_groups - g0);

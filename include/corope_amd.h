@@ -318,7 +318,7 @@ int64_t corope_gqa_bwd_min_workspace_bytes(int B, int Hq, int Hkv, int N, int D)
  * Like the reference's, it needs neither the forward's output nor its row statistics; `o` may be NULL.  When the forward's output is
  * passed, rowsum(O o dO) serves as a reference value that keeps dQ accurate for rows dominated by a single key (the
  * result is mathematically the same with or without it).  The workspace need not be initialised and may be any size from
- * corope_gqa_bwd_min_workspace_bytes up (see there).  Limit: B*Hq <= 65535. */
+ * corope_gqa_bwd_min_workspace_bytes up (see there). */
 int corope_gqa_bwd(const void *q, const void *k, const void *v, const void *o, const void *d_o,
                    void *dq, void *dk, void *dv,
                    int B, int Hq, int Hkv, int N, int D, float sm_scale, float theta,

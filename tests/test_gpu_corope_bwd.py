@@ -281,3 +281,26 @@ def test_corope_backward_fp16_scaled_upstream_gradient(pkg, kexp):
         err = (a - b).abs().max()
         print(f"  {name} at dO x 2^{kexp}: max-abs {err:.3e} (bar {bar * f:.3e}, max |ref| {b.abs().max():.3e})", flush=True)
         assert torch.isfinite(a).all() and err <= bar * f, name
+
+
+def test_corope_more_heads_than_a_grid_axis(pkg):
+    """B8200 Hq8 Hkv1 N16 D64: 65600 query heads, more than the 65535 a grid axis holds; the backward walks the groups in
+    passes.  The first and the last group against the same groups run on their own."""
+    mod = pkg.corope_gqa
+    dev = torch.device("cuda:0")
+    B, Hq, Hkv, N, D = 8200, 8, 1, 16, 64
+    g = torch.Generator(device=dev).manual_seed(3)
+    q, d_o = (torch.randn((B, Hq, N, D), device=dev, dtype=torch.bfloat16, generator=g) for _ in range(2))
+    k, v = (torch.randn((B, Hkv, N, D), device=dev, dtype=torch.bfloat16, generator=g) for _ in range(2))
+    o = pkg.corope_attention(q, k, v, True, 0.125, 1e4)
+    grads = mod.corope_gqa_backward(q, k, v, d_o, 0.125, 1e4)
+    torch.cuda.synchronize()
+    for b in (0, 4100, B - 1):
+        sl = slice(b, b + 1)
+        o1 = pkg.corope_attention(q[sl], k[sl], v[sl], True, 0.125, 1e4)
+        g1 = mod.corope_gqa_backward(q[sl], k[sl], v[sl], d_o[sl], 0.125, 1e4)
+        torch.cuda.synchronize()
+        assert torch.equal(o[sl], o1), b
+        for a, r in zip(grads, g1):
+            assert torch.equal(a[sl], r), b
+    mod.release_backward_workspace()
